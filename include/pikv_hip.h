@@ -1,0 +1,329 @@
+/*
+ * pikv_hip.h - C ABI of libpikv_hip.so: the routed, compressed KV-cache data
+ * path of PiKV as hand-written gfx950 (MI355X) HIP kernels.
+ *
+ * Conventions (shared by every entry point)
+ *   - Every pointer is a DEVICE pointer unless the name ends in _host.
+ *   - Tensors are row-major and contiguous; shapes are given in the comments.
+ *   - The caller allocates every output and every workspace; no entry point
+ *     allocates, frees or synchronises.  Work is enqueued on `stream`
+ *     (a hipStream_t passed as void*; NULL = the default stream).
+ *   - Return value: PIKV_OK (0) or a negative PIKV_ERR_* code.  Nothing is
+ *     enqueued when an error is returned.  pikv_status_string() names a code.
+ *   - Deterministic: no floating-point atomics; integer outputs (expert
+ *     indices, slots, codes, eviction sets) do not depend on launch geometry.
+ *   - Every top-k in this library orders by (value, index): larger value first
+ *     (or smaller first where stated), LOWER INDEX FIRST among equal values.
+ *
+ * The reference keeps its native surface in core/cuda/ as
+ *   extern "C" void launch_<name>(ptrs..., ints..., floats..., cudaStream_t)
+ * (core/cuda/pikv_routing_kernel.cu:404-511, pikv_compression_kernel.cu:463-623,
+ * pikv_scheduling_kernel.cu:504-676) and binds it from
+ * core/single/pikv_kernels.py:36-52.  Each entry point below names the
+ * reference interface it replaces.
+ *
+ * "Cache pool" layout used by the scatter / read / evict entry points
+ *   A pool holds n_caches independent caches (one per expert, or one per
+ *   sequence) in one row space.  Cache c owns rows
+ *   [cache_row_base[c], cache_row_base[c] + cache_cap[c]) of which the first
+ *   cache_fill[c] are valid.  Per row the pool stores, in separate planes,
+ *     codes  : int8  [rows, D]        (8-bit)   or uint8 [rows, D/2] (4-bit,
+ *              two codes per byte, low nibble = even element)
+ *     scale  : float [rows, D/group]  (8-bit)   or __half [rows, D/group] (4-bit)
+ *     zero   : same shape/type as scale; only for asymmetric schemes
+ *     acc,ts : float [rows]           H2O accumulator and access timestamp
+ *   with D = n_heads * head_dim, and `group` the quantisation domain
+ *   (D = per token, head_dim = per token per head, 32 = per group of 32).
+ *   Row layout inside a plane is [head][head_dim], as the reference's
+ *   k_cache[slot, head, head_dim] (core/single/pikv_attention.py:41-48).
+ */
+#ifndef PIKV_HIP_H
+#define PIKV_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes ------------------------------------------------------ */
+#define PIKV_OK                 0
+#define PIKV_ERR_NULL          -1   /* a required pointer is NULL            */
+#define PIKV_ERR_SHAPE         -2   /* a dimension is out of range           */
+#define PIKV_ERR_UNSUPPORTED   -3   /* valid request this build cannot serve */
+#define PIKV_ERR_WORKSPACE     -4   /* workspace too small                   */
+#define PIKV_ERR_LAUNCH        -5   /* the HIP runtime refused the launch    */
+
+/* ---- element types ------------------------------------------------------ */
+#define PIKV_F32   0
+#define PIKV_BF16  1
+
+/* ---- quantisation schemes (reference formula:
+ *      core/single/module/pikv_compression.py:945-1012) -------------------- */
+#define PIKV_Q_I8_SYM    0   /* codes -128..127, float scale                 */
+#define PIKV_Q_I8_ASYM   1   /* codes 0..255,    float scale + float zero    */
+#define PIKV_Q_I4_ASYM   2   /* codes 0..15,     half scale + half zero      */
+#define PIKV_Q_I4_SYM    3   /* codes -8..7,     half scale                  */
+
+/* ---- eviction policies (core/single/cache_scheduling.py:9-17) ----------- */
+#define PIKV_EVICT_H2O   0
+#define PIKV_EVICT_LRU   1
+
+const char* pikv_status_string(int status);
+
+/* Library/ABI version: major*1000 + minor. */
+int pikv_abi_version(void);
+
+/* ------------------------------------------------------------------------
+ * K1  fused router
+ * Replaces: BaseRouter.forward's tail - last nn.Linear of the gate, mask,
+ *   softmax, top-k, renormalise, capacity slots
+ *   (core/single/pikv_routing.py:65-82; capacity rule
+ *   core/single/module/pikv_routing.py:62-106); EPLBRouter's temperature and
+ *   expert_weights scaling (core/single/pikv_routing.py:653-660); native
+ *   precedents launch_adaptive_routing_kernel / launch_topk_routing_kernel /
+ *   launch_expert_capacity_kernel (core/cuda/pikv_routing_kernel.cu:404-511).
+ *
+ *   logits[t,e] = sum_h x[t,h]*w[e,h] + bias[e]          (fp32 accumulate)
+ *   logits     /= temperature            (if temperature != 1; true division)
+ *   logits     *= expert_scale[e]        (if expert_scale != NULL)
+ *   logits     += (1-expert_mask[e])*-1e9 (if expert_mask != NULL)
+ *   probs       = softmax_e(logits)
+ *   topk_idx    = k largest logits, (value desc, index asc)
+ *   topk_w      = probs[topk_idx] / (sum_j probs[topk_idx[j]] + renorm_eps)
+ *   slot[t,j]   = number of assignments (t',j') < (t,j) in token-major order
+ *                 with the same expert; -1 when that count >= capacity
+ *   count[e]    = number of assignments to e (kept or not)
+ *
+ *   x        [T,H]  x_dtype (PIKV_F32|PIKV_BF16)   w [E,H] same dtype
+ *   bias     [E] float or NULL        expert_scale, expert_mask [E] float|NULL
+ *   probs    [T,E] float or NULL      logits_out [T,E] float or NULL
+ *   topk_idx [T,k] int32              topk_w [T,k] float
+ *   slot     [T,k] int32 or NULL (then capacity/count/workspace are unused)
+ *   count    [E] int32 or NULL
+ *   1 <= E <= 64, 1 <= k <= min(E,8), H % 8 == 0
+ *   workspace: pikv_router_workspace_bytes(T,E,k) bytes, 256-byte aligned.
+ * ---------------------------------------------------------------------- */
+int pikv_router_fused(const void* x, const void* w, int x_dtype,
+                      const float* bias, const float* expert_scale,
+                      const float* expert_mask, float temperature,
+                      float renorm_eps,
+                      int64_t T, int H, int E, int k, int64_t capacity,
+                      float* probs, float* logits_out,
+                      int32_t* topk_idx, float* topk_w,
+                      int32_t* slot, int32_t* count,
+                      void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Router tail on precomputed logits.
+ * Replaces: PiKVRouter.forward's importance-gated blend of two gates,
+ *   cache_correction_factor and everything after
+ *   (core/single/pikv_routing.py:450-470), and PiKVKernels.top_k_routing
+ *   (core/single/pikv_kernels.py:54-99; use_softmax = 0 gives the raw top-k
+ *   of the logits that its fallback computes).
+ *   logits_b and select are optional: row t uses logits_a when
+ *   select[t] != 0 (or select == NULL) else logits_b.
+ *   With use_softmax = 0, probs is not written and topk_w holds the selected
+ *   logits themselves (no renormalisation).
+ *   Other arguments as in pikv_router_fused.
+ * ---------------------------------------------------------------------- */
+int pikv_router_tail(const float* logits_a, const float* logits_b,
+                     const uint8_t* select,
+                     const float* expert_scale, const float* expert_mask,
+                     float temperature, float renorm_eps, int use_softmax,
+                     int64_t T, int E, int k, int64_t capacity,
+                     float* probs, int32_t* topk_idx, float* topk_w,
+                     int32_t* slot, int32_t* count,
+                     void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Capacity slots alone, from expert indices in token-major order.
+ * Replaces: _create_dispatch_combine_tensors' sequential fill
+ *   (core/single/module/pikv_routing.py:93-104) in its compact form.
+ *   expert_idx [A] int32 in [0,E); slot [A]; count [E]. */
+int pikv_capacity_slots(const int32_t* expert_idx, int64_t A, int E,
+                        int64_t capacity, int32_t* slot, int32_t* count,
+                        void* workspace, int64_t workspace_bytes, void* stream);
+
+int64_t pikv_router_workspace_bytes(int64_t T, int E, int k);
+
+/* ------------------------------------------------------------------------
+ * K2  fused KV quantise + per-cache scatter (append)
+ * Replaces: QuantizedCompressor._quantize_tensor's formula
+ *   (core/single/module/pikv_compression.py:945-1012; asymmetric form also
+ *   core/single/pikv_compression.py:396-429) applied per `group` contiguous
+ *   elements of a token row, with the integer codes KEPT, followed by
+ *   CacheSchedulingManager.update_cache's append
+ *   (core/single/cache_scheduling.py:429-436) into each routed expert's cache;
+ *   native precedents launch_quantization_compression_kernel
+ *   (core/cuda/pikv_compression_kernel.cu:490-508) and
+ *   launch_lru_cache_management_kernel (pikv_scheduling_kernel.cu:506-529).
+ *
+ *   Source row s (0 <= s < n_src) is quantised once and written to the rows
+ *   of its `fanout` assignments a = s*fanout + j:
+ *     c = cache_id[a]; if slot[a] < 0 the assignment is dropped;
+ *     r = cache_fill[c] + slot[a]; dropped when r >= cache_cap[c]
+ *     (core/single/cache_scheduling.py:431-432: rows beyond the cache are
+ *     silently truncated); pool row = cache_row_base[c] + r.
+ *   n_src = T, fanout = k      : K/V shared by a token's k experts
+ *   n_src = T*k, fanout = 1    : K/V projected per assignment
+ *   cache_fill is NOT modified here (see pikv_cache_advance).
+ *
+ *   k_src, v_src [n_src, D] src_dtype; v_src and its outputs may be NULL.
+ *   scheme       PIKV_Q_*; group: power of two, 16 <= group <= 1024 for
+ *                8-bit, 32 <= group <= 2048 for 4-bit, D % group == 0.
+ *   k_codes/v_codes, k_scale/v_scale, k_zero/v_zero: pool planes (see top);
+ *                zero planes are required for asymmetric schemes only.
+ *   row_acc,row_ts [rows] float or NULL: set to 0 and `now` for written rows.
+ * ---------------------------------------------------------------------- */
+int pikv_quant_scatter(const void* k_src, const void* v_src, int src_dtype,
+                       int64_t n_src, int fanout, int D, int group, int scheme,
+                       const int32_t* cache_id, const int32_t* slot,
+                       const int64_t* cache_row_base, const int32_t* cache_fill,
+                       const int32_t* cache_cap, int n_caches,
+                       void* k_codes, void* v_codes,
+                       void* k_scale, void* v_scale,
+                       void* k_zero, void* v_zero,
+                       float* row_acc, float* row_ts, float now,
+                       void* stream);
+
+/* cache_fill[c] = min(cache_fill[c] + min(count[c], per_call_limit), cache_cap[c])
+ * Replaces: cache_size_current.fill_(end_idx)
+ *   (core/single/cache_scheduling.py:436).  per_call_limit is the router
+ *   capacity (rows with slot >= capacity were dropped); pass a negative value
+ *   for "no limit". */
+int pikv_cache_advance(int32_t* cache_fill, const int32_t* count,
+                       const int32_t* cache_cap, int n_caches,
+                       int64_t per_call_limit, void* stream);
+
+/* Quantise rows in place order (no routing): row i of the source goes to row
+ * dst_row0 + i of the planes.  Same formula as pikv_quant_scatter; used for
+ * QuantizedCompressor.quantize() and for bulk cache prefill. */
+int pikv_quantize_rows(const void* src, int src_dtype, int64_t n_rows, int D,
+                       int group, int scheme, int64_t dst_row0,
+                       void* codes, void* scale, void* zero, void* stream);
+
+/* ------------------------------------------------------------------------
+ * K3  gather + dequantise read path, attention scores, H2O accumulation
+ * Replaces: dq = (q - zero_point) * scale
+ *   (core/single/module/pikv_compression.py:1006), attention_scores =
+ *   matmul(q, k^T)/sqrt(head_dim) and softmax(dim=-1)
+ *   (core/single/pikv_attention.py:123,163), importance = probs.sum over
+ *   queries (core/single/pikv_moe.py:241-245) and
+ *   H2OScheduler.update_attention_scores
+ *   (core/single/cache_scheduling.py:69-73); native precedent
+ *   launch_cache_access_update_kernel (pikv_scheduling_kernel.cu:616-631).
+ * ---------------------------------------------------------------------- */
+
+/* out[i,:] = dequant(row rows[i]) (rows == NULL: row row0 + i).
+ * out [n, D] out_dtype (PIKV_F32 | PIKV_BF16, round-to-nearest-even). */
+int pikv_gather_dequant(const void* codes, const void* scale, const void* zero,
+                        int D, int group, int scheme,
+                        const int64_t* rows, int64_t row0, int64_t n,
+                        void* out, int out_dtype, void* stream);
+
+/* For every cache c and query head h (kv head g = h / (n_q_heads/n_kv_heads)):
+ *   scores[c,h,n] = dot(q[c,h,:], dequant(K[row_base[c]+n, g, :])) * scale_qk
+ *   for n < cache_fill[c]; entries n >= cache_fill[c] are not written.
+ *   q       [n_caches, n_q_heads, head_dim] q_dtype
+ *   scores  [n_caches, n_q_heads, score_stride] float
+ *   tile_max, tile_sum [n_caches, n_q_heads, n_tiles] float: per tile of
+ *   PIKV_SCORE_TILE cached tokens, max score and sum of exp(score - max);
+ *   n_tiles = ceil(max_len / PIKV_SCORE_TILE) with max_len <= score_stride
+ *   the largest cache_fill the caller wants covered.
+ *   D = n_kv_heads*head_dim; head_dim in {64,128}; group divides head_dim or
+ *   equals it. */
+#define PIKV_SCORE_TILE 64
+int pikv_gather_dequant_scores(const void* k_codes, const void* k_scale,
+                               const void* k_zero, int scheme, int group,
+                               int n_kv_heads, int n_q_heads, int head_dim,
+                               const void* q, int q_dtype, float scale_qk,
+                               const int64_t* cache_row_base,
+                               const int32_t* cache_fill, int n_caches,
+                               int64_t max_len, int64_t score_stride,
+                               float* scores, float* tile_max, float* tile_sum,
+                               void* stream);
+
+/* Softmax-normalise the scores over each cache's valid tokens, sum the
+ * probabilities over the n_q_heads heads and fold them into the H2O state:
+ *   acc[row] = acc[row]*decay + sum_h softmax_n(scores[c,h,:])[n]
+ *   ts[row]  = now                                  (row = row_base[c]+n)
+ *   decay = 1 reproduces core/single/cache_scheduling.py:69-73; decay = 0.95
+ *   the decay-first variant (core/single/module/pikv_scheduling.py:119-130).
+ *   If write_probs != 0 scores is overwritten with the probabilities.
+ *   importance_out [n_caches, score_stride] float or NULL receives the summed
+ *   probabilities.  head_stats [n_caches, n_q_heads, 2] float workspace
+ *   (final max and 1/sum per head). */
+int pikv_h2o_accumulate(float* scores, const float* tile_max,
+                        const float* tile_sum, int n_q_heads,
+                        const int64_t* cache_row_base,
+                        const int32_t* cache_fill, int n_caches,
+                        int64_t max_len, int64_t score_stride,
+                        float decay, float now, int write_probs,
+                        float* row_acc, float* row_ts, float* importance_out,
+                        float* head_stats, void* stream);
+
+/* ------------------------------------------------------------------------
+ * K4  eviction top-k + stable in-place compaction
+ * Replaces: H2OScheduler.select_eviction_candidates
+ *   (core/single/cache_scheduling.py:75-99), LRUScheduler's
+ *   (core/single/cache_scheduling.py:262-285), and the manager's compaction
+ *   keep = where(~mask); cache[:m] = cur[keep]
+ *   (core/single/cache_scheduling.py:418-424); native precedent
+ *   launch_cache_compaction_kernel (pikv_scheduling_kernel.cu:633-654).
+ *
+ *   For each cache c with len = cache_fill[c]:
+ *     H2O: keep = top-n_heavy[c] of row_acc  UNION  top-n_recent[c] of row_ts
+ *     LRU: evict the n_evict[c] rows with the smallest row_ts
+ *          (n_heavy is read as n_evict; n_recent is ignored)
+ *   keep_flag  [rows_total] uint8  : 1 for survivors (written for n < len)
+ *   keep_index [rows_total] int32  : ascending cache-local indices of the
+ *                                    survivors, at [row_base[c] .. +new_len)
+ *   new_len    [n_caches]  int32   : number of survivors
+ *   n_heavy/n_recent are per-cache DEVICE arrays so that no host read of
+ *   cache_fill is needed; pikv_h2o_budget fills them from the ratios.
+ * ---------------------------------------------------------------------- */
+int pikv_evict_select(int policy, const float* row_acc, const float* row_ts,
+                      const int64_t* cache_row_base, const int32_t* cache_fill,
+                      const int32_t* n_heavy, const int32_t* n_recent,
+                      int n_caches, uint8_t* keep_flag, int32_t* keep_index,
+                      int32_t* new_len, void* stream);
+
+/* n_heavy[c] = max(1,int(len*heavy_ratio)); n_recent[c] = max(1,int(len*recent_ratio))
+ * with len = cache_fill[c] and the product evaluated in double precision as
+ * Python does (core/single/cache_scheduling.py:83-84). */
+int pikv_h2o_budget(const int32_t* cache_fill, int n_caches,
+                    double heavy_ratio, double recent_ratio,
+                    int32_t* n_heavy, int32_t* n_recent, void* stream);
+
+/* Move surviving rows to the front of every cache, in place and in ascending
+ * order, for up to PIKV_MAX_PLANES planes (codes, scales, zeros, acc, ts ...),
+ * then set cache_fill[c] = new_len[c].
+ *   plane_ptrs_host  [n_planes] device pointers (the ARRAY itself is on the
+ *                    host); plane_row_bytes_host [n_planes] bytes per row,
+ *                    each a multiple of 4. */
+#define PIKV_MAX_PLANES 10
+int pikv_compact_rows(void* const* plane_ptrs_host,
+                      const int64_t* plane_row_bytes_host, int n_planes,
+                      const int64_t* cache_row_base, const int32_t* keep_index,
+                      const int32_t* new_len, int32_t* cache_fill,
+                      int n_caches, void* stream);
+
+/* ------------------------------------------------------------------------
+ * API-compatible fake quantisation of QuantizedCompressor.forward
+ * Replaces: core/single/pikv_compression.py:474-506 - min/max over ALL rows
+ *   of each block of `group` columns, asymmetric, output = dequantised floats.
+ *   x, out [N,H] float; stats [H/group (rounded up), 4] float workspace/out:
+ *   (min, max, scale, zero) per column block; sq_err [ceil(H/group)] float:
+ *   mean squared error per block (the reference's quantization_error is the
+ *   value of the LAST block processed).
+ * ---------------------------------------------------------------------- */
+int pikv_fakequant_colblocks(const float* x, int64_t N, int H, int group,
+                             int bits, int symmetric, float* out,
+                             float* stats, float* sq_err,
+                             void* workspace, int64_t workspace_bytes,
+                             void* stream);
+int64_t pikv_fakequant_workspace_bytes(int64_t N, int H, int group);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PIKV_HIP_H */

@@ -1,0 +1,218 @@
+// Shared device/host helpers for the gfx950 kernels of libpikv_hip.so.
+// Wavefront width is 64 everywhere; nothing here is written for 32-wide waves.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/pikv_hip.h"
+
+#define PIKV_WAVE 64
+
+#define PIKV_CHECK_LAUNCH()                              \
+  do {                                                   \
+    if (hipGetLastError() != hipSuccess) return PIKV_ERR_LAUNCH; \
+  } while (0)
+
+namespace pikv {
+
+// ---- scalar type conversion --------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) {
+  return __uint_as_float(b << 16);
+}
+
+// float -> bf16 bits, round to nearest even (NaN kept quiet).
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+// float -> half, round to nearest even, finite values saturate at +-65504.
+__device__ __forceinline__ _Float16 float_to_half_sat(float f) {
+  if (f > 65504.0f && f < __builtin_inff()) return (_Float16)65504.0f;
+  if (f < -65504.0f && f > -__builtin_inff()) return (_Float16)(-65504.0f);
+  _Float16 h = (_Float16)f;
+  if (__builtin_isinf((float)h) && !__builtin_isinf(f))
+    h = (_Float16)(f > 0.f ? 65504.0f : -65504.0f);
+  return h;
+}
+
+// ---- 16-byte global access -----------------------------------------------------
+__device__ __forceinline__ uint4 ld16(const void* p) {
+  return *reinterpret_cast<const uint4*>(p);
+}
+__device__ __forceinline__ void st16(void* p, uint4 v) {
+  *reinterpret_cast<uint4*>(p) = v;
+}
+
+// Load N consecutive source elements (N % 8 == 0) as float.
+template <int DT, int N>
+__device__ __forceinline__ void load_as_float(const void* base, int64_t elem_off,
+                                              float (&out)[N]) {
+  if constexpr (DT == PIKV_BF16) {
+    const char* p = reinterpret_cast<const char*>(base) + elem_off * 2;
+#pragma unroll
+    for (int i = 0; i < N / 8; ++i) {
+      uint4 v = ld16(p + 16 * i);
+      uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        out[8 * i + 2 * j] = __uint_as_float(w[j] << 16);
+        out[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      }
+    }
+  } else {
+    const char* p = reinterpret_cast<const char*>(base) + elem_off * 4;
+#pragma unroll
+    for (int i = 0; i < N / 4; ++i) {
+      uint4 v = ld16(p + 16 * i);
+      out[4 * i] = __uint_as_float(v.x);
+      out[4 * i + 1] = __uint_as_float(v.y);
+      out[4 * i + 2] = __uint_as_float(v.z);
+      out[4 * i + 3] = __uint_as_float(v.w);
+    }
+  }
+}
+
+// ---- cross-lane reductions over aligned groups of LANES lanes (power of two) -----
+template <int LANES>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+  for (int m = 1; m < LANES; m <<= 1) v = fmaxf(v, __shfl_xor(v, m, PIKV_WAVE));
+  return v;
+}
+template <int LANES>
+__device__ __forceinline__ float group_min(float v) {
+#pragma unroll
+  for (int m = 1; m < LANES; m <<= 1) v = fminf(v, __shfl_xor(v, m, PIKV_WAVE));
+  return v;
+}
+template <int LANES>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int m = 1; m < LANES; m <<= 1) v += __shfl_xor(v, m, PIKV_WAVE);
+  return v;
+}
+// Runtime-width variants (width = power of two <= 64).
+__device__ __forceinline__ float group_max_rt(float v, int width) {
+  for (int m = 1; m < width; m <<= 1) v = fmaxf(v, __shfl_xor(v, m, PIKV_WAVE));
+  return v;
+}
+__device__ __forceinline__ float group_min_rt(float v, int width) {
+  for (int m = 1; m < width; m <<= 1) v = fminf(v, __shfl_xor(v, m, PIKV_WAVE));
+  return v;
+}
+
+// ---- quantisation formula --------------------------------------------------------
+// Float32 arithmetic in the operation order of the reference's
+// QuantizedCompressor._quantize_tensor (core/single/module/pikv_compression.py:
+// 945-1012): true division, round-half-even, no reciprocal, no contraction.
+template <int SCHEME>
+struct QScheme {
+  static constexpr int bits = (SCHEME == PIKV_Q_I8_SYM || SCHEME == PIKV_Q_I8_ASYM) ? 8 : 4;
+  static constexpr bool sym = (SCHEME == PIKV_Q_I8_SYM || SCHEME == PIKV_Q_I4_SYM);
+  static constexpr int qmin = sym ? -(1 << (bits - 1)) : 0;
+  static constexpr int qmax = sym ? (1 << (bits - 1)) - 1 : (1 << bits) - 1;
+  static constexpr int epl = bits == 8 ? 16 : 32;  // elements per lane (16 code bytes)
+  static constexpr int meta_bytes = bits == 8 ? 4 : 2;
+};
+
+template <int SCHEME>
+__device__ __forceinline__ void quant_params(float mn, float mx, float& scale, float& zero) {
+  using Q = QScheme<SCHEME>;
+  if (mx == mn) mx = mn + 1e-5f;
+  const float qr = (float)(Q::qmax - Q::qmin);
+  if constexpr (Q::sym) {
+    float amax = fmaxf(fabsf(mn), fabsf(mx));
+    scale = (2.0f * amax) / qr;
+  } else {
+    scale = (mx - mn) / qr;
+  }
+  if constexpr (Q::bits == 4) scale = (float)float_to_half_sat(scale);
+  if constexpr (Q::sym) {
+    zero = 0.0f;
+  } else {
+    zero = (float)Q::qmin - rintf(mn / scale);
+    if constexpr (Q::bits == 4) zero = (float)float_to_half_sat(zero);
+  }
+}
+
+template <int SCHEME>
+__device__ __forceinline__ int quant_code(float x, float scale, float zero) {
+  using Q = QScheme<SCHEME>;
+  float y = x / scale;
+  y = y + zero;
+  y = rintf(y);
+  // NaN (0/0 from a zero scale) maps to qmin, as the CPU restatement does.
+  y = (y != y) ? (float)Q::qmin : y;
+  y = fminf(fmaxf(y, (float)Q::qmin), (float)Q::qmax);
+  return (int)y;
+}
+
+// Pack the codes of one lane (16 x 8-bit or 32 x 4-bit) into 16 bytes.
+template <int SCHEME>
+__device__ __forceinline__ uint4 pack_codes(const int* c) {
+  using Q = QScheme<SCHEME>;
+  uint32_t w[4];
+  if constexpr (Q::bits == 8) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      w[i] = (uint32_t)(c[4 * i] & 0xff) | ((uint32_t)(c[4 * i + 1] & 0xff) << 8) |
+             ((uint32_t)(c[4 * i + 2] & 0xff) << 16) | ((uint32_t)(c[4 * i + 3] & 0xff) << 24);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint32_t v = 0;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v |= (uint32_t)(c[8 * i + j] & 0xf) << (4 * j);
+      w[i] = v;
+    }
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// Unpack 16 bytes of codes into integers (sign-extended for symmetric schemes).
+template <int SCHEME>
+__device__ __forceinline__ void unpack_codes(uint4 v, int* c) {
+  using Q = QScheme<SCHEME>;
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  if constexpr (Q::bits == 8) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t b = (w[i] >> (8 * j)) & 0xff;
+        c[4 * i + j] = Q::sym ? (int)(int8_t)b : (int)b;
+      }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        int b = (int)((w[i] >> (4 * j)) & 0xf);
+        c[8 * i + j] = Q::sym ? ((b ^ 8) - 8) : b;
+      }
+  }
+}
+
+// Metadata (scale / zero) element access: float for 8-bit, half for 4-bit.
+template <int SCHEME>
+__device__ __forceinline__ void store_meta(void* plane, int64_t idx, float v) {
+  if constexpr (QScheme<SCHEME>::bits == 8)
+    reinterpret_cast<float*>(plane)[idx] = v;
+  else
+    reinterpret_cast<_Float16*>(plane)[idx] = (_Float16)v;  // exact: already half-valued
+}
+template <int SCHEME>
+__device__ __forceinline__ float load_meta(const void* plane, int64_t idx) {
+  if constexpr (QScheme<SCHEME>::bits == 8)
+    return reinterpret_cast<const float*>(plane)[idx];
+  else
+    return (float)reinterpret_cast<const _Float16*>(plane)[idx];
+}
+
+__host__ __device__ inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+
+}  // namespace pikv

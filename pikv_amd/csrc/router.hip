@@ -1,0 +1,397 @@
+// K1: fused router - gate projection, logit scaling/mask, softmax, top-k,
+// renormalisation - and the capacity-slot pass.
+//
+// Gate projection (skinny: E <= 64 outputs per token, HBM-bound for small E):
+// a wavefront owns a tile of TPW = 64/EPAD tokens (EPAD = E rounded up to
+// 8/16/32/64).  Lanes stride the hidden dimension with 128-bit loads; every lane
+// keeps TPW*EPAD = 64 partial sums, so a slice of W fetched once (from L2) is
+// used for all TPW tokens.  The 64 partial-sum vectors are then reduced with a
+// 63-shuffle transpose-reduction that leaves lane l holding the finished logit of
+// (token l / EPAD, expert l % EPAD): each token's experts sit in EPAD adjacent
+// lanes and the whole tail (softmax, k rounds of arg-max with lowest-index
+// tie-break via ballot, renormalisation) runs on those lane groups without LDS.
+//
+// Capacity slots: deterministic three-step histogram / scan / rank over the
+// assignments in token-major order (integer LDS atomics only feed counts, whose
+// value does not depend on arrival order).
+#include "common.hpp"
+
+namespace pikv {
+
+constexpr int kSlotChunk = 2048;  // assignments per block in the slot pass
+
+struct TailParams {
+  const float* bias;
+  const float* expert_scale;
+  const float* expert_mask;
+  float temperature;
+  float renorm_eps;
+  int use_softmax;
+  int E;
+  int k;
+  int64_t T;
+  float* probs;
+  float* logits_out;
+  int32_t* topk_idx;
+  float* topk_w;
+};
+
+// 64 values per lane -> lane l ends with the wave-wide sum of v[l].  Each step
+// halves the live values: a lane keeps the half selected by one bit of its lane
+// id and receives the partner's partial sums for that half.
+template <int HALF>
+__device__ __forceinline__ void transpose_reduce_step(float (&v)[64], int lane) {
+  const bool up = (lane & HALF) != 0;
+#pragma unroll
+  for (int i = 0; i < HALF; ++i) {
+    const float keep = up ? v[i + HALF] : v[i];
+    const float send = up ? v[i] : v[i + HALF];
+    v[i] = keep + __shfl_xor(send, HALF, PIKV_WAVE);
+  }
+}
+__device__ __forceinline__ float wave_transpose_reduce(float (&v)[64], int lane) {
+  transpose_reduce_step<32>(v, lane);
+  transpose_reduce_step<16>(v, lane);
+  transpose_reduce_step<8>(v, lane);
+  transpose_reduce_step<4>(v, lane);
+  transpose_reduce_step<2>(v, lane);
+  transpose_reduce_step<1>(v, lane);
+  return v[0];
+}
+
+// Lane holds the raw logit of (token t, expert e); groups of EPAD adjacent lanes
+// form one token.  Writes probs / top-k for the token.
+template <int EPAD>
+__device__ __forceinline__ void router_tail_lanes(float lg, int64_t t, int e, int lane,
+                                                  const TailParams& p) {
+  const bool valid = (t < p.T) && (e < p.E);
+  if (valid) {
+    if (p.bias) lg = lg + p.bias[e];
+    if (p.temperature != 1.0f) lg = lg / p.temperature;
+    if (p.expert_scale) lg = lg * p.expert_scale[e];
+    if (p.expert_mask) {
+      const float pen = (1.0f - p.expert_mask[e]) * -1e9f;
+      lg = lg + pen;
+    }
+    if (p.logits_out) p.logits_out[t * p.E + e] = lg;
+  } else {
+    lg = -__builtin_inff();
+  }
+  float prob = 0.f;
+  if (p.use_softmax) {
+    const float m = group_max<EPAD>(lg);
+    const float ex = valid ? expf(lg - m) : 0.f;
+    const float sum = group_sum<EPAD>(ex);
+    prob = ex / sum;
+    if (valid && p.probs) p.probs[t * p.E + e] = prob;
+  }
+  const float carried = p.use_softmax ? prob : lg;
+
+  const int gstart = lane & ~(EPAD - 1);
+  const uint64_t gmask = (EPAD == 64) ? ~0ull : (((1ull << EPAD) - 1ull) << gstart);
+  bool remaining = valid;
+  int my_idx = 0;
+  float my_val = 0.f;
+  for (int j = 0; j < p.k; ++j) {
+    const float key = remaining ? lg : -__builtin_inff();
+    const float mx = group_max<EPAD>(key);
+    uint64_t cand = __ballot(remaining && key == mx) & gmask;
+    if (cand == 0) cand = __ballot(remaining) & gmask;  // only NaNs left
+    int win = e;  // padding tokens (no candidates at all) stay harmless
+    if (cand != 0) win = (int)__builtin_ctzll(cand) - gstart;
+    const float wv = __shfl(carried, gstart + win, PIKV_WAVE);
+    if (e == j) {
+      my_idx = win;
+      my_val = wv;
+    }
+    if (e == win) remaining = false;
+  }
+  if (p.use_softmax) {
+    float s = 0.f;
+    for (int j = 0; j < p.k; ++j) s = s + __shfl(my_val, gstart + j, PIKV_WAVE);
+    if (p.renorm_eps != 0.f) s = s + p.renorm_eps;
+    my_val = my_val / s;
+  }
+  if (t < p.T && e < p.k) {
+    p.topk_idx[t * p.k + e] = my_idx;
+    p.topk_w[t * p.k + e] = my_val;
+  }
+}
+
+template <int EPAD, int DT>
+__global__ __launch_bounds__(256) void router_gate_kernel(const void* __restrict__ x,
+                                                          const void* __restrict__ w, int H,
+                                                          TailParams p) {
+  constexpr int TPW = 64 / EPAD;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t tile = (int64_t)blockIdx.x * 4 + wave;
+  const int64_t tok0 = tile * TPW;
+  if (tok0 >= p.T) return;  // whole wavefront leaves together
+
+  float acc[64];
+#pragma unroll
+  for (int i = 0; i < 64; ++i) acc[i] = 0.f;
+
+  for (int h0 = 0; h0 < H; h0 += 512) {
+    const int h = h0 + lane * 8;
+    if (h < H) {
+      float xs[TPW][8];
+#pragma unroll
+      for (int t = 0; t < TPW; ++t) {
+        if (tok0 + t < p.T) {
+          load_as_float<DT, 8>(x, (tok0 + t) * H + h, xs[t]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) xs[t][i] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < EPAD; ++e) {
+        if (e < p.E) {
+          float we[8];
+          load_as_float<DT, 8>(w, (int64_t)e * H + h, we);
+#pragma unroll
+          for (int t = 0; t < TPW; ++t)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[t * EPAD + e] = fmaf(xs[t][i], we[i], acc[t * EPAD + e]);
+        }
+      }
+    }
+  }
+  const float lg = wave_transpose_reduce(acc, lane);
+  router_tail_lanes<EPAD>(lg, tok0 + lane / EPAD, lane % EPAD, lane, p);
+}
+
+template <int EPAD>
+__global__ __launch_bounds__(256) void router_tail_kernel(const float* __restrict__ la,
+                                                          const float* __restrict__ lb,
+                                                          const uint8_t* __restrict__ select,
+                                                          TailParams p) {
+  constexpr int TPW = 64 / EPAD;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t tile = (int64_t)blockIdx.x * 4 + wave;
+  const int64_t t = tile * TPW + lane / EPAD;
+  const int e = lane % EPAD;
+  if (tile * TPW >= p.T) return;
+  float lg = 0.f;
+  if (t < p.T && e < p.E) {
+    const bool use_a = (lb == nullptr) || (select == nullptr) || (select[t] != 0);
+    lg = use_a ? la[t * p.E + e] : lb[t * p.E + e];
+  }
+  router_tail_lanes<EPAD>(lg, t, e, lane, p);
+}
+
+// ---- capacity slots -------------------------------------------------------------
+__global__ __launch_bounds__(256) void slot_hist_kernel(const int32_t* __restrict__ idx, int64_t A,
+                                                        int E, int32_t* __restrict__ ws) {
+  __shared__ int hist[64];
+  if (threadIdx.x < 64) hist[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t base = (int64_t)blockIdx.x * kSlotChunk;
+  for (int i = threadIdx.x; i < kSlotChunk; i += 256) {
+    const int64_t a = base + i;
+    if (a < A) {
+      const int e = idx[a];
+      if ((unsigned)e < (unsigned)E) atomicAdd(&hist[e], 1);
+    }
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < E) ws[(int64_t)blockIdx.x * E + threadIdx.x] = hist[threadIdx.x];
+}
+
+// One thread per expert: exclusive scan of the per-chunk histograms, in place.
+__global__ void slot_scan_kernel(int32_t* __restrict__ ws, int64_t n_chunks, int E,
+                                 int32_t* __restrict__ count) {
+  const int e = threadIdx.x;
+  if (e >= E) return;
+  int run = 0;
+  for (int64_t b = 0; b < n_chunks; ++b) {
+    const int v = ws[b * E + e];
+    ws[b * E + e] = run;
+    run += v;
+  }
+  if (count) count[e] = run;
+}
+
+__global__ __launch_bounds__(256) void slot_rank_kernel(const int32_t* __restrict__ idx, int64_t A,
+                                                        int E, int64_t capacity,
+                                                        const int32_t* __restrict__ ws,
+                                                        int32_t* __restrict__ slot) {
+  __shared__ int running[64];
+  __shared__ int wcnt[4][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  if ((int)threadIdx.x < 64)
+    running[threadIdx.x] = ((int)threadIdx.x < E) ? ws[(int64_t)blockIdx.x * E + threadIdx.x] : 0;
+  const int64_t base = (int64_t)blockIdx.x * kSlotChunk;
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int step = 0; step < kSlotChunk / 256; ++step) {
+    wcnt[wave][lane] = 0;
+    __syncthreads();
+    const int64_t a = base + step * 256 + threadIdx.x;
+    int e = -1;
+    if (a < A) {
+      e = idx[a];
+      if ((unsigned)e >= (unsigned)E) e = -1;  // out-of-range ids get slot -1
+    }
+    const bool valid = e >= 0;
+    int rank = 0;
+    uint64_t todo = __ballot(valid);
+    while (todo) {
+      const int leader = (int)__builtin_ctzll(todo);
+      const int e0 = __shfl(e, leader, PIKV_WAVE);
+      const uint64_t m = __ballot(valid && e == e0);
+      if (valid && e == e0) rank = __popcll(m & lt_mask);
+      if (lane == leader) wcnt[wave][e0] = __popcll(m);
+      todo &= ~m;
+    }
+    __syncthreads();
+    if (valid) {
+      int pos = running[e] + rank;
+      for (int w2 = 0; w2 < wave; ++w2) pos += wcnt[w2][e];
+      slot[a] = ((int64_t)pos < capacity) ? pos : -1;
+    } else if (a < A) {
+      slot[a] = -1;
+    }
+    __syncthreads();
+    if (threadIdx.x < 64)
+      running[threadIdx.x] += wcnt[0][threadIdx.x] + wcnt[1][threadIdx.x] + wcnt[2][threadIdx.x] +
+                              wcnt[3][threadIdx.x];
+    __syncthreads();
+  }
+}
+
+static int64_t slot_chunks(int64_t A) { return (A + kSlotChunk - 1) / kSlotChunk; }
+
+static int64_t slot_workspace_bytes(int64_t A, int E) {
+  int64_t b = slot_chunks(A) * E * (int64_t)sizeof(int32_t);
+  return (b + 255) / 256 * 256;
+}
+
+static int launch_slots(const int32_t* idx, int64_t A, int E, int64_t capacity, int32_t* slot,
+                        int32_t* count, void* ws, int64_t ws_bytes, hipStream_t st) {
+  if (A == 0) {
+    if (count) {
+      // count must still be defined: scan over zero chunks writes zeros.
+      hipLaunchKernelGGL(slot_scan_kernel, dim3(1), dim3(64), 0, st, (int32_t*)ws, (int64_t)0, E, count);
+      PIKV_CHECK_LAUNCH();
+    }
+    return PIKV_OK;
+  }
+  if (!ws) return PIKV_ERR_NULL;
+  if (ws_bytes < slot_workspace_bytes(A, E)) return PIKV_ERR_WORKSPACE;
+  const int64_t nb = slot_chunks(A);
+  if (nb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+  hipLaunchKernelGGL(slot_hist_kernel, dim3((unsigned)nb), dim3(256), 0, st, idx, A, E, (int32_t*)ws);
+  hipLaunchKernelGGL(slot_scan_kernel, dim3(1), dim3(64), 0, st, (int32_t*)ws, nb, E, count);
+  hipLaunchKernelGGL(slot_rank_kernel, dim3((unsigned)nb), dim3(256), 0, st, idx, A, E, capacity,
+                     (const int32_t*)ws, slot);
+  PIKV_CHECK_LAUNCH();
+  return PIKV_OK;
+}
+
+static int epad_of(int E) { return E <= 8 ? 8 : E <= 16 ? 16 : E <= 32 ? 32 : 64; }
+
+template <int DT>
+static void launch_gate(int epad, unsigned blocks, hipStream_t st, const void* x, const void* w,
+                        int H, const TailParams& p) {
+  switch (epad) {
+    case 8: hipLaunchKernelGGL((router_gate_kernel<8, DT>), dim3(blocks), dim3(256), 0, st, x, w, H, p); break;
+    case 16: hipLaunchKernelGGL((router_gate_kernel<16, DT>), dim3(blocks), dim3(256), 0, st, x, w, H, p); break;
+    case 32: hipLaunchKernelGGL((router_gate_kernel<32, DT>), dim3(blocks), dim3(256), 0, st, x, w, H, p); break;
+    default: hipLaunchKernelGGL((router_gate_kernel<64, DT>), dim3(blocks), dim3(256), 0, st, x, w, H, p); break;
+  }
+}
+
+}  // namespace pikv
+
+using namespace pikv;
+
+extern "C" int64_t pikv_router_workspace_bytes(int64_t T, int E, int k) {
+  if (T < 0 || E < 1 || k < 1) return 0;
+  return slot_workspace_bytes(T * k, E);
+}
+
+extern "C" int pikv_capacity_slots(const int32_t* expert_idx, int64_t A, int E, int64_t capacity,
+                                   int32_t* slot, int32_t* count, void* workspace,
+                                   int64_t workspace_bytes, void* stream) {
+  if (!expert_idx || !slot) return PIKV_ERR_NULL;
+  if (A < 0 || A > 0x7fffffffLL || E < 1 || E > 64 || capacity < 0) return PIKV_ERR_SHAPE;
+  return launch_slots(expert_idx, A, E, capacity, slot, count, workspace, workspace_bytes,
+                      (hipStream_t)stream);
+}
+
+static int check_router_dims(int64_t T, int E, int k, int64_t capacity) {
+  if (T < 0 || E < 1 || E > 64 || k < 1 || k > 8 || k > E || capacity < 0) return PIKV_ERR_SHAPE;
+  if (T * k > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+  return PIKV_OK;
+}
+
+extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, const float* bias,
+                                 const float* expert_scale, const float* expert_mask,
+                                 float temperature, float renorm_eps, int64_t T, int H, int E,
+                                 int k, int64_t capacity, float* probs, float* logits_out,
+                                 int32_t* topk_idx, float* topk_w, int32_t* slot, int32_t* count,
+                                 void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!x || !w || !topk_idx || !topk_w) return PIKV_ERR_NULL;
+  if (x_dtype != PIKV_F32 && x_dtype != PIKV_BF16) return PIKV_ERR_UNSUPPORTED;
+  int rc = check_router_dims(T, E, k, capacity);
+  if (rc != PIKV_OK) return rc;
+  if (H < 8) return PIKV_ERR_SHAPE;
+  if (H % 8 != 0) return PIKV_ERR_UNSUPPORTED;
+  if (slot) {
+    if (!workspace && T > 0) return PIKV_ERR_NULL;
+    if (workspace_bytes < slot_workspace_bytes(T * k, E)) return PIKV_ERR_WORKSPACE;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (T > 0) {
+    TailParams p{bias, expert_scale, expert_mask, temperature, renorm_eps, 1, E, k, T,
+                 probs, logits_out, topk_idx, topk_w};
+    const int epad = epad_of(E);
+    const int64_t tiles = (T + (64 / epad) - 1) / (64 / epad);
+    const int64_t blocks = (tiles + 3) / 4;
+    if (blocks > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+    if (x_dtype == PIKV_BF16)
+      launch_gate<PIKV_BF16>(epad, (unsigned)blocks, st, x, w, H, p);
+    else
+      launch_gate<PIKV_F32>(epad, (unsigned)blocks, st, x, w, H, p);
+    PIKV_CHECK_LAUNCH();
+  }
+  if (slot) return launch_slots(topk_idx, T * k, E, capacity, slot, count, workspace, workspace_bytes, st);
+  return PIKV_OK;
+}
+
+extern "C" int pikv_router_tail(const float* logits_a, const float* logits_b, const uint8_t* select,
+                                const float* expert_scale, const float* expert_mask,
+                                float temperature, float renorm_eps, int use_softmax, int64_t T,
+                                int E, int k, int64_t capacity, float* probs, int32_t* topk_idx,
+                                float* topk_w, int32_t* slot, int32_t* count, void* workspace,
+                                int64_t workspace_bytes, void* stream) {
+  if (!logits_a || !topk_idx || !topk_w) return PIKV_ERR_NULL;
+  int rc = check_router_dims(T, E, k, capacity);
+  if (rc != PIKV_OK) return rc;
+  if (slot) {
+    if (!workspace && T > 0) return PIKV_ERR_NULL;
+    if (workspace_bytes < slot_workspace_bytes(T * k, E)) return PIKV_ERR_WORKSPACE;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (T > 0) {
+    TailParams p{nullptr, expert_scale, expert_mask, temperature, renorm_eps, use_softmax ? 1 : 0,
+                 E, k, T, use_softmax ? probs : nullptr, nullptr, topk_idx, topk_w};
+    const int epad = epad_of(E);
+    const int64_t tiles = (T + (64 / epad) - 1) / (64 / epad);
+    const int64_t blocks = (tiles + 3) / 4;
+    if (blocks > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+    switch (epad) {
+      case 8: hipLaunchKernelGGL((router_tail_kernel<8>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p); break;
+      case 16: hipLaunchKernelGGL((router_tail_kernel<16>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p); break;
+      case 32: hipLaunchKernelGGL((router_tail_kernel<32>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p); break;
+      default: hipLaunchKernelGGL((router_tail_kernel<64>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p); break;
+    }
+    PIKV_CHECK_LAUNCH();
+  }
+  if (slot) return launch_slots(topk_idx, T * k, E, capacity, slot, count, workspace, workspace_bytes, st);
+  return PIKV_OK;
+}

@@ -1,0 +1,190 @@
+"""GPU parity: K3 (scores over the compressed cache, softmax statistics, H2O
+accumulation) and K4 (eviction top-k, stable in-place compaction) through the
+C ABI against the numpy restatement.
+
+Scores and importance are float results: tolerance 1e-3 relative to the
+root-mean-square score of the row (float32 path; the bound stated for this
+path), checked against a float64 evaluation of the same formula on the same
+dequantised codes.  Eviction sets, survivor order, compacted bytes and fill
+counts are bit-exact, ties broken towards the lower index."""
+import numpy as np
+import pytest
+
+import pikv_oracle as O
+from util import codes_np, kv_like, np_of, rng, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
+    """Build a device pool and its numpy mirror with lens[c] rows in cache c."""
+    import torch
+    from pikv_amd import ops
+    D = heads * dh
+    pool = ops.CachePool(caps, heads, dh, group, scheme, dev)
+    ref = O.CachePool(caps, D, group, scheme)
+    n = int(sum(lens))
+    ks, vs = kv_like(r, n, D, dtype=dtype), kv_like(r, n, D, dtype=dtype)
+    cid = np.concatenate([np.full(l, c, dtype=np.int32) for c, l in enumerate(lens)])
+    slot = np.concatenate([np.arange(l, dtype=np.int32) for l in lens])
+    pool.quant_scatter(to_dev(ks, dev, dtype), to_dev(vs, dev, dtype), to_dev(cid, dev),
+                       to_dev(slot, dev), 1, now=0.0)
+    cnt = np.array(lens, dtype=np.int32)
+    pool.advance(to_dev(cnt, dev))
+    ref.quant_scatter(ks, vs, cid, slot, 1, now=0.0)
+    ref.advance(cnt)
+    assert np.array_equal(np_of(pool.fill), ref.fill)
+    return pool, ref
+
+
+@pytest.mark.parametrize("scheme,group,heads,hq,dh", [
+    (O.Q_I4_ASYM, 32, 8, 32, 128),     # decode read path shape (GQA 4:1)
+    (O.Q_I8_SYM, 128, 4, 4, 128),      # int8 per token per head, MHA
+    (O.Q_I8_SYM, 256, 4, 8, 64),       # per-token scale
+    (O.Q_I8_ASYM, 64, 2, 16, 64),
+    (O.Q_I4_SYM, 64, 4, 4, 64),
+])
+@pytest.mark.parametrize("qdtype", ["f32", "bf16"])
+def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
+    r = rng(scheme * 7 + heads)
+    caps = [300, 64, 130, 10]
+    lens = [257, 64, 1, 0]            # ragged: partial tile, full tile, single row, empty
+    pool, ref = _fill_pool(dev, r, caps, lens, heads, dh, group, scheme)
+    q = r.standard_normal((len(caps), hq, dh)).astype(np.float32)
+    if qdtype == "bf16":
+        q = O.bf16_round(q)
+    scale_qk = 1.0 / np.sqrt(dh)
+    scores, tmax, tsum = pool.scores(to_dev(q, dev, qdtype), hq)
+    sc = np_of(scores)
+    imp_ref_all = []
+    for c, L in enumerate(lens):
+        if L == 0:
+            continue
+        rows = ref.valid_rows(c)
+        k_hat = O.dequantize_groups(ref.k_codes[rows], ref.k_scale[rows], ref.k_zero[rows], group)
+        s_ref = O.attention_scores(q[c], k_hat, heads, scale_qk)
+        rms = np.sqrt((s_ref.astype(np.float64) ** 2).mean()) + 1e-12
+        assert np.abs(sc[c, :, :L] - s_ref).max() <= 1e-3 * rms, (c, np.abs(sc[c, :, :L] - s_ref).max(), rms)
+        imp_ref_all.append((c, rows, O.h2o_importance(s_ref)))
+    # accumulate twice (second time with decay) and compare the running state
+    acc_ref, ts_ref = ref.acc.copy(), ref.ts.copy()
+    imp = pool.h2o_accumulate(scores, tmax, tsum, now=5.0, return_importance=True)
+    for c, rows, (p_ref, i_ref) in imp_ref_all:
+        O.h2o_accumulate(acc_ref, ts_ref, rows, i_ref, 5.0)
+        assert np.allclose(np_of(imp)[c, :len(rows)], i_ref, rtol=1e-3, atol=1e-6)
+        assert abs(np_of(imp)[c, :len(rows)].sum() - hq) < 1e-3 * hq
+    assert np.allclose(np_of(pool.acc), acc_ref, rtol=1e-3, atol=1e-6)
+    assert np.array_equal(np_of(pool.ts), ts_ref)
+    scores2, tmax2, tsum2 = pool.scores(to_dev(q, dev, qdtype), hq)
+    pool.h2o_accumulate(scores2, tmax2, tsum2, now=6.0, decay=0.95, write_probs=True)
+    for c, rows, (p_ref, i_ref) in imp_ref_all:
+        O.h2o_accumulate(acc_ref, ts_ref, rows, i_ref, 6.0, decay=0.95)
+        assert np.allclose(np_of(scores2)[c, :, :len(rows)], p_ref, rtol=1e-3, atol=1e-7)
+    assert np.allclose(np_of(pool.acc), acc_ref, rtol=1e-3, atol=1e-6)
+    assert np.array_equal(np_of(pool.ts), ts_ref)
+
+
+def _set_state(pool, ref, r, ties):
+    """Random accumulators / timestamps (with many exact ties when asked)."""
+    acc = r.random(pool.rows).astype(np.float32)
+    ts = r.integers(0, 50, pool.rows).astype(np.float32)
+    if ties:
+        acc = np.round(acc * 8) / 8
+        acc[::7] = 0.0
+        acc[3::11] = -0.0
+    ref.acc[:], ref.ts[:] = acc, ts
+    pool.acc.copy_(to_dev(acc, pool.device))
+    pool.ts.copy_(to_dev(ts, pool.device))
+
+
+def _check_compacted(pool, ref, scheme, keep_masks):
+    for c, keep in enumerate(keep_masks):
+        rows = ref.valid_rows(c)
+        if len(rows) == 0:
+            continue
+        planes = [ref.k_codes, ref.k_scale, ref.k_zero, ref.v_codes, ref.v_scale, ref.v_zero,
+                  ref.acc, ref.ts]
+        views = [p[rows[0]:rows[0] + len(rows)] for p in planes]
+        m = O.compact(keep, *views)
+        ref.fill[c] = m
+    assert np.array_equal(np_of(pool.fill), ref.fill)
+    for c in range(len(keep_masks)):
+        rows = ref.valid_rows(c)
+        assert np.array_equal(codes_np(pool.k_codes, scheme)[rows], ref.k_codes[rows])
+        assert np.array_equal(codes_np(pool.v_codes, scheme)[rows], ref.v_codes[rows])
+        assert np.array_equal(np_of(pool.k_scale)[rows].astype(np.float32), ref.k_scale[rows])
+        if pool.k_zero is not None:
+            assert np.array_equal(np_of(pool.v_zero)[rows].astype(np.float32), ref.v_zero[rows])
+        assert np.array_equal(np_of(pool.acc)[rows], ref.acc[rows])
+        assert np.array_equal(np_of(pool.ts)[rows], ref.ts[rows])
+
+
+@pytest.mark.parametrize("ties", [False, True])
+@pytest.mark.parametrize("scheme,group,heads,dh", [(O.Q_I4_ASYM, 32, 8, 128), (O.Q_I8_SYM, 64, 4, 64)])
+def test_h2o_evict_and_compact(dev, ties, scheme, group, heads, dh):
+    r = rng(31 + ties)
+    caps = [3000, 1024, 40, 5, 16]
+    lens = [2999, 1024, 33, 1, 0]
+    pool, ref = _fill_pool(dev, r, caps, lens, heads, dh, group, scheme)
+    _set_state(pool, ref, r, ties)
+    heavy, recent = 0.0625, 0.03
+    pool.evict_select(0, heavy_ratio=heavy, recent_ratio=recent)
+    keeps = []
+    for c, L in enumerate(lens):
+        rows = ref.valid_rows(c)
+        if L == 0:
+            keeps.append(np.zeros(0, dtype=bool))
+            continue
+        nh, nr = O.h2o_budget(L, heavy, recent)
+        keep = O.h2o_keep(ref.acc[rows], ref.ts[rows], nh, nr)
+        keeps.append(keep)
+        got = np_of(pool.keep_flag)[rows].astype(bool)
+        assert np.array_equal(got, keep), (c, np.argwhere(got != keep)[:5])
+        m = int(np_of(pool.new_len)[c])
+        assert m == keep.sum()
+        assert np.array_equal(np_of(pool.keep_index)[rows[0]:rows[0] + m], np.nonzero(keep)[0])
+    assert int(np_of(pool.new_len)[4]) == 0
+    pool.compact()
+    _check_compacted(pool, ref, scheme, keeps)
+
+
+@pytest.mark.parametrize("ties", [False, True])
+def test_lru_evict_and_compact(dev, ties):
+    scheme, group, heads, dh = O.Q_I8_SYM, 256, 4, 64   # config-0 layout: one scale per token
+    r = rng(41 + ties)
+    caps = [128, 128, 128, 128]
+    lens = [128, 100, 128, 7]
+    pool, ref = _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="f32")
+    _set_state(pool, ref, r, ties)
+    n_evict = np.array([32, 0, 128, 3], dtype=np.int32)
+    pool.evict_select(1, n_evict=to_dev(n_evict, dev))
+    keeps = []
+    for c, L in enumerate(lens):
+        rows = ref.valid_rows(c)
+        keep = O.lru_keep(ref.ts[rows], int(n_evict[c]))
+        keeps.append(keep)
+        assert np.array_equal(np_of(pool.keep_flag)[rows].astype(bool), keep), c
+    pool.compact()
+    _check_compacted(pool, ref, scheme, keeps)
+
+
+def test_select_brute_force_small(dev):
+    """Tiny caches against an O(n^2) ranking: element i is kept iff fewer than
+    m elements precede it in (value desc, index asc) order."""
+    r = rng(5)
+    caps = [16] * 32
+    lens = [int(v) for v in r.integers(1, 17, 32)]
+    pool, ref = _fill_pool(dev, r, caps, lens, 1, 64, 64, O.Q_I8_SYM, dtype="f32")
+    _set_state(pool, ref, r, True)
+    nh = np.array([int(v) for v in r.integers(0, 6, 32)], dtype=np.int32)
+    nr = np.array([int(v) for v in r.integers(0, 4, 32)], dtype=np.int32)
+    pool.evict_select(0, n_heavy=to_dev(nh, dev), n_recent=to_dev(nr, dev))
+    flags = np_of(pool.keep_flag)
+    for c, L in enumerate(lens):
+        rows = ref.valid_rows(c)
+        a, t = ref.acc[rows] + 0.0, ref.ts[rows]
+        for i in range(L):
+            before_a = sum((a[j] > a[i]) or (a[j] == a[i] and j < i) for j in range(L))
+            before_t = sum((t[j] > t[i]) or (t[j] == t[i] and j < i) for j in range(L))
+            want = before_a < nh[c] or before_t < nr[c]
+            assert bool(flags[rows[i]]) == want, (c, i)

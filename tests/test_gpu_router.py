@@ -1,0 +1,125 @@
+"""GPU parity: K1 router (gate projection, softmax, top-k, renormalise, capacity
+slots) through the C ABI against the numpy restatement.
+
+Bit-exact: expert indices and slots whenever the logits are given (tail entry
+point), including ties (lowest index wins), masks, scaling and the two-gate
+select.  For the fused gate projection the float32 summation order differs
+from any CPU order, so indices are compared exactly wherever the float64 gap
+between the k-th and (k+1)-th logit exceeds 1e-4 (relative to the logit range)
+and the capacity slots are checked for exact consistency with the indices the
+GPU produced.  Probabilities and weights: |diff| <= 1e-5 (float32) /
+1e-3 relative of the logit scale for bf16 inputs."""
+import numpy as np
+import pytest
+
+import pikv_oracle as O
+from util import np_of, rng, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("E,k", [(4, 2), (8, 2), (6, 3), (16, 4), (64, 8), (33, 1), (1, 1)])
+def test_router_tail_bit_exact(dev, E, k):
+    from pikv_amd import ops
+    r = rng(E * 10 + k)
+    T = 1000
+    lg = r.standard_normal((T, E)).astype(np.float32)
+    # force ties: duplicate columns and quantise some rows coarsely
+    lg[::3] = np.round(lg[::3] * 2) / 2
+    if E > 2:
+        lg[::5, 1] = lg[::5, 0]
+    lg_b = r.standard_normal((T, E)).astype(np.float32)
+    sel = (r.random(T) > 0.5)
+    scale = (0.5 + r.random(E)).astype(np.float32)
+    mask = (r.random(E) > 0.3).astype(np.float32)
+    if mask.sum() < k:
+        mask[:] = 1
+    cap = O.compute_capacity(1, T, 1.25, k, E)
+    for kw in [dict(), dict(temperature=0.7, expert_scale=scale),
+               dict(expert_mask=mask), dict(logits_b=lg_b, select=sel, expert_scale=scale),
+               dict(renorm_eps=1e-8)]:
+        okw = dict(kw)
+        dkw = {key: (to_dev(v, dev) if isinstance(v, np.ndarray) and v.dtype != bool else v)
+               for key, v in kw.items()}
+        if "select" in dkw:
+            dkw["select"] = to_dev(sel.astype(np.uint8), dev)
+        out = ops.router_tail(to_dev(lg, dev), top_k=k, capacity=cap, **dkw)
+        probs, idx, w, _ = O.router_tail(lg, k, **okw)
+        assert np.array_equal(np_of(out.topk_idx), idx), kw.keys()
+        assert np.allclose(np_of(out.probs), probs, atol=2e-6, rtol=1e-5)
+        assert np.allclose(np_of(out.topk_w), w, atol=2e-6, rtol=1e-5)
+        slot, count = O.capacity_slots(idx, E, cap)
+        assert np.array_equal(np_of(out.slot), slot)
+        assert np.array_equal(np_of(out.count), count)
+    # raw top-k of logits (the facade's top_k_routing): values are the logits
+    out = ops.router_tail(to_dev(lg, dev), top_k=k, use_softmax=False)
+    _, idx, vals, _ = O.router_tail(lg, k, use_softmax=False)
+    assert np.array_equal(np_of(out.topk_idx), idx)
+    assert np.array_equal(np_of(out.topk_w), vals)
+
+
+@pytest.mark.parametrize("A,E,cap", [(1, 4, 1), (2047, 8, 100), (2049, 8, 3), (100000, 64, 1500),
+                                      (65536, 8, 10240), (5000, 3, 0)])
+def test_capacity_slots_exact(dev, A, E, cap):
+    from pikv_amd import ops
+    r = rng(A + E)
+    # Zipf-like skew so that some experts overflow
+    p = 1.0 / np.arange(1, E + 1) ** 1.2
+    idx = r.choice(E, size=A, p=p / p.sum()).astype(np.int32)
+    slot, count = ops.capacity_slots(to_dev(idx, dev), E, cap)
+    s_ref, c_ref = O.capacity_slots(idx, E, cap)
+    assert np.array_equal(np_of(slot), s_ref)
+    assert np.array_equal(np_of(count), c_ref)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("T,H,E,k", [(128, 256, 4, 2), (1000, 512, 8, 2), (257, 1024, 16, 4),
+                                      (130, 7168, 64, 8), (64, 264, 5, 2)])
+def test_router_fused(dev, dtype, T, H, E, k):
+    from pikv_amd import ops
+    r = rng(T + H + E)
+    x = r.standard_normal((T, H)).astype(np.float32)
+    w = (0.02 * r.standard_normal((E, H))).astype(np.float32)
+    b = (0.1 * r.standard_normal(E)).astype(np.float32)
+    if dtype == "bf16":
+        x, w = O.bf16_round(x), O.bf16_round(w)
+    cap = O.compute_capacity(1, T, 1.25, k, E)
+    out = ops.router_fused(to_dev(x, dev, dtype), to_dev(w, dev, dtype), to_dev(b, dev),
+                           top_k=k, capacity=cap, return_logits=True)
+    lg64 = x.astype(np.float64) @ w.astype(np.float64).T + b
+    lg = lg64.astype(np.float32)
+    probs, idx, wts, _ = O.router_tail(lg, k)
+    assert np.allclose(np_of(out.logits), lg, atol=1e-5 * np.sqrt(H), rtol=1e-5)
+    assert np.allclose(np_of(out.probs), probs, atol=1e-5)
+    got = np_of(out.topk_idx)
+    # set of the k-th / (k+1)-th gap per row, in float64
+    srt = -np.sort(-lg64, axis=1)
+    gaps = np.abs(np.diff(srt, axis=1))[:, :k].min(axis=1) if E > 1 else np.ones(T)
+    clear = gaps > 1e-4
+    assert clear.mean() > 0.9
+    assert np.array_equal(got[clear], idx[clear])
+    # rows with a near-tie must still select valid, distinct experts
+    assert ((got >= 0) & (got < E)).all()
+    assert all(len(set(row)) == k for row in got)
+    assert np.allclose(np_of(out.topk_w)[clear], wts[clear], atol=1e-5)
+    assert np.allclose(np_of(out.topk_w).sum(1), 1.0, atol=1e-5)
+    # slots are exactly the token-major rule applied to the indices the GPU chose
+    slot, count = O.capacity_slots(got, E, cap)
+    assert np.array_equal(np_of(out.slot), slot)
+    assert np.array_equal(np_of(out.count), count)
+
+
+def test_router_empty_and_errors(dev):
+    import torch
+    from pikv_amd import ops
+    out = ops.router_fused(torch.zeros(0, 64, device=dev), torch.zeros(4, 64, device=dev),
+                           top_k=2, capacity=4)
+    assert out.topk_idx.shape == (0, 2) and int(out.count.sum()) == 0
+    with pytest.raises(ValueError):
+        ops.router_fused(torch.zeros(4, 63, device=dev), torch.zeros(4, 63, device=dev))
+    with pytest.raises(ValueError):
+        ops.router_fused(torch.zeros(4, 64, device=dev), torch.zeros(80, 64, device=dev))
+    with pytest.raises(ValueError):
+        ops.router_fused(torch.zeros(4, 64, device=dev), torch.zeros(4, 64, device=dev), top_k=5)
+    with pytest.raises(ValueError):
+        ops.router_fused(torch.zeros(4, 64), torch.zeros(4, 64))
