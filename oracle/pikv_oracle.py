@@ -253,7 +253,10 @@ def quant_params(x_min: np.ndarray, x_max: np.ndarray, scheme: int):
         else:
             scale = ((x_max - x_min).astype(F32) / qr).astype(F32)
         if bits == 4:
+            # a scale that underflows to zero in float16 becomes 2**-24, the
+            # smallest positive float16, so nothing divides by zero
             scale = _to_half_sat(scale).astype(F32)
+            scale = np.where(scale == 0, F32(2.0 ** -24), scale).astype(F32)
         if sym:
             zero = np.zeros_like(scale)
         else:

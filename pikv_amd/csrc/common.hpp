@@ -130,7 +130,12 @@ __device__ __forceinline__ void quant_params(float mn, float mx, float& scale, f
   } else {
     scale = (mx - mn) / qr;
   }
-  if constexpr (Q::bits == 4) scale = (float)float_to_half_sat(scale);
+  if constexpr (Q::bits == 4) {
+    // stored as half: a scale that underflows to zero becomes the smallest
+    // positive half (2^-24) so that encoder and decoder never divide by zero
+    scale = (float)float_to_half_sat(scale);
+    if (scale == 0.0f) scale = 5.9604644775390625e-08f;
+  }
   if constexpr (Q::sym) {
     zero = 0.0f;
   } else {

@@ -172,6 +172,10 @@ def router_fused(x, weight, bias=None, *, top_k=2, capacity=None, expert_scale=N
     expert_mask = _vecf(expert_mask, "expert_mask", E, dev)
     probs, logits, idx, w, slot, count, ws, ws_bytes = _router_common(
         T, E, top_k, capacity, dev, True, return_logits)
+    if T == 0:  # nothing to route (empty tensors have no device address)
+        if count is not None:
+            count.zero_()
+        return RouterOut(probs, idx, w, slot, count, logits, capacity)
     N.call("pikv_router_fused", _ptr(x), _ptr(weight), dt, _ptr(bias), _ptr(expert_scale),
            _ptr(expert_mask), float(temperature), float(renorm_eps), T, H, E, top_k,
            int(capacity or 0), _ptr(probs), _ptr(logits), _ptr(idx), _ptr(w), _ptr(slot),
@@ -199,6 +203,10 @@ def router_tail(logits, *, top_k=2, capacity=None, logits_b=None, select=None,
     expert_mask = _vecf(expert_mask, "expert_mask", E, dev)
     probs, _, idx, w, slot, count, ws, ws_bytes = _router_common(
         T, E, top_k, capacity, dev, bool(use_softmax), False)
+    if T == 0:
+        if count is not None:
+            count.zero_()
+        return RouterOut(probs, idx, w, slot, count, None, capacity)
     N.call("pikv_router_tail", _ptr(logits), _ptr(logits_b), _ptr(select), _ptr(expert_scale),
            _ptr(expert_mask), float(temperature), float(renorm_eps), int(bool(use_softmax)),
            T, E, top_k, int(capacity or 0), _ptr(probs), _ptr(idx), _ptr(w), _ptr(slot),
@@ -219,6 +227,8 @@ def capacity_slots(expert_idx, num_experts: int, capacity: int):
     count = torch.empty(num_experts, dtype=torch.int32, device=dev)
     ws_bytes = int(N.lib().pikv_router_workspace_bytes(A, num_experts, 1))
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+    if A == 0:
+        return slot, count.zero_()
     N.call("pikv_capacity_slots", _ptr(expert_idx), A, num_experts, int(capacity), _ptr(slot),
            _ptr(count), _ptr(ws), ws_bytes, _stream())
     return slot, count
@@ -239,6 +249,8 @@ def quantize_rows(x, group: int, scheme: int):
     codes = _code_plane(n, D, scheme, dev)
     scale = torch.empty(n, D // group, dtype=_meta_dtype(scheme), device=dev)
     zero = torch.empty_like(scale) if _scheme_asym(scheme) else None
+    if n == 0:
+        return codes, scale, zero
     N.call("pikv_quantize_rows", _ptr(x), dt, n, D, group, scheme, 0, _ptr(codes), _ptr(scale),
            _ptr(zero), _stream())
     return codes, scale, zero
@@ -267,6 +279,8 @@ def dequantize_rows(codes, scale, zero, group: int, scheme: int, out_dtype=torch
     if out_dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("out_dtype must be float32 or bfloat16")
     out = torch.empty(cnt, D, dtype=out_dtype, device=codes.device)
+    if cnt == 0:
+        return out
     N.call("pikv_gather_dequant", _ptr(codes), _ptr(scale), _ptr(zero), D, group, scheme,
            _ptr(rows), row0, cnt, _ptr(out), F32 if out_dtype == torch.float32 else BF16,
            _stream())
@@ -365,6 +379,8 @@ class CachePool:
             raise ValueError("fanout must be in [1,8]")
         if cache_id.numel() != n_src * fanout or slot.numel() != n_src * fanout:
             raise ValueError(f"cache_id/slot must have n_src*fanout = {n_src * fanout} elements")
+        if n_src == 0:
+            return
         N.call("pikv_quant_scatter", _ptr(k2), _ptr(v2), dt, n_src, fanout, self.D, self.group,
                self.scheme, _ptr(cache_id), _ptr(slot), _ptr(self.row_base), _ptr(self.fill),
                _ptr(self.cap), self.n_caches, _ptr(self.k_codes), _ptr(self.v_codes),
