@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Benchmark of the routed, compressed KV-cache data path on one MI355X.
+
+A step is one pass of the hot path over one prefill batch of the
+"prefill compress-write" workload (hidden 4096, 8 experts top-2, capacity
+factor 1.25, 32 heads x 128, bf16, batch 16 x seq 2048 = 32768 tokens, 1 % outlier
+channels x20, int8 symmetric per token per head, 8 caches x 8192 slots):
+
+    reset fill -> K1 fused router (+capacity slots)
+               -> K2 fused quantise + scatter of K and V into the routed caches
+               -> K3 gather + dequantise + QK^T scores over the 8 caches
+               -> softmax-normalised H2O importance accumulation
+
+Inputs are synthetic, seeded, and resident in HBM before the timed region.
+Prints ONE JSON line.  `value` = tokens routed and cached per second over the
+whole step; `roofline` is for the dominant kernel (K2), from HIP events recorded
+around that kernel inside the timed steps; `cpu_baseline` times the C restatement
+of the same step (oracle/pikv_oracle.c) on the host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "routed KV tokens/s (quant+scatter+gather+dequant), 1 MI355X; % HBM peak"
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOAD = dict(name="prefill compress-write", batch=16, seq=2048, hidden=4096, experts=8, top_k=2,
+                capacity_factor=1.25, heads=32, head_dim=128, cache_slots=8192,
+                quant="int8 symmetric per token per head", outlier_frac=0.01, outlier_scale=20.0,
+                seed=1)
+
+
+def make_inputs(torch, dev, w):
+    g = torch.Generator(device="cpu").manual_seed(w["seed"])
+    T, H, E = w["batch"] * w["seq"], w["hidden"], w["experts"]
+    D = w["heads"] * w["head_dim"]
+    gd = torch.Generator(device=dev).manual_seed(w["seed"])
+    hidden = torch.randn(T, H, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    gate_w = (0.02 * torch.randn(E, H, generator=g)).to(dev).to(torch.bfloat16)
+    n_out = max(1, int(D * w["outlier_frac"]))
+    ch = torch.randperm(D, generator=g)[:n_out].to(dev)
+    kv = []
+    for _ in range(2):
+        t = torch.randn(T, D, generator=gd, device=dev, dtype=torch.float32)
+        t[:, ch] *= w["outlier_scale"]
+        kv.append(t.to(torch.bfloat16))
+    q = torch.randn(E, w["heads"], w["head_dim"], generator=gd, device=dev).to(torch.bfloat16)
+    return hidden, gate_w, kv[0], kv[1], q
+
+
+def cpu_baseline(torch, w, hidden, gate_w, k_src, v_src, q, reps=2):
+    """Time the C restatement of the same step on the host (all of the batch)."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import c_oracle as CO
+    import pikv_oracle as O
+
+    def bits(t):
+        return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+    T = hidden.shape[0]
+    E, k = w["experts"], w["top_k"]
+    D = w["heads"] * w["head_dim"]
+    xh, wh, kh, vh, qh = bits(hidden), bits(gate_w), bits(k_src), bits(v_src), bits(q)
+    cap = O.compute_capacity(w["batch"], w["seq"], w["capacity_factor"], k, E)
+    times = []
+    for _ in range(reps):
+        pool = CO.CPool([w["cache_slots"]] * E, D, w["head_dim"], O.Q_I8_SYM)
+        t0 = time.perf_counter()
+        _, _, idx, _ = CO.router(xh, wh, None, k)
+        slot, count = CO.capacity_slots(idx, E, cap)
+        pool.quant_scatter(kh, vh, idx, slot, k, now=1.0)
+        pool.advance(count, cap)
+        pool.scores_h2o(qh, w["heads"], w["heads"], w["head_dim"], 1.0 / w["head_dim"] ** 0.5,
+                        now=1.0, want_scores=False)
+        times.append(time.perf_counter() - t0)
+    best = min(times)
+    return {"value": T / best, "unit": "tokens/s", "cores": CO.threads(), "kind": "port",
+            "sample": f"whole batch of {T} tokens, best of {reps} runs of oracle/pikv_oracle.c "
+                      f"(OpenMP, {CO.threads()} threads), {best:.2f} s per step"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from pikv_amd import ops
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    w = WORKLOAD
+    T, E, k = w["batch"] * w["seq"], w["experts"], w["top_k"]
+    heads, dh = w["heads"], w["head_dim"]
+    D = heads * dh
+    hidden, gate_w, k_src, v_src, q = make_inputs(torch, dev, w)
+    cap = int(w["batch"] * w["seq"] * w["capacity_factor"] * k / E)
+    pool = ops.CachePool([w["cache_slots"]] * E, heads, dh, dh, ops.Q_I8_SYM, dev)
+
+    def step(ev=None, now=1.0):
+        pool.fill.zero_()
+        if ev: ev[0].record()
+        r = ops.router_fused(hidden, gate_w, top_k=k, capacity=cap)
+        if ev: ev[1].record()
+        pool.quant_scatter(k_src, v_src, r.topk_idx, r.slot, k, now=now)
+        if ev: ev[2].record()
+        pool.advance(r.count, cap)
+        scores, tmax, tsum = pool.scores(q, heads)
+        if ev: ev[3].record()
+        pool.h2o_accumulate(scores, tmax, tsum, now=now)
+        if ev: ev[4].record()
+        return r
+
+    for i in range(args.warmup):
+        r = step()
+    torch.cuda.synchronize()
+    kept = int(pool.fill.sum().item())
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(events[i], now=float(i + 2))
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+
+    def avg(a, b):
+        return sum(ev[a].elapsed_time(ev[b]) for ev in events) / len(events)
+
+    t_router, t_quant, t_scores, t_h2o = avg(0, 1), avg(1, 2), avg(2, 3), avg(3, 4)
+    A = T * k
+    # algorithmic bytes of one launch
+    b_quant = T * 2 * D * 2 + kept * (2 * D + 2 * heads * 4) + A * 8
+    b_router = T * w["hidden"] * 2 + T * E * 4 + A * 12
+    b_scores = kept * (D + heads * 4) + kept * heads * 4
+    b_h2o = kept * heads * 4 + kept * 8
+    gbps = lambda b, ms: b / (ms * 1e-3) / 1e9
+    out = {
+        "metric": METRIC, "value": T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "prefill compress-write: T=32768 (16x2048), hidden 4096, 8 experts top-2 "
+                               "cf 1.25, 32 heads x 128 bf16, int8 sym per token per head, 8 caches x 8192 slots",
+                   "kept_assignments": kept, "assignments": A},
+        "roofline": {"bound": "hbm", "kernel": "quant_scatter_kernel<I8_SYM,bf16>",
+                     "achieved": gbps(b_quant, t_quant), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": gbps(b_quant, t_quant) / HBM_PEAK_GBPS, "traffic": None,
+                     "algorithmic_bytes": b_quant, "avg_launch_ms": t_quant},
+        "kernels": {
+            "router": {"ms": t_router, "GBps": gbps(b_router, t_router)},
+            "quant_scatter": {"ms": t_quant, "GBps": gbps(b_quant, t_quant),
+                              "tokens_per_s": T / (t_quant * 1e-3)},
+            "scores": {"ms": t_scores, "GBps": gbps(b_scores, t_scores),
+                       "cached_token_reads_per_s": kept / (t_scores * 1e-3)},
+            "h2o_accumulate": {"ms": t_h2o, "GBps": gbps(b_h2o, t_h2o)},
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, w, hidden, gate_w, k_src, v_src, q)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
