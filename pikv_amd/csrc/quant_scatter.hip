@@ -8,6 +8,10 @@
 // stored to each of the row's `fanout` destination rows, so HBM sees the
 // algorithmic traffic only: D*sizeof(src) bytes in, fanout*(D*bits/8 + metadata)
 // bytes out per source row, all as 128-bit accesses contiguous across lanes.
+// The K and V loads of a lane are issued together before any arithmetic, and
+// the per-element division of the reference formula is replaced by one division
+// per group plus an exactness check (see quantize_lane), which is what takes
+// the kernel from VALU-bound to HBM-bound.
 #include "common.hpp"
 
 namespace pikv {
@@ -34,9 +38,50 @@ struct QuantScatterArgs {
   int group;
   int n_tensors;        // 1 (K only) or 2 (K and V)
   int n_caches;
+  int lpr_shift;        // log2(lanes per row) or -1 when it is not a power of two
+  int lpg_shift;        // log2(lanes per group)
 };
 
-template <int SCHEME, int SRC_DT>
+template <int DT, int EPL>
+struct RawRow {
+  static constexpr int kVec = (DT == PIKV_BF16) ? EPL / 8 : EPL / 4;
+  uint4 v[kVec];
+  __device__ __forceinline__ void load(const void* base, int64_t elem_off) {
+    const char* p = reinterpret_cast<const char*>(base) + elem_off * (DT == PIKV_BF16 ? 2 : 4);
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) v[i] = ld16(p + 16 * i);
+  }
+  __device__ __forceinline__ void zero_fill() {
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) v[i] = make_uint4(0, 0, 0, 0);
+  }
+  __device__ __forceinline__ void to_float(float (&x)[EPL]) const {
+    if constexpr (DT == PIKV_BF16) {
+#pragma unroll
+      for (int i = 0; i < kVec; ++i) {
+        const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          x[8 * i + 2 * j] = __uint_as_float(w[j] << 16);
+          x[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kVec; ++i) {
+        x[4 * i] = __uint_as_float(v[i].x);
+        x[4 * i + 1] = __uint_as_float(v[i].y);
+        x[4 * i + 2] = __uint_as_float(v[i].z);
+        x[4 * i + 3] = __uint_as_float(v[i].w);
+      }
+    }
+  }
+};
+
+// ROW_UNIFORM: lanes_per_row is a power of two >= 64, so a wavefront never spans two
+// source rows; the row index, its destinations and every address base are then
+// wave-uniform and live in scalar registers.
+template <int SCHEME, int SRC_DT, int FANOUT, bool ROW_UNIFORM>
 __global__ __launch_bounds__(256) void quant_scatter_kernel(QuantScatterArgs a) {
   using Q = QScheme<SCHEME>;
   constexpr int EPL = Q::epl;
@@ -44,17 +89,30 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(QuantScatterArgs a) 
   const int lanes_per_group = a.group / EPL;
   const int groups_per_row = a.D / a.group;
 
-  const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t s = g / lanes_per_row;
-  const int part = (int)(g - s * lanes_per_row);
+  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  int64_t s;
+  int part;
+  if constexpr (ROW_UNIFORM) {
+    const int64_t g0 = (int64_t)blockIdx.x * 256 + (threadIdx.x & ~63u);
+    const uint32_t g0lo = __builtin_amdgcn_readfirstlane((uint32_t)g0);
+    const uint32_t g0hi = __builtin_amdgcn_readfirstlane((uint32_t)(g0 >> 32));
+    const int64_t gu = (int64_t)(((uint64_t)g0hi << 32) | g0lo);
+    s = gu >> a.lpr_shift;
+    part = (int)(gu & (lanes_per_row - 1)) + (int)(threadIdx.x & 63u);
+  } else if (a.lpr_shift >= 0) {
+    s = g >> a.lpr_shift;
+    part = (int)(g & (lanes_per_row - 1));
+  } else {
+    s = g / lanes_per_row;
+    part = (int)(g - s * lanes_per_row);
+  }
   const bool valid = s < a.n_src;
 
-  // Destination rows of this source row (-1 = dropped).  Fixed-trip unrolled
-  // loops keep the array in registers.
-  int64_t dst[kMaxFanout];
+  // Destination rows of this source row (-1 = dropped).
+  int64_t dst[FANOUT];
   bool any = false;
 #pragma unroll
-  for (int j = 0; j < kMaxFanout; ++j) {
+  for (int j = 0; j < FANOUT; ++j) {
     dst[j] = -1;
     if (valid && j < a.fanout) {
       if (a.cache_id == nullptr) {
@@ -77,47 +135,48 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(QuantScatterArgs a) 
   // takes the same branch below, and cross-lane traffic stays inside the group.
   const bool live = valid && any;
 
-  for (int t = 0; t < a.n_tensors; ++t) {
-    float x[EPL];
-    if (live) {
-      load_as_float<SRC_DT, EPL>(a.src[t], s * a.D + (int64_t)part * EPL, x);
-    } else {
+  RawRow<SRC_DT, EPL> raw[2];
+  raw[0].zero_fill();
+  raw[1].zero_fill();
+  if (live) {
+    const int64_t off = s * a.D + (int64_t)part * EPL;
+    raw[0].load(a.src[0], off);
+    if (a.n_tensors > 1) raw[1].load(a.src[1], off);
+  }
+  const bool meta_lane = (part & (lanes_per_group - 1)) == 0;
+  const int grp = part >> a.lpg_shift;
+
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) x[i] = 0.f;
-    }
+  for (int t = 0; t < 2; ++t) {
+    if (t >= a.n_tensors) break;
+    float x[EPL];
+    raw[t].to_float(x);
     float mn = x[0], mx = x[0];
 #pragma unroll
     for (int i = 1; i < EPL; ++i) {
       mn = fminf(mn, x[i]);
       mx = fmaxf(mx, x[i]);
     }
-    mn = group_min_rt(mn, lanes_per_group);
-    mx = group_max_rt(mx, lanes_per_group);
-    float scale, zero;
-    quant_params<SCHEME>(mn, mx, scale, zero);
-    int c[EPL];
-#pragma unroll
-    for (int i = 0; i < EPL; ++i) c[i] = quant_code<SCHEME>(x[i], scale, zero);
-    const uint4 packed = pack_codes<SCHEME>(c);
+    group_minmax_dpp(mn, mx, lanes_per_group);
+    const GroupQuant gq = make_group_quant<SCHEME>(mn, mx);
+    const uint4 packed = quantize_lane<SCHEME>(x, gq);
     if (live) {
-      const bool meta_lane = (part % lanes_per_group) == 0;
-      const int grp = part / lanes_per_group;
 #pragma unroll
-      for (int j = 0; j < kMaxFanout; ++j) {
+      for (int j = 0; j < FANOUT; ++j) {
         const int64_t row = dst[j];
         if (row < 0) continue;
         char* cp = reinterpret_cast<char*>(a.codes[t]) + (row * lanes_per_row + part) * 16;
-        st16(cp, packed);
+        st16_stream(cp, packed);
         if (meta_lane) {
-          store_meta<SCHEME>(a.scale[t], row * groups_per_row + grp, scale);
-          if constexpr (!Q::sym) store_meta<SCHEME>(a.zero[t], row * groups_per_row + grp, zero);
+          store_meta<SCHEME>(a.scale[t], row * groups_per_row + grp, gq.scale);
+          if constexpr (!Q::sym) store_meta<SCHEME>(a.zero[t], row * groups_per_row + grp, gq.zero);
         }
       }
     }
   }
   if (live && part == 0) {
 #pragma unroll
-    for (int j = 0; j < kMaxFanout; ++j) {
+    for (int j = 0; j < FANOUT; ++j) {
       if (dst[j] < 0) continue;
       if (a.row_acc) a.row_acc[dst[j]] = 0.f;
       if (a.row_ts) a.row_ts[dst[j]] = a.now;
@@ -125,17 +184,41 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(QuantScatterArgs a) 
   }
 }
 
+template <int SCHEME, int SRC_DT, bool RU>
+static void launch_quant_f(int fanout, unsigned blocks, hipStream_t st, const QuantScatterArgs& a) {
+  if (fanout <= 1)
+    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 1, RU>), dim3(blocks), dim3(256), 0, st, a);
+  else if (fanout <= 2)
+    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 2, RU>), dim3(blocks), dim3(256), 0, st, a);
+  else if (fanout <= 4)
+    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 4, RU>), dim3(blocks), dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 8, RU>), dim3(blocks), dim3(256), 0, st, a);
+}
+
 template <int SCHEME>
-static int launch_quant(const QuantScatterArgs& a, int src_dtype, hipStream_t st) {
+static int launch_quant(QuantScatterArgs a, int src_dtype, hipStream_t st) {
   using Q = QScheme<SCHEME>;
-  const int64_t lanes = a.n_src * (a.D / Q::epl);
+  const int lanes_per_row = a.D / Q::epl;
+  a.lpr_shift = -1;
+  if (is_pow2(lanes_per_row)) {
+    a.lpr_shift = 0;
+    while ((1 << a.lpr_shift) < lanes_per_row) ++a.lpr_shift;
+  }
+  a.lpg_shift = 0;
+  while ((Q::epl << a.lpg_shift) < a.group) ++a.lpg_shift;
+  const int64_t lanes = a.n_src * lanes_per_row;
   if (lanes == 0) return PIKV_OK;
   const int64_t blocks = (lanes + 255) / 256;
   if (blocks > 0x7fffffffLL) return PIKV_ERR_SHAPE;
-  if (src_dtype == PIKV_BF16)
-    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, PIKV_BF16>), dim3((unsigned)blocks), dim3(256), 0, st, a);
-  else
-    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, PIKV_F32>), dim3((unsigned)blocks), dim3(256), 0, st, a);
+  const bool ru = a.lpr_shift >= 6;
+  if (src_dtype == PIKV_BF16) {
+    if (ru) launch_quant_f<SCHEME, PIKV_BF16, true>(a.fanout, (unsigned)blocks, st, a);
+    else launch_quant_f<SCHEME, PIKV_BF16, false>(a.fanout, (unsigned)blocks, st, a);
+  } else {
+    if (ru) launch_quant_f<SCHEME, PIKV_F32, true>(a.fanout, (unsigned)blocks, st, a);
+    else launch_quant_f<SCHEME, PIKV_F32, false>(a.fanout, (unsigned)blocks, st, a);
+  }
   PIKV_CHECK_LAUNCH();
   return PIKV_OK;
 }
@@ -219,7 +302,7 @@ extern "C" int pikv_quantize_rows(const void* src, int src_dtype, int64_t n_rows
   QuantScatterArgs a{};
   a.src[0] = src; a.codes[0] = codes; a.scale[0] = scale; a.zero[0] = zero;
   a.cache_id = nullptr; a.n_src = n_rows; a.dst_row0 = dst_row0; a.fanout = 1;
-  a.D = D; a.group = group; a.n_tensors = 1;
+  a.D = D; a.group = group; a.n_tensors = 1; a.n_caches = 1;
   return dispatch_quant(a, scheme, src_dtype, (hipStream_t)stream);
 }
 

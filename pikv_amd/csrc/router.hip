@@ -18,7 +18,7 @@
 
 namespace pikv {
 
-constexpr int kSlotChunk = 2048;  // assignments per block in the slot pass
+constexpr int kSlotChunk = 512;  // assignments per block in the slot pass
 
 struct TailParams {
   const float* bias;
@@ -181,6 +181,91 @@ __global__ __launch_bounds__(256) void router_tail_kernel(const float* __restric
     lg = use_a ? la[t * p.E + e] : lb[t * p.E + e];
   }
   router_tail_lanes<EPAD>(lg, t, e, lane, p);
+}
+
+// ---- bf16 gate projection on the matrix cores ------------------------------------
+// Measured on the prefill workload (T=32768, H=4096, E=8) the VALU kernel above
+// issues 25.8 M wavefront instructions - 42 us of pure issue time against 34 us of
+// HBM time - and has too few wavefronts to hide latency.  For bf16 inputs the
+// contraction over H therefore runs as v_mfma_f32_16x16x32_bf16: a block owns 16
+// tokens, its 8 wavefronts interleave over 32-wide slices of H (so the block
+// reads 512 contiguous bytes of each token row per sweep), every wavefront keeps
+// one 16x16 fp32 tile per group of 16 experts, and the partial tiles meet in LDS.
+// The kernel stays HBM-bound up to E = 64 (the MFMA work is ~1/7 of the HBM time
+// there), which the VALU formulation cannot be.
+typedef __bf16 pikv_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float pikv_f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kMfmaWaves = 8;
+
+template <int NT>  // NT = number of 16-expert tiles (1, 2 or 4)
+__global__ __launch_bounds__(kMfmaWaves * 64) void router_gate_mfma_kernel(
+    const void* __restrict__ x, const void* __restrict__ w, int H, TailParams p) {
+  constexpr int EP = 16 * NT;
+  __shared__ float red[kMfmaWaves][16][EP];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t tok0 = (int64_t)blockIdx.x * 16;
+  const int m = lane & 15;    // token row of the A operand / expert column of B and C
+  const int kg = lane >> 4;   // which 8 of the 32 k-values this lane feeds
+  const bool tok_ok = tok0 + m < p.T;
+  const char* xrow = reinterpret_cast<const char*>(x) + ((tok0 + m) * (int64_t)H + kg * 8) * 2;
+  const char* wrow[NT];
+  bool w_ok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int e = t * 16 + m;
+    w_ok[t] = e < p.E;
+    wrow[t] = reinterpret_cast<const char*>(w) + ((int64_t)(w_ok[t] ? e : 0) * H + kg * 8) * 2;
+  }
+  pikv_f32x4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int steps = H / 32;
+  constexpr int UN = 4;
+  for (int st0 = wave; st0 < steps; st0 += kMfmaWaves * UN) {
+    uint4 av[UN], bv[UN][NT];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int st = st0 + u * kMfmaWaves;
+      const bool ok = st < steps;
+      av[u] = (ok && tok_ok) ? ld16(xrow + (int64_t)st * 64) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        bv[u][t] = (ok && w_ok[t]) ? ld16(wrow[t] + (int64_t)st * 64) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const pikv_bf16x8 a8 = __builtin_bit_cast(pikv_bf16x8, av[u]);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a8, __builtin_bit_cast(pikv_bf16x8, bv[u][t]),
+                                                         acc[t], 0, 0, 0);
+    }
+  }
+  // C layout: lane holds rows 4*(lane/16)+i, column lane%16 of each tile.
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][4 * kg + i][t * 16 + m] = acc[t][i];
+  __syncthreads();
+  // Wavefront w finishes tokens 2w, 2w+1: lane -> (token, expert) with the experts
+  // of a token in EP adjacent lanes, as the tail expects.
+  constexpr int TPC = 64 / EP;  // tokens per tail call
+#pragma unroll
+  for (int c = 0; c < 2 / TPC + (2 % TPC != 0); ++c) {
+    const int tl = 2 * wave + c * TPC + lane / EP;
+    const int e = lane % EP;
+    const bool in_range = (c * TPC + lane / EP) < 2;
+    float lg = 0.f;
+    if (in_range) {
+#pragma unroll
+      for (int w2 = 0; w2 < kMfmaWaves; ++w2) lg += red[w2][tl][e];
+    }
+    // lanes beyond the two tokens of this wavefront present an out-of-range token
+    router_tail_lanes<EP>(lg, in_range ? tok0 + tl : p.T, e, lane, p);
+  }
 }
 
 // ---- capacity slots -------------------------------------------------------------
@@ -353,10 +438,21 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
     const int64_t tiles = (T + (64 / epad) - 1) / (64 / epad);
     const int64_t blocks = (tiles + 3) / 4;
     if (blocks > 0x7fffffffLL) return PIKV_ERR_SHAPE;
-    if (x_dtype == PIKV_BF16)
+    if (x_dtype == PIKV_BF16 && H % 32 == 0) {
+      const int64_t mb = (T + 15) / 16;
+      if (mb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+      const dim3 grid((unsigned)mb), blk(kMfmaWaves * 64);
+      if (E <= 16)
+        hipLaunchKernelGGL((router_gate_mfma_kernel<1>), grid, blk, 0, st, x, w, H, p);
+      else if (E <= 32)
+        hipLaunchKernelGGL((router_gate_mfma_kernel<2>), grid, blk, 0, st, x, w, H, p);
+      else
+        hipLaunchKernelGGL((router_gate_mfma_kernel<4>), grid, blk, 0, st, x, w, H, p);
+    } else if (x_dtype == PIKV_BF16) {
       launch_gate<PIKV_BF16>(epad, (unsigned)blocks, st, x, w, H, p);
-    else
+    } else {
       launch_gate<PIKV_F32>(epad, (unsigned)blocks, st, x, w, H, p);
+    }
     PIKV_CHECK_LAUNCH();
   }
   if (slot) return launch_slots(topk_idx, T * k, E, capacity, slot, count, workspace, workspace_bytes, st);

@@ -170,3 +170,30 @@ def test_fakequant_reference_domain(dev):
         assert np.array_equal(np_of(stats), st_ref)
         assert np.array_equal(np_of(dq), dq_ref)
         assert np.allclose(np_of(mse), mse_ref, rtol=1e-5)
+
+
+@pytest.mark.parametrize("scheme,group", [(O.Q_I8_SYM, 128), (O.Q_I8_ASYM, 128), (O.Q_I4_ASYM, 32), (O.Q_I4_SYM, 32)])
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_quantize_many_values_bit_exact(dev, scheme, group, dtype):
+    """8.4 M values per case: the kernel replaces the per-element division by a
+    per-group reciprocal with an exactness check, so the codes are compared on
+    enough data that thousands of elements fall next to a rounding tie, plus rows
+    that leave the fast path's range (large offsets, huge and tiny magnitudes)."""
+    from pikv_amd import ops
+    r = rng(900 + scheme)
+    n, D = 2048, 4096
+    x = kv_like(r, n, D, dtype="f32")
+    x[100:140] += 1000.0                       # large zero points -> exact path
+    x[200:220] *= 1e-20
+    x[300:320] *= 1e20
+    x[400:420] = np.round(x[400:420] * 4) / 4  # coarse grid: exact ties in many groups
+    if dtype == "bf16":
+        x = O.bf16_round(x)
+    codes, scale, zero = ops.quantize_rows(to_dev(x, dev, dtype), group, scheme)
+    q_ref, s_ref, z_ref = O.quantize_groups(x, group, scheme)
+    assert np.array_equal(np_of(scale).astype(np.float32), s_ref)
+    if zero is not None:
+        assert np.array_equal(np_of(zero).astype(np.float32), z_ref, equal_nan=True)
+    got = codes_np(codes, scheme)
+    bad = np.argwhere(got != q_ref)
+    assert bad.size == 0, f"{len(bad)} codes differ, first {bad[:5]}"
