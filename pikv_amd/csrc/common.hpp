@@ -344,6 +344,34 @@ __device__ __forceinline__ void unpack_codes(uint4 v, int* c) {
   }
 }
 
+// Codes of one lane as floats of (code - qmin), i.e. the unsigned stored form: the
+// byte extractions below compile to v_cvt_f32_ubyteN (one instruction per code),
+// and the caller folds qmin into the zero point.
+template <int SCHEME>
+__device__ __forceinline__ void unpack_codes_unsigned(uint4 v, float* f) {
+  using Q = QScheme<SCHEME>;
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  if constexpr (Q::bits == 8) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t u = Q::sym ? (w[i] ^ 0x80808080u) : w[i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) f[4 * i + j] = (float)((u >> (8 * j)) & 0xffu);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t u = Q::sym ? (w[i] ^ 0x88888888u) : w[i];
+      const uint32_t ev = u & 0x0f0f0f0fu, od = (u >> 4) & 0x0f0f0f0fu;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        f[8 * i + 2 * j] = (float)((ev >> (8 * j)) & 0xffu);
+        f[8 * i + 2 * j + 1] = (float)((od >> (8 * j)) & 0xffu);
+      }
+    }
+  }
+}
+
 // Metadata (scale / zero) element access: float for 8-bit, half for 4-bit.
 template <int SCHEME>
 __device__ __forceinline__ void store_meta(void* plane, int64_t idx, float v) {

@@ -116,42 +116,58 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   const int kvh = part / lanes_per_head;
   const int d0 = (part % lanes_per_head) * EPL;
 
-  // Query slices of the REP heads that read this kv head.
+  // Query slices of the REP heads that read this kv head, and their sums (for the
+  // zero-point term: dot(q, (c - z) * s) = s * (dot(q, c) - z * sum(q))).
   float qv[REP][EPL];
+  float qsum[REP];
 #pragma unroll
   for (int r = 0; r < REP; ++r) {
     const int hq = kvh * REP + r;
     load_as_float<Q_DT, EPL>(a.q, ((int64_t)c * a.n_q_heads + hq) * a.head_dim + d0, qv[r]);
+    float sacc = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) sacc += qv[r][j];
+    qsum[r] = sacc;
   }
   const int64_t base_row = a.row_base[c];
+  constexpr int UN = 4;  // token steps in flight per lane
 
-  for (int s0 = 0; s0 < kTile; s0 += tok_per_step) {
-    const int tl = s0 + tok_in_step;  // token within the tile
-    const int64_t n = n0 + tl;
-    float dot[REP];
+  for (int s0 = 0; s0 < kTile; s0 += tok_per_step * UN) {
+    uint4 v[UN];
+    float sc[UN], zr[UN];
+    bool ok[UN];
 #pragma unroll
-    for (int r = 0; r < REP; ++r) dot[r] = 0.f;
-    if (n < len) {
-      const int64_t row = base_row + n;
-      const uint4 v = ld16(reinterpret_cast<const char*>(a.codes) + (row * lanes_per_row + part) * 16);
-      const int64_t mi = row * groups_per_row + (part * EPL) / a.group;
-      const float sc = load_meta<SCHEME>(a.scale, mi);
-      const float zr = Q::sym ? 0.f : load_meta<SCHEME>(a.zero, mi);
-      int cd[EPL];
-      unpack_codes<SCHEME>(v, cd);
-#pragma unroll
-      for (int j = 0; j < EPL; ++j) {
-        const float kf = ((float)cd[j] - zr) * sc;
-#pragma unroll
-        for (int r = 0; r < REP; ++r) dot[r] = fmaf(qv[r][j], kf, dot[r]);
+    for (int u = 0; u < UN; ++u) {
+      const int tl = s0 + u * tok_per_step + tok_in_step;
+      const int64_t n = n0 + tl;
+      ok[u] = tl < kTile && n < len;
+      v[u] = make_uint4(0, 0, 0, 0);
+      sc[u] = 0.f;
+      zr[u] = 0.f;
+      if (ok[u]) {
+        const int64_t row = base_row + n;
+        v[u] = ld16(reinterpret_cast<const char*>(a.codes) + (row * lanes_per_row + part) * 16);
+        const int64_t mi = row * groups_per_row + (part * EPL) / a.group;
+        sc[u] = load_meta<SCHEME>(a.scale, mi);
+        if constexpr (!Q::sym) zr[u] = load_meta<SCHEME>(a.zero, mi);
       }
     }
 #pragma unroll
-    for (int r = 0; r < REP; ++r) {
-      float d = dot[r];
-      for (int m = 1; m < lanes_per_head; m <<= 1) d += __shfl_xor(d, m, PIKV_WAVE);
-      if ((part % lanes_per_head) == 0)
-        stage[(kvh * REP + r) * kTile + tl] = (n < len) ? d * a.scale_qk : -__builtin_inff();
+    for (int u = 0; u < UN; ++u) {
+      const int tl = s0 + u * tok_per_step + tok_in_step;
+      float cf[EPL];
+      unpack_codes_unsigned<SCHEME>(v[u], cf);
+      const float zu = zr[u] - (float)Q::qmin;  // zero point of the unsigned stored form
+#pragma unroll
+      for (int r = 0; r < REP; ++r) {
+        float d = 0.f;
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) d = fmaf(qv[r][j], cf[j], d);
+        d = (d - zu * qsum[r]) * sc[u];
+        for (int m = 1; m < lanes_per_head; m <<= 1) d += __shfl_xor(d, m, PIKV_WAVE);
+        if ((part % lanes_per_head) == 0 && tl < kTile)
+          stage[(kvh * REP + r) * kTile + tl] = ok[u] ? d * a.scale_qk : -__builtin_inff();
+      }
     }
   }
   __syncthreads();

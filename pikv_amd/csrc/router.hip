@@ -286,18 +286,31 @@ __global__ __launch_bounds__(256) void slot_hist_kernel(const int32_t* __restric
   if ((int)threadIdx.x < E) ws[(int64_t)blockIdx.x * E + threadIdx.x] = hist[threadIdx.x];
 }
 
-// One thread per expert: exclusive scan of the per-chunk histograms, in place.
-__global__ void slot_scan_kernel(int32_t* __restrict__ ws, int64_t n_chunks, int E,
-                                 int32_t* __restrict__ count) {
-  const int e = threadIdx.x;
-  if (e >= E) return;
-  int run = 0;
-  for (int64_t b = 0; b < n_chunks; ++b) {
+// One wavefront per expert: exclusive scan of the per-chunk histograms, in place.
+// Lane l owns a contiguous run of chunks; the lane totals are scanned across the
+// wavefront with shuffles, so the chain of dependent global loads is n_chunks/64
+// long instead of n_chunks.
+__global__ __launch_bounds__(64) void slot_scan_kernel(int32_t* __restrict__ ws, int64_t n_chunks,
+                                                       int E, int32_t* __restrict__ count) {
+  const int e = blockIdx.x;
+  const int lane = threadIdx.x;
+  const int64_t per = (n_chunks + 63) / 64;
+  const int64_t b0 = lane * per;
+  const int64_t b1 = (b0 + per < n_chunks) ? b0 + per : n_chunks;
+  int total = 0;
+  for (int64_t b = b0; b < b1; ++b) total += ws[b * E + e];
+  int incl = total;
+  for (int d = 1; d < 64; d <<= 1) {
+    const int up = __shfl_up(incl, d, PIKV_WAVE);
+    if (lane >= d) incl += up;
+  }
+  int run = incl - total;
+  for (int64_t b = b0; b < b1; ++b) {
     const int v = ws[b * E + e];
     ws[b * E + e] = run;
     run += v;
   }
-  if (count) count[e] = run;
+  if (count && lane == 63) count[e] = incl;
 }
 
 __global__ __launch_bounds__(256) void slot_rank_kernel(const int32_t* __restrict__ idx, int64_t A,
@@ -360,7 +373,7 @@ static int launch_slots(const int32_t* idx, int64_t A, int E, int64_t capacity, 
   if (A == 0) {
     if (count) {
       // count must still be defined: scan over zero chunks writes zeros.
-      hipLaunchKernelGGL(slot_scan_kernel, dim3(1), dim3(64), 0, st, (int32_t*)ws, (int64_t)0, E, count);
+      hipLaunchKernelGGL(slot_scan_kernel, dim3((unsigned)E), dim3(64), 0, st, (int32_t*)ws, (int64_t)0, E, count);
       PIKV_CHECK_LAUNCH();
     }
     return PIKV_OK;
@@ -370,7 +383,7 @@ static int launch_slots(const int32_t* idx, int64_t A, int E, int64_t capacity, 
   const int64_t nb = slot_chunks(A);
   if (nb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
   hipLaunchKernelGGL(slot_hist_kernel, dim3((unsigned)nb), dim3(256), 0, st, idx, A, E, (int32_t*)ws);
-  hipLaunchKernelGGL(slot_scan_kernel, dim3(1), dim3(64), 0, st, (int32_t*)ws, nb, E, count);
+  hipLaunchKernelGGL(slot_scan_kernel, dim3((unsigned)E), dim3(64), 0, st, (int32_t*)ws, nb, E, count);
   hipLaunchKernelGGL(slot_rank_kernel, dim3((unsigned)nb), dim3(256), 0, st, idx, A, E, capacity,
                      (const int32_t*)ws, slot);
   PIKV_CHECK_LAUNCH();
