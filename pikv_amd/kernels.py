@@ -1,0 +1,110 @@
+"""PiKVKernels facade: the reference's kernel-binding class
+(core/single/pikv_kernels.py:20-422) with the same enums, method names, argument
+order and return tuples, dispatching into libpikv_hip.so.
+
+  top_k_routing(routing_logits, k) -> (indices, values)              :54-99
+      the fallback there is torch.topk on the raw logits; ties go to the lower
+      index here (torch's tie order is unspecified).
+  compress_kv(keys, values, mode, lora_params) -> (k', v', meta)       :101-287
+      QUANT8: per-row 8-bit codes.  The facade's own algebra
+      (q = round((x-min)/s), dq = q*s+min, :215-232) is kept for the returned
+      float tensors' meaning; the codes come from the library's asymmetric 8-bit
+      formula (zero point rounded to an integer), see meta['k_codes'].
+      NONE returns the inputs; LORA and MASK are dense/elementwise torch and not
+      part of the native path.
+  evict_cache(keys, values, timestamps, usage, now, policy, window, thr)
+      -> (keys, values, timestamps, usage, new_size)                   :289-422
+      SLIDING keeps rows with now - ts <= window; QUEST keeps rows with
+      ||k|| * usage >= threshold; survivors are compacted in order by
+      pikv_compact_rows.
+Where the reference silently falls back to torch when its library is missing
+(:44-52), this class raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from enum import IntEnum
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _native as N
+from . import ops
+
+
+class CompressionMode(IntEnum):
+    NONE = 0
+    LORA = 1
+    QUANT8 = 2
+    MASK = 3
+
+
+class EvictionPolicy(IntEnum):
+    SLIDING = 0
+    QUEST = 1
+
+
+class PiKVKernels:
+    def __init__(self, lib_path: Optional[str] = None):
+        if lib_path is not None:
+            N.LIB_PATH = lib_path
+        self.lib = N.lib()          # raises if the library is not built
+        self.hip_enabled = True
+
+    # ---- routing ---------------------------------------------------------------
+    def top_k_routing(self, routing_logits: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        out = ops.router_tail(routing_logits.float().contiguous(), top_k=k, use_softmax=False)
+        return out.topk_idx, out.topk_w
+
+    # ---- compression -------------------------------------------------------------
+    def compress_kv(self, keys: torch.Tensor, values: torch.Tensor,
+                    compression_mode: CompressionMode = CompressionMode.QUANT8,
+                    lora_params: Optional[Dict[str, torch.Tensor]] = None):
+        mode = CompressionMode(compression_mode)
+        if mode == CompressionMode.NONE:
+            return keys, values, {"compression_type": "none"}
+        if mode != CompressionMode.QUANT8:
+            raise NotImplementedError(f"{mode.name}: only NONE and QUANT8 run on the native path")
+        n, hidden = keys.shape
+        group = hidden
+        if group & (group - 1) or not (16 <= group <= 1024):
+            raise ValueError("QUANT8 needs a power-of-two row width in [16,1024]")
+        kc, ks, kz = ops.quantize_rows(keys.contiguous(), group, ops.Q_I8_ASYM)
+        vc, vs, vz = ops.quantize_rows(values.contiguous(), group, ops.Q_I8_ASYM)
+        ck = ops.dequantize_rows(kc, ks, kz, group, ops.Q_I8_ASYM)
+        cv = ops.dequantize_rows(vc, vs, vz, group, ops.Q_I8_ASYM)
+        meta = {"compression_type": "quant8", "k_scale": ks, "k_min": -kz * ks, "v_scale": vs,
+                "v_min": -vz * vs, "k_codes": kc, "v_codes": vc, "k_zero": kz, "v_zero": vz}
+        return ck.to(keys.dtype), cv.to(values.dtype), meta
+
+    # ---- eviction ------------------------------------------------------------------
+    def evict_cache(self, keys, values, timestamps, usage_counts, current_time: int,
+                    policy: EvictionPolicy, window_threshold: int = 1024,
+                    quest_threshold: float = 0.1):
+        n, hidden = keys.shape
+        dev = keys.device
+        if dev.type != "cuda":
+            raise ValueError("evict_cache needs GPU tensors; there is no CPU path")
+        if EvictionPolicy(policy) == EvictionPolicy.SLIDING:
+            valid = (current_time - timestamps) <= window_threshold
+        else:
+            valid = torch.linalg.vector_norm(keys.float(), dim=1) * usage_counts >= quest_threshold
+        keep_index = torch.nonzero(valid, as_tuple=False).reshape(-1).to(torch.int32).contiguous()
+        new_size = int(keep_index.numel())
+        if new_size == 0:
+            return keys[:0], values[:0], timestamps[:0], usage_counts[:0], 0
+        planes = [keys.clone().contiguous(), values.clone().contiguous(),
+                  timestamps.clone().contiguous(), usage_counts.clone().contiguous()]
+        if any((p[0].numel() * p.element_size()) % 4 for p in planes):
+            raise ValueError("rows must be a multiple of 4 bytes")
+        # one cache spanning all rows: keep_index is already the ascending survivor list
+        kidx = torch.zeros(n, dtype=torch.int32, device=dev)
+        kidx[:new_size] = keep_index
+        row_base = torch.zeros(1, dtype=torch.int64, device=dev)
+        new_len = torch.tensor([new_size], dtype=torch.int32, device=dev)
+        ptrs = (C.c_void_p * 4)(*[p.data_ptr() for p in planes])
+        rbs = (C.c_int64 * 4)(*[(p[0].numel() if p.dim() > 1 else 1) * p.element_size() for p in planes])
+        N.call("pikv_compact_rows", ptrs, rbs, 4, row_base.data_ptr(), kidx.data_ptr(),
+               new_len.data_ptr(), None, 1, torch.cuda.current_stream().cuda_stream)
+        return (planes[0][:new_size], planes[1][:new_size], planes[2][:new_size],
+                planes[3][:new_size], new_size)

@@ -1,0 +1,249 @@
+"""Routers with the reference's interface (core/single/pikv_routing.py), whose
+tail - last gate Linear, logit scaling / mask, softmax, top-k, renormalisation,
+capacity slots - runs in the fused HIP router.
+
+  BaseRouter ........... :7-161    forward(hidden_states, expert_mask=None)
+                                   -> (dispatch, combine, router_probs, aux_loss)
+  TopKBalancedRouter ... :163-222  (+ entropy / cv / l2 balance term)
+  PiKVRouter ........... :380-549  two gates chosen per token by an importance
+                                   mask, cache-usage correction factor, 5-tuple
+  EPLBRouter ........... :551-735  /temperature then *expert_weights, KL + z loss
+
+The hidden layers of the gate MLPs and the auxiliary losses stay in torch (dense
+GEMMs and scalar reductions); everything after the last hidden activation goes
+through pikv_router_fused / pikv_router_tail.  Capacity slots follow the
+token-major sequential rule of core/single/module/pikv_routing.py:93-104 (the
+vectorised loop of core/single/pikv_routing.py:107-128 gives every token of a
+round the same slot; it is not reproduced).  Ties in the top-k go to the lower
+expert index.
+
+Every forward also accepts return_compact=True and then returns the RouterOut
+(topk_idx, topk_w, slot, count, probs) instead of the dense tensors, which at
+production shapes cannot exist ([T, E, capacity] floats).
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+
+# dense [T, E, capacity] tensors are only built below this many elements
+DENSE_LIMIT = 1 << 28
+
+
+def _dense_dispatch_combine(r: ops.RouterOut, batch_size, seq_len, num_experts, capacity):
+    T = batch_size * seq_len
+    if T * num_experts * max(capacity, 1) > DENSE_LIMIT:
+        raise ValueError(
+            f"dense dispatch/combine tensors of shape [{T},{num_experts},{capacity}] are too large; "
+            "call forward(..., return_compact=True)")
+    dev = r.topk_idx.device
+    disp = torch.zeros(T, num_experts, capacity, device=dev)
+    comb = torch.zeros(T, num_experts, capacity, device=dev)
+    keep = r.slot >= 0
+    t_idx = torch.arange(T, device=dev).unsqueeze(1).expand_as(r.slot)[keep]
+    e_idx = r.topk_idx[keep].long()
+    s_idx = r.slot[keep].long()
+    disp[t_idx, e_idx, s_idx] = 1.0
+    comb[t_idx, e_idx, s_idx] = r.topk_w[keep]
+    return (disp.view(batch_size, seq_len, num_experts, capacity),
+            comb.view(batch_size, seq_len, num_experts, capacity))
+
+
+def _gate_tail(hidden: torch.Tensor, linear: nn.Linear, **kw) -> ops.RouterOut:
+    """hidden [T,H'] (activation before the last Linear) -> fused router."""
+    x = hidden.contiguous()
+    w = linear.weight.detach().to(x.dtype).contiguous()
+    b = None if linear.bias is None else linear.bias.detach().float()
+    return ops.router_fused(x, w, b, **kw)
+
+
+class BaseRouter(nn.Module):
+    def __init__(self, hidden_size: int, num_experts: int, top_k: int = 2,
+                 capacity_factor: float = 1.5, expert_backend: str = "fairscale"):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.num_experts = num_experts
+        self.top_k = min(top_k, num_experts)
+        self.capacity_factor = capacity_factor
+        self.expert_backend = expert_backend
+        self.router = nn.Sequential(nn.Linear(hidden_size, hidden_size), nn.ReLU(),
+                                    nn.Linear(hidden_size, num_experts))
+
+    def _compute_capacity(self, batch_size: int, seq_len: int) -> int:
+        return int(batch_size * seq_len * self.capacity_factor * self.top_k / self.num_experts)
+
+    def _hidden_before_gate(self, seq: nn.Sequential, x2d: torch.Tensor) -> torch.Tensor:
+        h = x2d
+        for layer in list(seq)[:-1]:
+            h = layer(h)
+        return h
+
+    def _route(self, hidden_states, expert_mask=None, *, seq=None, **scale_kw) -> ops.RouterOut:
+        B, S, H = hidden_states.shape
+        seq = self.router if seq is None else seq
+        with torch.no_grad():
+            h = self._hidden_before_gate(seq, hidden_states.reshape(B * S, H))
+        cap = self._compute_capacity(B, S)
+        return _gate_tail(h, seq[-1], top_k=self.top_k, capacity=cap, expert_mask=expert_mask, **scale_kw)
+
+    def _aux_loss(self, router_probs: torch.Tensor) -> torch.Tensor:
+        p = router_probs.mean(dim=[0, 1])
+        return torch.sum(p * torch.log(p * self.num_experts + 1e-9))
+
+    def _finish(self, r, B, S, return_compact):
+        probs = r.probs.view(B, S, self.num_experts)
+        if return_compact:
+            return r, probs
+        disp, comb = _dense_dispatch_combine(r, B, S, self.num_experts, r.capacity)
+        return (disp, comb), probs
+
+    def forward(self, hidden_states: torch.Tensor, expert_mask: Optional[torch.Tensor] = None,
+                return_compact: bool = False):
+        B, S, _ = hidden_states.shape
+        r = self._route(hidden_states, expert_mask)
+        out, probs = self._finish(r, B, S, return_compact)
+        aux = self._aux_loss(probs)
+        if return_compact:
+            return out, probs, aux
+        return out[0], out[1], probs, aux
+
+
+class TopKBalancedRouter(BaseRouter):
+    def __init__(self, hidden_size, num_experts, top_k=2, capacity_factor=1.5,
+                 expert_backend="fairscale", balance_coefficient=0.01, balance_mode="entropy"):
+        super().__init__(hidden_size, num_experts, top_k, capacity_factor, expert_backend)
+        self.balance_coefficient = balance_coefficient
+        self.balance_mode = balance_mode
+
+    def _balance(self, probs):
+        p = probs.mean(dim=[0, 1])
+        if self.balance_mode == "entropy":
+            term = -torch.sum(p * torch.log(p + 1e-9)) / math.log(self.num_experts)
+            return -self.balance_coefficient * term
+        if self.balance_mode == "cv":
+            return self.balance_coefficient * (p.std() / (p.mean() + 1e-9))
+        uniform = torch.ones_like(p) / self.num_experts
+        return self.balance_coefficient * torch.sum((p - uniform) ** 2)
+
+    def forward(self, hidden_states, expert_mask=None, return_compact=False):
+        res = super().forward(hidden_states, expert_mask, return_compact)
+        probs = res[-2]
+        aux = res[-1] + self._balance(probs)
+        return (*res[:-1], aux)
+
+
+class EPLBRouter(BaseRouter):
+    def __init__(self, hidden_size, num_experts, top_k=2, capacity_factor=1.5,
+                 expert_backend="fairscale", balance_coefficient=0.01, temperature=1.0,
+                 use_auxiliary_loss=True, use_z_loss=True, z_loss_coefficient=1e-3):
+        super().__init__(hidden_size, num_experts, top_k, capacity_factor, expert_backend)
+        self.balance_coefficient = balance_coefficient
+        self.temperature = temperature
+        self.use_auxiliary_loss = use_auxiliary_loss
+        self.use_z_loss = use_z_loss
+        self.z_loss_coefficient = z_loss_coefficient
+        self.global_step = 0
+        self.router = nn.Sequential(nn.Linear(hidden_size, hidden_size * 2), nn.GELU(), nn.Dropout(0.1),
+                                    nn.Linear(hidden_size * 2, hidden_size), nn.GELU(), nn.Dropout(0.1),
+                                    nn.Linear(hidden_size, num_experts))
+        self.register_buffer("expert_weights", torch.ones(num_experts))
+
+    def _update_expert_weights(self, expert_usage):
+        # core/single/pikv_routing.py:628-640 (the "momentum" there is the identity)
+        self.expert_weights = expert_usage.mean() / (expert_usage + 1e-8)
+
+    def forward(self, hidden_states, expert_mask=None, return_compact=False):
+        B, S, _ = hidden_states.shape
+        B_S = B * S
+        # /temperature, then *expert_weights, then mask: the order of :653-660
+        seq = self.router
+        with torch.no_grad():
+            h = self._hidden_before_gate(seq, hidden_states.reshape(B_S, -1))
+        cap = self._compute_capacity(B, S)
+        r = ops.router_fused(h.contiguous(), seq[-1].weight.detach().to(h.dtype).contiguous(),
+                             seq[-1].bias.detach().float(), top_k=self.top_k, capacity=cap,
+                             expert_scale=self.expert_weights, expert_mask=expert_mask,
+                             temperature=self.temperature, return_logits=True)
+        out, probs = self._finish(r, B, S, return_compact)
+        aux = torch.zeros((), device=probs.device)
+        usage = r.count.float()
+        if self.use_auxiliary_loss:
+            u = usage / (B_S * self.top_k)
+            kl = F.kl_div(torch.log(u + 1e-8), torch.full_like(u, 1.0 / self.num_experts), reduction="sum")
+            aux = aux + self.balance_coefficient * kl
+        if self.use_z_loss:
+            aux = aux + self.z_loss_coefficient * torch.mean(torch.logsumexp(r.logits, dim=-1) ** 2)
+        self._update_expert_weights(usage)
+        self.global_step += 1
+        if return_compact:
+            return out, probs, aux
+        return out[0], out[1], probs, aux
+
+
+class AdaptiveRouter(BaseRouter):
+    """core/single/pikv_routing.py:224-377: importance predictor + two gates."""
+
+    def __init__(self, hidden_size, num_experts, top_k=2, capacity_factor=1.5,
+                 expert_backend="fairscale", imp_threshold=0.5):
+        super().__init__(hidden_size, num_experts, top_k, capacity_factor, expert_backend)
+        self.importance_predictor = nn.Sequential(nn.Linear(hidden_size, hidden_size // 2), nn.ReLU(),
+                                                  nn.Linear(hidden_size // 2, 1), nn.Sigmoid())
+        self.imp_threshold = imp_threshold
+        mk = lambda: nn.Sequential(nn.Linear(hidden_size, hidden_size), nn.ReLU(),
+                                   nn.Linear(hidden_size, num_experts))
+        self.router_important = mk()
+        self.router_unimportant = mk()
+
+    def _two_gate_route(self, hidden_states, importance, expert_mask, expert_scale=None):
+        B, S, H = hidden_states.shape
+        x2 = hidden_states.reshape(B * S, H)
+        with torch.no_grad():
+            la = self.router_important(x2).float().contiguous()
+            lb = self.router_unimportant(x2).float().contiguous()
+        sel = (importance.reshape(-1) > self.imp_threshold)
+        cap = self._compute_capacity(B, S)
+        return ops.router_tail(la, top_k=self.top_k, capacity=cap, logits_b=lb, select=sel,
+                               expert_scale=expert_scale, expert_mask=expert_mask)
+
+
+class PiKVRouter(AdaptiveRouter):
+    def __init__(self, hidden_size, num_experts, top_k=2, capacity_factor=1.5,
+                 expert_backend="fairscale", imp_threshold=0.5, cache_update_interval=100):
+        super().__init__(hidden_size, num_experts, top_k, capacity_factor, expert_backend, imp_threshold)
+        self.register_buffer("cache_usage_history", torch.zeros(num_experts))
+        self.kv_importance_model = nn.Sequential(nn.Linear(hidden_size, hidden_size // 2), nn.ReLU(),
+                                                 nn.Linear(hidden_size // 2, 1), nn.Sigmoid())
+        self.cache_correction_factor = nn.Parameter(torch.ones(num_experts))
+        self.register_buffer("update_counter", torch.tensor(0))
+        self.cache_update_interval = cache_update_interval
+
+    def update_cache_usage(self, usage_vector: torch.Tensor):
+        self.cache_usage_history = 0.9 * self.cache_usage_history + 0.1 * usage_vector
+        self.update_counter += 1
+        if self.update_counter % self.cache_update_interval == 0:
+            f = 1.0 / (self.cache_usage_history + 0.5)
+            self.cache_correction_factor.data = f / f.mean()
+
+    def forward(self, hidden_states, kv_states=None, expert_mask=None, return_compact=False):
+        B, S, _ = hidden_states.shape
+        importance = self.importance_predictor(hidden_states)
+        if kv_states is not None:
+            importance = (importance + self.kv_importance_model(kv_states)) / 2
+        r = self._two_gate_route(hidden_states, importance.detach(), expert_mask,
+                                 expert_scale=self.cache_correction_factor.detach())
+        out, probs = self._finish(r, B, S, return_compact)
+        usage = probs.sum(dim=[0, 1])
+        usage_norm = usage / usage.sum()
+        self.update_cache_usage(usage_norm.detach())
+        p = probs.mean(dim=[0, 1])
+        aux = torch.sum(p * torch.log(p * self.num_experts + 1e-9))
+        aux = aux + 0.05 * torch.sum(self.cache_usage_history * usage_norm)
+        if return_compact:
+            return out, probs, aux, importance
+        return out[0], out[1], probs, aux, importance

@@ -1,0 +1,241 @@
+"""GPU tests of the host-side mirror of the reference's Python interface: same
+constructors, argument meaning, return arity / shapes / dtypes and error
+behaviour, with results checked against the oracle."""
+import numpy as np
+import pytest
+
+import pikv_oracle as O
+from util import np_of, rng
+
+pytestmark = pytest.mark.gpu
+
+
+def _mlp_hidden(seq, x2d):
+    import torch
+    h = x2d
+    with torch.no_grad():
+        for layer in list(seq)[:-1]:
+            h = layer(h)
+    return h
+
+
+def test_base_and_balanced_router_dense_outputs(dev):
+    """Config-0 shape: batch 2 x seq 64, hidden 256, 4 experts top-2, cf 1.5."""
+    import torch
+    from pikv_amd.routing import BaseRouter, TopKBalancedRouter
+    torch.manual_seed(0)
+    for cls in (BaseRouter, TopKBalancedRouter):
+        r = cls(256, 4, top_k=2, capacity_factor=1.5).to(dev)
+        for lin in (r.router[0], r.router[2]):
+            torch.nn.init.normal_(lin.weight, std=0.02)
+        x = torch.randn(2, 64, 256, device=dev)
+        disp, comb, probs, aux = r(x)
+        cap = O.compute_capacity(2, 64, 1.5, 2, 4)
+        assert cap == 96
+        assert disp.shape == (2, 64, 4, cap) and comb.shape == disp.shape and probs.shape == (2, 64, 4)
+        h = _mlp_hidden(r.router, x.reshape(128, 256)).cpu().numpy()
+        w = r.router[2].weight.detach().cpu().numpy()
+        b = r.router[2].bias.detach().cpu().numpy()
+        p_ref, idx, wts, _ = O.router_tail(O.gate_logits(h, w, b), 2)
+        slot, count = O.capacity_slots(idx, 4, cap)
+        d_ref, c_ref = O.dense_dispatch_combine(idx, wts, slot, 4, cap)
+        assert np.allclose(np_of(probs).reshape(128, 4), p_ref, atol=1e-5)
+        assert np.array_equal(np_of(disp).reshape(128, 4, cap), d_ref)
+        assert np.allclose(np_of(comb).reshape(128, 4, cap), c_ref, atol=1e-5)
+        pm = p_ref.reshape(128, 4).mean(0)
+        base = float(np.sum(pm * np.log(pm * 4 + 1e-9)))
+        if cls is TopKBalancedRouter:
+            ent = -np.sum(pm * np.log(pm + 1e-9)) / np.log(4)
+            base += -0.01 * ent
+        assert abs(float(aux) - base) < 1e-4
+        # compact form
+        out, probs2, _ = r(x, return_compact=True)
+        assert np.array_equal(np_of(out.topk_idx), idx) and np.array_equal(np_of(out.slot), slot)
+        # expert mask: masked experts get no tokens
+        mask = torch.tensor([1.0, 0.0, 1.0, 1.0], device=dev)
+        out, _, _ = r(x, expert_mask=mask, return_compact=True)
+        assert (np_of(out.topk_idx) != 1).all()
+
+
+def test_eplb_and_pikv_router(dev):
+    import torch
+    from pikv_amd.routing import EPLBRouter, PiKVRouter
+    torch.manual_seed(1)
+    r = EPLBRouter(128, 8, top_k=2, temperature=0.7).to(dev).eval()
+    x = torch.randn(2, 32, 128, device=dev)
+    r.expert_weights = torch.linspace(0.5, 1.5, 8, device=dev)
+    ew = r.expert_weights.clone()
+    disp, comb, probs, aux = r(x)
+    h = _mlp_hidden(r.router, x.reshape(64, 128)).cpu().numpy()
+    lg = O.gate_logits(h, r.router[-1].weight.detach().cpu().numpy(), r.router[-1].bias.detach().cpu().numpy())
+    p_ref, idx, wts, _ = O.router_tail(lg, 2, temperature=0.7, expert_scale=ew.cpu().numpy())
+    assert np.allclose(np_of(probs).reshape(64, 8), p_ref, atol=1e-5)
+    cap = O.compute_capacity(2, 32, 1.5, 2, 8)
+    slot, count = O.capacity_slots(idx, 8, cap)
+    d_ref, _ = O.dense_dispatch_combine(idx, wts, slot, 8, cap)
+    assert np.array_equal(np_of(disp).reshape(64, 8, cap), d_ref)
+    # expert_weights updated from usage: mean / (usage + 1e-8)
+    usage = count.astype(np.float32)
+    assert np.allclose(np_of(r.expert_weights), usage.mean() / (usage + 1e-8), rtol=1e-5)
+    assert r.global_step == 1 and float(aux) == float(aux)
+
+    p = PiKVRouter(128, 4, top_k=2).to(dev).eval()
+    with torch.no_grad():
+        p.cache_correction_factor.copy_(torch.tensor([1.0, 0.5, 2.0, 1.0]))
+    x = torch.randn(2, 16, 128, device=dev)
+    disp, comb, probs, aux, imp = p(x, kv_states=torch.randn(2, 16, 128, device=dev))
+    assert imp.shape == (2, 16, 1) and disp.shape[:3] == (2, 16, 4)
+    x2 = x.reshape(32, 128)
+    with torch.no_grad():
+        la = p.router_important(x2).cpu().numpy()
+        lb = p.router_unimportant(x2).cpu().numpy()
+    sel = (np_of(imp).reshape(-1) > 0.5)
+    p_ref, idx, _, _ = O.router_tail(la, 2, logits_b=lb, select=sel,
+                                     expert_scale=np.array([1.0, 0.5, 2.0, 1.0], np.float32))
+    assert np.allclose(np_of(probs).reshape(32, 4), p_ref, atol=1e-5)
+    assert int(p.update_counter) == 1
+
+
+def test_quantized_compressor(dev):
+    import torch
+    from pikv_amd.compression import QuantizedCompressor
+    r = rng(3)
+    c = QuantizedCompressor(256, bits=8, group_size=128).to(dev)
+    k = torch.from_numpy(r.standard_normal((4, 32, 256)).astype(np.float32)).to(dev)
+    v = torch.from_numpy(r.standard_normal((4, 32, 256)).astype(np.float32)).to(dev)
+    dk, dv = c(k, v)
+    assert dk.shape == k.shape and dk.dtype == k.dtype
+    ref_k, _, mse_k = O.fakequant_colblocks(np_of(k).reshape(-1, 256), 128)
+    ref_v, _, mse_v = O.fakequant_colblocks(np_of(v).reshape(-1, 256), 128)
+    assert np.array_equal(np_of(dk).reshape(-1, 256), ref_k)
+    assert np.array_equal(np_of(dv).reshape(-1, 256), ref_v)
+    st = c.get_compression_stats()
+    assert set(st) == {"compression_ratio", "memory_reduction", "bits", "quantization_error",
+                       "group_size", "num_samples"}
+    assert st["compression_ratio"] == 0.25 and abs(st["quantization_error"] - mse_v[-1]) < 1e-8
+    assert st["num_samples"] == 4            # two column blocks for keys, two for values
+    q, dq, scale = c._quantize(k[0])
+    ref, stats, _ = O.fakequant_colblocks(np_of(k[0]).reshape(1, -1), k[0].numel())
+    assert np.array_equal(np_of(dq).reshape(1, -1), ref) and float(scale) == stats[0, 2]
+    assert float(q.min()) >= 0 and float(q.max()) <= 255
+    # integer-code interface
+    codes, s, z = c.quantize(k, granularity="token_head", head_dim=64)
+    q_ref, s_ref, z_ref = O.quantize_groups(np_of(k).reshape(-1, 256), 64, O.Q_I8_ASYM)
+    assert np.array_equal(np_of(codes).astype(np.int16), q_ref) and np.array_equal(np_of(s), s_ref)
+    back = c.dequantize(codes, s, z, granularity="token_head", head_dim=64)
+    assert np.array_equal(np_of(back), O.dequantize_groups(q_ref, s_ref, z_ref, 64))
+    with pytest.raises(ValueError):
+        QuantizedCompressor(256, bits=3)
+
+
+def test_schedulers_select(dev):
+    import torch
+    from pikv_amd.scheduling import H2OScheduler, LRUScheduler
+    r = rng(4)
+    h = H2OScheduler(64, 32, heavy_ratio=0.25, recent_ratio=0.1).to(dev)
+    idx = torch.arange(50, device=dev)
+    w = torch.from_numpy((np.round(r.random(50) * 4) / 4).astype(np.float32)).to(dev)
+    h.update_attention_scores(idx, w)
+    h.update_attention_scores(idx[:10], w[:10])
+    keys = torch.zeros(50, 32, device=dev)
+    mask = h.select_eviction_candidates(keys, keys, {})
+    nh, nr = O.h2o_budget(50, 0.25, 0.1)
+    keep = O.h2o_keep(np_of(h.attention_accumulator)[:50], np_of(h.access_timestamps)[:50], nh, nr)
+    assert mask.dtype == torch.bool and np.array_equal(np_of(mask), ~keep)
+    l = LRUScheduler(40, 32).to(dev)
+    for t in range(5):
+        l.update_access_time(torch.from_numpy(r.permutation(40)[:20]).to(dev))   # indices inside the 40-entry table
+    m = l.select_eviction_candidates(keys, keys, {})
+    # 50 rows shown to a 40-row scheduler: rows beyond its table count as never accessed
+    times = np.concatenate([np_of(l.access_times), np.zeros(10, np.float32)])
+    assert np.array_equal(np_of(m), ~O.lru_keep(times, 10))
+    assert not np_of(l.select_eviction_candidates(keys[:40], keys[:40], {})).any()
+
+
+@pytest.mark.parametrize("policy_name", ["LRU", "H2O"])
+def test_cache_scheduling_manager(dev, policy_name):
+    """Cache of 128 rows x 256, int8 symmetric per token (the config-0 cache)."""
+    import torch
+    from pikv_amd.scheduling import CacheSchedulingManager, SchedulingPolicy
+    r = rng(6)
+    policy = SchedulingPolicy[policy_name]
+    m = CacheSchedulingManager(128, 256, policy, heavy_ratio=0.25, recent_ratio=0.125)
+    ref = O.CachePool([128], 256, 256, O.Q_I8_SYM)
+    t = 0
+    evicted = 0
+    for step in range(5):
+        k = r.standard_normal((2, 24, 256)).astype(np.float32)
+        v = r.standard_normal((2, 24, 256)).astype(np.float32)
+        m.update_cache(torch.from_numpy(k).to(dev), torch.from_numpy(v).to(dev))
+        n, cur = 48, int(ref.fill[0])
+        if cur + n > 128:
+            rows = ref.valid_rows(0)
+            if policy_name == "H2O":
+                nh, nr = O.h2o_budget(cur, 0.25, 0.125)
+                keep = O.h2o_keep(ref.acc[rows], ref.ts[rows], nh, nr)
+            else:
+                keep = O.lru_keep(ref.ts[rows], cur + n - 128)
+            planes = [ref.k_codes, ref.k_scale, ref.k_zero, ref.v_codes, ref.v_scale, ref.v_zero, ref.acc, ref.ts]
+            new = O.compact(keep, *[p[:cur] for p in planes])
+            evicted += cur - new
+            ref.fill[0] = new
+        t += 1
+        ref.quant_scatter(k.reshape(-1, 256), v.reshape(-1, 256), np.zeros(n, np.int32),
+                          np.arange(n, dtype=np.int32), 1, now=float(t))
+        ref.advance([n])
+        st = m.get_cache_stats()
+        assert st["cache_size"] == int(ref.fill[0]) and st["policy"] == policy.value
+        assert st["eviction_count"] == evicted
+        rows = ref.valid_rows(0)
+        want = O.dequantize_groups(ref.k_codes[rows], ref.k_scale[rows], ref.k_zero[rows], 256)
+        assert np.array_equal(np_of(m.cache_keys)[:len(rows)], want)
+    assert set(st) == {"cache_size", "cache_utilization", "policy", "hit_rate", "eviction_count"}
+    m.reset_cache()
+    assert m.get_cache_stats()["cache_size"] == 0
+    m.change_policy(SchedulingPolicy.NONE)
+    m.update_cache(torch.zeros(1, 1, 256, device=dev), torch.zeros(1, 1, 256, device=dev))
+    assert m.get_cache_stats()["cache_size"] == 0     # no policy: update is a no-op, as in the reference
+    with pytest.raises(ValueError):
+        CacheSchedulingManager(8, 256, "bogus")
+
+
+def test_kernels_facade(dev):
+    import torch
+    from pikv_amd.kernels import CompressionMode, EvictionPolicy, PiKVKernels
+    r = rng(8)
+    K = PiKVKernels()
+    lg = r.standard_normal((32, 64)).astype(np.float32)
+    idx, val = K.top_k_routing(torch.from_numpy(lg).to(dev), 8)
+    _, i_ref, v_ref, _ = O.router_tail(lg, 8, use_softmax=False)
+    assert np.array_equal(np_of(idx), i_ref) and np.array_equal(np_of(val), v_ref)
+    keys = r.standard_normal((32, 512)).astype(np.float32)
+    vals = r.standard_normal((32, 512)).astype(np.float32)
+    ck, cv, meta = K.compress_kv(torch.from_numpy(keys).to(dev), torch.from_numpy(vals).to(dev),
+                                 CompressionMode.QUANT8)
+    q_ref, s_ref, z_ref = O.quantize_groups(keys, 512, O.Q_I8_ASYM)
+    assert meta["compression_type"] == "quant8"
+    assert np.array_equal(np_of(meta["k_codes"]).astype(np.int16), q_ref)
+    assert np.array_equal(np_of(ck), O.dequantize_groups(q_ref, s_ref, z_ref, 512))
+    assert np.abs(np_of(ck) - keys).max() <= s_ref.max() * 0.51
+    # eviction: sliding window, stable compaction
+    n = 2048
+    keys = r.standard_normal((n, 512)).astype(np.float32)
+    vals = r.standard_normal((n, 512)).astype(np.float32)
+    ts = r.integers(0, 1000, n).astype(np.float32)
+    use = r.integers(1, 10, n).astype(np.float32)
+    out = K.evict_cache(*[torch.from_numpy(a).to(dev) for a in (keys, vals, ts, use)], 1000,
+                        EvictionPolicy.SLIDING, window_threshold=600)
+    valid = (1000 - ts) <= 600
+    assert out[4] == valid.sum()
+    assert np.array_equal(np_of(out[0]), keys[valid]) and np.array_equal(np_of(out[1]), vals[valid])
+    assert np.array_equal(np_of(out[2]), ts[valid]) and np.array_equal(np_of(out[3]), use[valid])
+    score = np.linalg.norm(keys.astype(np.float64), axis=1) * use
+    srt = np.sort(score)
+    gap = np.argmax(np.diff(srt[900:1100])) + 900          # threshold inside the widest nearby gap
+    thr = float((srt[gap] + srt[gap + 1]) / 2)
+    out = K.evict_cache(*[torch.from_numpy(a).to(dev) for a in (keys, vals, ts, use)], 1000,
+                        EvictionPolicy.QUEST, quest_threshold=thr)
+    valid = score >= thr
+    assert out[4] == valid.sum() and np.array_equal(np_of(out[0]), keys[valid])
+    with pytest.raises(NotImplementedError):
+        K.compress_kv(torch.zeros(4, 64, device=dev), torch.zeros(4, 64, device=dev), CompressionMode.LORA)
