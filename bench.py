@@ -30,6 +30,11 @@ sys.path.insert(0, ROOT)
 
 METRIC = "routed KV tokens/s (quant+scatter+gather+dequant), 1 MI355X; % HBM peak"
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the quantise+scatter kernel on this workload, from the
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
+# profiles/bench_prefill_compress_write.md (counters scaled by what a plain 1 GiB
+# device copy reads on them: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
+K2_TRAFFIC_BYTES_PROFILED = 1099.1e6
 
 WORKLOAD = dict(name="prefill compress-write", batch=16, seq=2048, hidden=4096, experts=8, top_k=2,
                 capacity_factor=1.25, heads=32, head_dim=128, cache_slots=8192,
@@ -55,7 +60,7 @@ def make_inputs(torch, dev, w):
     return hidden, gate_w, kv[0], kv[1], q
 
 
-def cpu_baseline(torch, w, hidden, gate_w, k_src, v_src, q, reps=2):
+def cpu_baseline(torch, w, hidden, gate_w, k_src, v_src, q, reps=5):
     """Time the C restatement of the same step on the host (all of the batch)."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import numpy as np
@@ -93,6 +98,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain 1 GiB device copy (a kernel of known traffic, to scale "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -105,6 +113,16 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
+    if args.calibrate_copy:
+        n = 1 << 30
+        src = torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": n, "calibrate_copy_bytes_written": n,
+                          "kernel": "torch elementwise copy (5 launches)"}))
+        return
     w = WORKLOAD
     T, E, k = w["batch"] * w["seq"], w["experts"], w["top_k"]
     heads, dh = w["heads"], w["head_dim"]
@@ -161,7 +179,7 @@ def main():
                    "kept_assignments": kept, "assignments": A},
         "roofline": {"bound": "hbm", "kernel": "quant_scatter_kernel<I8_SYM,bf16>",
                      "achieved": gbps(b_quant, t_quant), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": gbps(b_quant, t_quant) / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": gbps(b_quant, t_quant) / HBM_PEAK_GBPS, "traffic": K2_TRAFFIC_BYTES_PROFILED,
                      "algorithmic_bytes": b_quant, "avg_launch_ms": t_quant},
         "kernels": {
             "router": {"ms": t_router, "GBps": gbps(b_router, t_router)},
