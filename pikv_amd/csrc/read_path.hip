@@ -191,6 +191,356 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   }
 }
 
+// ---- 4-bit scores on the matrix cores ------------------------------------------------
+// The VALU kernel above is instruction-bound for grouped 4-bit caches read by
+// several query heads per kv head (decode, GQA): 4 heads x 128 dims per cached
+// token-head against a budget of ~4 instructions per element at the HBM rate
+// (measured: 1.18 ms where HBM allows 0.24 ms).  Here the contraction over a
+// 32-element quantisation group is one v_mfma_f32_16x16x32_bf16:
+//   A (16 x 32) = the query heads of one kv head (rows >= rep are zero),
+//   B (32 x 16) = the codes of one group for 16 cached tokens, expanded to bf16
+//                 as 0x4300|u = 128 + u (exact), u = unsigned stored code,
+//   C           = 128*Qs + sum q*u per (head, token); the group scale and zero
+//                 point are applied in the epilogue:
+//                 s * (C - (z + bias) * Qs),  Qs = sum of q over the group.
+// Loads stay 16 bytes per lane and contiguous: lane (token n, j) fetches group j
+// of its token, and a 4x4 transpose across the four 16-lane rows
+// (v_permlane16_swap / v_permlane32_swap) hands lane (n, kg) the k-slice kg of
+// every group, which is the operand layout the MFMA wants.
+typedef __bf16 pikv_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float pikv_f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void transpose4x4_rows(uint32_t (&v)[4]) {
+  auto a = __builtin_amdgcn_permlane16_swap(v[0], v[1], false, false);
+  auto b = __builtin_amdgcn_permlane16_swap(v[2], v[3], false, false);
+  auto c = __builtin_amdgcn_permlane32_swap(a[0], b[0], false, false);
+  auto d = __builtin_amdgcn_permlane32_swap(a[1], b[1], false, false);
+  v[0] = c[0]; v[2] = c[1]; v[1] = d[0]; v[3] = d[1];
+}
+
+template <int SCHEME>
+__global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
+  using Q = QScheme<SCHEME>;
+  static_assert(Q::bits == 4, "4-bit schemes only");
+  __shared__ float stage[kMaxQHeads * kTile];  // [q head][token in tile]
+  __shared__ float qs[kMaxQHeads * 4];         // sum of q over each 32-wide group
+
+  const int c = blockIdx.y;
+  const int64_t tile = blockIdx.x;
+  const int len = a.fill[c];
+  const int64_t n0 = tile * kTile;
+  if (n0 >= len) return;  // uniform for the block
+  const int rep = a.n_q_heads / a.n_kv_heads;
+  const int lanes_per_row = a.n_kv_heads * 4;   // 16-byte groups per cached row
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nl = lane & 15;   // token column / query-head row
+  const int rg = lane >> 4;   // group fetched by this lane; k-slice after the transpose
+  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * 128;
+
+  // Group sums of the query (float32), one (head, group) pair per thread.
+  for (int i = threadIdx.x; i < a.n_q_heads * 4; i += 256) {
+    const uint16_t* qp = qbase + (int64_t)(i >> 2) * 128 + (i & 3) * 32;
+    float sacc = 0.f;
+    for (int k = 0; k < 32; ++k) sacc += bf16_bits_to_float(qp[k]);
+    qs[i] = sacc;
+  }
+  __syncthreads();
+
+  const float zbias = 128.0f - (float)Q::qmin;  // 128 (asymmetric) or 136 (symmetric)
+  const int64_t base_row = a.row_base[c];
+
+  for (int g = wave; g < a.n_kv_heads; g += 4) {
+    // A operands of this kv head: lane (row m = nl, k-slice rg) of group gq holds
+    // q[g*rep + m][32*gq + 8*rg + {0,4,1,5,2,6,3,7}] - the element order in which
+    // the codes come out of the nibble expansion below.
+    pikv_bf16x8 amat[4];
+    float qsum[4][4];  // [gq][i] for C rows 4*rg + i
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      uint4 d = make_uint4(0, 0, 0, 0);
+      if (nl < rep) d = ld16(qbase + (int64_t)(g * rep + nl) * 128 + gq * 32 + rg * 8);
+      const uint4 p = make_uint4((d.x & 0xffffu) | (d.z << 16), (d.x >> 16) | (d.z & 0xffff0000u),
+                                 (d.y & 0xffffu) | (d.w << 16), (d.y >> 16) | (d.w & 0xffff0000u));
+      amat[gq] = __builtin_bit_cast(pikv_bf16x8, p);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 4 * rg + i;
+        qsum[gq][i] = (r < rep) ? qs[(g * rep + r) * 4 + gq] : 0.f;
+      }
+    }
+    // All four 16-token slices of the tile are fetched before any of them is used:
+    // four 16-byte loads (plus metadata) in flight per lane.
+    constexpr int NTG = kTile / 16;
+    uint32_t v[NTG][4], meta1[NTG];
+    bool ok[NTG];
+#pragma unroll
+    for (int tg = 0; tg < NTG; ++tg) {
+      const int64_t n = n0 + tg * 16 + nl;
+      ok[tg] = n < len;
+      v[tg][0] = v[tg][1] = v[tg][2] = v[tg][3] = 0;
+      meta1[tg] = 0;
+      if (ok[tg]) {
+        const int64_t gi = (base_row + n) * lanes_per_row + g * 4 + rg;
+        const uint4 cv = ld16(reinterpret_cast<const char*>(a.codes) + gi * 16);
+        v[tg][0] = cv.x; v[tg][1] = cv.y; v[tg][2] = cv.z; v[tg][3] = cv.w;
+        uint32_t m = reinterpret_cast<const uint16_t*>(a.scale)[gi];
+        if constexpr (!Q::sym) m |= (uint32_t) reinterpret_cast<const uint16_t*>(a.zero)[gi] << 16;
+        meta1[tg] = m;
+      }
+    }
+#pragma unroll
+    for (int tg = 0; tg < NTG; ++tg) {
+      const int tl = tg * 16 + nl;
+      uint32_t meta[4] = {meta1[tg], meta1[tg], meta1[tg], meta1[tg]};
+      transpose4x4_rows(v[tg]);  // v[gq] = k-slice rg of group gq of token nl
+      transpose4x4_rows(meta);   // meta[gq] = (scale, zero) of group gq of token nl
+      pikv_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
+        const uint32_t w = Q::sym ? (v[tg][gq] ^ 0x88888888u) : v[tg][gq];
+        const uint4 b = make_uint4((w & 0x000f000fu) | 0x43004300u, ((w >> 4) & 0x000f000fu) | 0x43004300u,
+                                   ((w >> 8) & 0x000f000fu) | 0x43004300u,
+                                   ((w >> 12) & 0x000f000fu) | 0x43004300u);
+        const pikv_f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+        const pikv_f32x4 pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            amat[gq], __builtin_bit_cast(pikv_bf16x8, b), zero4, 0, 0, 0);
+        const _Float16 sh = __builtin_bit_cast(_Float16, (uint16_t)(meta[gq] & 0xffffu));
+        const _Float16 zh = __builtin_bit_cast(_Float16, (uint16_t)(meta[gq] >> 16));
+        const float sc = (float)sh;
+        const float zq = (Q::sym ? 0.f : (float)zh) + zbias;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = fmaf(sc, fmaf(-zq, qsum[gq][i], pc[i]), acc[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 4 * rg + i;
+        if (r < rep) stage[(g * rep + r) * kTile + tl] = ok[tg] ? acc[i] * a.scale_qk : -__builtin_inff();
+      }
+    }
+  }
+  __syncthreads();
+
+  for (int hq = wave; hq < a.n_q_heads; hq += 4) {
+    const float sv = stage[hq * kTile + lane];
+    const bool ok = n0 + lane < len;
+    if (ok) a.scores[((int64_t)c * a.n_q_heads + hq) * a.score_stride + n0 + lane] = sv;
+    const float m = group_max<64>(ok ? sv : -__builtin_inff());
+    const float e = ok ? expf(sv - m) : 0.f;
+    const float sum = group_sum<64>(e);
+    if (lane == 0) {
+      const int64_t ti = ((int64_t)c * a.n_q_heads + hq) * a.n_tiles + tile;
+      a.tile_max[ti] = m;
+      a.tile_sum[ti] = sum;
+    }
+  }
+}
+
+// Variant for at most 4 query heads per kv head (the usual GQA ratios), where the
+// layout above leaves 12 of the 16 tile rows empty.  Here the 16 rows are
+// (group gq, head r) and the A operand is block-diagonal in the k-slices: the
+// k-slice kg of MFMA #b multiplies q[r][32*gq + 8*b ..] only in rows with gq == kg.
+// Four MFMAs accumulate into one tile that holds, in row-group rg, the partial dot
+// products of group rg for the lane's own token - so every lane uses the codes and
+// the (scale, zero) it loaded itself: no transpose, one epilogue per 16 tokens
+// instead of one per MFMA, and a 3-swap transpose-reduction over the four
+// row-groups leaves row-group r with the finished score of head r.
+constexpr int kGqaTilesPerBlock = 4;   // consecutive 64-token tiles handled by one block
+constexpr int kGqaMaxKvHeads = 16;     // code vectors of one 16-token slice kept in registers
+
+// LDS bytes of scores_mfma_i4_gqa_kernel: score staging, query sums, compact A
+// operands, and the (scale, zero) rows of one tile.
+static size_t gqa_lds_bytes(int n_q_heads, int n_kv_heads) {
+  return (size_t)n_q_heads * (kTile + 4) * sizeof(float) + (size_t)n_kv_heads * 4 * 16 * 16 +
+         2 * (size_t)kTile * (n_kv_heads * 4 + 2) * sizeof(uint16_t);
+}
+
+// A wavefront owns one 16-token slice of the tile and walks over ALL kv heads, so
+// its loads cover 16 whole cached rows (n_kv_heads * 64 contiguous bytes each),
+// issued back to back - HBM sees complete rows instead of 64-byte pieces that are
+// revisited later.  The next tile's rows are prefetched while the current ones are
+// multiplied.
+template <int SCHEME, int NKV>  // NKV = n_kv_heads rounded up to 4/8/16
+__global__ __launch_bounds__(256) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
+  using Q = QScheme<SCHEME>;
+  static_assert(Q::bits == 4, "4-bit schemes only");
+  extern __shared__ float gqa_lds[];
+  float* stage = gqa_lds;                            // [q head][token in tile]
+  float* qs = stage + a.n_q_heads * kTile;           // [q head][group]: sum of q over the group
+  uint4* alds = reinterpret_cast<uint4*>(qs + a.n_q_heads * 4);  // [kv head][b][gq*4 + r]
+  const int meta_stride = a.n_kv_heads * 4 + 2;      // halves; +2 spreads the tokens over banks
+  uint16_t* smeta = reinterpret_cast<uint16_t*>(alds + a.n_kv_heads * 64);
+  uint16_t* zmeta = smeta + kTile * meta_stride;
+
+  const int c = blockIdx.y;
+  const int len = a.fill[c];
+  const int64_t tile0 = (int64_t)blockIdx.x * kGqaTilesPerBlock;
+  const int64_t tok0 = tile0 * kTile;
+  if (tok0 >= len) return;  // uniform for the block
+  const int rep = a.n_q_heads / a.n_kv_heads;  // <= 4
+  const int lanes_per_row = a.n_kv_heads * 4;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nl = lane & 15;
+  const int rg = lane >> 4;
+  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * 128;
+  const int64_t base_row = a.row_base[c];
+
+  // Code vectors of this wavefront's slice of tile tt: one 16-byte load per kv head.
+  auto issue = [&](int tt, uint4 (&cv)[NKV]) {
+    const int64_t n = tok0 + tt * kTile + wave * 16 + nl;
+    const bool okn = n < len;
+    const char* rowp = reinterpret_cast<const char*>(a.codes) + ((base_row + n) * lanes_per_row + rg) * 16;
+#pragma unroll
+    for (int g = 0; g < NKV; ++g) {
+      cv[g] = make_uint4(0, 0, 0, 0);
+      if (okn && g < a.n_kv_heads) cv[g] = ld16(rowp + g * 64);
+    }
+  };
+  uint4 cur[NKV], nxt[NKV];
+  issue(0, cur);  // in flight while the prologue runs
+
+  // Prologue: group sums of q, and the non-zero part of the block-diagonal A
+  // operands: entry (g, b, gq, r) = q[g*rep + r][32*gq + 8*b + {0,4,1,5,2,6,3,7}].
+  for (int i = threadIdx.x; i < a.n_q_heads * 4; i += 256) {
+    float h32[32];
+    load_as_float<PIKV_BF16, 32>(qbase, (int64_t)i * 32, h32);
+    float sacc = 0.f;
+#pragma unroll
+    for (int k = 0; k < 32; ++k) sacc += h32[k];
+    qs[i] = sacc;
+  }
+  for (int i = threadIdx.x; i < a.n_kv_heads * 64; i += 256) {
+    const int g = i >> 6, b2 = (i >> 4) & 3, gq = (i >> 2) & 3, r = i & 3;
+    uint4 d = make_uint4(0, 0, 0, 0);
+    if (r < rep) d = ld16(qbase + (int64_t)(g * rep + r) * 128 + gq * 32 + b2 * 8);
+    alds[i] = make_uint4((d.x & 0xffffu) | (d.z << 16), (d.x >> 16) | (d.z & 0xffff0000u),
+                         (d.y & 0xffffu) | (d.w << 16), (d.y >> 16) | (d.w & 0xffff0000u));
+  }
+
+  const float zbias = 128.0f - (float)Q::qmin;  // 128 (asymmetric) or 136 (symmetric)
+  const bool a_on = (nl >> 2) == rg;            // this lane's k-slice meets its row's group
+
+  for (int tt = 0; tt < kGqaTilesPerBlock; ++tt) {
+    const int64_t tile = tile0 + tt;
+    const int64_t n0 = tile * kTile;
+    if (n0 >= len) break;  // uniform
+    // (scale, zero) of the tile: 8-byte loads, one per (token, kv head)
+    for (int ch = threadIdx.x; ch < kTile * a.n_kv_heads; ch += 256) {
+      const int tok = ch / a.n_kv_heads, hd = ch - tok * a.n_kv_heads;
+      uint2 sv = make_uint2(0, 0), zv = make_uint2(0, 0);
+      if (n0 + tok < len) {
+        const int64_t mi = (base_row + n0 + tok) * lanes_per_row + hd * 4;
+        sv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.scale) + mi);
+        if constexpr (!Q::sym) zv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.zero) + mi);
+      }
+      uint32_t* sd = reinterpret_cast<uint32_t*>(smeta + tok * meta_stride + hd * 4);
+      sd[0] = sv.x; sd[1] = sv.y;
+      if constexpr (!Q::sym) {
+        uint32_t* zd = reinterpret_cast<uint32_t*>(zmeta + tok * meta_stride + hd * 4);
+        zd[0] = zv.x; zd[1] = zv.y;
+      }
+    }
+    if ((tt + 1 < kGqaTilesPerBlock) && (n0 + kTile < len)) issue(tt + 1, nxt);
+    __syncthreads();  // metadata (and, first time, qs / alds) visible
+
+    const int tl = wave * 16 + nl;
+    const bool okt = n0 + tl < len;
+#pragma unroll
+    for (int g = 0; g < NKV; ++g) {
+      if (g < a.n_kv_heads) {
+        const uint32_t wv[4] = {cur[g].x, cur[g].y, cur[g].z, cur[g].w};
+        pikv_f32x4 pc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int b2 = 0; b2 < 4; ++b2) {
+          const uint32_t w = Q::sym ? (wv[b2] ^ 0x88888888u) : wv[b2];
+          const uint4 bb = make_uint4((w & 0x000f000fu) | 0x43004300u, ((w >> 4) & 0x000f000fu) | 0x43004300u,
+                                      ((w >> 8) & 0x000f000fu) | 0x43004300u,
+                                      ((w >> 12) & 0x000f000fu) | 0x43004300u);
+          uint4 av = make_uint4(0, 0, 0, 0);
+          if (a_on) av = alds[(g * 4 + b2) * 16 + nl];
+          pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, av),
+                                                       __builtin_bit_cast(pikv_bf16x8, bb), pc, 0, 0, 0);
+        }
+        const int mo = tl * meta_stride + g * 4 + rg;
+        const float sc = (float)__builtin_bit_cast(_Float16, smeta[mo]);
+        const float zq = (Q::sym ? 0.f : (float)__builtin_bit_cast(_Float16, zmeta[mo])) + zbias;
+        float t[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float qsi = (i < rep) ? qs[(g * rep + i) * 4 + rg] : 0.f;
+          t[i] = sc * fmaf(-zq, qsi, pc[i]);
+        }
+        // sum over the four row-groups; row-group r ends with head r
+        auto s01 = __builtin_amdgcn_permlane16_swap(__float_as_uint(t[0]), __float_as_uint(t[1]), false, false);
+        auto s23 = __builtin_amdgcn_permlane16_swap(__float_as_uint(t[2]), __float_as_uint(t[3]), false, false);
+        const float u01 = __uint_as_float(s01[0]) + __uint_as_float(s01[1]);
+        const float u23 = __uint_as_float(s23[0]) + __uint_as_float(s23[1]);
+        auto sf = __builtin_amdgcn_permlane32_swap(__float_as_uint(u01), __float_as_uint(u23), false, false);
+        const float score = (__uint_as_float(sf[0]) + __uint_as_float(sf[1])) * a.scale_qk;
+        if (rg < rep) stage[(g * rep + rg) * kTile + tl] = okt ? score : -__builtin_inff();
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < NKV; ++g) cur[g] = nxt[g];
+    __syncthreads();
+
+    // Tile statistics and score rows, four heads per wavefront pass: lane (rg, nl)
+    // owns tokens nl, nl+16, nl+32, nl+48 of head h4 + rg; the 16 lanes of a row
+    // reduce with DPP.
+    for (int h4 = wave * 4; h4 < a.n_q_heads; h4 += 16) {
+      const int hq = h4 + rg;
+      const bool hok = hq < a.n_q_heads;
+      float x[4];
+      bool okk[4];
+      float m = -__builtin_inff();
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        okk[k] = hok && (n0 + nl + 16 * k < len);
+        x[k] = okk[k] ? stage[hq * kTile + nl + 16 * k] : -__builtin_inff();
+        m = fmaxf(m, x[k]);
+      }
+      PIKV_DPP_INPLACE("v_max_f32_dpp", m, "quad_perm:[1,0,3,2]");
+      PIKV_DPP_INPLACE("v_max_f32_dpp", m, "quad_perm:[2,3,0,1]");
+      PIKV_DPP_INPLACE("v_max_f32_dpp", m, "row_half_mirror");
+      PIKV_DPP_INPLACE("v_max_f32_dpp", m, "row_mirror");
+      float sum = 0.f;
+      float* out = a.scores + ((int64_t)c * a.n_q_heads + (hok ? hq : 0)) * a.score_stride + n0 + nl;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (okk[k]) {
+          sum += __builtin_amdgcn_exp2f((x[k] - m) * 1.4426950408889634f);
+          out[16 * k] = x[k];
+        }
+      }
+      PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "quad_perm:[1,0,3,2]");
+      PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "quad_perm:[2,3,0,1]");
+      PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "row_half_mirror");
+      PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "row_mirror");
+      if (nl == 0 && hok) {
+        const int64_t ti = ((int64_t)c * a.n_q_heads + hq) * a.n_tiles + tile;
+        a.tile_max[ti] = m;
+        a.tile_sum[ti] = sum;
+      }
+    }
+    __syncthreads();  // stage and the metadata rows are reused by the next tile
+  }
+}
+
+template <int SCHEME>
+static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
+  const size_t lds = gqa_lds_bytes(a.n_q_heads, a.n_kv_heads);
+  if (lds > 64 * 1024 || a.n_kv_heads > kGqaMaxKvHeads) return PIKV_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
+  if (a.n_kv_heads <= 4)
+    hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4>), grid, dim3(256), lds, st, a);
+  else if (a.n_kv_heads <= 8)
+    hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8>), grid, dim3(256), lds, st, a);
+  else
+    hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 16>), grid, dim3(256), lds, st, a);
+  return PIKV_OK;
+}
+
 // Final max and sum per (cache, q head) from the tile statistics.
 __global__ __launch_bounds__(64) void head_stats_kernel(const float* __restrict__ tile_max,
                                                         const float* __restrict__ tile_sum,
@@ -345,6 +695,22 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   const dim3 grid((unsigned)n_tiles, (unsigned)n_caches);
   hipStream_t st = (hipStream_t)stream;
   const int rep = n_q_heads / n_kv_heads;
+  // grouped 4-bit caches read with bf16 queries go to the matrix-core kernel
+  if (!eight && group == 32 && head_dim == 128 && q_dtype == PIKV_BF16 && rep <= 16) {
+    int grc = PIKV_ERR_UNSUPPORTED;
+    if (rep <= 4)
+      grc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(a, n_caches, n_tiles, st)
+                                       : launch_gqa<PIKV_Q_I4_SYM>(a, n_caches, n_tiles, st);
+    if (grc == PIKV_OK) {
+      // launched above
+    } else if (scheme == PIKV_Q_I4_ASYM) {
+      hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_ASYM>), grid, dim3(256), 0, st, a);
+    } else {
+      hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_SYM>), grid, dim3(256), 0, st, a);
+    }
+    PIKV_CHECK_LAUNCH();
+    return PIKV_OK;
+  }
   int rc = PIKV_ERR_UNSUPPORTED;
   switch (scheme) {
     case PIKV_Q_I8_SYM: rc = launch_scores<PIKV_Q_I8_SYM>(rep, grid, st, q_dtype, a); break;
