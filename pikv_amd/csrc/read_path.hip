@@ -345,31 +345,40 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 // the (scale, zero) it loaded itself: no transpose, one epilogue per 16 tokens
 // instead of one per MFMA, and a 3-swap transpose-reduction over the four
 // row-groups leaves row-group r with the finished score of head r.
+// (x & m) | o in one instruction (one scalar operand at most per instruction).
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(m), "v"(o));
+  return r;
+}
+
 constexpr int kGqaTilesPerBlock = 4;   // consecutive 64-token tiles handled by one block
 constexpr int kGqaMaxKvHeads = 16;     // code vectors of one 16-token slice kept in registers
 
 // LDS bytes of scores_mfma_i4_gqa_kernel: score staging, query sums, compact A
-// operands, and the (scale, zero) rows of one tile.
+// operands plus an all-zero twin, and the (scale, zero) rows of one tile.
 static size_t gqa_lds_bytes(int n_q_heads, int n_kv_heads) {
-  return (size_t)n_q_heads * (kTile + 4) * sizeof(float) + (size_t)n_kv_heads * 4 * 16 * 16 +
-         2 * (size_t)kTile * (n_kv_heads * 4 + 2) * sizeof(uint16_t);
+  return (size_t)n_q_heads * kTile * sizeof(float) + (size_t)n_kv_heads * 16 * sizeof(float) +
+         2 * (size_t)n_kv_heads * 4 * 16 * 16 + 2 * (size_t)kTile * (n_kv_heads * 4 + 2) * sizeof(uint16_t);
 }
 
 // A wavefront owns one 16-token slice of the tile and walks over ALL kv heads, so
 // its loads cover 16 whole cached rows (n_kv_heads * 64 contiguous bytes each),
 // issued back to back - HBM sees complete rows instead of 64-byte pieces that are
 // revisited later.  The next tile's rows are prefetched while the current ones are
-// multiplied.
+// multiplied (two register sets, used alternately).
 template <int SCHEME, int NKV>  // NKV = n_kv_heads rounded up to 4/8/16
-__global__ __launch_bounds__(256) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 4 : 2))) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
+  static_assert(kGqaTilesPerBlock % 2 == 0, "tiles are processed in pairs");
   extern __shared__ float gqa_lds[];
   float* stage = gqa_lds;                            // [q head][token in tile]
-  float* qs = stage + a.n_q_heads * kTile;           // [q head][group]: sum of q over the group
-  uint4* alds = reinterpret_cast<uint4*>(qs + a.n_q_heads * 4);  // [kv head][b][gq*4 + r]
+  float4* qs4 = reinterpret_cast<float4*>(stage + a.n_q_heads * kTile);  // [kv head][group]: q sums of its <=4 heads
+  uint4* alds = reinterpret_cast<uint4*>(qs4 + a.n_kv_heads * 4);        // [kv head][b][gq*4 + r]
+  uint4* azero = alds + a.n_kv_heads * 64;                                // same shape, all zero
   const int meta_stride = a.n_kv_heads * 4 + 2;      // halves; +2 spreads the tokens over banks
-  uint16_t* smeta = reinterpret_cast<uint16_t*>(alds + a.n_kv_heads * 64);
+  uint16_t* smeta = reinterpret_cast<uint16_t*>(azero + a.n_kv_heads * 64);
   uint16_t* zmeta = smeta + kTile * meta_stride;
 
   const int c = blockIdx.y;
@@ -386,29 +395,52 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
   const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * 128;
   const int64_t base_row = a.row_base[c];
 
-  // Code vectors of this wavefront's slice of tile tt: one 16-byte load per kv head.
-  auto issue = [&](int tt, uint4 (&cv)[NKV]) {
-    const int64_t n = tok0 + tt * kTile + wave * 16 + nl;
+  // Code vectors of this wavefront's slice of tile tt (one 16-byte load per kv
+  // head) and this thread's share of the tile's (scale, zero) rows: chunk
+  // j*256 + thread = (token, kv head), 8 bytes each.
+  constexpr int NM = NKV / 4;
+  struct TileRegs {
+    uint4 cv[NKV];
+    uint2 sv[NM], zv[NM];
+  };
+  auto issue = [&](int tt, TileRegs& t) {
+    const int64_t t0 = tok0 + tt * kTile;
+    const int64_t n = t0 + wave * 16 + nl;
     const bool okn = n < len;
     const char* rowp = reinterpret_cast<const char*>(a.codes) + ((base_row + n) * lanes_per_row + rg) * 16;
 #pragma unroll
     for (int g = 0; g < NKV; ++g) {
-      cv[g] = make_uint4(0, 0, 0, 0);
-      if (okn && g < a.n_kv_heads) cv[g] = ld16(rowp + g * 64);
+      t.cv[g] = make_uint4(0, 0, 0, 0);
+      if (okn && g < a.n_kv_heads) t.cv[g] = ld16(rowp + g * 64);
+    }
+#pragma unroll
+    for (int j = 0; j < NM; ++j) {
+      const int ch = j * 256 + threadIdx.x;
+      const int tok = ch / a.n_kv_heads, hd = ch - tok * a.n_kv_heads;
+      t.sv[j] = make_uint2(0, 0);
+      t.zv[j] = make_uint2(0, 0);
+      if (tok < kTile && t0 + tok < len) {
+        const int64_t mi = (base_row + t0 + tok) * lanes_per_row + hd * 4;
+        t.sv[j] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.scale) + mi);
+        if constexpr (!Q::sym) t.zv[j] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.zero) + mi);
+      }
     }
   };
-  uint4 cur[NKV], nxt[NKV];
-  issue(0, cur);  // in flight while the prologue runs
+  TileRegs ra, rb;
+  issue(0, ra);  // in flight while the prologue runs
 
   // Prologue: group sums of q, and the non-zero part of the block-diagonal A
   // operands: entry (g, b, gq, r) = q[g*rep + r][32*gq + 8*b + {0,4,1,5,2,6,3,7}].
-  for (int i = threadIdx.x; i < a.n_q_heads * 4; i += 256) {
-    float h32[32];
-    load_as_float<PIKV_BF16, 32>(qbase, (int64_t)i * 32, h32);
+  for (int i = threadIdx.x; i < a.n_kv_heads * 16; i += 256) {
+    const int g = i >> 4, gq = (i >> 2) & 3, r = i & 3;
     float sacc = 0.f;
+    if (r < rep) {
+      float h32[32];
+      load_as_float<PIKV_BF16, 32>(qbase, (int64_t)(g * rep + r) * 128 + gq * 32, h32);
 #pragma unroll
-    for (int k = 0; k < 32; ++k) sacc += h32[k];
-    qs[i] = sacc;
+      for (int k = 0; k < 32; ++k) sacc += h32[k];
+    }
+    reinterpret_cast<float*>(qs4)[i] = sacc;
   }
   for (int i = threadIdx.x; i < a.n_kv_heads * 64; i += 256) {
     const int g = i >> 6, b2 = (i >> 4) & 3, gq = (i >> 2) & 3, r = i & 3;
@@ -416,64 +448,61 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
     if (r < rep) d = ld16(qbase + (int64_t)(g * rep + r) * 128 + gq * 32 + b2 * 8);
     alds[i] = make_uint4((d.x & 0xffffu) | (d.z << 16), (d.x >> 16) | (d.z & 0xffff0000u),
                          (d.y & 0xffffu) | (d.w << 16), (d.y >> 16) | (d.w & 0xffff0000u));
+    azero[i] = make_uint4(0, 0, 0, 0);
   }
 
   const float zbias = 128.0f - (float)Q::qmin;  // 128 (asymmetric) or 136 (symmetric)
-  const bool a_on = (nl >> 2) == rg;            // this lane's k-slice meets its row's group
+  // a lane whose k-slice does not meet its row's group reads zeros
+  const uint4* a_lane = (((nl >> 2) == rg) ? alds : azero) + nl;
+  const uint32_t kNib = 0x000f000fu, kExp = 0x43004300u;  // two nibbles -> two bf16 values 128 + code
 
-  for (int tt = 0; tt < kGqaTilesPerBlock; ++tt) {
+  // One tile: returns false when the block has run past the cache's fill.
+  auto do_tile = [&](int tt, TileRegs& cur, TileRegs& nxt) -> bool {
     const int64_t tile = tile0 + tt;
     const int64_t n0 = tile * kTile;
-    if (n0 >= len) break;  // uniform
-    // (scale, zero) of the tile: 8-byte loads, one per (token, kv head)
-    for (int ch = threadIdx.x; ch < kTile * a.n_kv_heads; ch += 256) {
+    if (n0 >= len) return false;  // uniform
+    // (scale, zero) rows of the tile into LDS, then start the next tile's loads
+#pragma unroll
+    for (int j = 0; j < NM; ++j) {
+      const int ch = j * 256 + threadIdx.x;
       const int tok = ch / a.n_kv_heads, hd = ch - tok * a.n_kv_heads;
-      uint2 sv = make_uint2(0, 0), zv = make_uint2(0, 0);
-      if (n0 + tok < len) {
-        const int64_t mi = (base_row + n0 + tok) * lanes_per_row + hd * 4;
-        sv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.scale) + mi);
-        if constexpr (!Q::sym) zv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.zero) + mi);
-      }
-      uint32_t* sd = reinterpret_cast<uint32_t*>(smeta + tok * meta_stride + hd * 4);
-      sd[0] = sv.x; sd[1] = sv.y;
-      if constexpr (!Q::sym) {
-        uint32_t* zd = reinterpret_cast<uint32_t*>(zmeta + tok * meta_stride + hd * 4);
-        zd[0] = zv.x; zd[1] = zv.y;
+      if (tok < kTile) {
+        uint32_t* sd = reinterpret_cast<uint32_t*>(smeta + tok * meta_stride + hd * 4);
+        sd[0] = cur.sv[j].x; sd[1] = cur.sv[j].y;
+        if constexpr (!Q::sym) {
+          uint32_t* zd = reinterpret_cast<uint32_t*>(zmeta + tok * meta_stride + hd * 4);
+          zd[0] = cur.zv[j].x; zd[1] = cur.zv[j].y;
+        }
       }
     }
     if ((tt + 1 < kGqaTilesPerBlock) && (n0 + kTile < len)) issue(tt + 1, nxt);
-    __syncthreads();  // metadata (and, first time, qs / alds) visible
+    __syncthreads();  // metadata (and, first time, qs4 / alds) visible
 
     const int tl = wave * 16 + nl;
     const bool okt = n0 + tl < len;
 #pragma unroll
     for (int g = 0; g < NKV; ++g) {
       if (g < a.n_kv_heads) {
-        const uint32_t wv[4] = {cur[g].x, cur[g].y, cur[g].z, cur[g].w};
+        const uint32_t wv[4] = {cur.cv[g].x, cur.cv[g].y, cur.cv[g].z, cur.cv[g].w};
         pikv_f32x4 pc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int b2 = 0; b2 < 4; ++b2) {
           const uint32_t w = Q::sym ? (wv[b2] ^ 0x88888888u) : wv[b2];
-          const uint4 bb = make_uint4((w & 0x000f000fu) | 0x43004300u, ((w >> 4) & 0x000f000fu) | 0x43004300u,
-                                      ((w >> 8) & 0x000f000fu) | 0x43004300u,
-                                      ((w >> 12) & 0x000f000fu) | 0x43004300u);
-          uint4 av = make_uint4(0, 0, 0, 0);
-          if (a_on) av = alds[(g * 4 + b2) * 16 + nl];
+          const uint4 bb = make_uint4(and_or(w, kNib, kExp), and_or(w >> 4, kNib, kExp),
+                                      and_or(w >> 8, kNib, kExp), and_or(w >> 12, kNib, kExp));
+          const uint4 av = a_lane[(g * 4 + b2) * 16];
           pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, av),
                                                        __builtin_bit_cast(pikv_bf16x8, bb), pc, 0, 0, 0);
         }
         const int mo = tl * meta_stride + g * 4 + rg;
         const float sc = (float)__builtin_bit_cast(_Float16, smeta[mo]);
         const float zq = (Q::sym ? 0.f : (float)__builtin_bit_cast(_Float16, zmeta[mo])) + zbias;
-        float t[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float qsi = (i < rep) ? qs[(g * rep + i) * 4 + rg] : 0.f;
-          t[i] = sc * fmaf(-zq, qsi, pc[i]);
-        }
+        const float4 qv = qs4[g * 4 + rg];
+        const float t0 = sc * fmaf(-zq, qv.x, pc[0]), t1 = sc * fmaf(-zq, qv.y, pc[1]);
+        const float t2 = sc * fmaf(-zq, qv.z, pc[2]), t3 = sc * fmaf(-zq, qv.w, pc[3]);
         // sum over the four row-groups; row-group r ends with head r
-        auto s01 = __builtin_amdgcn_permlane16_swap(__float_as_uint(t[0]), __float_as_uint(t[1]), false, false);
-        auto s23 = __builtin_amdgcn_permlane16_swap(__float_as_uint(t[2]), __float_as_uint(t[3]), false, false);
+        auto s01 = __builtin_amdgcn_permlane16_swap(__float_as_uint(t0), __float_as_uint(t1), false, false);
+        auto s23 = __builtin_amdgcn_permlane16_swap(__float_as_uint(t2), __float_as_uint(t3), false, false);
         const float u01 = __uint_as_float(s01[0]) + __uint_as_float(s01[1]);
         const float u23 = __uint_as_float(s23[0]) + __uint_as_float(s23[1]);
         auto sf = __builtin_amdgcn_permlane32_swap(__float_as_uint(u01), __float_as_uint(u23), false, false);
@@ -481,8 +510,6 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
         if (rg < rep) stage[(g * rep + rg) * kTile + tl] = okt ? score : -__builtin_inff();
       }
     }
-#pragma unroll
-    for (int g = 0; g < NKV; ++g) cur[g] = nxt[g];
     __syncthreads();
 
     // Tile statistics and score rows, four heads per wavefront pass: lane (rg, nl)
@@ -524,6 +551,12 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
       }
     }
     __syncthreads();  // stage and the metadata rows are reused by the next tile
+    return true;
+  };
+
+  for (int tt = 0; tt < kGqaTilesPerBlock; tt += 2) {
+    if (!do_tile(tt, ra, rb)) break;
+    if (!do_tile(tt + 1, rb, ra)) break;
   }
 }
 
