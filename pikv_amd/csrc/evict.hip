@@ -2,9 +2,10 @@
 //
 // Selection: one 1024-thread block per cache.  A float is mapped to a 32-bit key
 // whose unsigned order is the float order; an MSB-first radix select (4 passes of
-// 8 bits, LDS histogram) finds the key of the m-th largest element, and an
-// ordered marking pass takes every larger element plus the first (lowest-index)
-// elements equal to it.  Total order = (value desc, index asc); the "smallest m"
+// 8 bits, one LDS histogram per wavefront) finds the key of the m-th largest
+// element, and an ordered marking pass takes every larger element plus the first
+// (lowest-index) elements equal to it.  Caches of up to 32768 rows keep their keys
+// in registers between the passes.  Total order = (value desc, index asc); the "smallest m"
 // variant runs the same code on the complemented key.
 //
 // Compaction: survivors move to the front in ascending order.  A block owns one
@@ -20,6 +21,7 @@ namespace pikv {
 
 constexpr int kSelThreads = 1024;
 constexpr int kSelWaves = kSelThreads / 64;
+constexpr int kSelItems = 32;  // keys a thread keeps in registers (caches of <= 32768 rows)
 
 __device__ __forceinline__ uint32_t order_key(float v, bool smallest) {
   v = v + 0.0f;  // -0 -> +0 so that they tie
@@ -28,78 +30,200 @@ __device__ __forceinline__ uint32_t order_key(float v, bool smallest) {
   return smallest ? ~u : u;
 }
 
-// Exclusive prefix count of a per-thread flag over the block, in thread order.
-// sh must hold kSelWaves ints.  Returns the prefix; total gets the block sum.
-__device__ __forceinline__ int block_flag_scan(bool f, int* sh, int& total) {
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const uint64_t b = __ballot(f);
-  const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-  const int in_wave = __popcll(b & lt);
-  __syncthreads();  // previous use of sh is over
-  if (lane == 0) sh[wave] = __popcll(b);
+struct SelShared {
+  int whist[kSelWaves][256];  // one digit histogram per wavefront
+  int hist[256];
+  int wtot[kSelWaves];
+  int pick_digit, pick_rem;
+};
+
+// Element order inside the block: wavefront w owns the contiguous segment
+// [w*items*64, (w+1)*items*64); its round j covers 64 consecutive elements, one
+// per lane.  Prefix counts in index order are then ballots inside a round, a
+// running count over the rounds of a wavefront, and one 16-entry scan across
+// wavefronts.
+struct SelGeom {
+  int len, items, lane, wave, seg0;
+  __device__ __forceinline__ int index(int j) const { return seg0 + j * 64 + lane; }
+};
+
+// Exclusive prefix over the wavefronts of a per-wavefront total (uniform in the
+// wavefront).  All threads call.
+__device__ __forceinline__ int wave_base(int total, const SelGeom& g, SelShared& s) {
+  __syncthreads();  // previous use of wtot is over
+  if (g.lane == 0) s.wtot[g.wave] = total;
   __syncthreads();
-  int pre = 0, tot = 0;
+  int pre = 0;
 #pragma unroll
-  for (int w = 0; w < kSelWaves; ++w) {
-    const int v = sh[w];
-    if (w < wave) pre += v;
-    tot += v;
+  for (int w = 0; w < kSelWaves; ++w)
+    if (w < g.wave) pre += s.wtot[w];
+  return pre;
+}
+
+// Run f(j) for every round of this thread; fully unrolled when the keys sit in
+// registers so that the register array is indexed by constants only.
+template <bool CACHED, typename F>
+__device__ __forceinline__ void for_rounds(const SelGeom& g, F&& f) {
+  if constexpr (CACHED) {
+#pragma unroll
+    for (int j = 0; j < kSelItems; ++j) {
+      if (j < g.items) f(j);  // uniform
+    }
+  } else {
+    for (int j = 0; j < g.items; ++j) f(j);
   }
-  total = tot;
-  return pre + in_wave;
 }
 
 // Mark the m top elements of v[0..len): flag[i] = mark.  All threads must call.
-__device__ void block_select_mark(const float* __restrict__ v, int len, int m, bool smallest,
-                                  uint8_t* __restrict__ flag, uint8_t mark, int* hist /*256*/,
-                                  int* sh /*kSelWaves + 2*/) {
+// CACHED: every thread holds its <= kSelItems keys in registers across the passes.
+template <bool CACHED>
+__device__ void block_select_mark(const float* __restrict__ v, int m, bool smallest,
+                                  uint8_t* __restrict__ flag, uint8_t mark, const SelGeom& g,
+                                  SelShared& s) {
+  const int len = g.len;
   if (m <= 0 || len <= 0) return;  // uniform
-  if (m >= len) {
-    for (int i = threadIdx.x; i < len; i += kSelThreads) flag[i] = mark;
+  if (m >= len) {  // every thread marks its own elements
+    for (int j = 0; j < g.items; ++j)
+      if (g.index(j) < len) flag[g.index(j)] = mark;
     return;
   }
+  uint32_t kreg[CACHED ? kSelItems : 1];
+  uint32_t vbits = 0;  // CACHED: bit j = round j holds an element
+  if (CACHED) {
+#pragma unroll
+    for (int j = 0; j < kSelItems; ++j) {
+      const int i = g.index(j);
+      kreg[j] = 0;
+      if (j < g.items && i < len) {
+        kreg[j] = order_key(v[i], smallest);
+        vbits |= 1u << j;
+      }
+    }
+  }
+  auto fetch = [&](int j, uint32_t& key) -> bool {
+    if (CACHED) {
+      key = kreg[j];
+      return (vbits >> j) & 1u;
+    }
+    const int i = g.index(j);
+    if (i >= len) return false;
+    key = order_key(v[i], smallest);
+    return true;
+  };
+  const uint64_t lt = (g.lane == 0) ? 0ull : (~0ull >> (64 - g.lane));
+
   uint32_t prefix = 0, pmask = 0;
   int remaining = m;
   for (int shift = 24; shift >= 0; shift -= 8) {
+    __syncthreads();  // the histograms of the previous pass have been read
+    *reinterpret_cast<int4*>(&s.whist[g.wave][g.lane * 4]) = make_int4(0, 0, 0, 0);
+    for_rounds<CACHED>(g, [&](int j) {
+      uint32_t key = 0;
+      bool act = fetch(j, key);
+      act = act && ((key & pmask) == prefix);
+      const uint64_t am = __ballot(act);
+      if (am == 0) return;  // uniform
+      const int d = (key >> shift) & 255u;
+      // floats of similar magnitude share their leading digit: count the first
+      // active lane's digit with one ballot, the rest with LDS atomics
+      const int lead = __builtin_ctzll(am);
+      const int ld = __builtin_amdgcn_readlane(d, lead);
+      const uint64_t mm = __ballot(act && d == ld);
+      if (g.lane == lead) atomicAdd(&s.whist[g.wave][ld], __popcll(mm));
+      if (act && d != ld) atomicAdd(&s.whist[g.wave][d], 1);
+    });
     __syncthreads();
-    if (threadIdx.x < 256) hist[threadIdx.x] = 0;
-    __syncthreads();
-    for (int i = threadIdx.x; i < len; i += kSelThreads) {
-      const uint32_t key = order_key(v[i], smallest);
-      if ((key & pmask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1);
+    if (threadIdx.x < 256) {
+      int h = 0;
+#pragma unroll
+      for (int w = 0; w < kSelWaves; ++w) h += s.whist[w][threadIdx.x];
+      s.hist[threadIdx.x] = h;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      int cum = 0, d = 255;
-      for (; d > 0; --d) {
-        if (cum + hist[d] >= remaining) break;
-        cum += hist[d];
+    if (g.wave == 0) {
+      // lane l owns digits 255-4l .. 252-4l (descending); find the digit where the
+      // running count from the top first reaches `remaining`
+      int cnt[4], tot = 0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        cnt[k] = s.hist[255 - 4 * g.lane - k];
+        tot += cnt[k];
       }
-      sh[kSelWaves] = d;
-      sh[kSelWaves + 1] = remaining - cum;
+      int incl = tot;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int o = __shfl_up(incl, off, 64);
+        if (g.lane >= off) incl += o;
+      }
+      int before = incl - tot;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (before < remaining && remaining <= before + cnt[k]) {
+          s.pick_digit = 255 - 4 * g.lane - k;
+          s.pick_rem = remaining - before;
+        }
+        before += cnt[k];
+      }
     }
     __syncthreads();
-    prefix |= (uint32_t)sh[kSelWaves] << shift;
+    prefix |= (uint32_t)s.pick_digit << shift;
     pmask |= 255u << shift;
-    remaining = sh[kSelWaves + 1];
+    remaining = s.pick_rem;
   }
-  // prefix = key of the m-th element; `remaining` of the elements equal to it are taken.
-  int taken_eq = 0;
-  for (int i0 = 0; i0 < len; i0 += kSelThreads) {
-    const int i = i0 + threadIdx.x;
+  // prefix = key of the m-th element; `remaining` of the elements equal to it are
+  // taken, lowest index first.
+  int weq = 0;
+  for_rounds<CACHED>(g, [&](int j) {
     uint32_t key = 0;
-    bool eq = false, gt = false;
-    if (i < len) {
-      key = order_key(v[i], smallest);
-      eq = key == prefix;
-      gt = key > prefix;
-    }
-    int tot;
-    const int r = block_flag_scan(eq, sh, tot);
-    if (gt || (eq && taken_eq + r < remaining)) flag[i] = mark;
-    taken_eq += tot;
+    const bool ok = fetch(j, key);
+    weq += __popcll(__ballot(ok && key == prefix));
+  });
+  int rank = wave_base(weq, g, s);
+  for_rounds<CACHED>(g, [&](int j) {
+    uint32_t key = 0;
+    const bool ok = fetch(j, key);
+    const bool eq = ok && key == prefix;
+    const bool gt = ok && key > prefix;
+    const uint64_t eb = __ballot(eq);
+    if (gt || (eq && rank + __popcll(eb & lt) < remaining)) flag[g.index(j)] = mark;
+    rank += __popcll(eb);
+  });
+}
+
+template <bool CACHED>
+__device__ void evict_select_body(int policy, const float* __restrict__ acc,
+                                  const float* __restrict__ ts, int n_heavy, int n_recent,
+                                  uint8_t* __restrict__ flag, int32_t* __restrict__ out,
+                                  int32_t* __restrict__ new_len_c, const SelGeom& g, SelShared& s) {
+  const int rounds = g.items;
+  // a thread initialises, marks and later reads only its own flags: no barrier needed for them
+  const uint8_t init = (policy == PIKV_EVICT_H2O) ? 0 : 1;
+  for (int j = 0; j < rounds; ++j) {
+    const int i = g.index(j);
+    if (i < g.len) flag[i] = init;
   }
+  if (policy == PIKV_EVICT_H2O) {
+    block_select_mark<CACHED>(acc, n_heavy, false, flag, 1, g, s);
+    block_select_mark<CACHED>(ts, n_recent, false, flag, 1, g, s);
+  } else {
+    block_select_mark<CACHED>(ts, n_heavy, true, flag, 0, g, s);
+  }
+  // Ascending list of survivors.
+  const uint64_t lt = (g.lane == 0) ? 0ull : (~0ull >> (64 - g.lane));
+  int wk = 0;
+  for (int j = 0; j < rounds; ++j) {
+    const int i = g.index(j);
+    wk += __popcll(__ballot(i < g.len && flag[i] != 0));
+  }
+  int pos = wave_base(wk, g, s);
+  for (int j = 0; j < rounds; ++j) {
+    const int i = g.index(j);
+    const bool k = i < g.len && flag[i] != 0;
+    const uint64_t kb = __ballot(k);
+    if (k) out[pos + __popcll(kb & lt)] = i;
+    pos += __popcll(kb);
+  }
+  if (threadIdx.x == kSelThreads - 1) *new_len_c = pos;  // the last wavefront ends at the total
 }
 
 __global__ __launch_bounds__(kSelThreads) void evict_select_kernel(
@@ -107,40 +231,29 @@ __global__ __launch_bounds__(kSelThreads) void evict_select_kernel(
     const int64_t* __restrict__ row_base, const int32_t* __restrict__ fill,
     const int32_t* __restrict__ n_heavy, const int32_t* __restrict__ n_recent,
     uint8_t* __restrict__ keep_flag, int32_t* __restrict__ keep_index, int32_t* __restrict__ new_len) {
-  __shared__ int hist[256];
-  __shared__ int sh[kSelWaves + 2];
+  __shared__ SelShared s;
   const int c = blockIdx.x;
   const int len = fill[c];
   const int64_t base = row_base[c];
-  uint8_t* flag = keep_flag + base;
   if (len <= 0) {
     if (threadIdx.x == 0) new_len[c] = 0;
     return;
   }
-  if (policy == PIKV_EVICT_H2O) {
-    for (int i = threadIdx.x; i < len; i += kSelThreads) flag[i] = 0;
-    __syncthreads();
-    block_select_mark(row_acc + base, len, n_heavy[c], false, flag, 1, hist, sh);
-    __syncthreads();
-    block_select_mark(row_ts + base, len, n_recent[c], false, flag, 1, hist, sh);
-  } else {
-    for (int i = threadIdx.x; i < len; i += kSelThreads) flag[i] = 1;
-    __syncthreads();
-    block_select_mark(row_ts + base, len, n_heavy[c], true, flag, 0, hist, sh);
-  }
-  __syncthreads();
-  // Ascending list of survivors.
-  int32_t* out = keep_index + base;
-  int kept = 0;
-  for (int i0 = 0; i0 < len; i0 += kSelThreads) {
-    const int i = i0 + threadIdx.x;
-    const bool k = (i < len) && flag[i] != 0;
-    int tot;
-    const int r = block_flag_scan(k, sh, tot);
-    if (k) out[kept + r] = i;
-    kept += tot;
-  }
-  if (threadIdx.x == 0) new_len[c] = kept;
+  SelGeom g;
+  g.len = len;
+  g.items = (len + kSelThreads - 1) / kSelThreads;
+  g.lane = threadIdx.x & 63;
+  g.wave = threadIdx.x >> 6;
+  g.seg0 = g.wave * g.items * 64;
+  const float* acc = row_acc ? row_acc + base : nullptr;
+  const int nh = n_heavy[c];
+  const int nr = (policy == PIKV_EVICT_H2O) ? n_recent[c] : 0;
+  if (g.items <= kSelItems)
+    evict_select_body<true>(policy, acc, row_ts + base, nh, nr, keep_flag + base, keep_index + base,
+                            new_len + c, g, s);
+  else
+    evict_select_body<false>(policy, acc, row_ts + base, nh, nr, keep_flag + base, keep_index + base,
+                             new_len + c, g, s);
 }
 
 __global__ void h2o_budget_kernel(const int32_t* __restrict__ fill, int n, double heavy_ratio,

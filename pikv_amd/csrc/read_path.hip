@@ -599,31 +599,82 @@ __global__ __launch_bounds__(64) void head_stats_kernel(const float* __restrict_
   }
 }
 
+// VEC consecutive tokens per thread (16-byte accesses when VEC = 4) and four q
+// heads per round, their loads issued before any store of the round.
+template <int VEC, bool WRITE_PROBS>
 __global__ __launch_bounds__(256) void h2o_accumulate_kernel(
     float* __restrict__ scores, const float* __restrict__ head_stats, int n_q_heads,
     const int64_t* __restrict__ row_base, const int32_t* __restrict__ fill, int64_t score_stride,
-    float decay, float now, int write_probs, float* __restrict__ row_acc, float* __restrict__ row_ts,
+    float decay, float now, float* __restrict__ row_acc, float* __restrict__ row_ts,
     float* __restrict__ importance_out) {
+  constexpr int UN = 4;
   const int c = blockIdx.y;
-  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (n >= fill[c]) return;
-  float imp = 0.f;
-  for (int hq = 0; hq < n_q_heads; ++hq) {
-    const int64_t si = ((int64_t)c * n_q_heads + hq) * score_stride + n;
-    const float m = head_stats[((int64_t)c * n_q_heads + hq) * 2];
-    const float z = head_stats[((int64_t)c * n_q_heads + hq) * 2 + 1];
-    const float p = expf(scores[si] - m) / z;
-    if (write_probs) scores[si] = p;
-    imp = imp + p;
+  const int64_t n0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  const int64_t len = fill[c];
+  if (n0 >= len) return;
+  const int cnt = (len - n0 < VEC) ? (int)(len - n0) : VEC;
+  const float* hs = head_stats + (int64_t)c * n_q_heads * 2;
+  float* sc = scores + (int64_t)c * n_q_heads * score_stride + n0;
+  float imp[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) imp[j] = 0.f;
+  for (int h0 = 0; h0 < n_q_heads; h0 += UN) {
+    float x[UN][VEC];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int hq = h0 + u;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) x[u][j] = -__builtin_inff();
+      if (hq < n_q_heads) {
+        const float* p = sc + (int64_t)hq * score_stride;
+        if (VEC == 4 && cnt == 4) {
+          const float4 v = *reinterpret_cast<const float4*>(p);
+          x[u][0] = v.x; x[u][1] = v.y; x[u][2] = v.z; x[u][3] = v.w;
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j)
+            if (j < cnt) x[u][j] = p[j];
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int hq = h0 + u;
+      if (hq < n_q_heads) {
+        const float m = hs[hq * 2];
+        const float rz = 1.0f / hs[hq * 2 + 1];
+        float pr[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          pr[j] = __builtin_amdgcn_exp2f((x[u][j] - m) * 1.4426950408889634f) * rz;
+          imp[j] = imp[j] + pr[j];
+        }
+        if (WRITE_PROBS) {
+          float* p = sc + (int64_t)hq * score_stride;
+          if (VEC == 4 && cnt == 4) {
+            *reinterpret_cast<float4*>(p) = make_float4(pr[0], pr[1], pr[2], pr[3]);
+          } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+              if (j < cnt) p[j] = pr[j];
+          }
+        }
+      }
+    }
   }
-  const int64_t row = row_base[c] + n;
-  if (row_acc) {
-    float acc = row_acc[row];
-    if (decay != 1.0f) acc = acc * decay;
-    row_acc[row] = acc + imp;
+  const int64_t row = row_base[c] + n0;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    if (j < cnt) {
+      if (row_acc) {
+        float acc = row_acc[row + j];
+        if (decay != 1.0f) acc = acc * decay;
+        row_acc[row + j] = acc + imp[j];
+      }
+      if (row_ts) row_ts[row + j] = now;
+      if (importance_out) importance_out[(int64_t)c * score_stride + n0 + j] = imp[j];
+    }
   }
-  if (row_ts) row_ts[row] = now;
-  if (importance_out) importance_out[(int64_t)c * score_stride + n] = imp;
 }
 
 template <int SCHEME, int OUT_DT>
@@ -772,11 +823,22 @@ extern "C" int pikv_h2o_accumulate(float* scores, const float* tile_max, const f
   hipStream_t st = (hipStream_t)stream;
   hipLaunchKernelGGL(head_stats_kernel, dim3((unsigned)n_q_heads, (unsigned)n_caches), dim3(64), 0,
                      st, tile_max, tile_sum, cache_fill, n_q_heads, n_tiles, head_stats);
-  const int64_t nb = (max_len + 255) / 256;
+  // 16-byte accesses need every score row to start on a 16-byte boundary
+  const bool vec4 = (score_stride % 4 == 0) && ((reinterpret_cast<uintptr_t>(scores) & 15) == 0);
+  const int per_block = 256 * (vec4 ? 4 : 1);
+  const int64_t nb = (max_len + per_block - 1) / per_block;
   if (nb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
-  hipLaunchKernelGGL(h2o_accumulate_kernel, dim3((unsigned)nb, (unsigned)n_caches), dim3(256), 0, st,
-                     scores, head_stats, n_q_heads, cache_row_base, cache_fill, score_stride, decay,
-                     now, write_probs, row_acc, row_ts, importance_out);
+  const dim3 grid((unsigned)nb, (unsigned)n_caches);
+#define PIKV_H2O_LAUNCH(V, W)                                                                       \
+  hipLaunchKernelGGL((h2o_accumulate_kernel<V, W>), grid, dim3(256), 0, st, scores, head_stats,     \
+                     n_q_heads, cache_row_base, cache_fill, score_stride, decay, now, row_acc,      \
+                     row_ts, importance_out)
+  if (vec4) {
+    if (write_probs) PIKV_H2O_LAUNCH(4, true); else PIKV_H2O_LAUNCH(4, false);
+  } else {
+    if (write_probs) PIKV_H2O_LAUNCH(1, true); else PIKV_H2O_LAUNCH(1, false);
+  }
+#undef PIKV_H2O_LAUNCH
   PIKV_CHECK_LAUNCH();
   return PIKV_OK;
 }

@@ -193,3 +193,29 @@ def test_select_brute_force_small(dev):
             before_t = sum((t[j] > t[i]) or (t[j] == t[i] and j < i) for j in range(L))
             want = before_a < nh[c] or before_t < nr[c]
             assert bool(flags[rows[i]]) == want, (c, i)
+
+
+@pytest.mark.parametrize("ties", [False, True])
+def test_h2o_select_long_cache(dev, ties):
+    """Caches longer than 32768 rows take the selection path that re-reads its keys
+    from memory in every pass; one shorter cache rides along on the register path."""
+    r = rng(77 + ties)
+    caps = [70000, 33000, 32768]
+    lens = [69999, 32769, 32768]
+    pool, ref = _fill_pool(dev, r, caps, lens, 1, 32, 32, O.Q_I8_SYM, dtype="f32")
+    _set_state(pool, ref, r, ties)
+    nh = np.array([4375, 1, 2048], dtype=np.int32)
+    nr = np.array([546, 32769, 256], dtype=np.int32)
+    pool.evict_select(0, n_heavy=to_dev(nh, dev), n_recent=to_dev(nr, dev))
+    keeps = []
+    for c, L in enumerate(lens):
+        rows = ref.valid_rows(c)
+        keep = O.h2o_keep(ref.acc[rows], ref.ts[rows], int(nh[c]), int(nr[c]))
+        keeps.append(keep)
+        got = np_of(pool.keep_flag)[rows].astype(bool)
+        assert np.array_equal(got, keep), (c, np.argwhere(got != keep)[:5])
+        m = int(np_of(pool.new_len)[c])
+        assert m == keep.sum()
+        assert np.array_equal(np_of(pool.keep_index)[rows[0]:rows[0] + m], np.nonzero(keep)[0])
+    pool.compact()
+    _check_compacted(pool, ref, O.Q_I8_SYM, keeps)
