@@ -194,8 +194,35 @@ int pikv_cache_advance(int32_t* cache_fill, const int32_t* count,
                        const int32_t* cache_cap, int n_caches,
                        int64_t per_call_limit, void* stream);
 
+/* Pyramid compression: quantise a SELECTED subset of source rows into the caches,
+ * in list order.  For cache c and j < n_take[c], the source row
+ *     src_row_base[c] + src_index[src_row_base[c] + j]
+ * is quantised (same formula as pikv_quant_scatter) and appended at cache row
+ * cache_fill[c] + j; rows past cache_cap[c] are dropped; cache_fill is not advanced.
+ * src_index is an ascending survivor list in the SOURCE row space, as
+ * pikv_evict_select writes it when it is handed the source geometry
+ * (cache_row_base = src_row_base, cache_fill = rows per layer, n_heavy = keep_l,
+ * n_recent = 0): top-keep_l by score, ties to the lower index, original order kept.
+ * A gathered row starts with accumulator src_score[source row] (0 when src_score
+ * is NULL) and timestamp `now`.
+ * Replaces: the importance-descending partition of PyramidCompressor.forward
+ *   (core/single/pikv_compression.py:145-160) followed by per-level compression,
+ *   with the per-layer budgets of PiKVMoE.pyramidal_cache_allocation
+ *   (core/single/pikv_moe.py:218-224); max_take >= max_c n_take[c] sizes the grid. */
+int pikv_quant_gather(const void* k_src, const void* v_src, int src_dtype,
+                      int D, int group, int scheme,
+                      const int64_t* src_row_base, const int32_t* src_index,
+                      const int32_t* n_take, int64_t max_take, const float* src_score,
+                      const int64_t* cache_row_base, const int32_t* cache_fill,
+                      const int32_t* cache_cap, int n_caches,
+                      void* k_codes, void* v_codes,
+                      void* k_scale, void* v_scale,
+                      void* k_zero, void* v_zero,
+                      float* row_acc, float* row_ts, float now,
+                      void* stream);
+
 /* Quantise rows in place order (no routing): row i of the source goes to row
- * dst_row0 + i of the planes.  Same formula as pikv_quant_scatter; used for
+ * dst_row0 + i of the planes. Same formula as pikv_quant_scatter; used for
  * QuantizedCompressor.quantize() and for bulk cache prefill. */
 int pikv_quantize_rows(const void* src, int src_dtype, int64_t n_rows, int D,
                        int group, int scheme, int64_t dst_row0,

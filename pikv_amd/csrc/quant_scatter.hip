@@ -31,6 +31,13 @@ struct QuantScatterArgs {
   float* row_acc;
   float* row_ts;
   float now;
+  // gather mode (seg_index != nullptr): grid row y = cache c; logical source j of
+  // cache c is source row seg_src_base[c] + seg_index[seg_src_base[c] + j],
+  // j < seg_count[c], appended at cache row fill[c] + j
+  const int64_t* seg_src_base;
+  const int32_t* seg_index;
+  const int32_t* seg_count;
+  const float* seg_score;  // optional: initial accumulator of a gathered row, by source row
   int64_t n_src;
   int64_t dst_row0;     // used when cache_id == nullptr
   int fanout;
@@ -106,7 +113,19 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(QuantScatterArgs a) 
     s = g / lanes_per_row;
     part = (int)(g - s * lanes_per_row);
   }
-  const bool valid = s < a.n_src;
+  bool valid = s < a.n_src;
+  int64_t srow = s;  // row of src[] this lane reads
+  int64_t gather_dst = -1;
+  if (a.seg_index != nullptr) {
+    const int c = blockIdx.y;
+    valid = valid && s < a.seg_count[c];
+    if (valid) {
+      const int64_t sb = a.seg_src_base[c];
+      srow = sb + a.seg_index[sb + s];
+      const int64_t r = (int64_t)a.fill[c] + s;
+      if (r < a.cap[c]) gather_dst = a.row_base[c] + r;
+    }
+  }
 
   // Destination rows of this source row (-1 = dropped).
   int64_t dst[FANOUT];
@@ -115,7 +134,9 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(QuantScatterArgs a) 
   for (int j = 0; j < FANOUT; ++j) {
     dst[j] = -1;
     if (valid && j < a.fanout) {
-      if (a.cache_id == nullptr) {
+      if (a.seg_index != nullptr) {
+        dst[j] = gather_dst;
+      } else if (a.cache_id == nullptr) {
         dst[j] = a.dst_row0 + s;
       } else {
         const int64_t as = s * a.fanout + j;
@@ -139,7 +160,7 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(QuantScatterArgs a) 
   raw[0].zero_fill();
   raw[1].zero_fill();
   if (live) {
-    const int64_t off = s * a.D + (int64_t)part * EPL;
+    const int64_t off = srow * a.D + (int64_t)part * EPL;
     raw[0].load(a.src[0], off);
     if (a.n_tensors > 1) raw[1].load(a.src[1], off);
   }
@@ -178,7 +199,7 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(QuantScatterArgs a) 
 #pragma unroll
     for (int j = 0; j < FANOUT; ++j) {
       if (dst[j] < 0) continue;
-      if (a.row_acc) a.row_acc[dst[j]] = 0.f;
+      if (a.row_acc) a.row_acc[dst[j]] = a.seg_score ? a.seg_score[srow] : 0.f;
       if (a.row_ts) a.row_ts[dst[j]] = a.now;
     }
   }
@@ -186,14 +207,15 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(QuantScatterArgs a) 
 
 template <int SCHEME, int SRC_DT, bool RU>
 static void launch_quant_f(int fanout, unsigned blocks, hipStream_t st, const QuantScatterArgs& a) {
+  const dim3 grid(blocks, a.seg_index ? (unsigned)a.n_caches : 1u);
   if (fanout <= 1)
-    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 1, RU>), dim3(blocks), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 1, RU>), grid, dim3(256), 0, st, a);
   else if (fanout <= 2)
-    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 2, RU>), dim3(blocks), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 2, RU>), grid, dim3(256), 0, st, a);
   else if (fanout <= 4)
-    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 4, RU>), dim3(blocks), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 4, RU>), grid, dim3(256), 0, st, a);
   else
-    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 8, RU>), dim3(blocks), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((quant_scatter_kernel<SCHEME, SRC_DT, 8, RU>), grid, dim3(256), 0, st, a);
 }
 
 template <int SCHEME>
@@ -284,6 +306,39 @@ extern "C" int pikv_quant_scatter(const void* k_src, const void* v_src, int src_
   a.fill = cache_fill; a.cap = cache_cap;
   a.row_acc = row_acc; a.row_ts = row_ts; a.now = now;
   a.n_src = n_src; a.dst_row0 = 0; a.fanout = fanout; a.D = D; a.group = group;
+  a.n_tensors = v_src ? 2 : 1;
+  a.n_caches = n_caches;
+  return dispatch_quant(a, scheme, src_dtype, (hipStream_t)stream);
+}
+
+extern "C" int pikv_quant_gather(const void* k_src, const void* v_src, int src_dtype, int D,
+                                 int group, int scheme, const int64_t* src_row_base,
+                                 const int32_t* src_index, const int32_t* n_take, int64_t max_take,
+                                 const float* src_score, const int64_t* cache_row_base,
+                                 const int32_t* cache_fill, const int32_t* cache_cap, int n_caches,
+                                 void* k_codes, void* v_codes, void* k_scale, void* v_scale,
+                                 void* k_zero, void* v_zero, float* row_acc, float* row_ts,
+                                 float now, void* stream) {
+  if (!k_src || !k_codes || !k_scale || !src_row_base || !src_index || !n_take || !cache_row_base ||
+      !cache_fill || !cache_cap)
+    return PIKV_ERR_NULL;
+  if (src_dtype != PIKV_F32 && src_dtype != PIKV_BF16) return PIKV_ERR_UNSUPPORTED;
+  if (max_take < 0 || n_caches < 1 || n_caches > 65535) return PIKV_ERR_SHAPE;
+  int rc = check_quant_shape(D, group, scheme);
+  if (rc != PIKV_OK) return rc;
+  const bool asym = (scheme == PIKV_Q_I8_ASYM || scheme == PIKV_Q_I4_ASYM);
+  if (asym && !k_zero) return PIKV_ERR_NULL;
+  if (v_src && (!v_codes || !v_scale || (asym && !v_zero))) return PIKV_ERR_NULL;
+  QuantScatterArgs a{};
+  a.src[0] = k_src; a.src[1] = v_src;
+  a.codes[0] = k_codes; a.codes[1] = v_codes;
+  a.scale[0] = k_scale; a.scale[1] = v_scale;
+  a.zero[0] = k_zero; a.zero[1] = v_zero;
+  a.row_base = cache_row_base; a.fill = cache_fill; a.cap = cache_cap;
+  a.seg_src_base = src_row_base; a.seg_index = src_index; a.seg_count = n_take;
+  a.seg_score = src_score;
+  a.row_acc = row_acc; a.row_ts = row_ts; a.now = now;
+  a.n_src = max_take; a.dst_row0 = 0; a.fanout = 1; a.D = D; a.group = group;
   a.n_tensors = v_src ? 2 : 1;
   a.n_caches = n_caches;
   return dispatch_quant(a, scheme, src_dtype, (hipStream_t)stream);

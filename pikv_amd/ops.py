@@ -310,6 +310,31 @@ def fakequant_colblocks(x, group: int, bits: int = 8, symmetric: bool = False):
 # cache pool
 # --------------------------------------------------------------------------
 
+def select_top_rows(score, seg_base, seg_len, n_keep):
+    """Per segment c of a flat score array (rows seg_base[c] .. +seg_len[c]): keep
+    the n_keep[c] largest scores, ties to the lower index.  Returns (keep_flag
+    uint8 [rows], keep_index int32 [rows], n_kept int32 [segments]); segment c's
+    ascending survivor list sits at keep_index[seg_base[c] : +n_kept[c]]."""
+    score = _need(score, "score", dtype=torch.float32, ndim=1)
+    seg_base = _need(seg_base, "seg_base", dtype=torch.int64, ndim=1)
+    seg_len = _need(seg_len, "seg_len", dtype=torch.int32, ndim=1)
+    n_keep = _need(n_keep, "n_keep", dtype=torch.int32, ndim=1)
+    n = seg_base.numel()
+    if seg_len.numel() != n or n_keep.numel() != n:
+        raise ValueError("seg_base, seg_len and n_keep must have the same length")
+    dev = score.device
+    flag = torch.zeros(score.numel(), dtype=torch.uint8, device=dev)
+    index = torch.zeros(score.numel(), dtype=torch.int32, device=dev)
+    kept = torch.zeros(n, dtype=torch.int32, device=dev)
+    if n == 0 or score.numel() == 0:
+        return flag, index, kept
+    zero = torch.zeros(n, dtype=torch.int32, device=dev)
+    # H2O selection with an empty "recent" budget; the score doubles as the (unused) timestamp
+    N.call("pikv_evict_select", EVICT_H2O, _ptr(score), _ptr(score), _ptr(seg_base), _ptr(seg_len),
+           _ptr(n_keep), _ptr(zero), n, _ptr(flag), _ptr(index), _ptr(kept), _stream())
+    return flag, index, kept
+
+
 class CachePool:
     """n_caches quantised KV caches (one per expert or per sequence) sharing a
     row space in HBM; see include/pikv_hip.h for the plane layout.  State
@@ -386,6 +411,41 @@ class CachePool:
                _ptr(self.cap), self.n_caches, _ptr(self.k_codes), _ptr(self.v_codes),
                _ptr(self.k_scale), _ptr(self.v_scale), _ptr(self.k_zero), _ptr(self.v_zero),
                _ptr(self.acc), _ptr(self.ts), float(now), _stream())
+
+    def quant_gather(self, k_src, v_src, src_row_base, src_index, n_take, max_take: int,
+                     src_score=None, now: float = 0.0):
+        """Quantise the listed source rows into the caches in list order: for
+        cache c and j < n_take[c], source row src_row_base[c] +
+        src_index[src_row_base[c] + j] goes to cache row fill[c] + j.  fill is
+        not advanced."""
+        k_src = _need(k_src, "k_src")
+        dt = _dt(k_src, "k_src")
+        k2 = k_src.reshape(-1, self.D)
+        v2 = None
+        if self.with_v:
+            v_src = _need(v_src, "v_src", dtype=k_src.dtype)
+            v2 = v_src.reshape(-1, self.D)
+            if v2.shape != k2.shape:
+                raise ValueError("v_src must match k_src")
+        src_row_base = _need(src_row_base, "src_row_base", dtype=torch.int64, ndim=1)
+        src_index = _need(src_index, "src_index", dtype=torch.int32, ndim=1)
+        n_take = _need(n_take, "n_take", dtype=torch.int32, ndim=1)
+        if src_row_base.numel() != self.n_caches or n_take.numel() != self.n_caches:
+            raise ValueError("src_row_base / n_take must have one entry per cache")
+        if src_index.numel() < k2.shape[0]:
+            raise ValueError("src_index must cover the source row space")
+        if src_score is not None:
+            src_score = _need(src_score, "src_score", dtype=torch.float32)
+            if src_score.numel() != k2.shape[0]:
+                raise ValueError("src_score must have one entry per source row")
+        if max_take <= 0 or k2.shape[0] == 0:
+            return
+        N.call("pikv_quant_gather", _ptr(k2), _ptr(v2), dt, self.D, self.group, self.scheme,
+               _ptr(src_row_base), _ptr(src_index), _ptr(n_take), int(max_take), _ptr(src_score),
+               _ptr(self.row_base), _ptr(self.fill), _ptr(self.cap), self.n_caches,
+               _ptr(self.k_codes), _ptr(self.v_codes), _ptr(self.k_scale), _ptr(self.v_scale),
+               _ptr(self.k_zero), _ptr(self.v_zero), _ptr(self.acc), _ptr(self.ts), float(now),
+               _stream())
 
     def advance(self, count, per_call_limit: int = -1):
         """fill[c] = min(fill[c] + min(count[c], limit), cap[c])."""
