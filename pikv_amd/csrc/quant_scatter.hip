@@ -155,6 +155,9 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(QuantScatterArgs a) 
   // Lanes of one group share s, hence the same destinations: the whole group
   // takes the same branch below, and cross-lane traffic stays inside the group.
   const bool live = valid && any;
+  // A group never straddles a wavefront, so a wavefront without live lanes has
+  // nothing to reduce or store.
+  if (__ballot(live) == 0) return;
 
   RawRow<SRC_DT, EPL> raw[2];
   raw[0].zero_fill();
