@@ -102,7 +102,10 @@ int pikv_abi_version(void);
  *   slot     [T,k] int32 or NULL (then capacity/count/workspace are unused)
  *   count    [E] int32 or NULL
  *   1 <= E <= 64, 1 <= k <= min(E,8), H % 8 == 0
- *   workspace: pikv_router_workspace_bytes(T,E,k) bytes, 256-byte aligned.
+ *   workspace: pikv_router_fused_workspace_bytes(T,H,E,k) bytes, 256-byte aligned
+ *              (slot scan counters, and the gate weights re-laid per 32-wide
+ *              k-step for the bf16 matrix-core projection); required whenever
+ *              slot != NULL or x_dtype == PIKV_BF16.
  * ---------------------------------------------------------------------- */
 int pikv_router_fused(const void* x, const void* w, int x_dtype,
                       const float* bias, const float* expert_scale,
@@ -143,7 +146,9 @@ int pikv_capacity_slots(const int32_t* expert_idx, int64_t A, int E,
                         int64_t capacity, int32_t* slot, int32_t* count,
                         void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Workspace of pikv_router_tail / pikv_capacity_slots, and of pikv_router_fused. */
 int64_t pikv_router_workspace_bytes(int64_t T, int E, int k);
+int64_t pikv_router_fused_workspace_bytes(int64_t T, int H, int E, int k);
 
 /* ------------------------------------------------------------------------
  * K2  fused KV quantise + per-cache scatter (append)

@@ -35,6 +35,7 @@ SIGNATURES = {
                               _p, _p, _p, _p, _p, _p, _l, _p]),
     "pikv_capacity_slots": (_i, [_p, _l, _i, _l, _p, _p, _p, _l, _p]),
     "pikv_router_workspace_bytes": (_l, [_l, _i, _i]),
+    "pikv_router_fused_workspace_bytes": (_l, [_l, _i, _i, _i]),
     "pikv_quant_scatter": (_i, [_p, _p, _i, _l, _i, _i, _i, _i, _p, _p, _p, _p, _p, _i,
                                 _p, _p, _p, _p, _p, _p, _p, _p, _f, _p]),
     "pikv_cache_advance": (_i, [_p, _p, _p, _i, _l, _p]),

@@ -197,73 +197,103 @@ typedef __bf16 pikv_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float pikv_f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMfmaWaves = 8;
+#ifndef PIKV_GATE_MT16
+#define PIKV_GATE_MT16 4
+#endif
 
-template <int NT>  // NT = number of 16-expert tiles (1, 2 or 4)
+// Gate weights re-laid for the matrix-core kernel: wb[step][expert (padded to EP)][32 k]
+// so that the B operands of one k-step are EP*64 contiguous bytes.  Rows of the
+// original [E,H] layout are a multiple of 2 KB apart for the usual hidden sizes and
+// would all fall into the same L2 channel.
+__global__ __launch_bounds__(256) void gate_weight_relayout_kernel(const uint16_t* __restrict__ w, int H,
+                                                                  int E, int EP, uint4* __restrict__ wb) {
+  const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;  // 16-byte chunk of wb
+  const int64_t total = (int64_t)(H / 32) * EP * 4;
+  if (chunk >= total) return;
+  const int kg = (int)(chunk & 3);
+  const int e = (int)((chunk >> 2) % EP);
+  const int64_t st = (chunk >> 2) / EP;
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (e < E) v = ld16(w + (int64_t)e * H + st * 32 + kg * 8);
+  wb[chunk] = v;
+}
+
+template <int NT, int MT>  // NT 16-expert tiles (1, 2 or 4) x MT 16-token tiles per block
 __global__ __launch_bounds__(kMfmaWaves * 64) void router_gate_mfma_kernel(
-    const void* __restrict__ x, const void* __restrict__ w, int H, TailParams p) {
+    const void* __restrict__ x, const void* __restrict__ wb, int H, TailParams p) {
   constexpr int EP = 16 * NT;
-  __shared__ float red[kMfmaWaves][16][EP];
+  constexpr int TB = 16 * MT;  // tokens per block
+  __shared__ float red[kMfmaWaves][TB][EP];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int64_t tok0 = (int64_t)blockIdx.x * 16;
+  const int64_t tok0 = (int64_t)blockIdx.x * TB;
   const int m = lane & 15;    // token row of the A operand / expert column of B and C
   const int kg = lane >> 4;   // which 8 of the 32 k-values this lane feeds
-  const bool tok_ok = tok0 + m < p.T;
-  const char* xrow = reinterpret_cast<const char*>(x) + ((tok0 + m) * (int64_t)H + kg * 8) * 2;
-  const char* wrow[NT];
-  bool w_ok[NT];
+  const char* xrow[MT];
+  bool tok_ok[MT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int e = t * 16 + m;
-    w_ok[t] = e < p.E;
-    wrow[t] = reinterpret_cast<const char*>(w) + ((int64_t)(w_ok[t] ? e : 0) * H + kg * 8) * 2;
+  for (int mt = 0; mt < MT; ++mt) {
+    tok_ok[mt] = tok0 + mt * 16 + m < p.T;
+    xrow[mt] = reinterpret_cast<const char*>(x) +
+               ((tok_ok[mt] ? tok0 + mt * 16 + m : 0) * (int64_t)H + kg * 8) * 2;
   }
-  pikv_f32x4 acc[NT];
+  const char* wlane = reinterpret_cast<const char*>(wb) + (m * 32 + kg * 8) * 2;
+  pikv_f32x4 acc[MT][NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[mt][t] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // the k-steps are dealt round-robin to the wavefronts; each keeps UN steps in flight
   const int steps = H / 32;
-  constexpr int UN = 4;
+  constexpr int UN = (MT + NT > 4) ? 2 : 4;
   for (int st0 = wave; st0 < steps; st0 += kMfmaWaves * UN) {
-    uint4 av[UN], bv[UN][NT];
+    uint4 av[UN][MT], bv[UN][NT];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int st = st0 + u * kMfmaWaves;
       const bool ok = st < steps;
-      av[u] = (ok && tok_ok) ? ld16(xrow + (int64_t)st * 64) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        av[u][mt] = (ok && tok_ok[mt]) ? ld16(xrow[mt] + (int64_t)st * 64) : make_uint4(0, 0, 0, 0);
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        bv[u][t] = (ok && w_ok[t]) ? ld16(wrow[t] + (int64_t)st * 64) : make_uint4(0, 0, 0, 0);
+        bv[u][t] = ok ? ld16(wlane + ((int64_t)st * EP + t * 16) * 64) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const pikv_bf16x8 a8 = __builtin_bit_cast(pikv_bf16x8, av[u]);
+    for (int u = 0; u < UN; ++u)
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a8, __builtin_bit_cast(pikv_bf16x8, bv[u][t]),
-                                                         acc[t], 0, 0, 0);
-    }
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(pikv_bf16x8, av[u][mt]), __builtin_bit_cast(pikv_bf16x8, bv[u][t]),
+              acc[mt][t], 0, 0, 0);
   }
   // C layout: lane holds rows 4*(lane/16)+i, column lane%16 of each tile.
 #pragma unroll
-  for (int t = 0; t < NT; ++t)
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][4 * kg + i][t * 16 + m] = acc[t][i];
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][mt * 16 + 4 * kg + i][t * 16 + m] = acc[mt][t][i];
   __syncthreads();
-  // Wavefront w finishes tokens 2w, 2w+1: lane -> (token, expert) with the experts
-  // of a token in EP adjacent lanes, as the tail expects.
-  constexpr int TPC = 64 / EP;  // tokens per tail call
+  // Wavefront w finishes tokens TW*w .. TW*w+TW-1: lane -> (token, expert) with the
+  // experts of a token in EP adjacent lanes, as the tail expects.
+  constexpr int TW = TB / kMfmaWaves;  // tokens finished by one wavefront
+  constexpr int TPC = 64 / EP;         // tokens per tail call
 #pragma unroll
-  for (int c = 0; c < 2 / TPC + (2 % TPC != 0); ++c) {
-    const int tl = 2 * wave + c * TPC + lane / EP;
+  for (int c = 0; c < (TW + TPC - 1) / TPC; ++c) {
+    const int tw = c * TPC + lane / EP;
+    const int tl = TW * wave + tw;
     const int e = lane % EP;
-    const bool in_range = (c * TPC + lane / EP) < 2;
+    const bool in_range = tw < TW;
     float lg = 0.f;
     if (in_range) {
 #pragma unroll
       for (int w2 = 0; w2 < kMfmaWaves; ++w2) lg += red[w2][tl][e];
     }
-    // lanes beyond the two tokens of this wavefront present an out-of-range token
+    // lanes beyond this wavefront's tokens present an out-of-range token
     router_tail_lanes<EP>(lg, in_range ? tok0 + tl : p.T, e, lane, p);
   }
 }
@@ -412,6 +442,15 @@ extern "C" int64_t pikv_router_workspace_bytes(int64_t T, int E, int k) {
   return slot_workspace_bytes(T * k, E);
 }
 
+static int gate_epad(int E) { return E <= 16 ? 16 : E <= 32 ? 32 : 64; }
+static int64_t gate_weight_bytes(int H, int E) { return (int64_t)H * gate_epad(E) * 2; }
+static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+
+extern "C" int64_t pikv_router_fused_workspace_bytes(int64_t T, int H, int E, int k) {
+  if (T < 0 || H < 1 || E < 1 || k < 1) return 0;
+  return align256(slot_workspace_bytes(T * k, E)) + gate_weight_bytes(H, E);
+}
+
 extern "C" int pikv_capacity_slots(const int32_t* expert_idx, int64_t A, int E, int64_t capacity,
                                    int32_t* slot, int32_t* count, void* workspace,
                                    int64_t workspace_bytes, void* stream) {
@@ -439,10 +478,15 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
   if (rc != PIKV_OK) return rc;
   if (H < 8) return PIKV_ERR_SHAPE;
   if (H % 8 != 0) return PIKV_ERR_UNSUPPORTED;
-  if (slot) {
-    if (!workspace && T > 0) return PIKV_ERR_NULL;
-    if (workspace_bytes < slot_workspace_bytes(T * k, E)) return PIKV_ERR_WORKSPACE;
+  const bool mfma = x_dtype == PIKV_BF16 && H % 32 == 0;
+  const int64_t slot_ws = align256(slot_workspace_bytes(T * k, E));
+  if ((slot || mfma) && T > 0) {
+    if (!workspace) return PIKV_ERR_NULL;
+    if (workspace_bytes < (slot ? slot_ws : 0) + (mfma ? gate_weight_bytes(H, E) : 0))
+      return PIKV_ERR_WORKSPACE;
   }
+  // the re-laid gate weights sit behind the slot area when both are in use
+  char* wb = reinterpret_cast<char*>(workspace) + (slot ? slot_ws : 0);
   hipStream_t st = (hipStream_t)stream;
   if (T > 0) {
     TailParams p{bias, expert_scale, expert_mask, temperature, renorm_eps, 1, E, k, T,
@@ -451,16 +495,21 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
     const int64_t tiles = (T + (64 / epad) - 1) / (64 / epad);
     const int64_t blocks = (tiles + 3) / 4;
     if (blocks > 0x7fffffffLL) return PIKV_ERR_SHAPE;
-    if (x_dtype == PIKV_BF16 && H % 32 == 0) {
-      const int64_t mb = (T + 15) / 16;
+    if (mfma) {
+      const int ep = gate_epad(E);
+      const int mt = (ep == 16) ? PIKV_GATE_MT16 : 2;  // 16-token tiles per block
+      const int64_t mb = (T + 16 * mt - 1) / (16 * mt);
       if (mb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+      const int64_t chunks = (int64_t)(H / 32) * ep * 4;
+      hipLaunchKernelGGL(gate_weight_relayout_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256),
+                         0, st, (const uint16_t*)w, H, E, ep, (uint4*)wb);
       const dim3 grid((unsigned)mb), blk(kMfmaWaves * 64);
       if (E <= 16)
-        hipLaunchKernelGGL((router_gate_mfma_kernel<1>), grid, blk, 0, st, x, w, H, p);
+        hipLaunchKernelGGL((router_gate_mfma_kernel<1, PIKV_GATE_MT16>), grid, blk, 0, st, x, wb, H, p);
       else if (E <= 32)
-        hipLaunchKernelGGL((router_gate_mfma_kernel<2>), grid, blk, 0, st, x, w, H, p);
+        hipLaunchKernelGGL((router_gate_mfma_kernel<2, 2>), grid, blk, 0, st, x, wb, H, p);
       else
-        hipLaunchKernelGGL((router_gate_mfma_kernel<4>), grid, blk, 0, st, x, w, H, p);
+        hipLaunchKernelGGL((router_gate_mfma_kernel<4, 2>), grid, blk, 0, st, x, wb, H, p);
     } else if (x_dtype == PIKV_BF16) {
       launch_gate<PIKV_BF16>(epad, (unsigned)blocks, st, x, w, H, p);
     } else {

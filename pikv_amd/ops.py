@@ -172,6 +172,8 @@ def router_fused(x, weight, bias=None, *, top_k=2, capacity=None, expert_scale=N
     expert_mask = _vecf(expert_mask, "expert_mask", E, dev)
     probs, logits, idx, w, slot, count, ws, ws_bytes = _router_common(
         T, E, top_k, capacity, dev, True, return_logits)
+    ws_bytes = int(N.lib().pikv_router_fused_workspace_bytes(T, H, E, top_k))
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
     if T == 0:  # nothing to route (empty tensors have no device address)
         if count is not None:
             count.zero_()
