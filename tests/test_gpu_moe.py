@@ -1,0 +1,176 @@
+"""GPU parity of the PiKVMoE mirror at the small CPU-runnable configuration
+(batch 2, seq 64, hidden 256, 4 experts top-2, 4 heads x 64, 128-slot caches,
+int8 symmetric per token, LRU): the native cache traffic of several consecutive
+forwards against the numpy restatement fed with the same routed rows.
+
+Bit-exact: slots, counts, eviction sets, cache codes / scales / timestamps / fill.
+Expert indices are exact wherever the float64 gap between the k-th and (k+1)-th
+logit exceeds 1e-5.  Logits: <= 1e-3 relative (float32 path) against a float64
+evaluation of the same module graph that uses the restatement's cache means."""
+import numpy as np
+import pytest
+
+import pikv_oracle as O
+from util import np_of
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def small_config():
+    from pikv_amd.config import config
+    saved = dict(config)
+    config.update(vocab_size=512, cache_decrement=0, kv_heads=4, kv_quant='int8', kv_group=None,
+                  hidden_size=256, num_experts=4, kv_cache_size=128, top_k=2, capacity_factor=1.5)
+    yield config
+    config.clear()
+    config.update(saved)
+
+
+def _f64(t):
+    return t.detach().double().cpu().numpy()
+
+
+def _lora(layer, x):
+    return (x @ _f64(layer.lora_A) @ _f64(layer.lora_B)) * layer.scaling
+
+
+def _linear(lin, x):
+    return x @ _f64(lin.weight).T + _f64(lin.bias)
+
+
+@pytest.mark.parametrize("policy", ["lru", "h2o"])
+def test_pikvmoe_small_config(dev, small_config, policy):
+    import torch
+    from pikv_amd import moe
+    from pikv_amd.scheduling import SchedulingPolicy
+    torch.manual_seed(0)
+    pol = SchedulingPolicy.LRU if policy == "lru" else SchedulingPolicy.H2O
+    model = moe.PiKVMoE(use_cache_scheduling=True, cache_scheduling_policy=pol).to(dev)
+    gate = model.router.router[-1]
+    with torch.no_grad():
+        gate.weight.normal_(0.0, 0.02)
+        gate.bias.zero_()
+        for e in model.experts:          # non-zero LoRA so that the term is exercised
+            e.lora.lora_B.normal_(0.0, 0.05)
+    model.eval()
+    model.debug_capture = True
+    assert model.cache_sizes == [128, 128, 128, 128]
+    E, H, k, C = 4, 256, 2, 128
+    ref = O.CachePool([C] * E, H, H, O.Q_I8_SYM)
+    g = torch.Generator().manual_seed(0)
+    for step in range(1, 5):
+        x = torch.randn(2, 64, H, generator=g).to(dev)
+        with torch.no_grad():
+            logits = model(x)
+        cap = model.captured
+        r = cap["router"]
+        T = 128
+        assert r.capacity == O.compute_capacity(2, 64, 1.5, k, E) == 96
+        # --- router: indices against the restatement on the same gate input
+        x2 = x.reshape(T, H)
+        with torch.no_grad():
+            h = model.router._hidden_before_gate(model.router.router, x2)
+        lg64 = _f64(h) @ _f64(gate.weight).T + _f64(gate.bias)
+        order = np.sort(lg64, axis=1)[:, ::-1]
+        clear = (order[:, k - 1] - order[:, k]) > 1e-5
+        _, idx_ref, _, _ = O.router_tail(lg64.astype(np.float32), k)
+        idx = np_of(r.topk_idx)
+        assert clear.mean() > 0.9
+        assert np.array_equal(idx[clear], idx_ref[clear])
+        slot_ref, count_ref = O.capacity_slots(idx, E, r.capacity)
+        assert np.array_equal(np_of(r.slot), slot_ref)
+        assert np.array_equal(np_of(r.count), count_ref)
+        # --- cache means used by this forward = means of the restatement's state
+        means = np.zeros((E, H))
+        for c in range(E):
+            rows = ref.valid_rows(c)
+            if len(rows):
+                means[c] = O.dequantize_groups(ref.v_codes[rows], ref.v_scale[rows], ref.v_zero[rows], H).astype(np.float64).mean(0)
+        assert np.allclose(np_of(cap["cached"]), means, rtol=1e-5, atol=1e-6)
+        # --- logits against a float64 evaluation of the same graph
+        x64 = _f64(x2)
+        w = np.zeros((T, E))
+        np.put_along_axis(w, idx.astype(np.int64), np_of(r.topk_w).astype(np.float64), axis=1)
+        out = np.zeros((T, H))
+        for i, ex in enumerate(model.experts):
+            cm = means[i] + _lora(model.kv_caches[i].value_lora, means[i])
+            o = np.maximum(_linear(ex.dense, x64) + _lora(ex.lora, x64), 0.0) + cm
+            out += o * w[:, i:i + 1]
+        lref = _linear(model.vocab_proj, out)
+        got = _f64(logits).reshape(T, -1)
+        assert np.abs(got - lref).max() <= 1e-3 * np.sqrt((lref ** 2).mean())
+        # --- cache update: evict, compact, append on the restatement with the same rows
+        n_new = np.minimum(np.minimum(count_ref, r.capacity), C).astype(np.int32)
+        assert np.array_equal(np_of(cap["n_new"]), n_new)
+        for c in range(E):
+            rows = ref.valid_rows(c)
+            L = len(rows)
+            over = max(0, L + int(n_new[c]) - C)
+            if policy == "lru":
+                keep = O.lru_keep(ref.ts[rows], min(over, L))
+            elif over == 0:
+                keep = np.ones(L, dtype=bool)
+            else:
+                nh, nr = O.h2o_budget(L, 0.1, 0.1)
+                keep = O.h2o_keep(ref.acc[rows], ref.ts[rows], nh, nr)
+            if L:
+                planes = [ref.k_codes, ref.k_scale, ref.v_codes, ref.v_scale, ref.acc, ref.ts]
+                ref.fill[c] = O.compact(keep, *[p[rows[0]:rows[0] + L] for p in planes])
+        assert np.array_equal(np_of(cap["fill_before"]), ref.fill)
+        ks, vs = np_of(cap["keys"]), np_of(cap["values"])
+        ref.quant_scatter(ks, vs, idx.reshape(-1), slot_ref.reshape(-1), 1, now=float(step))
+        ref.advance(count_ref, r.capacity)
+        pool = model.pool
+        assert np.array_equal(np_of(pool.fill), ref.fill)
+        if policy == "h2o":
+            # the importance accumulation touches every valid row: timestamp = this
+            # step, accumulator grows by a distribution that sums to the head count
+            before = ref.acc.copy()
+            ref.acc[:] = np_of(pool.acc)
+            for c in range(E):
+                rows = ref.valid_rows(c)
+                ref.ts[rows] = np.float32(step)
+                gain = (ref.acc[rows] - before[rows]).astype(np.float64)
+                assert gain.min() >= 0 and abs(gain.sum() - pool.n_heads) < 1e-3 * pool.n_heads
+        for c in range(E):
+            rows = ref.valid_rows(c)
+            assert np.array_equal(np_of(pool.k_codes)[rows], ref.k_codes[rows]), (step, c)
+            assert np.array_equal(np_of(pool.v_codes)[rows], ref.v_codes[rows]), (step, c)
+            assert np.array_equal(np_of(pool.k_scale)[rows], ref.k_scale[rows])
+            assert np.array_equal(np_of(pool.v_scale)[rows], ref.v_scale[rows])
+            assert np.array_equal(np_of(pool.ts)[rows], ref.ts[rows])
+    stats = model.get_cache_stats()
+    assert set(stats) == {f"expert_{i}" for i in range(E)}
+    assert all(0 < s["cache_utilization"] <= 1.0 for s in stats.values())
+    if policy == "lru":   # the caches are full after four forwards of ~64 rows per expert
+        assert max(s["cache_size"] for s in stats.values()) == C
+
+
+def test_kvcache_standalone(dev, small_config):
+    import torch
+    from pikv_amd import moe
+    from pikv_amd.scheduling import SchedulingPolicy
+    torch.manual_seed(1)
+    cache = moe.KVCache(32, use_scheduling=True, scheduling_policy=SchedulingPolicy.LRU).to(dev)
+    assert float(cache.get_all().abs().sum()) == 0.0
+    ref = O.CachePool([32], 256, 256, O.Q_I8_SYM)
+    g = torch.Generator().manual_seed(1)
+    for step in range(4):
+        kx = torch.randn(12, 256, generator=g)
+        vx = torch.randn(12, 256, generator=g)
+        cache.update(step, kx.to(dev), vx.to(dev), None)
+        rows = ref.valid_rows(0)
+        over = max(0, len(rows) + 12 - 32)
+        if len(rows):
+            keep = O.lru_keep(ref.ts[rows], over)
+            planes = [ref.k_codes, ref.k_scale, ref.v_codes, ref.v_scale, ref.acc, ref.ts]
+            ref.fill[0] = O.compact(keep, *[p[:len(rows)] for p in planes])
+        ref.quant_scatter(kx.numpy(), vx.numpy(), np.zeros(12, np.int32), np.arange(12, dtype=np.int32), 1,
+                          now=float(step + 1))
+        ref.advance(np.array([12], np.int32))
+        rows = ref.valid_rows(0)
+        assert cache.get_cache_stats()["cache_size"] == len(rows)
+        assert np.array_equal(np_of(cache.pool.v_codes)[rows], ref.v_codes[rows])
+        want = O.dequantize_groups(ref.v_codes[rows], ref.v_scale[rows], ref.v_zero[rows], 256).mean(0)
+        assert np.allclose(np_of(cache.get_all()), want, rtol=1e-5, atol=1e-6)
