@@ -92,12 +92,149 @@ def cpu_baseline(torch, w, hidden, gate_w, k_src, v_src, q, reps=5):
                       f"(OpenMP, {CO.threads()} threads), {best:.2f} s per step"}
 
 
+def _median_ms(torch, fn, iters, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+           for _ in range(iters)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in evs)
+    return ts[len(ts) // 2]
+
+
+def _entry(ms, nbytes, **extra):
+    d = {"ms": ms, "algorithmic_bytes": nbytes, "GBps": nbytes / (ms * 1e-3) / 1e9,
+         "hbm_frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    d.update(extra)
+    return d
+
+
+def decode_read_workload(torch, ops, dev, iters):
+    """Decode read path: 64 sequences x 32768 cached tokens, 8 KV heads (GQA from 32
+    q heads) x 128, int4 asymmetric, group 32, fp16 scale/zero; H2O keeps 2048 heavy
+    + 256 recent."""
+    B, N, hkv, hq, dh = 64, 32768, 8, 32, 128
+    D = hkv * dh
+    g = torch.Generator(device=dev).manual_seed(2)
+    pool = ops.CachePool([N] * B, hkv, dh, 32, ops.Q_I4_ASYM, dev, with_v=False)
+    chunk = 4
+    slot = torch.arange(N, device=dev, dtype=torch.int32).repeat(chunk)
+    t_write = None
+    for b0 in range(0, B, chunk):
+        ks = torch.randn(chunk * N, D, generator=g, device=dev).to(torch.bfloat16)
+        cid = torch.arange(b0, b0 + chunk, device=dev, dtype=torch.int32).repeat_interleave(N)
+        if b0 == 0:
+            t_write = _median_ms(torch, lambda: pool.quant_scatter(ks, None, cid, slot, 1), iters)
+        pool.quant_scatter(ks, None, cid, slot, 1)
+    pool.fill.fill_(N)
+    q = torch.randn(B, hq, dh, generator=g, device=dev).to(torch.bfloat16)
+    t_scores = _median_ms(torch, lambda: pool.scores(q, hq), iters)
+    sc, tm, tsu = pool.scores(q, hq)
+    t_h2o = _median_ms(torch, lambda: pool.h2o_accumulate(sc, tm, tsu, now=1.0), iters)
+    t_sel = _median_ms(torch, lambda: pool.evict_select(0, heavy_ratio=1 / 16, recent_ratio=1 / 128), iters)
+
+    def evict():
+        pool.fill.fill_(N)
+        pool.evict(0, heavy_ratio=1 / 16, recent_ratio=1 / 128)
+    t_evict = _median_ms(torch, evict, iters)
+    rows = B * N
+    k_bytes = rows * (D // 2 + (D // 32) * 4)
+    return {
+        "workload": "decode read: 64 seq x 32768 cached tokens, 8 KV heads x 128 (32 q heads), int4 asym g32",
+        "quant_scatter_i4": _entry(t_write, chunk * N * (D * 2 + D // 2 + (D // 32) * 4 + 8),
+                                   rows=chunk * N),
+        "gather_dequant_scores": _entry(t_scores, k_bytes, cached_tokens_per_s=rows / (t_scores * 1e-3),
+                                        bytes_with_score_store=k_bytes + rows * hq * 4),
+        "h2o_accumulate": _entry(t_h2o, rows * hq * 4 + rows * 12),
+        "evict_select": _entry(t_sel, rows * 8 + rows * 5),
+        "evict_select_plus_compact": {"ms": t_evict},
+    }
+
+
+def wide_routing_workload(torch, ops, dev, iters):
+    """Wide MoE routing: 65536 tokens, hidden 7168, 64 experts top-8, Zipf(1.2) expert
+    popularity, EPLB-style per-expert logit scale; int8 KV of 8 heads x 128 scattered
+    to per-expert caches sized by the observed load."""
+    T, H, E, k, heads, dh = 65536, 7168, 64, 8, 8, 128
+    D = heads * dh
+    gc = torch.Generator().manual_seed(3)
+    g = torch.Generator(device=dev).manual_seed(3)
+    hidden = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    gw = (0.02 * torch.randn(E, H, generator=gc)).to(dev).to(torch.bfloat16)
+    rank = torch.randperm(E, generator=gc).float() + 1
+    pop = rank ** -1.2
+    bias = (pop / pop.sum()).log().to(dev)
+    ks = torch.randn(T, D, generator=g, device=dev).to(torch.bfloat16)
+    vs = torch.randn(T, D, generator=g, device=dev).to(torch.bfloat16)
+    warm = ops.router_fused(hidden, gw, bias, top_k=k, capacity=T)
+    load = warm.count.float() / warm.count.float().mean()
+    ew = (1.0 / load.clamp_min(0.1)).clamp(0.5, 2.0)
+    r = ops.router_fused(hidden, gw, bias, top_k=k, capacity=T, expert_scale=ew)
+    counts = r.count.cpu().tolist()
+    t_router = _median_ms(torch, lambda: ops.router_fused(hidden, gw, bias, top_k=k, capacity=T,
+                                                          expert_scale=ew), iters)
+    pool = ops.CachePool(counts, heads, dh, dh, ops.Q_I8_SYM, dev)
+    t_q = _median_ms(torch, lambda: pool.quant_scatter(ks, vs, r.topk_idx, r.slot, k), iters)
+    A = T * k
+    return {
+        "workload": "wide MoE routing: T=65536, hidden 7168, 64 experts top-8, Zipf 1.2, int8 KV 8x128",
+        "router": _entry(t_router, T * H * 2 + T * E * 4 + A * 12, tflops=2.0 * T * H * E / (t_router * 1e-3) / 1e12,
+                         tokens_per_s=T / (t_router * 1e-3)),
+        "quant_scatter": _entry(t_q, T * 2 * D * 2 + A * (2 * D + 2 * heads * 4) + A * 8,
+                                assignments_per_s=A / (t_q * 1e-3)),
+        "expert_load_max_over_mean": max(counts) / (sum(counts) / E),
+    }
+
+
+def pyramid_workload(torch, ops, dev, iters):
+    """Long-context pyramid compression: 131072 tokens, 32 layers, 8 KV heads x 128
+    bf16; layer l keeps int(N*(1-0.75*l/31)) rows by score, then int8 per token per
+    head."""
+    from pikv_amd import pyramid
+    L, N, heads, dh = 32, 131072, 8, 128
+    D = heads * dh
+    g = torch.Generator(device=dev).manual_seed(4)
+    keep = pyramid.linear_keep_budget(N, L)
+    ks = torch.empty(L, N, D, dtype=torch.bfloat16, device=dev)
+    vs = torch.empty(L, N, D, dtype=torch.bfloat16, device=dev)
+    for l in range(L):
+        ks[l] = torch.randn(N, D, generator=g, device=dev).to(torch.bfloat16)
+        vs[l] = torch.randn(N, D, generator=g, device=dev).to(torch.bfloat16)
+    z = torch.randn(L, N, generator=g, device=dev)
+    heavy = torch.rand(L, N, generator=g, device=dev) < 0.05
+    sc = torch.softmax(z + 4.0 * heavy, dim=-1).contiguous()
+    pc = pyramid.PyramidCache(keep, heads, dh, scheme=ops.Q_I8_SYM, device=dev)
+    seg_base = torch.arange(L, dtype=torch.int64, device=dev) * N
+    seg_len = torch.full((L,), N, dtype=torch.int32, device=dev)
+    nk = torch.tensor(keep, dtype=torch.int32, device=dev)
+    flat = sc.reshape(-1)
+    t_sel = _median_ms(torch, lambda: ops.select_top_rows(flat, seg_base, seg_len, nk), iters)
+    _, index, kept = ops.select_top_rows(flat, seg_base, seg_len, nk)
+    pc.pool.fill.zero_()
+    t_g = _median_ms(torch, lambda: pc.pool.quant_gather(ks, vs, seg_base, index, kept, max(keep),
+                                                         src_score=flat), iters)
+    rows = sum(keep)
+    return {
+        "workload": "pyramid compression: 32 layers x 131072 tokens, 8 heads x 128 bf16, budget 100% -> 25%, int8",
+        "select_top_rows": _entry(t_sel, L * N * 4 + L * N * 5),
+        "quant_gather": _entry(t_g, rows * (2 * D * 2 + 2 * D + 2 * heads * 4), rows=rows,
+                               rows_per_s=rows / (t_g * 1e-3)),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only-headline", action="store_true",
+                    help="skip the per-kernel figures of the decode, wide-routing and pyramid workloads")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device copy (a kernel of known traffic, to scale "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit")
@@ -190,6 +327,13 @@ def main():
             "h2o_accumulate": {"ms": t_h2o, "GBps": gbps(b_h2o, t_h2o)},
         },
     }
+    if not args.only_headline:
+        it = max(5, min(args.steps, 20))
+        out["other_workloads"] = {}
+        for name, fn in (("decode_read", decode_read_workload), ("wide_routing", wide_routing_workload),
+                         ("pyramid", pyramid_workload)):
+            out["other_workloads"][name] = fn(torch, ops, dev, it)
+            torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, w, hidden, gate_w, k_src, v_src, q)
     else:
