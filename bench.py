@@ -32,9 +32,9 @@ METRIC = "routed KV tokens/s (quant+scatter+gather+dequant), 1 MI355X; % HBM pea
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the quantise+scatter kernel on this workload, from the
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
-# profiles/bench_prefill_compress_write.md (counters scaled by what a plain 1 GiB
+# profiles/bench_all_workloads.md (counters scaled by what a plain 1 GiB
 # device copy reads on them: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
-K2_TRAFFIC_BYTES_PROFILED = 1099.1e6
+K2_TRAFFIC_BYTES_PROFILED = 1099.2e6
 
 WORKLOAD = dict(name="prefill compress-write", batch=16, seq=2048, hidden=4096, experts=8, top_k=2,
                 capacity_factor=1.25, heads=32, head_dim=128, cache_slots=8192,
