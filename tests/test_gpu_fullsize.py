@@ -1,0 +1,232 @@
+"""GPU checks at the full sizes of the benchmark workloads, through properties
+that do not need a CPU evaluation of the whole workload: round trips within half
+a quantisation step, slot/capacity invariants, exact homogeneity of the scores,
+threshold and order properties of the selections, exact row moves of the
+compaction.  The checker is torch on the GPU; the code under test is the C ABI."""
+import math
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _slot_invariants(torch, idx, slot, count, E, cap):
+    """Token-major sequential rule: the kept slots of an expert are 0..kept-1 in
+    assignment order; an assignment is dropped iff its rank >= capacity."""
+    A = idx.numel()
+    idx, slot = idx.reshape(-1).long(), slot.reshape(-1).long()
+    assert int(count.sum()) == A
+    assert torch.equal(torch.bincount(idx, minlength=E).int(), count)
+    order = torch.argsort(idx, stable=True)          # groups by expert, keeps assignment order
+    start = torch.cumsum(count.long(), 0) - count.long()
+    rank = torch.arange(A, device=idx.device) - start[idx[order]]
+    want = torch.where(rank < cap, rank, torch.full_like(rank, -1))
+    assert torch.equal(slot[order], want)
+
+
+def test_prefill_compress_write_full(dev):
+    import torch
+    from pikv_amd import ops
+    T, H, E, k, heads, dh, C = 32768, 4096, 8, 2, 32, 128, 8192
+    D = heads * dh
+    g = torch.Generator(device=dev).manual_seed(1)
+    hidden = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    gw = (0.02 * torch.randn(E, H, generator=g, device=dev)).to(torch.bfloat16)
+    ks = torch.randn(T, D, generator=g, device=dev)
+    ks[:, torch.randperm(D, generator=torch.Generator().manual_seed(1))[:41].to(dev)] *= 20
+    ks = ks.to(torch.bfloat16)
+    vs = torch.randn(T, D, generator=g, device=dev).to(torch.bfloat16)
+    cap = int(16 * 2048 * 1.25 * k / E)
+    assert cap == 10240
+    r = ops.router_fused(hidden, gw, top_k=k, capacity=cap, return_logits=True)
+    # router: softmax rows, distinct experts, descending probabilities, renormalised weights
+    assert torch.allclose(r.probs.sum(1), torch.ones(T, device=dev), atol=1e-5)
+    assert bool((r.topk_idx[:, 0] != r.topk_idx[:, 1]).all())
+    p = torch.gather(r.probs, 1, r.topk_idx.long())
+    assert bool((p[:, 0] >= p[:, 1]).all())
+    rest = r.probs.clone().scatter_(1, r.topk_idx.long(), -1.0)
+    assert bool((rest.max(1).values <= p[:, 1]).all())
+    assert torch.allclose(r.topk_w.sum(1), torch.ones(T, device=dev), atol=1e-5)
+    ref = torch.softmax(hidden.float() @ gw.float().T, dim=-1)
+    assert torch.allclose(r.probs, ref, atol=2e-4)
+    _slot_invariants(torch, r.topk_idx, r.slot, r.count, E, cap)
+    # write + read back: every kept assignment's row decodes to within half a step of its source
+    pool = ops.CachePool([C] * E, heads, dh, dh, ops.Q_I8_SYM, dev)
+    pool.quant_scatter(ks, vs, r.topk_idx, r.slot, k, now=1.0)
+    pool.advance(r.count, cap)
+    assert torch.equal(pool.fill, torch.minimum(r.count, torch.full_like(r.count, C)))
+    slot, eid = r.slot.reshape(-1).long(), r.topk_idx.reshape(-1).long()
+    kept = (slot >= 0) & (slot < C)
+    rows = pool.row_base[eid[kept]] + slot[kept]
+    src = torch.arange(T, device=dev).repeat_interleave(k)[kept]
+    assert rows.unique().numel() == rows.numel() == int(pool.fill.sum())
+    for which, x in (("k", ks), ("v", vs)):
+        codes, scale, _ = pool._planes(which)
+        xs = x[src].float().view(-1, heads, dh)
+        amax = xs.abs().amax(-1)
+        want_scale = torch.where(amax > 0, 2 * amax / 255, torch.full_like(amax, 1e-5 / 255))
+        # torch divides by a scalar through its reciprocal on the GPU: one ulp of slack
+        assert torch.allclose(scale[rows], want_scale, rtol=3e-7, atol=0)
+        dq = pool.gather_dequant(which, rows=rows).view(-1, heads, dh)
+        err = (dq - xs).abs()
+        steps = err / scale[rows].unsqueeze(-1)                          # error in quantisation steps
+        inside = xs < (127.4 * scale[rows].unsqueeze(-1))                # +absmax (code 127.5) saturates at 127
+        # exact .5 ties are common in bf16 data; q*scale rounds at 127 steps' magnitude
+        assert float(steps[inside].max()) <= 0.5 + 1e-4, float(steps[inside].max())
+        assert float(steps.max()) <= 1.0 + 1e-4
+        assert int(codes[rows].min()) >= -128 and int(codes[rows].max()) <= 127
+    assert bool((pool.ts[rows] == 1.0).all()) and bool((pool.acc[rows] == 0).all())
+
+
+def test_decode_read_full(dev):
+    import torch
+    from pikv_amd import ops
+    B, N, hkv, hq, dh = 64, 32768, 8, 32, 128
+    D = hkv * dh
+    g = torch.Generator(device=dev).manual_seed(2)
+    pool = ops.CachePool([N] * B, hkv, dh, 32, ops.Q_I4_ASYM, dev, with_v=False)
+    chunk = 8
+    slot = torch.arange(N, device=dev, dtype=torch.int32).repeat(chunk)
+    keep_src = None
+    for b0 in range(0, B, chunk):
+        ks = torch.randn(chunk * N, D, generator=g, device=dev).to(torch.bfloat16)
+        cid = torch.arange(b0, b0 + chunk, device=dev, dtype=torch.int32).repeat_interleave(N)
+        pool.quant_scatter(ks, None, cid, slot, 1)
+        if b0 == 0:
+            keep_src = ks[:N].float()                                    # sequence 0
+    pool.fill.fill_(N)
+    # int4 round trip of sequence 0: within half a step wherever the value is inside the code range
+    dq = pool.gather_dequant("k", row0=0, n=N)
+    sc = pool.k_scale[:N].float().repeat_interleave(32, dim=1)
+    zp = pool.k_zero[:N].float().repeat_interleave(32, dim=1)
+    lo, hi = (0 - zp) * sc, (15 - zp) * sc
+    inside = (keep_src >= lo) & (keep_src <= hi)
+    assert inside.float().mean() > 0.95
+    assert bool(((dq - keep_src).abs()[inside] <= (0.5 * sc * (1 + 1e-3))[inside] + 1e-6).all())
+    q = torch.randn(B, hq, dh, generator=g, device=dev).to(torch.bfloat16)
+    s1, tm, tsu = pool.scores(q, hq)
+    # scores of sequences 0 and 63 against dequantise + matmul in float32
+    for b in (0, B - 1):
+        kh = pool.gather_dequant("k", row0=b * N, n=N).view(N, hkv, dh)
+        want = torch.einsum("hd,nhd->hn", q[b].float().view(hkv, 4, dh).reshape(hq, dh),
+                            kh.repeat_interleave(4, dim=1)) / math.sqrt(dh)
+        rms = want.pow(2).mean().sqrt()
+        assert float((s1[b] - want).abs().max()) <= 1e-3 * float(rms)
+    # exact homogeneity: doubling the query doubles every score bit for bit
+    s2, _, _ = pool.scores((q * 2).contiguous(), hq)
+    assert torch.equal(s2, s1 * 2)
+    # importance: a distribution per q head, summed over heads
+    imp = pool.h2o_accumulate(s1, tm, tsu, now=7.0, return_importance=True)
+    assert torch.allclose(imp.sum(1), torch.full((B,), float(hq), device=dev), rtol=1e-3)
+    assert torch.allclose(pool.acc.view(B, N), imp, rtol=1e-6, atol=0)
+    assert bool((pool.ts == 7.0).all())
+    # make the timestamps distinct so that "recent" is well defined, then select
+    pool.ts.copy_(torch.arange(N, device=dev, dtype=torch.float32).repeat(B))
+    acc_before, ts_before = pool.acc.clone(), pool.ts.clone()
+    codes_before = pool.k_codes.clone()
+    pool.evict_select(0, heavy_ratio=1 / 16, recent_ratio=1 / 128)
+    flag = pool.keep_flag.view(B, N).bool()
+    m = pool.new_len.long()
+    assert torch.equal(flag.sum(1), m)
+    assert bool(((m >= 2048) & (m <= 2304)).all())
+    assert bool(flag[:, N - 256:].all())                                 # the 256 most recent rows
+    accv = acc_before.view(B, N)
+    heavy_only = flag.clone()
+    heavy_only[:, N - 256:] = False
+    # threshold property: every row kept as heavy scores at least as high as every dropped row
+    kept_min = torch.where(heavy_only, accv, torch.full_like(accv, float("inf"))).min(1).values
+    drop_max = torch.where(~flag, accv, torch.full_like(accv, -float("inf"))).max(1).values
+    assert bool((kept_min >= drop_max).all())
+    top = torch.topk(accv, 2048, dim=1).values[:, -1]
+    assert bool((torch.where(flag, accv, torch.full_like(accv, float("inf"))).min(1).values <= top).all())
+    assert bool(((accv > top.unsqueeze(1)) <= flag).all())              # everything above the cut is kept
+    idx = pool.keep_index.view(B, N)
+    for b in (0, 17, B - 1):
+        mb = int(m[b])
+        assert torch.equal(idx[b, :mb].long(), torch.nonzero(flag[b]).reshape(-1))
+    pool.compact()
+    assert torch.equal(pool.fill.long(), m)
+    for b in (0, 17, B - 1):
+        mb = int(m[b])
+        src = b * N + idx[b, :mb].long()
+        assert torch.equal(pool.acc[b * N:b * N + mb], acc_before[src])
+        assert torch.equal(pool.ts[b * N:b * N + mb], ts_before[src])
+        assert torch.equal(pool.k_codes[b * N:b * N + mb], codes_before[src])
+    # idempotence: a second eviction with budgets that cover the cache keeps everything in place
+    pool.evict_select(0, n_heavy=pool.fill.clone(), n_recent=torch.zeros_like(pool.fill))
+    assert torch.equal(pool.new_len, pool.fill)
+    k0 = pool.k_codes.clone()
+    pool.compact()
+    assert torch.equal(pool.k_codes, k0)
+
+
+def test_wide_routing_full(dev):
+    import torch
+    from pikv_amd import ops
+    T, H, E, k, heads, dh = 65536, 7168, 64, 8, 8, 128
+    D = heads * dh
+    g = torch.Generator(device=dev).manual_seed(3)
+    gc = torch.Generator().manual_seed(3)
+    hidden = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    gw = (0.02 * torch.randn(E, H, generator=gc)).to(dev).to(torch.bfloat16)
+    pop = (torch.randperm(E, generator=gc).float() + 1) ** -1.2
+    bias = (pop / pop.sum()).log().to(dev)
+    ew = (0.5 + torch.rand(E, generator=gc)).to(dev)
+    r = ops.router_fused(hidden, gw, bias, top_k=k, capacity=T, expert_scale=ew, return_logits=True)
+    lg = (hidden.float() @ gw.float().T + bias) * ew
+    assert torch.allclose(r.logits, lg, atol=2e-3, rtol=1e-4)
+    # top-k of the logits the kernel itself produced: exact, ties to the lower index
+    order = torch.sort(r.logits, dim=1, descending=True, stable=True).indices[:, :k]
+    assert torch.equal(r.topk_idx.long(), order)
+    assert torch.allclose(r.topk_w.sum(1), torch.ones(T, device=dev), atol=1e-5)
+    _slot_invariants(torch, r.topk_idx, r.slot, r.count, E, T)
+    counts = r.count.cpu().tolist()
+    assert max(counts) > 3 * (T * k / E)                                 # the skew is there
+    pool = ops.CachePool(counts, heads, dh, dh, ops.Q_I8_SYM, dev)
+    ks = torch.randn(T, D, generator=g, device=dev).to(torch.bfloat16)
+    vs = torch.randn(T, D, generator=g, device=dev).to(torch.bfloat16)
+    pool.quant_scatter(ks, vs, r.topk_idx, r.slot, k)
+    pool.advance(r.count)
+    assert torch.equal(pool.fill, r.count)
+    rows = pool.row_base[r.topk_idx.reshape(-1).long()] + r.slot.reshape(-1).long()
+    assert rows.unique().numel() == T * k == pool.rows                   # every row written exactly once
+    codes1, scale1, _ = ops.quantize_rows(ks, dh, ops.Q_I8_SYM)
+    src = torch.arange(T, device=dev).repeat_interleave(k)
+    assert torch.equal(pool.k_codes[rows], codes1[src])
+    assert torch.equal(pool.k_scale[rows], scale1[src])
+
+
+def test_pyramid_full(dev):
+    import torch
+    from pikv_amd import ops, pyramid
+    L, N, heads, dh = 32, 131072, 8, 128
+    D = heads * dh
+    keep = pyramid.linear_keep_budget(N, L)
+    assert keep[0] == N and keep[-1] == N // 4 and sum(keep) == 2621425
+    g = torch.Generator(device=dev).manual_seed(4)
+    ks = torch.empty(L, N, D, dtype=torch.bfloat16, device=dev)
+    vs = torch.empty(L, N, D, dtype=torch.bfloat16, device=dev)
+    for l in range(L):
+        ks[l] = torch.randn(N, D, generator=g, device=dev).to(torch.bfloat16)
+        vs[l] = torch.randn(N, D, generator=g, device=dev).to(torch.bfloat16)
+    z = torch.randn(L, N, generator=g, device=dev)
+    sc = torch.softmax(z + 4.0 * (torch.rand(L, N, generator=g, device=dev) < 0.05), dim=-1).contiguous()
+    pc = pyramid.PyramidCache(keep, heads, dh, scheme=ops.Q_I8_SYM, device=dev)
+    index, kept = pc.compress(ks, vs, sc, now=2.0)
+    pool = pc.pool
+    want = torch.tensor(keep, dtype=torch.int32, device=dev)
+    assert torch.equal(kept, want) and torch.equal(pool.fill, want)
+    idx = index.view(L, N).long()
+    for l in (0, 1, 13, L - 1):
+        kl = keep[l]
+        sel = idx[l, :kl]
+        assert bool((sel[1:] > sel[:-1]).all())                          # original order kept
+        # the kept set is the top-keep_l in (score desc, index asc) order
+        order = torch.sort(sc[l], descending=True, stable=True).indices[:kl]
+        assert torch.equal(sel, torch.sort(order).values)
+        base = int(pool.row_base[l])
+        codes1, scale1, _ = ops.quantize_rows(vs[l][sel].contiguous(), dh, ops.Q_I8_SYM)
+        assert torch.equal(pool.v_codes[base:base + kl], codes1)
+        assert torch.equal(pool.v_scale[base:base + kl], scale1)
+        assert torch.equal(pool.acc[base:base + kl], sc[l][sel])
