@@ -21,6 +21,8 @@ Pinning status (what, besides this file, fixes each function's output):
                                        restatement
   scores / h2o ....................... float64 closed forms, C restatement
   select / compact ................... brute force on tiny inputs, invariants
+  streaming / quest / flexgen / lru+ . hand-computed known answers, brute-force
+                                       ranking on tiny inputs
 The reference's own tests hold no golden vectors for any of these.
 """
 from __future__ import annotations
@@ -502,6 +504,58 @@ def lru_keep(access_times: np.ndarray, n_evict: int) -> np.ndarray:
     if n_evict > 0:
         keep[topk_asc(access_times[None, :], min(n_evict, L))[0]] = False
     return keep
+
+
+def streaming_keep(cache_len: int, start_size: int, recent_size: int) -> np.ndarray:
+    """Keep the first start_size rows and the rows from
+    max(start_size, cache_len - recent_size) on (core/single/cache_scheduling.py:125-132)."""
+    keep = np.zeros(cache_len, dtype=bool)
+    keep[:start_size] = True
+    keep[max(start_size, cache_len - recent_size):] = True
+    return keep
+
+
+def quest_utility(quality, frequency, last_access, now, decay_factor) -> np.ndarray:
+    """utility = quality * frequency * decay^(now - last access)
+    (core/single/cache_scheduling.py:166-176), float32."""
+    decay = np.power(F32(decay_factor), (F32(now) - np.asarray(last_access, F32))).astype(F32)
+    return (np.asarray(quality, F32) * np.asarray(frequency, F32) * decay).astype(F32)
+
+
+def evict_lowest(score: np.ndarray, n_evict: int) -> np.ndarray:
+    """EVICT mask of the n_evict lowest scores (topk largest=False,
+    core/single/cache_scheduling.py:197,245,343), ties to the lower index."""
+    L = score.shape[0]
+    ev = np.zeros(L, dtype=bool)
+    if n_evict > 0:
+        ev[topk_asc(np.asarray(score, F32)[None, :], min(n_evict, L))[0]] = True
+    return ev
+
+
+def quest_evict(utility: np.ndarray, threshold: float, n_evict: int) -> np.ndarray:
+    """Rows below the threshold go; when they are fewer than n_evict, the n_evict
+    lowest go instead (core/single/cache_scheduling.py:190-201)."""
+    below = np.asarray(utility, F32) < F32(threshold)
+    if below.sum() < n_evict:
+        return evict_lowest(utility, n_evict)
+    return below
+
+
+def flexgen_benefit(frequency, cost) -> np.ndarray:
+    """benefit = access frequency / access cost (core/single/cache_scheduling.py:241)."""
+    return (np.asarray(frequency, F32) / np.asarray(cost, F32)).astype(F32)
+
+
+def lruplus_priority(times, frequency, importance, frequency_weight=0.3,
+                     importance_weight=0.4) -> np.ndarray:
+    """priority = w_r*t/(max t + 1e-8) + w_f*f/(max f + 1e-8) + w_i*importance with
+    w_r = 1 - w_f - w_i (core/single/cache_scheduling.py:296,311-327), float32."""
+    t, f = np.asarray(times, F32), np.asarray(frequency, F32)
+    w_r = 1.0 - frequency_weight - importance_weight
+    rec = (t / (t.max() + F32(1e-8))).astype(F32)
+    frq = (f / (f.max() + F32(1e-8))).astype(F32)
+    return (F32(w_r) * rec + F32(frequency_weight) * frq
+            + F32(importance_weight) * np.asarray(importance, F32)).astype(F32)
 
 
 def compact(keep: np.ndarray, *planes):

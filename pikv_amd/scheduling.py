@@ -4,8 +4,17 @@
   SchedulingPolicy ................ :9-17
   BaseScheduler ................... :19-51   (hit/miss/eviction counters)
   H2OScheduler .................... :53-99   (accumulator, timestamps, heavy/recent keep set)
+  StreamingLLMScheduler ........... :101-134 (first tokens + recent window)
+  QUESTScheduler .................. :136-203 (quality x frequency x time decay, threshold)
+  FlexGenScheduler ................ :205-251 (access frequency / access cost)
   LRUScheduler .................... :253-285
+  LRUPlusScheduler ................ :287-349 (recency + frequency + importance)
   CacheSchedulingManager .......... :351-467 (append / evict / compact / stats)
+
+Every policy is "a score per row, then keep the top / drop the bottom": the score
+is a handful of elementwise operations on [cache_size] buffers (left to torch),
+the selection - exact top-k with ties to the lower index - runs in
+pikv_evict_select, as does everything that moves rows.
 
 Selection and compaction run in pikv_evict_select / pikv_compact_rows; the
 manager stores its rows as integer codes in a one-cache CachePool (quantise +
@@ -66,7 +75,7 @@ class BaseScheduler(nn.Module):
 
 
 def _one_cache_select(policy: int, acc: Optional[torch.Tensor], ts: torch.Tensor, length: int,
-                      *, heavy_ratio=0.1, recent_ratio=0.1, n_evict=0) -> torch.Tensor:
+                      *, heavy_ratio=0.1, recent_ratio=0.1, n_evict=0, budgets=None) -> torch.Tensor:
     """Run the native selection on a single cache of `length` rows whose state is
     acc/ts (float32, >= length entries).  Returns the bool EVICT mask [length]."""
     from . import _native as N
@@ -83,7 +92,10 @@ def _one_cache_select(policy: int, acc: Optional[torch.Tensor], ts: torch.Tensor
     kidx = torch.empty(length, **i32)
     new_len = torch.empty(1, **i32)
     st = torch.cuda.current_stream().cuda_stream
-    if policy == ops.EVICT_H2O:
+    if policy == ops.EVICT_H2O and budgets is not None:   # explicit (n_heavy, n_recent)
+        nh.fill_(int(budgets[0]))
+        nr.fill_(int(budgets[1]))
+    elif policy == ops.EVICT_H2O:
         N.call("pikv_h2o_budget", fill.data_ptr(), 1, float(heavy_ratio), float(recent_ratio),
                nh.data_ptr(), nr.data_ptr(), st)
     else:
@@ -142,6 +154,173 @@ class LRUScheduler(BaseScheduler):
                                  n_evict=cache_len - self.cache_size)
 
 
+def _evict_lowest(score: torch.Tensor, cache_len: int, n_evict: int) -> torch.Tensor:
+    """EVICT mask of the n_evict lowest scores among the first cache_len (ties: the
+    lower index goes first), through the native smallest-n selection."""
+    if n_evict <= 0:
+        return torch.zeros(cache_len, dtype=torch.bool, device=score.device)
+    return _one_cache_select(ops.EVICT_LRU, None, score[:cache_len].float().contiguous(), cache_len,
+                             n_evict=min(n_evict, cache_len))
+
+
+def _padded(buf: torch.Tensor, n: int, fill: float = 0.0) -> torch.Tensor:
+    """First n entries of a per-slot buffer; slots beyond the tracked range read `fill`."""
+    if buf.numel() >= n:
+        return buf[:n]
+    return torch.cat([buf, torch.full((n - buf.numel(),), fill, dtype=buf.dtype, device=buf.device)])
+
+
+class StreamingLLMScheduler(BaseScheduler):
+    """Keep the first start_size rows and the last recent_size rows (:101-134)."""
+
+    def __init__(self, cache_size: int, hidden_size: int, start_size: int = 4,
+                 recent_size: Optional[int] = None):
+        super().__init__(cache_size, hidden_size)
+        self.start_size = start_size
+        self.recent_size = recent_size if recent_size is not None else (cache_size - start_size)
+        self.register_buffer("position_counter", torch.tensor(0))
+
+    def keep_budgets(self, cache_len: int):
+        """(rows kept at the front, rows kept at the back) of a cache_len-row cache."""
+        n_start = min(self.start_size, cache_len)
+        recent_start = max(self.start_size, cache_len - self.recent_size)
+        return n_start, max(0, cache_len - recent_start)
+
+    def select_eviction_candidates(self, keys, values, metadata) -> torch.Tensor:
+        cache_len = keys.size(0)
+        if cache_len <= self.cache_size:
+            return torch.zeros(cache_len, dtype=torch.bool, device=keys.device)
+        return self.evict_mask(cache_len, keys.device)
+
+    def evict_mask(self, cache_len: int, device) -> torch.Tensor:
+        # position is the score: the "heavy" set takes the lowest positions, the
+        # "recent" set the highest
+        pos = torch.arange(cache_len, dtype=torch.float32, device=device)
+        n_start, n_recent = self.keep_budgets(cache_len)
+        return _one_cache_select(ops.EVICT_H2O, (-pos).contiguous(), pos, cache_len,
+                                 budgets=(n_start, n_recent))
+
+
+class QUESTScheduler(BaseScheduler):
+    """utility = quality * usage frequency * decay^(now - last access); rows below
+    the threshold go, or the lowest cache_len - cache_size when those are too few
+    (:136-203)."""
+
+    def __init__(self, cache_size: int, hidden_size: int, quality_threshold: float = 0.1,
+                 decay_factor: float = 0.95):
+        super().__init__(cache_size, hidden_size)
+        self.quality_threshold = quality_threshold
+        self.decay_factor = decay_factor
+        self.register_buffer("quality_scores", torch.zeros(cache_size))
+        self.register_buffer("usage_frequency", torch.zeros(cache_size))
+        self.register_buffer("last_access_time", torch.zeros(cache_size))
+        self.register_buffer("global_time", torch.tensor(0))
+
+    def update_quality_scores(self, indices: torch.Tensor, reconstruction_errors: torch.Tensor):
+        self.quality_scores[indices] = 1.0 / (1.0 + reconstruction_errors)
+        self.usage_frequency[indices] += 1
+        self.last_access_time[indices] = self.global_time.float()
+        self.global_time += 1
+
+    def compute_utility_scores(self, cache_len: int) -> torch.Tensor:
+        last = _padded(self.last_access_time, cache_len)
+        decay = torch.pow(torch.tensor(self.decay_factor, device=last.device),
+                          self.global_time.float() - last)
+        return _padded(self.quality_scores, cache_len) * _padded(self.usage_frequency, cache_len) * decay
+
+    def row_buffers(self):
+        return [self.quality_scores, self.usage_frequency, self.last_access_time]
+
+    def evict_mask(self, cache_len: int, n_evict: int) -> torch.Tensor:
+        utility = self.compute_utility_scores(cache_len)
+        below = utility < self.quality_threshold
+        if int(below.sum()) < n_evict:
+            return _evict_lowest(utility, cache_len, n_evict)
+        return below
+
+    def select_eviction_candidates(self, keys, values, metadata) -> torch.Tensor:
+        cache_len = keys.size(0)
+        if cache_len <= self.cache_size:
+            return torch.zeros(cache_len, dtype=torch.bool, device=keys.device)
+        return self.evict_mask(cache_len, cache_len - self.cache_size)
+
+
+class FlexGenScheduler(BaseScheduler):
+    """benefit = access frequency / access cost; the lowest go (:205-251)."""
+
+    def __init__(self, cache_size: int, hidden_size: int, gpu_ratio: float = 0.3,
+                 cpu_ratio: float = 0.5):
+        super().__init__(cache_size, hidden_size)
+        self.gpu_ratio, self.cpu_ratio = gpu_ratio, cpu_ratio
+        self.gpu_cache_size = int(cache_size * gpu_ratio)
+        self.cpu_cache_size = int(cache_size * cpu_ratio)
+        self.disk_cache_size = cache_size - self.gpu_cache_size - self.cpu_cache_size
+        self.register_buffer("access_frequency", torch.zeros(cache_size))
+        self.register_buffer("access_cost", torch.ones(cache_size))
+        self.register_buffer("cache_level", torch.zeros(cache_size, dtype=torch.long))
+
+    def update_access_patterns(self, indices: torch.Tensor, access_costs: torch.Tensor):
+        self.access_frequency[indices] += 1
+        self.access_cost[indices] = access_costs
+
+    def compute_benefit_scores(self, cache_len: int) -> torch.Tensor:
+        return _padded(self.access_frequency, cache_len) / _padded(self.access_cost, cache_len, 1.0)
+
+    def row_buffers(self):
+        return [self.access_frequency, self.access_cost]
+
+    def evict_mask(self, cache_len: int, n_evict: int) -> torch.Tensor:
+        return _evict_lowest(self.compute_benefit_scores(cache_len), cache_len, n_evict)
+
+    def select_eviction_candidates(self, keys, values, metadata) -> torch.Tensor:
+        cache_len = keys.size(0)
+        if cache_len <= self.cache_size:
+            return torch.zeros(cache_len, dtype=torch.bool, device=keys.device)
+        return self.evict_mask(cache_len, cache_len - self.cache_size)
+
+
+class LRUPlusScheduler(BaseScheduler):
+    """priority = w_r * recency + w_f * frequency + w_i * importance, recency and
+    frequency normalised by their maxima; the lowest go (:287-349)."""
+
+    def __init__(self, cache_size: int, hidden_size: int, frequency_weight: float = 0.3,
+                 importance_weight: float = 0.4):
+        super().__init__(cache_size, hidden_size)
+        self.frequency_weight = frequency_weight
+        self.importance_weight = importance_weight
+        self.recency_weight = 1.0 - frequency_weight - importance_weight
+        self.register_buffer("access_times", torch.zeros(cache_size))
+        self.register_buffer("access_frequency", torch.zeros(cache_size))
+        self.register_buffer("importance_scores", torch.zeros(cache_size))
+        self.register_buffer("global_time", torch.tensor(0))
+
+    def update_access_info(self, indices: torch.Tensor, importance: torch.Tensor):
+        self.access_times[indices] = self.global_time.float()
+        self.access_frequency[indices] += 1
+        self.importance_scores[indices] = importance
+        self.global_time += 1
+
+    def compute_priority_scores(self, cache_len: int) -> torch.Tensor:
+        times = _padded(self.access_times, cache_len)
+        freq = _padded(self.access_frequency, cache_len)
+        recency = times / (times.max() + 1e-8)
+        frequency = freq / (freq.max() + 1e-8)
+        return (self.recency_weight * recency + self.frequency_weight * frequency +
+                self.importance_weight * _padded(self.importance_scores, cache_len))
+
+    def row_buffers(self):
+        return [self.access_times, self.access_frequency, self.importance_scores]
+
+    def evict_mask(self, cache_len: int, n_evict: int) -> torch.Tensor:
+        return _evict_lowest(self.compute_priority_scores(cache_len), cache_len, n_evict)
+
+    def select_eviction_candidates(self, keys, values, metadata) -> torch.Tensor:
+        cache_len = keys.size(0)
+        if cache_len <= self.cache_size:
+            return torch.zeros(cache_len, dtype=torch.bool, device=keys.device)
+        return self.evict_mask(cache_len, cache_len - self.cache_size)
+
+
 _NATIVE = {SchedulingPolicy.H2O: ops.EVICT_H2O, SchedulingPolicy.LRU: ops.EVICT_LRU}
 
 
@@ -191,9 +370,14 @@ class CacheSchedulingManager(nn.Module):
             return H2OScheduler(self.cache_size, self.hidden_size, self.heavy_ratio, self.recent_ratio)
         if policy == SchedulingPolicy.LRU:
             return LRUScheduler(self.cache_size, self.hidden_size)
-        if isinstance(policy, SchedulingPolicy):
-            raise NotImplementedError(
-                f"{policy.value}: only H2O and LRU run on the native selection kernel in this build")
+        if policy == SchedulingPolicy.STREAMING_LLM:
+            return StreamingLLMScheduler(self.cache_size, self.hidden_size)
+        if policy == SchedulingPolicy.QUEST:
+            return QUESTScheduler(self.cache_size, self.hidden_size)
+        if policy == SchedulingPolicy.FLEXGEN:
+            return FlexGenScheduler(self.cache_size, self.hidden_size)
+        if policy == SchedulingPolicy.LRU_PLUS:
+            return LRUPlusScheduler(self.cache_size, self.hidden_size)
         raise ValueError(f"Unknown scheduling policy: {policy}")
 
     def _ensure_pool(self, device):
@@ -244,12 +428,16 @@ class CacheSchedulingManager(nn.Module):
         n = k2.shape[0]
         cur = self._fill_host
         if cur + n > self.cache_size and cur > 0:
+            n_ev = min(cur, cur + n - self.cache_size)
             if self.policy == SchedulingPolicy.H2O:
                 pool.evict(ops.EVICT_H2O, heavy_ratio=self.scheduler.heavy_ratio,
                            recent_ratio=self.scheduler.recent_ratio)
-            elif not self.legacy_no_evict:
-                n_ev = min(cur, cur + n - self.cache_size)
+            elif self.legacy_no_evict:
+                pass
+            elif self.policy == SchedulingPolicy.LRU:
                 pool.evict(ops.EVICT_LRU, n_evict=torch.tensor([n_ev], dtype=torch.int32, device=pool.device))
+            else:
+                self._evict_by_scheduler(pool, cur, n_ev)
             new_cur = int(pool.fill.item())
             self.scheduler.eviction_count += cur - new_cur
             cur = new_cur
@@ -261,6 +449,31 @@ class CacheSchedulingManager(nn.Module):
         pool.advance(torch.tensor([n], dtype=torch.int32, device=dev))
         self._fill_host = min(cur + n, self.cache_size)
         self.cache_valid = torch.arange(self.cache_size) < self._fill_host
+
+    def _evict_by_scheduler(self, pool, cur: int, n_ev: int):
+        """StreamingLLM / QUEST / FlexGen / LRU+: the scheduler scores its slots, the
+        native selection turns the score into a keep list, and the compaction moves
+        the scheduler's per-slot buffers together with the rows."""
+        sch = self.scheduler.to(pool.device)
+        if isinstance(sch, StreamingLLMScheduler):
+            # room for the new rows: the window shrinks to what fits beside the start tokens
+            n_start = min(sch.start_size, cur)
+            n_recent = max(0, min(cur - n_start, cur - n_ev - n_start))
+            pos = torch.arange(pool.rows, dtype=torch.float32, device=pool.device)
+            evict = _one_cache_select(ops.EVICT_H2O, (-pos).contiguous(), pos, cur,
+                                      budgets=(n_start, n_recent))
+            extra = []
+        else:
+            evict = sch.evict_mask(cur, n_ev)
+            extra = sch.row_buffers()
+        keep = ~evict
+        m = int(keep.sum())
+        pool.keep_flag[:cur] = keep.to(torch.uint8)
+        pool.keep_index[:m] = torch.nonzero(keep).reshape(-1).to(torch.int32)
+        pool.new_len.fill_(m)
+        pool.compact(extra_planes=extra)
+        for b in extra:   # slots behind the survivors start fresh
+            b[m:] = 1.0 if b is getattr(sch, "access_cost", None) else 0.0
 
     def get_cache_stats(self) -> Dict[str, float]:
         stats = {"cache_size": self._fill_host,

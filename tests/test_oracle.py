@@ -351,3 +351,32 @@ def test_compact_is_stable_and_in_place():
     b = np.arange(16, dtype=np.int16).reshape(8, 2)
     m = O.compact(keep, a, b)
     assert m == 4 and a[:4].tolist() == [1, 2, 4, 7] and b[:4, 0].tolist() == [2, 4, 8, 14]
+
+
+def test_other_policies_known_answers():
+    """StreamingLLM / QUEST / FlexGen / LRU+ restatements against hand-computed values
+    and a brute-force ranking."""
+    # StreamingLLM: 10 rows, 2 start + 3 recent -> rows 0,1 and 7,8,9
+    assert O.streaming_keep(10, 2, 3).tolist() == [True, True] + [False] * 5 + [True] * 3
+    # window larger than the cache: everything stays
+    assert O.streaming_keep(5, 4, 124).all()
+    # QUEST: quality .5, used twice, last touched 2 ticks ago, decay .5 -> .5*2*.25 = .25
+    u = O.quest_utility([0.5, 1.0, 0.0], [2, 1, 5], [3, 5, 5], 5, 0.5)
+    assert np.allclose(u, [0.25, 1.0, 0.0])
+    assert O.quest_evict(u, 0.3, 1).tolist() == [True, False, True]     # two below the threshold
+    assert O.quest_evict(u, 0.1, 2).tolist() == [True, False, True]     # too few below: the two lowest
+    # FlexGen: freq/cost
+    b = O.flexgen_benefit([4, 1, 9, 0], [2, 1, 3, 1])
+    assert b.tolist() == [2.0, 1.0, 3.0, 0.0]
+    assert O.evict_lowest(b, 2).tolist() == [False, True, False, True]
+    # LRU+: weights .3/.3/.4, times [0,5,10], freq [1,2,4], importance [1,0,.5]
+    p = O.lruplus_priority([0, 5, 10], [1, 2, 4], [1.0, 0.0, 0.5])
+    assert np.allclose(p, [0.3 * 0.25 + 0.4, 0.3 * 0.5 + 0.3 * 0.5, 0.3 + 0.3 + 0.2], atol=1e-6)
+    # lowest-n against an O(n^2) ranking with ties (lower index goes first)
+    r = np.random.default_rng(11)
+    s = (np.round(r.random(40) * 6) / 6).astype(np.float32)
+    for n in (0, 1, 7, 40):
+        ev = O.evict_lowest(s, n)
+        for i in range(40):
+            before = sum((s[j] < s[i]) or (s[j] == s[i] and j < i) for j in range(40))
+            assert ev[i] == (before < n)
