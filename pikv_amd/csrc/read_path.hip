@@ -345,12 +345,10 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 // the (scale, zero) it loaded itself: no transpose, one epilogue per 16 tokens
 // instead of one per MFMA, and a 3-swap transpose-reduction over the four
 // row-groups leaves row-group r with the finished score of head r.
-// (x & m) | o in one instruction (one scalar operand at most per instruction).
-__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(m), "v"(o));
-  return r;
-}
+// (x & m) | o.  Plain C on purpose: the value feeds a matrix-core operand, and a
+// result produced inside an inline-asm block is invisible to the compiler's
+// hazard handling between vector and matrix-core instructions.
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) { return (x & m) | o; }
 
 constexpr int kGqaTilesPerBlock = 4;   // consecutive 64-token tiles handled by one block
 constexpr int kGqaMaxKvHeads = 16;     // code vectors of one 16-token slice kept in registers
