@@ -298,6 +298,27 @@ __device__ __forceinline__ void group_minmax_dpp(float& mn, float& mx, int lanes
   if (lanes >= 64) { mn = fminf(mn, __shfl_xor(mn, 32, PIKV_WAVE)); mx = fmaxf(mx, __shfl_xor(mx, 32, PIKV_WAVE)); }
 }
 
+// Sum / max over aligned groups of `lanes` (a power of two <= 64) adjacent lanes;
+// every lane of the group ends with the result.
+__device__ __forceinline__ float group_sum_dpp(float v, int lanes) {
+  if (lanes >= 2) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "quad_perm:[1,0,3,2]");
+  if (lanes >= 4) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "quad_perm:[2,3,0,1]");
+  if (lanes >= 8) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "row_half_mirror");
+  if (lanes >= 16) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "row_mirror");
+  if (lanes >= 32) v += __shfl_xor(v, 16, PIKV_WAVE);
+  if (lanes >= 64) v += __shfl_xor(v, 32, PIKV_WAVE);
+  return v;
+}
+__device__ __forceinline__ float group_max_dpp(float v, int lanes) {
+  if (lanes >= 2) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "quad_perm:[1,0,3,2]");
+  if (lanes >= 4) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "quad_perm:[2,3,0,1]");
+  if (lanes >= 8) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "row_half_mirror");
+  if (lanes >= 16) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "row_mirror");
+  if (lanes >= 32) v = fmaxf(v, __shfl_xor(v, 16, PIKV_WAVE));
+  if (lanes >= 64) v = fmaxf(v, __shfl_xor(v, 32, PIKV_WAVE));
+  return v;
+}
+
 // Pack the codes of one lane (16 x 8-bit or 32 x 4-bit) into 16 bytes.
 template <int SCHEME>
 __device__ __forceinline__ uint4 pack_codes(const int* c) {

@@ -93,27 +93,35 @@ struct ScoreArgs {
   int n_kv_heads;
   int n_q_heads;
   int head_dim;
+  int head_split;   // scores_kernel: blocks along z share a tile, each owns n_kv_heads/head_split heads
 };
 
 template <int SCHEME, int REP, int Q_DT>
 __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   using Q = QScheme<SCHEME>;
   constexpr int EPL = Q::epl;
-  __shared__ float stage[kMaxQHeads * kTile];  // [q head][token in tile]
+  __shared__ float stage[kMaxQHeads * kTile];  // [q head of this block][token in tile]
 
   const int c = blockIdx.y;
   const int64_t tile = blockIdx.x;
   const int len = a.fill[c];
   const int64_t n0 = tile * kTile;
   if (n0 >= len) return;  // uniform for the block
+  // A block owns the kv heads [kv0, kv0 + kv_blk) of its tile: wide rows are split
+  // over several blocks so that while one block reduces its tile, others still load.
+  const int kv_blk = a.n_kv_heads / a.head_split;
+  const int kv0 = blockIdx.z * kv_blk;
   const int D = a.n_kv_heads * a.head_dim;
-  const int lanes_per_row = D / EPL;           // <= 256, divides 256
-  const int lanes_per_head = a.head_dim / EPL; // power of two
+  const int lanes_per_row = D / EPL;                         // lanes of a whole cached row
+  const int lanes_per_head = a.head_dim / EPL;               // power of two
+  const int lanes_blk = kv_blk * lanes_per_head;             // <= 256, divides 256
   const int groups_per_row = D / a.group;
-  const int tok_per_step = 256 / lanes_per_row;
-  const int part = threadIdx.x % lanes_per_row;  // fixed (kv head, slice) of this lane
-  const int tok_in_step = threadIdx.x / lanes_per_row;
-  const int kvh = part / lanes_per_head;
+  const int tok_per_step = 256 / lanes_blk;
+  const int part_blk = threadIdx.x % lanes_blk;
+  const int part = kv0 * lanes_per_head + part_blk;          // fixed (kv head, slice) of this lane
+  const int tok_in_step = threadIdx.x / lanes_blk;
+  const int kvl = part_blk / lanes_per_head;                 // kv head inside the block
+  const int kvh = kv0 + kvl;
   const int d0 = (part % lanes_per_head) * EPL;
 
   // Query slices of the REP heads that read this kv head, and their sums (for the
@@ -164,9 +172,9 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
 #pragma unroll
         for (int j = 0; j < EPL; ++j) d = fmaf(qv[r][j], cf[j], d);
         d = (d - zu * qsum[r]) * sc[u];
-        for (int m = 1; m < lanes_per_head; m <<= 1) d += __shfl_xor(d, m, PIKV_WAVE);
+        d = group_sum_dpp(d, lanes_per_head);
         if ((part % lanes_per_head) == 0 && tl < kTile)
-          stage[(kvh * REP + r) * kTile + tl] = ok[u] ? d * a.scale_qk : -__builtin_inff();
+          stage[(kvl * REP + r) * kTile + tl] = ok[u] ? d * a.scale_qk : -__builtin_inff();
       }
     }
   }
@@ -176,13 +184,15 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   // reduce the tile's softmax statistics.
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  for (int hq = wave; hq < a.n_q_heads; hq += 4) {
-    const float s = stage[hq * kTile + lane];
+  const int hq_blk = kv_blk * REP;
+  for (int hl = wave; hl < hq_blk; hl += 4) {
+    const int hq = kv0 * REP + hl;
+    const float s = stage[hl * kTile + lane];
     const bool ok = n0 + lane < len;
     if (ok) a.scores[((int64_t)c * a.n_q_heads + hq) * a.score_stride + n0 + lane] = s;
-    const float m = group_max<64>(ok ? s : -__builtin_inff());
-    const float e = ok ? expf(s - m) : 0.f;
-    const float sum = group_sum<64>(e);
+    const float m = group_max_dpp(ok ? s : -__builtin_inff(), 64);
+    const float e = ok ? __builtin_amdgcn_exp2f((s - m) * 1.4426950408889634f) : 0.f;
+    const float sum = group_sum_dpp(e, 64);
     if (lane == 0) {
       const int64_t ti = ((int64_t)c * a.n_q_heads + hq) * a.n_tiles + tile;
       a.tile_max[ti] = m;
@@ -773,7 +783,7 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
   if (n_tiles > 0x7fffffffLL) return PIKV_ERR_SHAPE;
   ScoreArgs a{k_codes, k_scale, k_zero, q, cache_row_base, cache_fill, scores, tile_max, tile_sum,
-              score_stride, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim};
+              score_stride, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim, 1};
   const dim3 grid((unsigned)n_tiles, (unsigned)n_caches);
   hipStream_t st = (hipStream_t)stream;
   const int rep = n_q_heads / n_kv_heads;
@@ -793,12 +803,15 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
     PIKV_CHECK_LAUNCH();
     return PIKV_OK;
   }
+  // rows wider than one wavefront are split by kv heads over several blocks per tile
+  while (lanes_per_row / a.head_split > 64 && n_kv_heads % (a.head_split * 2) == 0) a.head_split *= 2;
+  const dim3 vgrid((unsigned)n_tiles, (unsigned)n_caches, (unsigned)a.head_split);
   int rc = PIKV_ERR_UNSUPPORTED;
   switch (scheme) {
-    case PIKV_Q_I8_SYM: rc = launch_scores<PIKV_Q_I8_SYM>(rep, grid, st, q_dtype, a); break;
-    case PIKV_Q_I8_ASYM: rc = launch_scores<PIKV_Q_I8_ASYM>(rep, grid, st, q_dtype, a); break;
-    case PIKV_Q_I4_ASYM: rc = launch_scores<PIKV_Q_I4_ASYM>(rep, grid, st, q_dtype, a); break;
-    case PIKV_Q_I4_SYM: rc = launch_scores<PIKV_Q_I4_SYM>(rep, grid, st, q_dtype, a); break;
+    case PIKV_Q_I8_SYM: rc = launch_scores<PIKV_Q_I8_SYM>(rep, vgrid, st, q_dtype, a); break;
+    case PIKV_Q_I8_ASYM: rc = launch_scores<PIKV_Q_I8_ASYM>(rep, vgrid, st, q_dtype, a); break;
+    case PIKV_Q_I4_ASYM: rc = launch_scores<PIKV_Q_I4_ASYM>(rep, vgrid, st, q_dtype, a); break;
+    case PIKV_Q_I4_SYM: rc = launch_scores<PIKV_Q_I4_SYM>(rep, vgrid, st, q_dtype, a); break;
   }
   if (rc != PIKV_OK) return rc;
   PIKV_CHECK_LAUNCH();
