@@ -298,15 +298,22 @@ __device__ __forceinline__ void group_minmax_dpp(float& mn, float& mx, int lanes
   if (lanes >= 64) { mn = fminf(mn, __shfl_xor(mn, 32, PIKV_WAVE)); mx = fmaxf(mx, __shfl_xor(mx, 32, PIKV_WAVE)); }
 }
 
+__device__ __forceinline__ float read_lane_f(float v, int l) {
+  return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), l));
+}
+
 // Sum / max over aligned groups of `lanes` (a power of two <= 64) adjacent lanes;
-// every lane of the group ends with the result.
+// every lane of the group ends with the result.  Rows of 16 lanes reduce with DPP;
+// a whole wavefront then combines its four rows through scalar registers.
 __device__ __forceinline__ float group_sum_dpp(float v, int lanes) {
   if (lanes >= 2) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "quad_perm:[1,0,3,2]");
   if (lanes >= 4) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "quad_perm:[2,3,0,1]");
   if (lanes >= 8) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "row_half_mirror");
   if (lanes >= 16) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "row_mirror");
-  if (lanes >= 32) v += __shfl_xor(v, 16, PIKV_WAVE);
-  if (lanes >= 64) v += __shfl_xor(v, 32, PIKV_WAVE);
+  if (lanes >= 64)
+    v = (read_lane_f(v, 0) + read_lane_f(v, 16)) + (read_lane_f(v, 32) + read_lane_f(v, 48));
+  else if (lanes >= 32)
+    v += __shfl_xor(v, 16, PIKV_WAVE);
   return v;
 }
 __device__ __forceinline__ float group_max_dpp(float v, int lanes) {
@@ -314,8 +321,10 @@ __device__ __forceinline__ float group_max_dpp(float v, int lanes) {
   if (lanes >= 4) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "quad_perm:[2,3,0,1]");
   if (lanes >= 8) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "row_half_mirror");
   if (lanes >= 16) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "row_mirror");
-  if (lanes >= 32) v = fmaxf(v, __shfl_xor(v, 16, PIKV_WAVE));
-  if (lanes >= 64) v = fmaxf(v, __shfl_xor(v, 32, PIKV_WAVE));
+  if (lanes >= 64)
+    v = fmaxf(fmaxf(read_lane_f(v, 0), read_lane_f(v, 16)), fmaxf(read_lane_f(v, 32), read_lane_f(v, 48)));
+  else if (lanes >= 32)
+    v = fmaxf(v, __shfl_xor(v, 16, PIKV_WAVE));
   return v;
 }
 

@@ -79,9 +79,9 @@ __device__ __forceinline__ void router_tail_lanes(float lg, int64_t t, int e, in
   }
   float prob = 0.f;
   if (p.use_softmax) {
-    const float m = group_max<EPAD>(lg);
+    const float m = group_max_dpp(lg, EPAD);
     const float ex = valid ? expf(lg - m) : 0.f;
-    const float sum = group_sum<EPAD>(ex);
+    const float sum = group_sum_dpp(ex, EPAD);
     prob = ex / sum;
     if (valid && p.probs) p.probs[t * p.E + e] = prob;
   }
@@ -92,14 +92,22 @@ __device__ __forceinline__ void router_tail_lanes(float lg, int64_t t, int e, in
   bool remaining = valid;
   int my_idx = 0;
   float my_val = 0.f;
+  float wsum = 0.f;  // sum of the selected values, in selection order
   for (int j = 0; j < p.k; ++j) {
     const float key = remaining ? lg : -__builtin_inff();
-    const float mx = group_max<EPAD>(key);
+    const float mx = group_max_dpp(key, EPAD);
     uint64_t cand = __ballot(remaining && key == mx) & gmask;
     if (cand == 0) cand = __ballot(remaining) & gmask;  // only NaNs left
     int win = e;  // padding tokens (no candidates at all) stay harmless
     if (cand != 0) win = (int)__builtin_ctzll(cand) - gstart;
-    const float wv = __shfl(carried, gstart + win, PIKV_WAVE);
+    float wv;
+    if constexpr (EPAD == 64) {
+      // one token per wavefront: the winner is wave-uniform
+      wv = read_lane_f(carried, __builtin_amdgcn_readfirstlane(win));
+    } else {
+      wv = __shfl(carried, gstart + win, PIKV_WAVE);
+    }
+    wsum = wsum + wv;
     if (e == j) {
       my_idx = win;
       my_val = wv;
@@ -107,8 +115,7 @@ __device__ __forceinline__ void router_tail_lanes(float lg, int64_t t, int e, in
     if (e == win) remaining = false;
   }
   if (p.use_softmax) {
-    float s = 0.f;
-    for (int j = 0; j < p.k; ++j) s = s + __shfl(my_val, gstart + j, PIKV_WAVE);
+    float s = wsum;
     if (p.renorm_eps != 0.f) s = s + p.renorm_eps;
     my_val = my_val / s;
   }
@@ -196,10 +203,6 @@ __global__ __launch_bounds__(256) void router_tail_kernel(const float* __restric
 typedef __bf16 pikv_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float pikv_f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kMfmaWaves = 8;
-#ifndef PIKV_GATE_MT16
-#define PIKV_GATE_MT16 4
-#endif
 
 // Gate weights re-laid for the matrix-core kernel: wb[step][expert (padded to EP)][32 k]
 // so that the B operands of one k-step are EP*64 contiguous bytes.  Rows of the
@@ -218,12 +221,13 @@ __global__ __launch_bounds__(256) void gate_weight_relayout_kernel(const uint16_
   wb[chunk] = v;
 }
 
-template <int NT, int MT>  // NT 16-expert tiles (1, 2 or 4) x MT 16-token tiles per block
-__global__ __launch_bounds__(kMfmaWaves * 64) void router_gate_mfma_kernel(
+// NT 16-expert tiles (1, 2 or 4) x MT 16-token tiles per block; WAVES wavefronts share the k-steps
+template <int NT, int MT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void router_gate_mfma_kernel(
     const void* __restrict__ x, const void* __restrict__ wb, int H, TailParams p) {
   constexpr int EP = 16 * NT;
   constexpr int TB = 16 * MT;  // tokens per block
-  __shared__ float red[kMfmaWaves][TB][EP];
+  __shared__ float red[WAVES][TB][EP];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int64_t tok0 = (int64_t)blockIdx.x * TB;
@@ -247,11 +251,11 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void router_gate_mfma_kernel(
   // the k-steps are dealt round-robin to the wavefronts; each keeps UN steps in flight
   const int steps = H / 32;
   constexpr int UN = (MT + NT > 4) ? 2 : 4;
-  for (int st0 = wave; st0 < steps; st0 += kMfmaWaves * UN) {
+  for (int st0 = wave; st0 < steps; st0 += WAVES * UN) {
     uint4 av[UN][MT], bv[UN][NT];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int st = st0 + u * kMfmaWaves;
+      const int st = st0 + u * WAVES;
       const bool ok = st < steps;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
@@ -280,7 +284,7 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void router_gate_mfma_kernel(
   __syncthreads();
   // Wavefront w finishes tokens TW*w .. TW*w+TW-1: lane -> (token, expert) with the
   // experts of a token in EP adjacent lanes, as the tail expects.
-  constexpr int TW = TB / kMfmaWaves;  // tokens finished by one wavefront
+  constexpr int TW = TB / WAVES;  // tokens finished by one wavefront
   constexpr int TPC = 64 / EP;         // tokens per tail call
 #pragma unroll
   for (int c = 0; c < (TW + TPC - 1) / TPC; ++c) {
@@ -291,7 +295,7 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void router_gate_mfma_kernel(
     float lg = 0.f;
     if (in_range) {
 #pragma unroll
-      for (int w2 = 0; w2 < kMfmaWaves; ++w2) lg += red[w2][tl][e];
+      for (int w2 = 0; w2 < WAVES; ++w2) lg += red[w2][tl][e];
     }
     // lanes beyond this wavefront's tokens present an out-of-range token
     router_tail_lanes<EP>(lg, in_range ? tok0 + tl : p.T, e, lane, p);
@@ -497,19 +501,21 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
     if (blocks > 0x7fffffffLL) return PIKV_ERR_SHAPE;
     if (mfma) {
       const int ep = gate_epad(E);
-      const int mt = (ep == 16) ? PIKV_GATE_MT16 : 2;  // 16-token tiles per block
-      const int64_t mb = (T + 16 * mt - 1) / (16 * mt);
-      if (mb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
       const int64_t chunks = (int64_t)(H / 32) * ep * 4;
       hipLaunchKernelGGL(gate_weight_relayout_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256),
                          0, st, (const uint16_t*)w, H, E, ep, (uint4*)wb);
-      const dim3 grid((unsigned)mb), blk(kMfmaWaves * 64);
-      if (E <= 16)
-        hipLaunchKernelGGL((router_gate_mfma_kernel<1, PIKV_GATE_MT16>), grid, blk, 0, st, x, wb, H, p);
-      else if (E <= 32)
-        hipLaunchKernelGGL((router_gate_mfma_kernel<2, 2>), grid, blk, 0, st, x, wb, H, p);
+      // 64 tokens per block.  Few experts: 8 wavefronts share the k-steps; many
+      // experts: 4 (the accumulators of 4 x 4 tiles and the partial sums in LDS
+      // leave room for two such blocks per compute unit)
+      const int64_t mb = (T + 63) / 64;
+      if (mb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+      const dim3 grid((unsigned)mb);
+      if (ep == 16)
+        hipLaunchKernelGGL((router_gate_mfma_kernel<1, 4, 8>), grid, dim3(512), 0, st, x, wb, H, p);
+      else if (ep == 32)
+        hipLaunchKernelGGL((router_gate_mfma_kernel<2, 4, 4>), grid, dim3(256), 0, st, x, wb, H, p);
       else
-        hipLaunchKernelGGL((router_gate_mfma_kernel<4, 2>), grid, blk, 0, st, x, wb, H, p);
+        hipLaunchKernelGGL((router_gate_mfma_kernel<4, 4, 4>), grid, dim3(256), 0, st, x, wb, H, p);
     } else if (x_dtype == PIKV_BF16) {
       launch_gate<PIKV_BF16>(epad, (unsigned)blocks, st, x, w, H, p);
     } else {
