@@ -282,8 +282,8 @@ int pikv_gather_dequant_scores(const void* k_codes, const void* k_scale,
  *   the decay-first variant (core/single/module/pikv_scheduling.py:119-130).
  *   If write_probs != 0 scores is overwritten with the probabilities.
  *   importance_out [n_caches, score_stride] float or NULL receives the summed
- *   probabilities.  head_stats [n_caches, n_q_heads, 2] float workspace
- *   (final max and 1/sum per head). */
+ *   probabilities.  head_stats [n_caches, n_q_heads, 2] float receives the final
+ *   (max, sum of exp(score - max)) of every head; pikv_attend_values takes it. */
 int pikv_h2o_accumulate(float* scores, const float* tile_max,
                         const float* tile_sum, int n_q_heads,
                         const int64_t* cache_row_base,
@@ -292,6 +292,31 @@ int pikv_h2o_accumulate(float* scores, const float* tile_max,
                         float decay, float now, int write_probs,
                         float* row_acc, float* row_ts, float* importance_out,
                         float* head_stats, void* stream);
+
+/* Attention output over the compressed V cache:
+ *   out[c,h,:] = sum_{n < cache_fill[c]} p[c,h,n] * dequant(V[c,n,h/rep,:])
+ *   p = exp(scores - head_stats[c,h,0]) / head_stats[c,h,1]   (head_stats != NULL:
+ *       raw scores of pikv_gather_dequant_scores + the statistics that
+ *       pikv_h2o_accumulate leaves in its head_stats argument), or
+ *   p = scores                                              (head_stats == NULL:
+ *       scores already hold probabilities, e.g. after write_probs = 1).
+ * Replaces: context = torch.matmul(attention_probs, v)
+ *   (core/single/pikv_attention.py:188) on a dequantised copy of the cache.
+ *   out [n_caches, n_q_heads, head_dim] float; V planes as in the pool layout;
+ *   workspace: pikv_attend_workspace_bytes(...) bytes (partial sums of token
+ *   ranges, added in a fixed order), 256-byte aligned.  Shape limits as for
+ *   pikv_gather_dequant_scores. */
+int pikv_attend_values(const float* scores, const float* head_stats,
+                       int64_t score_stride,
+                       const void* v_codes, const void* v_scale, const void* v_zero,
+                       int scheme, int group,
+                       int n_kv_heads, int n_q_heads, int head_dim,
+                       const int64_t* cache_row_base, const int32_t* cache_fill,
+                       int n_caches, int64_t max_len,
+                       float* out, void* workspace, int64_t workspace_bytes,
+                       void* stream);
+int64_t pikv_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim,
+                                    int64_t max_len);
 
 /* ------------------------------------------------------------------------
  * K4  eviction top-k + stable in-place compaction

@@ -467,6 +467,19 @@ def h2o_importance(scores: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
     return p.astype(F32), p.sum(axis=0).astype(F32)
 
 
+def attend_values(probs: np.ndarray, v_hat: np.ndarray, n_kv_heads: int) -> np.ndarray:
+    """context[h,:] = sum_n probs[h,n] * V^[n, h//rep, :]
+    (core/single/pikv_attention.py:188: matmul(attention_probs, v)).
+    probs [Hq,N]; v_hat [N, Hkv*dh] dequantised float32.  float64 accumulate."""
+    Hq, N = probs.shape
+    rep = Hq // n_kv_heads
+    vh = v_hat.reshape(N, n_kv_heads, -1).astype(np.float64)
+    out = np.empty((Hq, vh.shape[2]), dtype=np.float64)
+    for h in range(Hq):
+        out[h] = probs[h].astype(np.float64) @ vh[:, h // rep, :]
+    return out.astype(F32)
+
+
 def h2o_accumulate(acc, ts, rows, imp, now, decay=1.0):
     """acc[idx] += w; ts[idx] = t (core/single/cache_scheduling.py:69-73);
     decay-first variant core/single/module/pikv_scheduling.py:119-130."""

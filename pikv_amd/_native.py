@@ -47,6 +47,9 @@ SIGNATURES = {
                                         _p, _p, _i, _l, _l, _p, _p, _p, _p]),
     "pikv_h2o_accumulate": (_i, [_p, _p, _p, _i, _p, _p, _i, _l, _l, _f, _f, _i,
                                  _p, _p, _p, _p, _p]),
+    "pikv_attend_values": (_i, [_p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _i, _l,
+                                _p, _p, _l, _p]),
+    "pikv_attend_workspace_bytes": (_l, [_i, _i, _i, _l]),
     "pikv_evict_select": (_i, [_i, _p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _p]),
     "pikv_h2o_budget": (_i, [_p, _i, _d, _d, _p, _p, _p]),
     "pikv_compact_rows": (_i, [C.POINTER(_p), C.POINTER(_l), _i, _p, _p, _p, _p, _i, _p]),

@@ -515,7 +515,35 @@ class CachePool:
                _ptr(self.row_base), _ptr(self.fill), nc, stride, stride, float(decay), float(now),
                int(bool(write_probs)), _ptr(self.acc), _ptr(self.ts), _ptr(imp), _ptr(head_stats),
                _stream())
+        self.head_stats = head_stats   # (max, sum) per (cache, head): what attend_values normalises with
         return imp
+
+    def attend_values(self, scores, head_stats=None):
+        """out[c,h,:] = sum_n p[c,h,n] * dequant(V[c,n,h/rep,:]) over the valid rows.
+        scores [n_caches, n_q_heads, stride] float32: raw scores together with
+        head_stats [n_caches, n_q_heads, 2] (as left in self.head_stats by
+        h2o_accumulate), or probabilities when head_stats is None."""
+        if not self.with_v:
+            raise ValueError("this pool stores no V rows")
+        scores = _need(scores, "scores", dtype=torch.float32, ndim=3)
+        nc, hq, stride = scores.shape
+        if nc != self.n_caches or hq % self.n_heads:
+            raise ValueError("scores must be [n_caches, n_q_heads, stride] with n_q_heads a multiple of the kv heads")
+        if head_stats is not None:
+            head_stats = _need(head_stats, "head_stats", dtype=torch.float32, ndim=3)
+            if head_stats.shape != (nc, hq, 2):
+                raise ValueError("head_stats must be [n_caches, n_q_heads, 2]")
+        dev = self.device
+        out = torch.zeros(nc, hq, self.head_dim, dtype=torch.float32, device=dev)
+        if stride == 0:
+            return out
+        ws_bytes = int(N.lib().pikv_attend_workspace_bytes(nc, hq, self.head_dim, stride))
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+        N.call("pikv_attend_values", _ptr(scores), _ptr(head_stats), stride, _ptr(self.v_codes),
+               _ptr(self.v_scale), _ptr(self.v_zero), self.scheme, self.group, self.n_heads, hq,
+               self.head_dim, _ptr(self.row_base), _ptr(self.fill), nc, stride, _ptr(out), _ptr(ws),
+               ws_bytes, _stream())
+        return out
 
     # ---- eviction ----
     def evict_select(self, policy: int, *, heavy_ratio=0.1, recent_ratio=0.1,
