@@ -134,48 +134,62 @@ __global__ __launch_bounds__(256) void attend_valu_kernel(AttendArgs a) {
 // ---- matrix-core form -----------------------------------------------------------------
 typedef int pikv_i32x2 __attribute__((ext_vector_type(2)));
 
+constexpr int kAttARow = 144;  // bytes per staged A-operand row: 64 tokens x bf16 + 16 (bank spread)
+
 static size_t attend_mfma_lds_bytes(int n_kv_heads) {
-  // codes [64 tokens][n_kv_heads*64 + 8 bytes]; scale and zero + bias as float
-  // [kv head][group of 32][64 tokens + 8]
-  return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * (size_t)n_kv_heads * 4 * (kAttTile + 8) * sizeof(float);
+  // codes [64 tokens][n_kv_heads*64 + 8 bytes]; scale and zero + bias as float4 (4 groups)
+  // [kv head][64 tokens]; A operands per wavefront [4 groups][8 rows][kAttARow]
+  return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * (size_t)n_kv_heads * kAttTile * 16 +
+         4 * (size_t)4 * 8 * kAttARow;
 }
 
-template <int SCHEME>
+// HKS = log2(n_kv_heads); at most 4 query heads per kv head.
+template <int SCHEME, int HKS>
 __global__ __launch_bounds__(256) void attend_mfma_i4_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
-  constexpr int kMaxHeadsPerWave = 2;  // n_kv_heads <= 8
-  constexpr int MS = kAttTile + 8;     // floats per (kv head, group) row of the metadata
+  constexpr int HK = 1 << HKS;
+  constexpr int NH = (HK + 3) / 4;        // kv heads per wavefront
+  constexpr int RS = HK * 64 + 8;         // bytes per token row of staged codes
+  constexpr int LPR = HK * 4;             // 16-byte chunks per cached row
+  constexpr int NCH = kAttTile * LPR / 256 > 0 ? kAttTile * LPR / 256 : 1;  // code chunks per thread
+  constexpr int NMC = (kAttTile * HK + 255) / 256;                          // metadata chunks per thread
   extern __shared__ __align__(16) unsigned char att_lds[];
-  const int HK = a.n_kv_heads;
-  const int RS = HK * 64 + 8;          // bytes per token row of staged codes
   unsigned char* lcodes = att_lds;
-  float* lscale = reinterpret_cast<float*>(att_lds + (size_t)kAttTile * RS);
-  float* lzterm = lscale + HK * 4 * MS;
+  float4* lscale = reinterpret_cast<float4*>(att_lds + kAttTile * RS);  // [kv head][token] -> 4 groups
+  float4* lzterm = lscale + HK * kAttTile;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  unsigned char* abuf = reinterpret_cast<unsigned char*>(lzterm + HK * kAttTile) + wave * (4 * 8 * kAttARow);
 
   const int c = blockIdx.y;
   const int64_t len = a.fill[c];
   const int64_t t0 = (int64_t)blockIdx.x * kAttTokensPerBlock;
   const int64_t t1 = (t0 + kAttTokensPerBlock < len) ? t0 + kAttTokensPerBlock : len;
-  const int rep = a.n_q_heads / a.n_kv_heads;  // <= 8
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int i = lane & 15;   // A: row (head r = i/2, part h = i%2); B/C: dimension inside a block of 16
-  const int kg = lane >> 4;  // 16 tokens of the tile
-  const int r = i >> 1;
-  const bool lo_row = (i & 1) != 0;
+  if (t0 >= t1) {  // nothing cached in this range: the partial is zero
+    for (int idx = threadIdx.x; idx < a.n_q_heads * 128; idx += 256)
+      a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * 128 + idx] = 0.f;
+    return;
+  }
+  const int rep = a.n_q_heads / HK;  // <= 4
+  // matrix-core roles: A row / B,C column i, token group kg
+  const int i = lane & 15;
+  const int kg = lane >> 4;
+  // weight-preparation roles: head r of the kv group, tokens {tk, tk+4, tk+8, tk+12} of group wkg
+  const int r = lane >> 4;
+  const int wkg = (lane >> 2) & 3;
+  const int tk = wkg * 16 + (lane & 3);
   const bool row_on = r < rep;
   const bool normalise = a.head_stats != nullptr;
   const float zbias = 128.0f - (float)Q::qmin;
   const int64_t base_row = a.row_base[c];
-  const int lanes_per_row = HK * 4;
 
-  pikv_f32x4 C[kMaxHeadsPerWave][8];
-  float zacc[kMaxHeadsPerWave][4];
-  float mx[kMaxHeadsPerWave], rz[kMaxHeadsPerWave];
-  const float* srow[kMaxHeadsPerWave];
+  pikv_f32x4 C[NH][8];
+  float zacc[NH][4];
+  float mx[NH], rz[NH];
+  const float* srow[NH];
 #pragma unroll
-  for (int hs = 0; hs < kMaxHeadsPerWave; ++hs) {
+  for (int hs = 0; hs < NH; ++hs) {
     const int g = wave + 4 * hs;
     const int hq = (g < HK && row_on) ? g * rep + r : 0;
     srow[hs] = a.scores + ((int64_t)c * a.n_q_heads + hq) * a.score_stride;
@@ -191,141 +205,180 @@ __global__ __launch_bounds__(256) void attend_mfma_i4_kernel(AttendArgs a) {
     for (int sg = 0; sg < 4; ++sg) zacc[hs][sg] = 0.f;
   }
 
+  // registers that carry the next tile from HBM to LDS
+  uint4 pc[NCH];
+  uint2 ps[NMC], pz[NMC];
+  auto fetch = [&](int64_t n0) {
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+      const int ch = k * 256 + threadIdx.x;
+      const int tok = ch >> (HKS + 2), off = ch & (LPR - 1);
+      pc[k] = make_uint4(0, 0, 0, 0);
+      if (tok < kAttTile && n0 + tok < t1)
+        pc[k] = ld16(reinterpret_cast<const char*>(a.codes) + ((base_row + n0 + tok) * LPR + off) * 16);
+    }
+#pragma unroll
+    for (int k = 0; k < NMC; ++k) {
+      const int ch = k * 256 + threadIdx.x;
+      const int tok = ch >> HKS, hd = ch & (HK - 1);
+      ps[k] = make_uint2(0, 0);
+      pz[k] = make_uint2(0, 0);
+      if (tok < kAttTile && n0 + tok < t1) {
+        const int64_t mi = (base_row + n0 + tok) * LPR + hd * 4;
+        ps[k] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.scale) + mi);
+        if constexpr (!Q::sym) pz[k] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.zero) + mi);
+      }
+    }
+  };
+  auto h2f = [](uint32_t w, int hi) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> (16 * hi))); };
+  auto stage = [&]() {
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+      const int ch = k * 256 + threadIdx.x;
+      const int tok = ch >> (HKS + 2), off = ch & (LPR - 1);
+      if (tok < kAttTile) {
+        uint2* dst = reinterpret_cast<uint2*>(lcodes + tok * RS + off * 16);  // rows are 8-byte aligned only
+        dst[0] = make_uint2(pc[k].x, pc[k].y);
+        dst[1] = make_uint2(pc[k].z, pc[k].w);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < NMC; ++k) {
+      const int ch = k * 256 + threadIdx.x;
+      const int tok = ch >> HKS, hd = ch & (HK - 1);
+      if (tok < kAttTile) {
+        lscale[hd * kAttTile + tok] = make_float4(h2f(ps[k].x, 0), h2f(ps[k].x, 1), h2f(ps[k].y, 0), h2f(ps[k].y, 1));
+        lzterm[hd * kAttTile + tok] = make_float4(h2f(pz[k].x, 0) + zbias, h2f(pz[k].x, 1) + zbias,
+                                                  h2f(pz[k].y, 0) + zbias, h2f(pz[k].y, 1) + zbias);
+      }
+    }
+  };
+
+  fetch(t0);
   for (int64_t n0 = t0; n0 < t1; n0 += kAttTile) {
     __syncthreads();  // the previous tile has been consumed
-    // stage the codes of 64 tokens as they are (rows past the fill as zeros)
-    for (int ch = threadIdx.x; ch < kAttTile * lanes_per_row; ch += 256) {
-      const int tok = ch / lanes_per_row, off = ch - tok * lanes_per_row;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (n0 + tok < t1) v = ld16(reinterpret_cast<const char*>(a.codes) + ((base_row + n0 + tok) * lanes_per_row + off) * 16);
-      uint2* dst = reinterpret_cast<uint2*>(lcodes + tok * RS + off * 16);  // 8-byte aligned only
-      dst[0] = make_uint2(v.x, v.y);
-      dst[1] = make_uint2(v.z, v.w);
-    }
-    // scale and zero + bias of every (token, kv head, group), token-minor
-    for (int ch = threadIdx.x; ch < kAttTile * HK; ch += 256) {
-      const int tok = ch / HK, hd = ch - tok * HK;
-      uint2 sv = make_uint2(0, 0), zv = make_uint2(0, 0);
-      if (n0 + tok < t1) {
-        const int64_t mi = (base_row + n0 + tok) * lanes_per_row + hd * 4;
-        sv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.scale) + mi);
-        if constexpr (!Q::sym) zv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.zero) + mi);
-      }
-      const uint32_t sw[2] = {sv.x, sv.y}, zw[2] = {zv.x, zv.y};
-#pragma unroll
-      for (int sg = 0; sg < 4; ++sg) {
-        const float s = (float)__builtin_bit_cast(_Float16, (uint16_t)(sw[sg >> 1] >> (16 * (sg & 1))));
-        const float z = (float)__builtin_bit_cast(_Float16, (uint16_t)(zw[sg >> 1] >> (16 * (sg & 1))));
-        lscale[(hd * 4 + sg) * MS + tok] = s;
-        lzterm[(hd * 4 + sg) * MS + tok] = z + zbias;
-      }
-    }
+    stage();
     __syncthreads();
+    if (n0 + kAttTile < t1) fetch(n0 + kAttTile);  // in flight while this tile is multiplied
 
 #pragma unroll
-    for (int hs = 0; hs < kMaxHeadsPerWave; ++hs) {
+    for (int hs = 0; hs < NH; ++hs) {
       const int g = wave + 4 * hs;
-      if (g < HK) {  // uniform
-        // probabilities of this lane's head for its 16 tokens
-        float p[16];
+      if (g >= HK) continue;  // uniform
+      // ---- weights: this lane prepares head r for four tokens, all four groups ----
+      float p4[4];
+      float4 s4[4], z4[4];
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const int64_t n = n0 + kg * 16 + q4 * 4;
-          float4 sv = make_float4(0.f, 0.f, 0.f, 0.f);
-          if (row_on && n < t1) sv = *reinterpret_cast<const float4*>(srow[hs] + n);  // t1 - t0 and n are multiples of 4 apart
-          const float s4[4] = {sv.x, sv.y, sv.z, sv.w};
+      for (int j = 0; j < 4; ++j) {
+        const int64_t n = n0 + tk + 4 * j;
+        const bool ok = row_on && n < t1;
+        const float sv = ok ? srow[hs][n] : 0.f;
+        p4[j] = ok ? prob_of(sv, mx[hs], rz[hs], normalise) : 0.f;
+        s4[j] = lscale[g * kAttTile + tk + 4 * j];
+        z4[j] = lzterm[g * kAttTile + tk + 4 * j];
+      }
 #pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const float pv = prob_of(s4[k], mx[hs], rz[hs], normalise);
-            p[q4 * 4 + k] = (row_on && n + k < t1) ? pv : 0.f;
-          }
+      for (int sg = 0; sg < 4; ++sg) {
+        // w = p * scale cut into a bf16 high part and a bf16 remainder.  The zero-point
+        // sum uses the SAME two-part value, so that what the matrix core multiplies with
+        // 128 + u is taken off again exactly.
+        float hi[4], lo[4];
+        float zsum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float sc = sg == 0 ? s4[j].x : sg == 1 ? s4[j].y : sg == 2 ? s4[j].z : s4[j].w;
+          const float zt = sg == 0 ? z4[j].x : sg == 1 ? z4[j].y : sg == 2 ? z4[j].z : z4[j].w;
+          const float w = p4[j] * sc;
+          hi[j] = __uint_as_float(__float_as_uint(w) & 0xffff0000u);
+          lo[j] = __uint_as_float(__float_as_uint(w - hi[j]) & 0xffff0000u);
+          zsum = fmaf(hi[j] + lo[j], zt, zsum);
+        }
+        zacc[hs][sg] += zsum;
+        // operand order inside 8 tokens is {0,4,1,5,2,6,3,7}: tokens (k, k+4) share a dword
+        if (row_on) {
+          uint32_t* rowh = reinterpret_cast<uint32_t*>(abuf + (sg * 8 + 2 * r) * kAttARow + wkg * 32) + (lane & 3);
+          uint32_t* rowl = reinterpret_cast<uint32_t*>(abuf + (sg * 8 + 2 * r + 1) * kAttARow + wkg * 32) + (lane & 3);
+          rowh[0] = (__float_as_uint(hi[0]) >> 16) | __float_as_uint(hi[1]);
+          rowh[4] = (__float_as_uint(hi[2]) >> 16) | __float_as_uint(hi[3]);
+          rowl[0] = (__float_as_uint(lo[0]) >> 16) | __float_as_uint(lo[1]);
+          rowl[4] = (__float_as_uint(lo[2]) >> 16) | __float_as_uint(lo[3]);
+        }
+      }
+      // the rows were written by other lanes of this wavefront
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      // ---- products: rows 2r / 2r+1 of A against 16 dimensions of 64 tokens ----
+#pragma unroll
+      for (int sg = 0; sg < 4; ++sg) {
+        uint4 a1 = make_uint4(0, 0, 0, 0), a2 = make_uint4(0, 0, 0, 0);
+        if (i < 2 * rep) {
+          const uint4* ap = reinterpret_cast<const uint4*>(abuf + (sg * 8 + i) * kAttARow + kg * 32);
+          a1 = ap[0];
+          a2 = ap[1];
         }
 #pragma unroll
-        for (int sg = 0; sg < 4; ++sg) {
-          const float4* sp = reinterpret_cast<const float4*>(lscale + (g * 4 + sg) * MS + kg * 16);
-          const float4* zp = reinterpret_cast<const float4*>(lzterm + (g * 4 + sg) * MS + kg * 16);
-          // w = p * scale, cut into a bf16 high part and a bf16 remainder.  The
-          // zero-point sum uses the SAME two-part value, so that what the matrix core
-          // multiplies with 128 + u is subtracted again exactly; only the product with
-          // (u - zero) keeps the 2^-16 relative rounding of the split.
-          float x[16];
-          float zsum = 0.f;
+        for (int dbl = 0; dbl < 2; ++dbl) {
+          const int db = 2 * sg + dbl;
+          // lane i lends the 8 code bytes of token kg*16+i that cover dims db*16..+15 and
+          // receives the nibbles of dimension db*16+i from its 16 neighbours
+          const pikv_i32x2 tr = __builtin_amdgcn_ds_read_tr4_b64_v2i32(
+              (pikv_i32x2 __attribute__((address_space(3)))*)(lcodes + (kg * 16 + i) * RS + g * 64 + db * 8));
 #pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            const float4 s4 = sp[q4], z4 = zp[q4];
-            const float ss[4] = {s4.x, s4.y, s4.z, s4.w}, zz[4] = {z4.x, z4.y, z4.z, z4.w};
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-              const float w = p[q4 * 4 + k] * ss[k];
-              const float hi = __uint_as_float(__float_as_uint(w) & 0xffff0000u);
-              const float lo = __uint_as_float(__float_as_uint(w - hi) & 0xffff0000u);
-              zsum = fmaf(hi + lo, zz[k], zsum);
-              x[q4 * 4 + k] = lo_row ? lo : hi;
-            }
-          }
-          zacc[hs][sg] += zsum;
-          // token order {0,4,1,5,2,6,3,7} inside each half of 8 to match the nibble
-          // expansion below
-          uint32_t ab[8];
-#pragma unroll
-          for (int half = 0; half < 2; ++half)
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-              ab[half * 4 + k] = (__float_as_uint(x[half * 8 + k]) >> 16) | __float_as_uint(x[half * 8 + k + 4]);
-          const uint4 a1 = make_uint4(ab[0], ab[1], ab[2], ab[3]);
-          const uint4 a2 = make_uint4(ab[4], ab[5], ab[6], ab[7]);
-#pragma unroll
-          for (int dbl = 0; dbl < 2; ++dbl) {
-            const int db = 2 * sg + dbl;
-            // lane i lends the 8 code bytes of token kg*16+i that cover dims db*16..+15 and
-            // receives the nibbles of dimension db*16+i from its 16 neighbours
-            const pikv_i32x2 tr = __builtin_amdgcn_ds_read_tr4_b64_v2i32(
-                (pikv_i32x2 __attribute__((address_space(3)))*)(lcodes + (kg * 16 + i) * RS + g * 64 + db * 8));
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-              const uint32_t u = Q::sym ? ((uint32_t)tr[half] ^ 0x88888888u) : (uint32_t)tr[half];
-              const uint4 bb = make_uint4((u & 0x000f000fu) | 0x43004300u, ((u >> 4) & 0x000f000fu) | 0x43004300u,
-                                          ((u >> 8) & 0x000f000fu) | 0x43004300u,
-                                          ((u >> 12) & 0x000f000fu) | 0x43004300u);
-              C[hs][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  __builtin_bit_cast(pikv_bf16x8, half ? a2 : a1), __builtin_bit_cast(pikv_bf16x8, bb), C[hs][db], 0, 0, 0);
-            }
+          for (int half = 0; half < 2; ++half) {
+            const uint32_t u = Q::sym ? ((uint32_t)tr[half] ^ 0x88888888u) : (uint32_t)tr[half];
+            const uint4 bb = make_uint4((u & 0x000f000fu) | 0x43004300u, ((u >> 4) & 0x000f000fu) | 0x43004300u,
+                                        ((u >> 8) & 0x000f000fu) | 0x43004300u,
+                                        ((u >> 12) & 0x000f000fu) | 0x43004300u);
+            C[hs][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                __builtin_bit_cast(pikv_bf16x8, half ? a2 : a1), __builtin_bit_cast(pikv_bf16x8, bb), C[hs][db], 0, 0, 0);
           }
         }
       }
+      // the next head's rows go into the same buffer
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
   }
 
   // Epilogue.  C: lane (dimension i, rows 4*kg + q): rows 2r / 2r+1 are the two parts of
   // head r, so head 2*kg is q = 0,1 and head 2*kg+1 is q = 2,3.  The zero-point sums sit
-  // with the lanes of row 2r (all four token groups): they meet in LDS.
+  // spread over the 16 lanes that prepared head r.
   __syncthreads();
-  float* zl = reinterpret_cast<float*>(att_lds);  // [wave][head slot][kg][r][sg]
+  float* zl = reinterpret_cast<float*>(att_lds);  // [wave][head slot][r][sg]
 #pragma unroll
-  for (int hs = 0; hs < kMaxHeadsPerWave; ++hs)
-    if ((i & 1) == 0 && row_on)
+  for (int hs = 0; hs < NH; ++hs)
 #pragma unroll
-      for (int sg = 0; sg < 4; ++sg)
-        zl[((((wave * kMaxHeadsPerWave + hs) * 4 + kg) * 8) + r) * 4 + sg] = zacc[hs][sg];
+    for (int sg = 0; sg < 4; ++sg) {
+      const float z = group_sum_dpp(zacc[hs][sg], 16);
+      if ((lane & 15) == 0) zl[((wave * NH + hs) * 4 + r) * 4 + sg] = z;
+    }
   __syncthreads();
 #pragma unroll
-  for (int hs = 0; hs < kMaxHeadsPerWave; ++hs) {
+  for (int hs = 0; hs < NH; ++hs) {
     const int g = wave + 4 * hs;
     if (g >= HK) continue;
 #pragma unroll
     for (int rr = 0; rr < 2; ++rr) {
       const int ro = 2 * kg + rr;  // head (inside the kv group) held by this lane
       if (ro >= rep) continue;
-      float* o = a.partial + (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep + ro) * a.head_dim;
+      float* o = a.partial + (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep + ro) * 128;
 #pragma unroll
-      for (int db = 0; db < 8; ++db) {
-        float z = 0.f;
-#pragma unroll
-        for (int k2 = 0; k2 < 4; ++k2)
-          z += zl[((((wave * kMaxHeadsPerWave + hs) * 4 + k2) * 8) + ro) * 4 + (db >> 1)];
-        o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - z;
-      }
+      for (int db = 0; db < 8; ++db)
+        o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NH + hs) * 4 + ro) * 4 + (db >> 1)];
     }
+  }
+}
+
+template <int SCHEME>
+static void launch_attend_mfma(int n_kv_heads, dim3 grid, hipStream_t st, const AttendArgs& a) {
+  const size_t lds = attend_mfma_lds_bytes(n_kv_heads);
+  switch (n_kv_heads) {
+    case 1: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 0>), grid, dim3(256), lds, st, a); break;
+    case 2: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 1>), grid, dim3(256), lds, st, a); break;
+    case 4: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 2>), grid, dim3(256), lds, st, a); break;
+    default: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 3>), grid, dim3(256), lds, st, a); break;
   }
 }
 
@@ -392,14 +445,11 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
                (float*)workspace, score_stride, group, n_kv_heads, n_q_heads, head_dim, n_caches};
   const int rep = n_q_heads / n_kv_heads;
   if (max_len > 0) {
-    const bool aligned = (score_stride % 4 == 0) && ((reinterpret_cast<uintptr_t>(scores) & 15) == 0);
-    if (!eight && group == 32 && head_dim == 128 && rep <= 8 && n_kv_heads <= 8 && aligned) {
-      const size_t lds = attend_mfma_lds_bytes(n_kv_heads);
+    const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;
+    if (!eight && group == 32 && head_dim == 128 && rep <= 4 && hk_ok) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
-      if (scheme == PIKV_Q_I4_ASYM)
-        hipLaunchKernelGGL((attend_mfma_i4_kernel<PIKV_Q_I4_ASYM>), grid, dim3(256), lds, st, a);
-      else
-        hipLaunchKernelGGL((attend_mfma_i4_kernel<PIKV_Q_I4_SYM>), grid, dim3(256), lds, st, a);
+      if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(n_kv_heads, grid, st, a);
+      else launch_attend_mfma<PIKV_Q_I4_SYM>(n_kv_heads, grid, st, a);
     } else {
       // heads of a kv group per pass: the float accumulators of one lane must fit
       const int rp = eight ? (rep >= 4 ? 4 : rep >= 2 ? 2 : 1) : (rep >= 2 ? 2 : 1);
