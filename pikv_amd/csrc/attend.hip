@@ -136,16 +136,23 @@ typedef int pikv_i32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kAttARow = 144;  // bytes per staged A-operand row: 64 tokens x bf16 + 16 (bank spread)
 
+// Metadata of token t, kv head g (one float4 = the 4 groups of the head) sits at byte
+// t*(HK*16+16) + (t/16)*64 + g*16: the 16 tokens {k + 16w} that one pass of 16 lanes reads
+// fall into 16 different banks quads, and consecutive (token, head) writers stay contiguous.
+__host__ __device__ constexpr size_t att_meta_bytes(int hk) { return (size_t)kAttTile * (hk * 16 + 16) + 4 * 64; }
+__device__ __forceinline__ int att_meta_off(int tok, int g, int hk) {
+  return tok * (hk * 16 + 16) + (tok >> 4) * 64 + g * 16;
+}
+
 static size_t attend_mfma_lds_bytes(int n_kv_heads) {
   // codes [64 tokens][n_kv_heads*64 + 8 bytes]; scale and zero + bias as float4 (4 groups)
-  // [kv head][64 tokens]; A operands per wavefront [4 groups][8 rows][kAttARow]
-  return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * (size_t)n_kv_heads * kAttTile * 16 +
-         4 * (size_t)4 * 8 * kAttARow;
+  // [64 tokens][kv head] in padded token rows; A operands per wavefront [4 groups][8 rows][kAttARow]
+  return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * att_meta_bytes(n_kv_heads) + 4 * (size_t)4 * 8 * kAttARow;
 }
 
 // HKS = log2(n_kv_heads); at most 4 query heads per kv head.
 template <int SCHEME, int HKS>
-__global__ __launch_bounds__(256) void attend_mfma_i4_kernel(AttendArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i4_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
   constexpr int HK = 1 << HKS;
@@ -156,11 +163,11 @@ __global__ __launch_bounds__(256) void attend_mfma_i4_kernel(AttendArgs a) {
   constexpr int NMC = (kAttTile * HK + 255) / 256;                          // metadata chunks per thread
   extern __shared__ __align__(16) unsigned char att_lds[];
   unsigned char* lcodes = att_lds;
-  float4* lscale = reinterpret_cast<float4*>(att_lds + kAttTile * RS);  // [kv head][token] -> 4 groups
-  float4* lzterm = lscale + HK * kAttTile;
+  unsigned char* lscale = att_lds + kAttTile * RS;
+  unsigned char* lzterm = lscale + att_meta_bytes(HK);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  unsigned char* abuf = reinterpret_cast<unsigned char*>(lzterm + HK * kAttTile) + wave * (4 * 8 * kAttARow);
+  unsigned char* abuf = lzterm + att_meta_bytes(HK) + wave * (4 * 8 * kAttARow);
 
   const int c = blockIdx.y;
   const int64_t len = a.fill[c];
@@ -247,9 +254,11 @@ __global__ __launch_bounds__(256) void attend_mfma_i4_kernel(AttendArgs a) {
       const int ch = k * 256 + threadIdx.x;
       const int tok = ch >> HKS, hd = ch & (HK - 1);
       if (tok < kAttTile) {
-        lscale[hd * kAttTile + tok] = make_float4(h2f(ps[k].x, 0), h2f(ps[k].x, 1), h2f(ps[k].y, 0), h2f(ps[k].y, 1));
-        lzterm[hd * kAttTile + tok] = make_float4(h2f(pz[k].x, 0) + zbias, h2f(pz[k].x, 1) + zbias,
-                                                  h2f(pz[k].y, 0) + zbias, h2f(pz[k].y, 1) + zbias);
+        const int mo = att_meta_off(tok, hd, HK);
+        *reinterpret_cast<float4*>(lscale + mo) =
+            make_float4(h2f(ps[k].x, 0), h2f(ps[k].x, 1), h2f(ps[k].y, 0), h2f(ps[k].y, 1));
+        *reinterpret_cast<float4*>(lzterm + mo) = make_float4(h2f(pz[k].x, 0) + zbias, h2f(pz[k].x, 1) + zbias,
+                                                              h2f(pz[k].y, 0) + zbias, h2f(pz[k].y, 1) + zbias);
       }
     }
   };
@@ -274,8 +283,8 @@ __global__ __launch_bounds__(256) void attend_mfma_i4_kernel(AttendArgs a) {
         const bool ok = row_on && n < t1;
         const float sv = ok ? srow[hs][n] : 0.f;
         p4[j] = ok ? prob_of(sv, mx[hs], rz[hs], normalise) : 0.f;
-        s4[j] = lscale[g * kAttTile + tk + 4 * j];
-        z4[j] = lzterm[g * kAttTile + tk + 4 * j];
+        s4[j] = *reinterpret_cast<const float4*>(lscale + att_meta_off(tk + 4 * j, g, HK));
+        z4[j] = *reinterpret_cast<const float4*>(lzterm + att_meta_off(tk + 4 * j, g, HK));
       }
 #pragma unroll
       for (int sg = 0; sg < 4; ++sg) {
