@@ -121,21 +121,23 @@ def decode_read_workload(torch, ops, dev, iters):
     B, N, hkv, hq, dh = 64, 32768, 8, 32, 128
     D = hkv * dh
     g = torch.Generator(device=dev).manual_seed(2)
-    pool = ops.CachePool([N] * B, hkv, dh, 32, ops.Q_I4_ASYM, dev, with_v=False)
+    pool = ops.CachePool([N] * B, hkv, dh, 32, ops.Q_I4_ASYM, dev, with_v=True)
     chunk = 4
     slot = torch.arange(N, device=dev, dtype=torch.int32).repeat(chunk)
     t_write = None
     for b0 in range(0, B, chunk):
         ks = torch.randn(chunk * N, D, generator=g, device=dev).to(torch.bfloat16)
+        vs = torch.randn(chunk * N, D, generator=g, device=dev).to(torch.bfloat16)
         cid = torch.arange(b0, b0 + chunk, device=dev, dtype=torch.int32).repeat_interleave(N)
         if b0 == 0:
-            t_write = _median_ms(torch, lambda: pool.quant_scatter(ks, None, cid, slot, 1), iters)
-        pool.quant_scatter(ks, None, cid, slot, 1)
+            t_write = _median_ms(torch, lambda: pool.quant_scatter(ks, vs, cid, slot, 1), iters)
+        pool.quant_scatter(ks, vs, cid, slot, 1)
     pool.fill.fill_(N)
     q = torch.randn(B, hq, dh, generator=g, device=dev).to(torch.bfloat16)
     t_scores = _median_ms(torch, lambda: pool.scores(q, hq), iters)
     sc, tm, tsu = pool.scores(q, hq)
     t_h2o = _median_ms(torch, lambda: pool.h2o_accumulate(sc, tm, tsu, now=1.0), iters)
+    t_att = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats), iters)
     t_sel = _median_ms(torch, lambda: pool.evict_select(0, heavy_ratio=1 / 16, recent_ratio=1 / 128), iters)
 
     def evict():
@@ -146,11 +148,12 @@ def decode_read_workload(torch, ops, dev, iters):
     k_bytes = rows * (D // 2 + (D // 32) * 4)
     return {
         "workload": "decode read: 64 seq x 32768 cached tokens, 8 KV heads x 128 (32 q heads), int4 asym g32",
-        "quant_scatter_i4": _entry(t_write, chunk * N * (D * 2 + D // 2 + (D // 32) * 4 + 8),
+        "quant_scatter_i4": _entry(t_write, chunk * N * (2 * (D * 2 + D // 2 + (D // 32) * 4) + 8),
                                    rows=chunk * N),
         "gather_dequant_scores": _entry(t_scores, k_bytes, cached_tokens_per_s=rows / (t_scores * 1e-3),
                                         bytes_with_score_store=k_bytes + rows * hq * 4),
         "h2o_accumulate": _entry(t_h2o, rows * hq * 4 + rows * 12),
+        "attend_values": _entry(t_att, k_bytes + rows * hq * 4),
         "evict_select": _entry(t_sel, rows * 8 + rows * 5),
         "evict_select_plus_compact": {"ms": t_evict},
     }
