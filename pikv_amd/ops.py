@@ -385,6 +385,64 @@ class CachePool:
         self.n_heavy = torch.zeros(self.n_caches, dtype=torch.int32, device=dev)
         self.n_recent = torch.zeros(self.n_caches, dtype=torch.int32, device=dev)
 
+    # ---- checkpoint ----
+    _STATE_PLANES = ("k_codes", "k_scale", "k_zero", "v_codes", "v_scale", "v_zero", "acc", "ts")
+
+    def state_dict(self, trim: bool = True):
+        """Everything needed to restore the caches: geometry, fill counts and the
+        quantised planes (codes, scales, zero points, accumulators, timestamps) as
+        CPU tensors.  With trim=True only the valid rows of every cache are kept
+        (rows [row_base[c], row_base[c]+fill[c]), concatenated in cache order)."""
+        fill = self.fill.cpu()
+        sd = {"layout": torch.tensor([self.n_heads, self.head_dim, self.group, self.scheme,
+                                      int(self.with_v), int(trim)], dtype=torch.int64),
+              "cap": self.cap.cpu(), "fill": fill}
+        rows = None
+        if trim:
+            base = self.row_base.cpu()
+            rows = torch.cat([torch.arange(int(base[c]), int(base[c]) + int(fill[c]))
+                              for c in range(self.n_caches)]) if self.n_caches else torch.zeros(0, dtype=torch.int64)
+            rows = rows.to(self.device)
+        for name in self._STATE_PLANES:
+            t = getattr(self, name)
+            if t is not None:
+                sd[name] = (t.index_select(0, rows) if rows is not None else t).cpu()
+        return sd
+
+    def load_state_dict(self, sd):
+        """Restore what state_dict() saved into a pool of the same geometry."""
+        layout = [int(v) for v in sd["layout"]]
+        mine = [self.n_heads, self.head_dim, self.group, self.scheme, int(self.with_v)]
+        if layout[:5] != mine:
+            raise ValueError(f"checkpoint layout {layout[:5]} does not match this pool {mine}")
+        if not torch.equal(sd["cap"].to(torch.int32).cpu(), self.cap.cpu()):
+            raise ValueError("checkpoint cache capacities do not match this pool")
+        fill = sd["fill"].to(torch.int32)
+        if bool((fill > self.cap.cpu()).any()) or bool((fill < 0).any()):
+            raise ValueError("checkpoint fill counts exceed the capacities")
+        trim = bool(layout[5])
+        rows = None
+        if trim:
+            base = self.row_base.cpu()
+            rows = torch.cat([torch.arange(int(base[c]), int(base[c]) + int(fill[c]))
+                              for c in range(self.n_caches)]).to(self.device)
+        for name in self._STATE_PLANES:
+            t = getattr(self, name)
+            if t is None:
+                continue
+            src = sd[name].to(self.device)
+            if src.dtype != t.dtype or src.shape[1:] != t.shape[1:]:
+                raise ValueError(f"checkpoint plane {name} has the wrong dtype or row shape")
+            if rows is not None:
+                if src.shape[0] != rows.numel():
+                    raise ValueError(f"checkpoint plane {name} does not hold the saved rows")
+                t.index_copy_(0, rows, src)
+            else:
+                if src.shape != t.shape:
+                    raise ValueError(f"checkpoint plane {name} has the wrong number of rows")
+                t.copy_(src)
+        self.fill.copy_(fill.to(self.device))
+
     # ---- write path ----
     def quant_scatter(self, k_src, v_src, cache_id, slot, fanout: int, now: float = 0.0):
         """Quantise source rows once and append them to their routed caches.

@@ -239,3 +239,33 @@ def test_kernels_facade(dev):
     assert out[4] == valid.sum() and np.array_equal(np_of(out[0]), keys[valid])
     with pytest.raises(NotImplementedError):
         K.compress_kv(torch.zeros(4, 64, device=dev), torch.zeros(4, 64, device=dev), CompressionMode.LORA)
+
+
+@pytest.mark.parametrize("trim", [True, False])
+def test_cache_pool_checkpoint_round_trip(dev, trim, tmp_path):
+    """state_dict -> torch.save -> torch.load(weights_only=True) -> load_state_dict restores
+    codes, metadata, accumulators and fill exactly, and reads give identical scores."""
+    import torch
+    from pikv_amd import ops
+    from test_gpu_read_evict import _fill_pool
+    r = rng(12)
+    caps, lens = [70, 40, 16], [65, 0, 16]
+    pool, ref = _fill_pool(dev, r, caps, lens, 2, 64, 32, O.Q_I4_ASYM)
+    pool.acc.copy_(torch.rand(pool.rows, device=dev))
+    q = torch.randn(3, 4, 64, device=dev)
+    s0, _, _ = pool.scores(q, 4)
+    path = tmp_path / "pool.pt"
+    torch.save(pool.state_dict(trim=trim), path)
+    sd = torch.load(path, weights_only=True)
+    fresh = ops.CachePool(caps, 2, 64, 32, ops.Q_I4_ASYM, dev)
+    fresh.load_state_dict(sd)
+    assert torch.equal(fresh.fill, pool.fill)
+    for c in range(3):
+        rows = ref.valid_rows(c)
+        for name in ("k_codes", "k_scale", "k_zero", "v_codes", "v_scale", "v_zero", "acc", "ts"):
+            assert torch.equal(getattr(fresh, name)[rows], getattr(pool, name)[rows]), name
+    s1, _, _ = fresh.scores(q, 4)
+    assert torch.equal(s0[0, :, :65], s1[0, :, :65]) and torch.equal(s0[2, :, :16], s1[2, :, :16])
+    other = ops.CachePool(caps, 2, 64, 64, ops.Q_I4_ASYM, dev)
+    with pytest.raises(ValueError):
+        other.load_state_dict(sd)
