@@ -29,6 +29,8 @@ def test_header_declares_expected_surface():
                  "pikv_gather_dequant_scores", "pikv_h2o_accumulate", "pikv_evict_select",
                  "pikv_h2o_budget", "pikv_compact_rows", "pikv_fakequant_colblocks",
                  "pikv_router_workspace_bytes", "pikv_fakequant_workspace_bytes",
+                 "pikv_router_fused_workspace_bytes", "pikv_quant_gather", "pikv_attend_values",
+                 "pikv_attend_workspace_bytes",
                  "pikv_status_string", "pikv_abi_version"]:
         assert need in d
 
@@ -65,6 +67,18 @@ def test_pure_host_entry_points():
     assert lib.pikv_router_fused(1, 1, 7, None, None, None, 1.0, 0.0, 4, 64, 4, 2, 0,
                                  None, None, 1, 1, None, None, None, 0, None) == -3
     assert lib.pikv_evict_select(9, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, None) == -3
+    # bf16 router needs its workspace (re-laid gate weights): too small -> workspace status
+    need = lib.pikv_router_fused_workspace_bytes(64, 128, 8, 2)
+    assert need >= 128 * 16 * 2
+    assert lib.pikv_router_fused(1, 1, 1, None, None, None, 1.0, 0.0, 64, 128, 8, 2, 0,
+                                 None, None, 1, 1, None, None, 1, 128 * 16 * 2 - 1, None) == -4
+    # pyramid gather: NULL index list; attention output: heads must divide, workspace must fit
+    assert lib.pikv_quant_gather(1, None, 1, 128, 128, 0, 1, None, 1, 4, None, 1, 1, 1, 1,
+                                 1, None, 1, None, None, None, None, None, 0.0, None) == -1
+    assert lib.pikv_attend_values(1, None, 64, 1, 1, None, 0, 128, 3, 4, 128, 1, 1, 1, 64, 1, 1, 1 << 20, None) == -2
+    ws = lib.pikv_attend_workspace_bytes(2, 4, 128, 5000)
+    assert ws == 3 * 2 * 4 * 128 * 4
+    assert lib.pikv_attend_values(1, None, 5000, 1, 1, None, 0, 128, 4, 4, 128, 1, 1, 2, 5000, 1, 1, ws - 1, None) == -4
 
 
 def test_ops_reject_cpu_tensors():
