@@ -1,0 +1,216 @@
+"""PiKVAttention with the reference's interface (core/single/pikv_attention.py:7-283)
+on a quantised, natively read KV cache.
+
+The reference keeps `k_cache` / `v_cache` as float buffers `[cache_size, heads, head_dim]`
+that `forward` only ever writes (`_update_cache`, :74-102) and attends over the K/V of
+the current call.  Here every sequence of the batch owns one cache of a shared
+`CachePool` (rows = tokens, quantised on the way in by the fused quantise + scatter
+kernel), and a single-token call - the decode step - attends over the WHOLE cached
+context natively:
+
+    scores   = pikv_gather_dequant_scores   (QK^T over the compressed K rows, :123)
+    softmax  = pikv_h2o_accumulate          (:163; also feeds the H2O importance)
+    context  = pikv_attend_values           (probabilities x compressed V rows, :188)
+
+Multi-token calls (prefill) compute their attention in torch exactly as the reference
+does and write their K/V rows into the cache.  When a cache would overflow, the
+reference wipes it (:85-90); here H2O eviction keeps the heavy and the recent rows
+(`on_overflow="reset"` restores the wipe).
+
+`load_past_key_values` / `past_key_values` convert from and to the
+`[batch, heads, seq, head_dim]` tuples that Hugging Face style callers carry.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+
+_SCHEMES = {"int8": ops.Q_I8_SYM, "int8_asym": ops.Q_I8_ASYM, "int4": ops.Q_I4_ASYM,
+            "int4_sym": ops.Q_I4_SYM}
+
+
+class RotaryEmbedding(nn.Module):
+    """core/single/pikv_attention.py:285-363 (rotate-half form on [B,S,heads,dim])."""
+
+    def __init__(self, dim: int, max_position_embeddings: int = 2048):
+        super().__init__()
+        self.dim = dim
+        self.max_position_embeddings = max_position_embeddings
+        position = torch.arange(max_position_embeddings, dtype=torch.float).unsqueeze(1)
+        freq = 1.0 / (10000 ** (torch.arange(0, dim, step=2, dtype=torch.float) / dim))
+        self.register_buffer("cos_cached", torch.cos(position * freq), persistent=False)
+        self.register_buffer("sin_cached", torch.sin(position * freq), persistent=False)
+
+    def forward(self, q, k, position_ids):
+        cos = self.cos_cached[position_ids].unsqueeze(2)   # [B,S,1,dim/2]
+        sin = self.sin_cached[position_ids].unsqueeze(2)
+
+        def rot(x):
+            x1, x2 = x[..., 0::2], x[..., 1::2]
+            out = torch.empty_like(x)
+            out[..., 0::2] = x1 * cos - x2 * sin
+            out[..., 1::2] = x1 * sin + x2 * cos
+            return out
+        return rot(q), rot(k)
+
+
+class PiKVAttention(nn.Module):
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: Optional[int] = None,
+                 dropout: float = 0.1, use_rotary: bool = False,
+                 max_position_embeddings: int = 2048, cache_size: int = 4096, *,
+                 num_kv_heads: Optional[int] = None, kv_quant: str = "int4", kv_group: int = 32,
+                 heavy_ratio: float = 0.0625, recent_ratio: float = 0.0078125,
+                 on_overflow: str = "h2o"):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.head_dim = head_dim if head_dim is not None else hidden_size // num_heads
+        self.num_kv_heads = num_kv_heads or num_heads
+        if num_heads % self.num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        if on_overflow not in ("h2o", "reset"):
+            raise ValueError("on_overflow must be 'h2o' or 'reset'")
+        self.dropout = dropout
+        self.use_rotary = use_rotary
+        self.cache_size = cache_size
+        self.scheme = _SCHEMES[kv_quant]
+        self.kv_group = kv_group
+        self.heavy_ratio, self.recent_ratio = heavy_ratio, recent_ratio
+        self.on_overflow = on_overflow
+        self.q_proj = nn.Linear(hidden_size, num_heads * self.head_dim)
+        self.k_proj = nn.Linear(hidden_size, self.num_kv_heads * self.head_dim)
+        self.v_proj = nn.Linear(hidden_size, self.num_kv_heads * self.head_dim)
+        self.o_proj = nn.Linear(num_heads * self.head_dim, hidden_size)
+        self.attn_dropout = nn.Dropout(dropout)
+        if use_rotary:
+            self.rotary_emb = RotaryEmbedding(self.head_dim, max_position_embeddings)
+        for m in (self.q_proj, self.k_proj, self.v_proj, self.o_proj):
+            nn.init.normal_(m.weight, mean=0.0, std=0.02)
+            nn.init.zeros_(m.bias)
+        self.pool: Optional[ops.CachePool] = None
+        self.clock = 0
+
+    # ---- cache ---------------------------------------------------------------------
+    def _ensure_pool(self, batch_size: int, device) -> ops.CachePool:
+        if self.pool is None or self.pool.n_caches != batch_size:
+            self.pool = ops.CachePool([self.cache_size] * batch_size, self.num_kv_heads, self.head_dim,
+                                      self.kv_group, self.scheme, device)
+            self.clock = 0
+        return self.pool
+
+    @property
+    def cache_ptr(self) -> torch.Tensor:
+        """Rows cached per sequence (the reference's single write pointer, per sequence)."""
+        if self.pool is None:
+            return torch.zeros(1, dtype=torch.long)
+        return self.pool.fill.long()
+
+    def reset_cache(self):
+        if self.pool is not None:
+            self.pool.fill.zero_()
+
+    def _update_cache(self, k: torch.Tensor, v: torch.Tensor):
+        """Append k, v [B,S,kv_heads,head_dim] to the B caches (core/single/
+        pikv_attention.py:74-102), making room first when a cache would overflow."""
+        B, S = k.shape[0], k.shape[1]
+        pool = self._ensure_pool(B, k.device)
+        dev = pool.device
+        n_new = torch.full((B,), min(S, self.cache_size), dtype=torch.int32, device=dev)
+        over = (pool.fill + n_new - pool.cap).clamp_min(0)
+        if self.on_overflow == "reset":
+            pool.fill.copy_(torch.where(over > 0, torch.zeros_like(pool.fill), pool.fill))
+        else:
+            f = pool.fill.double()
+            nh = (f * self.heavy_ratio).floor().clamp_min(1).to(torch.int32)
+            nr = (f * self.recent_ratio).floor().clamp_min(1).to(torch.int32)
+            # never keep more than what leaves room for the new rows
+            room = (pool.cap - n_new).clamp_min(0)
+            nh = torch.minimum(nh, room)
+            nr = torch.minimum(nr, (room - nh).clamp_min(0))
+            keep_all = over == 0
+            pool.evict(ops.EVICT_H2O, n_heavy=torch.where(keep_all, pool.fill, nh).contiguous(),
+                       n_recent=torch.where(keep_all, torch.zeros_like(nr), nr).contiguous())
+        self.clock += 1
+        D = self.num_kv_heads * self.head_dim
+        dt = k.dtype if k.dtype in (torch.float32, torch.bfloat16) else torch.float32
+        cid = torch.arange(B, dtype=torch.int32, device=dev).repeat_interleave(S)
+        slot = torch.arange(S, dtype=torch.int32, device=dev).repeat(B)
+        pool.quant_scatter(k.reshape(B * S, D).to(dt).contiguous(), v.reshape(B * S, D).to(dt).contiguous(),
+                           cid, slot, 1, now=float(self.clock))
+        pool.advance(n_new)
+
+    def load_past_key_values(self, past_key_values: Tuple[torch.Tensor, torch.Tensor]):
+        """Fill the caches from (k, v) of shape [batch, kv_heads, seq, head_dim]."""
+        past_k, past_v = past_key_values
+        self.reset_cache()
+        self._update_cache(past_k.transpose(1, 2).contiguous(), past_v.transpose(1, 2).contiguous())
+
+    def past_key_values(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Dequantised caches as (k, v) [batch, kv_heads, max cached rows, head_dim]; rows past
+        a sequence's fill are zero."""
+        pool = self.pool
+        if pool is None:
+            raise RuntimeError("nothing cached yet")
+        B, L = pool.n_caches, int(pool.fill.max().item())
+        out = []
+        for which in ("k", "v"):
+            full = pool.gather_dequant(which).view(B, self.cache_size, self.num_kv_heads, self.head_dim)[:, :L]
+            mask = (torch.arange(L, device=pool.device).unsqueeze(0) < pool.fill.unsqueeze(1))
+            out.append((full * mask[:, :, None, None]).transpose(1, 2).contiguous())
+        return out[0], out[1]
+
+    # ---- attention --------------------------------------------------------------------
+    def _decode_attention(self, q: torch.Tensor) -> torch.Tensor:
+        """q [B, heads, head_dim] against the whole compressed cache of each sequence."""
+        pool = self.pool
+        qq = q.to(torch.bfloat16) if q.dtype == torch.bfloat16 else q.float()
+        scores, tmax, tsum = pool.scores(qq.contiguous(), self.num_heads, 1.0 / math.sqrt(self.head_dim))
+        pool.h2o_accumulate(scores, tmax, tsum, now=float(self.clock))
+        return pool.attend_values(scores, pool.head_stats)          # [B, heads, head_dim]
+
+    def _dense_attention(self, q, k, v, attention_mask, causal_mask):
+        """core/single/pikv_attention.py:104-191 on the K/V of this call."""
+        rep = self.num_heads // self.num_kv_heads
+        q = q.transpose(1, 2)
+        k = k.transpose(1, 2).repeat_interleave(rep, dim=1)
+        v = v.transpose(1, 2).repeat_interleave(rep, dim=1)
+        s = torch.matmul(q, k.transpose(-1, -2)) / math.sqrt(self.head_dim)
+        if attention_mask is not None:
+            if attention_mask.dim() != 4:
+                attention_mask = attention_mask.unsqueeze(1).unsqueeze(2)
+            s = s.masked_fill(attention_mask == 0, float("-inf"))
+        if causal_mask:
+            n, m = s.shape[-2], s.shape[-1]
+            tri = torch.triu(torch.ones(n, m, device=q.device), diagonal=1 + m - n).bool()
+            s = s.masked_fill(tri, float("-inf"))
+        p = self.attn_dropout(F.softmax(s, dim=-1))
+        return torch.matmul(p, v).transpose(1, 2)                   # [B,S,heads,head_dim]
+
+    def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                past_key_values: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                position_ids: Optional[torch.Tensor] = None, use_cache: bool = False,
+                causal_mask: bool = True, stream_mode: bool = False,
+                stream_position: Optional[int] = None):
+        B, S, _ = hidden_states.shape
+        q = self.q_proj(hidden_states).view(B, S, self.num_heads, self.head_dim)
+        k = self.k_proj(hidden_states).view(B, S, self.num_kv_heads, self.head_dim)
+        v = self.v_proj(hidden_states).view(B, S, self.num_kv_heads, self.head_dim)
+        if self.use_rotary and position_ids is not None:
+            q, k = self.rotary_emb(q, k, position_ids)
+        if past_key_values is not None:
+            self.load_past_key_values(past_key_values)
+        with torch.no_grad():
+            self._update_cache(k.detach(), v.detach())
+        if S == 1 and attention_mask is None:
+            context = self._decode_attention(q[:, 0]).unsqueeze(1)  # over everything cached
+        else:
+            context = self._dense_attention(q, k, v, attention_mask, causal_mask)
+        output = self.o_proj(context.reshape(B, S, self.num_heads * self.head_dim).to(hidden_states.dtype))
+        present = (k, v) if use_cache else None
+        return output, present
