@@ -277,7 +277,7 @@ struct CompactPlanes {
 };
 
 constexpr int kSlabBytes = 256;
-constexpr int kRowsUnroll = 4;
+constexpr int kRowsUnroll = 16;
 
 template <typename V>
 __device__ __forceinline__ void compact_slab(char* plane, int64_t row_bytes, int64_t base_row,
