@@ -528,6 +528,34 @@ def streaming_keep(cache_len: int, start_size: int, recent_size: int) -> np.ndar
     return keep
 
 
+def duo_keep(cache_len: int, sink_size: int, recent_size: int) -> np.ndarray:
+    """Keep rows [:sink_size] and [-recent_size:]
+    (core/single/module/pikv_scheduling.py:695-700)."""
+    keep = np.zeros(cache_len, dtype=bool)
+    keep[:sink_size] = True
+    if recent_size > 0:
+        keep[-recent_size:] = True
+    return keep
+
+
+def adakv_keep(scores: np.ndarray, compression_ratio: float, safeguard_ratio: float) -> np.ndarray:
+    """num_keep = int(len*(1-ratio)); the top int(num_keep*safeguard) scores are kept
+    first, then the top (num_keep - safeguarded) of the remaining ones
+    (core/single/module/pikv_scheduling.py:648-661).  Ties to the lower index."""
+    s = np.asarray(scores, F32)
+    L = s.shape[0]
+    num_keep = int(L * (1 - compression_ratio))
+    num_safe = int(num_keep * safeguard_ratio)
+    keep = np.zeros(L, dtype=bool)
+    safe = topk_desc(s[None, :], num_safe)[0] if num_safe > 0 else np.zeros(0, dtype=np.int64)
+    keep[safe] = True
+    rest = s.copy()
+    rest[safe] = -np.inf
+    if num_keep - num_safe > 0:
+        keep[topk_desc(rest[None, :], num_keep - num_safe)[0]] = True
+    return keep
+
+
 def quest_utility(quality, frequency, last_access, now, decay_factor) -> np.ndarray:
     """utility = quality * frequency * decay^(now - last access)
     (core/single/cache_scheduling.py:166-176), float32."""

@@ -9,6 +9,8 @@
   FlexGenScheduler ................ :205-251 (access frequency / access cost)
   LRUScheduler .................... :253-285
   LRUPlusScheduler ................ :287-349 (recency + frequency + importance)
+  AdaKVScheduler .................. core/single/module/pikv_scheduling.py:624-673
+  DuoAttentionScheduler ........... core/single/module/pikv_scheduling.py:675-710
   CacheSchedulingManager .......... :351-467 (append / evict / compact / stats)
 
 Every policy is "a score per row, then keep the top / drop the bottom": the score
@@ -47,6 +49,8 @@ class SchedulingPolicy(Enum):
     FLEXGEN = "flexgen"
     LRU = "lru"
     LRU_PLUS = "lru_plus"
+    ADAKV = "adakv"                 # core/single/module/pikv_scheduling.py:23-33
+    DUOATTENTION = "duoattention"
 
 
 class BaseScheduler(nn.Module):
@@ -321,6 +325,58 @@ class LRUPlusScheduler(BaseScheduler):
         return self.evict_mask(cache_len, cache_len - self.cache_size)
 
 
+
+class AdaKVScheduler(BaseScheduler):
+    """Keep the int(len*(1-compression_ratio)) rows with the highest linear importance
+    score (core/single/module/pikv_scheduling.py:624-673).  The reference picks a
+    safeguarded top slice first and fills up from the rest; both slices together are the
+    plain top-num_keep of one score, which is what the native selection returns."""
+
+    def __init__(self, cache_size: int, hidden_size: int, compression_ratio: float = 0.5,
+                 safeguard_ratio: float = 0.2):
+        super().__init__(cache_size, hidden_size)
+        self.compression_ratio = compression_ratio
+        self.safeguard_ratio = safeguard_ratio
+        self.register_buffer("importance_scores", torch.zeros(cache_size))
+        self.linear_proj = nn.Linear(hidden_size, 1)
+
+    def update_importance(self, indices: torch.Tensor, keys: torch.Tensor):
+        with torch.no_grad():
+            self.importance_scores[indices] = self.linear_proj(keys).squeeze(-1)
+
+    def row_buffers(self):
+        return [self.importance_scores]
+
+    def num_keep(self, cache_len: int) -> int:
+        return int(cache_len * (1 - self.compression_ratio))
+
+    def evict_mask(self, cache_len: int, n_evict: int = 0) -> torch.Tensor:
+        """n_evict > 0 (the manager making room) lowers the kept count when needed."""
+        scores = _padded(self.importance_scores, cache_len).float().contiguous()
+        keep = max(0, min(self.num_keep(cache_len), cache_len - n_evict))
+        return _one_cache_select(ops.EVICT_H2O, scores, scores, cache_len, budgets=(keep, 0))
+
+    def select_eviction_candidates(self, keys, values, metadata) -> torch.Tensor:
+        cache_len = keys.size(0)
+        if cache_len <= self.cache_size:
+            return torch.zeros(cache_len, dtype=torch.bool, device=keys.device)
+        return self.evict_mask(cache_len)
+
+
+class DuoAttentionScheduler(StreamingLLMScheduler):
+    """Keep sink_size rows at the front and recent_size rows at the back
+    (core/single/module/pikv_scheduling.py:675-710)."""
+
+    def __init__(self, cache_size: int, hidden_size: int, sink_size: int = 64, recent_size: int = 512):
+        super().__init__(cache_size, hidden_size, start_size=sink_size, recent_size=recent_size)
+        self.sink_size = sink_size
+
+    def keep_budgets(self, cache_len: int):
+        # the reference keeps [:sink] and [-recent:] independently (they may overlap)
+        n_start = min(self.sink_size, cache_len)
+        return n_start, min(self.recent_size, cache_len)
+
+
 _NATIVE = {SchedulingPolicy.H2O: ops.EVICT_H2O, SchedulingPolicy.LRU: ops.EVICT_LRU}
 
 
@@ -378,6 +434,12 @@ class CacheSchedulingManager(nn.Module):
             return FlexGenScheduler(self.cache_size, self.hidden_size)
         if policy == SchedulingPolicy.LRU_PLUS:
             return LRUPlusScheduler(self.cache_size, self.hidden_size)
+        if policy == SchedulingPolicy.ADAKV:
+            return AdaKVScheduler(self.cache_size, self.hidden_size)
+        if policy == SchedulingPolicy.DUOATTENTION:
+            return DuoAttentionScheduler(self.cache_size, self.hidden_size,
+                                         sink_size=max(1, self.cache_size // 16),
+                                         recent_size=max(1, self.cache_size // 2))
         raise ValueError(f"Unknown scheduling policy: {policy}")
 
     def _ensure_pool(self, device):
@@ -451,7 +513,7 @@ class CacheSchedulingManager(nn.Module):
         self.cache_valid = torch.arange(self.cache_size) < self._fill_host
 
     def _evict_by_scheduler(self, pool, cur: int, n_ev: int):
-        """StreamingLLM / QUEST / FlexGen / LRU+: the scheduler scores its slots, the
+        """StreamingLLM / DuoAttention / QUEST / FlexGen / LRU+ / AdaKV: the scheduler scores its slots, the
         native selection turns the score into a keep list, and the compaction moves
         the scheduler's per-slot buffers together with the rows."""
         sch = self.scheduler.to(pool.device)

@@ -122,3 +122,28 @@ def test_manager_other_policies(dev, policy_name):
         assert np.array_equal(np_of(m.pool.ts)[rows], ref.ts[rows])
     assert m.get_cache_stats()["policy"] == SchedulingPolicy[policy_name].value
     assert m.get_cache_stats()["eviction_count"] > 0
+
+
+def test_adakv_and_duoattention_schedulers(dev):
+    import torch
+    from pikv_amd.scheduling import AdaKVScheduler, CacheSchedulingManager, DuoAttentionScheduler, SchedulingPolicy
+    r = rng(44)
+    C, L = 40, 60
+    a = AdaKVScheduler(C, 16, compression_ratio=0.5, safeguard_ratio=0.2).to(dev)
+    keys = torch.from_numpy(np.round(r.standard_normal((C, 16)) * 2).astype(np.float32) / 2).to(dev)
+    a.update_importance(torch.arange(C, device=dev), keys)
+    sc = np.pad(np_of(a.importance_scores), (0, L - C))
+    big = torch.zeros(L, 16, device=dev)
+    ev = np_of(a.select_eviction_candidates(big, big, {}))
+    assert np.array_equal(ev, ~O.adakv_keep(sc, 0.5, 0.2))
+    assert (~ev).sum() == int(L * 0.5)
+    assert not np_of(a.select_eviction_candidates(big[:C], big[:C], {})).any()
+    d = DuoAttentionScheduler(32, 16, sink_size=4, recent_size=10).to(dev)
+    ev = np_of(d.select_eviction_candidates(big, big, {}))
+    assert np.array_equal(ev, ~O.duo_keep(L, 4, 10))
+    for name in ("ADAKV", "DUOATTENTION"):
+        m = CacheSchedulingManager(32, 64, SchedulingPolicy[name])
+        for step in range(4):
+            m.update_cache(torch.randn(1, 12, 64, device=dev), torch.randn(1, 12, 64, device=dev))
+            assert 0 < m.get_cache_stats()["cache_size"] <= 32
+        assert m.get_cache_stats()["eviction_count"] > 0

@@ -380,3 +380,20 @@ def test_other_policies_known_answers():
         for i in range(40):
             before = sum((s[j] < s[i]) or (s[j] == s[i] and j < i) for j in range(40))
             assert ev[i] == (before < n)
+
+
+def test_adakv_duo_known_answers():
+    s = np.array([0.1, 0.9, 0.5, 0.9, -1.0, 0.3, 0.2, 0.8, 0.0, 0.4], dtype=np.float32)
+    # keep 5 of 10; safeguard 1 (the first 0.9), then the next four: 0.9(idx 3), 0.8, 0.5, 0.4
+    k = O.adakv_keep(s, 0.5, 0.2)
+    assert np.nonzero(k)[0].tolist() == [1, 2, 3, 7, 9]
+    # the two-stage pick equals the plain top-num_keep under the tie rule
+    r = np.random.default_rng(2)
+    for _ in range(20):
+        x = (np.round(r.standard_normal(37) * 3) / 3).astype(np.float32)
+        kk = O.adakv_keep(x, 0.4, 0.3)
+        want = np.zeros(37, dtype=bool)
+        want[O.topk_desc(x[None, :], int(37 * 0.6))[0]] = True
+        assert np.array_equal(kk, want)
+    assert O.duo_keep(10, 2, 3).tolist() == [True, True] + [False] * 5 + [True] * 3
+    assert O.duo_keep(4, 3, 3).all()
