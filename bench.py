@@ -139,6 +139,23 @@ def decode_read_workload(torch, ops, dev, iters):
     sc, tm, tsu = pool.scores(q, hq)
     t_h2o = _median_ms(torch, lambda: pool.h2o_accumulate(sc, tm, tsu, now=1.0), iters)
     t_att = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats), iters)
+    # one whole decode step: append the new token of every sequence, read the cache
+    pool.fill.fill_(N - 1)
+    new_k = torch.randn(B, D, generator=g, device=dev).to(torch.bfloat16)
+    new_v = torch.randn(B, D, generator=g, device=dev).to(torch.bfloat16)
+    seq_id = torch.arange(B, device=dev, dtype=torch.int32)
+    zero_slot = torch.zeros(B, device=dev, dtype=torch.int32)
+    one = torch.ones(B, device=dev, dtype=torch.int32)
+
+    def decode_step():
+        pool.fill.fill_(N - 1)
+        pool.quant_scatter(new_k, new_v, seq_id, zero_slot, 1, now=2.0)
+        pool.advance(one)
+        s_, m_, z_ = pool.scores(q, hq)
+        pool.h2o_accumulate(s_, m_, z_, now=2.0)
+        return pool.attend_values(s_, pool.head_stats)
+    t_step = _median_ms(torch, decode_step, iters)
+    pool.fill.fill_(N)
     t_sel = _median_ms(torch, lambda: pool.evict_select(0, heavy_ratio=1 / 16, recent_ratio=1 / 128), iters)
 
     def evict():
@@ -155,6 +172,10 @@ def decode_read_workload(torch, ops, dev, iters):
                                         bytes_with_score_store=k_bytes + rows * hq * 4),
         "h2o_accumulate": _entry(t_h2o, rows * hq * 4 + rows * 12),
         "attend_values": _entry(t_att, k_bytes + rows * hq * 4),
+        "decode_step": {"ms": t_step, "what": "append 1 token per sequence + scores + H2O accumulate + attention output",
+                        "cached_tokens_per_s": rows / (t_step * 1e-3),
+                        "algorithmic_bytes": 2 * k_bytes + 2 * rows * hq * 4 + rows * 12,
+                        "GBps": (2 * k_bytes + 2 * rows * hq * 4 + rows * 12) / (t_step * 1e-3) / 1e9},
         "evict_select": _entry(t_sel, rows * 8 + rows * 5),
         "evict_select_plus_compact": {"ms": t_evict},
     }
