@@ -337,12 +337,18 @@ int64_t pikv_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim,
  *   new_len    [n_caches]  int32   : number of survivors
  *   n_heavy/n_recent are per-cache DEVICE arrays so that no host read of
  *   cache_fill is needed; pikv_h2o_budget fills them from the ratios.
+ *   max_len >= max_c cache_fill[c] sizes the launch.  workspace (optional,
+ *   pikv_evict_workspace_bytes(n_caches, max_len) bytes, 256-byte aligned) lets long
+ *   caches be selected by several blocks each; with workspace == NULL one block
+ *   serves a cache whatever its length.  Both forms give identical results.
  * ---------------------------------------------------------------------- */
 int pikv_evict_select(int policy, const float* row_acc, const float* row_ts,
                       const int64_t* cache_row_base, const int32_t* cache_fill,
                       const int32_t* n_heavy, const int32_t* n_recent,
-                      int n_caches, uint8_t* keep_flag, int32_t* keep_index,
-                      int32_t* new_len, void* stream);
+                      int n_caches, int64_t max_len,
+                      uint8_t* keep_flag, int32_t* keep_index, int32_t* new_len,
+                      void* workspace, int64_t workspace_bytes, void* stream);
+int64_t pikv_evict_workspace_bytes(int n_caches, int64_t max_len);
 
 /* n_heavy[c] = max(1,int(len*heavy_ratio)); n_recent[c] = max(1,int(len*recent_ratio))
  * with len = cache_fill[c] and the product evaluated in double precision as

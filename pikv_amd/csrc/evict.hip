@@ -256,6 +256,265 @@ __global__ __launch_bounds__(kSelThreads) void evict_select_kernel(
                              new_len + c, g, s);
 }
 
+// ---- multi-block selection ---------------------------------------------------------
+// Long caches are cut into chunks of kMbChunk rows, one 256-thread block each.  The
+// order-preserving key is split into three digits (11 + 11 + 10 bits); pass p builds
+// the histogram of digit p over the keys that match the digits already chosen
+// (integer atomics into a per-cache table, so the result does not depend on
+// scheduling), and every later kernel re-derives the chosen digits from the tables.
+// Kernels, in stream order: zero tables | hist 0 | hist 1 | hist 2 | mark | list.
+// A thread owns 16 CONSECUTIVE rows, so ranks in index order are a thread-local count
+// plus one block scan plus the per-chunk counts of the earlier chunks.
+constexpr int kMbThreads = 256;
+constexpr int kMbItems = 16;
+constexpr int kMbChunk = kMbThreads * kMbItems;
+constexpr int kMbBins = 2048;
+
+struct MbArgs {
+  int policy;
+  const float* acc;
+  const float* ts;
+  const int64_t* row_base;
+  const int32_t* fill;
+  const int32_t* n_heavy;
+  const int32_t* n_recent;
+  uint8_t* keep_flag;
+  int32_t* keep_index;
+  int32_t* new_len;
+  int* hist;       // [cache][pass 0..2][slot 0..1][kMbBins]
+  int* blk_hist2;  // [cache][chunk][slot][1024]: last-digit histogram of every chunk
+  int* blk_kept;   // [cache][chunk]
+  int n_chunks;
+};
+
+__device__ __forceinline__ int mb_digit(uint32_t key, int pass) {
+  return pass == 0 ? (int)(key >> 21) : pass == 1 ? (int)((key >> 10) & 2047u) : (int)(key & 1023u);
+}
+__device__ __forceinline__ uint32_t mb_mask(int passes_done) {
+  return passes_done == 0 ? 0u : passes_done == 1 ? 0xffe00000u : passes_done == 2 ? 0xfffffc00u : 0xffffffffu;
+}
+
+// Selection `slot` of cache c: H2O slot 0 = n_heavy largest of acc, slot 1 = n_recent
+// largest of ts; LRU slot 0 = n_evict smallest of ts.  m is clamped to [0, len].
+struct MbSel {
+  const float* v;
+  bool smallest;
+  int m;
+  bool used;     // the slot exists for this policy
+  bool partial;  // 0 < m < len: a threshold has to be found
+};
+__device__ __forceinline__ MbSel mb_sel(const MbArgs& a, int c, int slot, int len) {
+  MbSel s;
+  const int64_t base = a.row_base[c];
+  if (a.policy == PIKV_EVICT_H2O) {
+    s.v = (slot == 0 ? a.acc : a.ts) + base;
+    s.smallest = false;
+    s.m = slot == 0 ? a.n_heavy[c] : a.n_recent[c];
+    s.used = true;
+  } else {
+    s.v = a.ts + base;
+    s.smallest = true;
+    s.m = a.n_heavy[c];
+    s.used = slot == 0;
+  }
+  s.m = s.m < 0 ? 0 : (s.m > len ? len : s.m);
+  s.partial = s.used && s.m > 0 && s.m < len;
+  return s;
+}
+
+// Exclusive prefix of v over the 256 threads (thread order); total to all.
+__device__ __forceinline__ int mb_block_scan(int v, int* sh /*4*/, int& total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = v;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int o = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += o;
+  }
+  __syncthreads();
+  if (lane == 63) sh[wave] = incl;
+  __syncthreads();
+  int pre = 0, tot = 0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const int t = sh[w];
+    if (w < wave) pre += t;
+    tot += t;
+  }
+  total = tot;
+  return pre + incl - v;
+}
+
+// Digit at which the running count from the top first reaches `remaining`; remaining
+// becomes the count still to take inside that digit.  All threads call; nb is 2048 or 1024.
+__device__ __forceinline__ int mb_pick(const int* __restrict__ hist, int nb, int& remaining, int* sh /*6*/) {
+  const int per = nb / kMbThreads;  // 8 or 4
+  int cnt[8], tot = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    cnt[k] = k < per ? hist[nb - 1 - (threadIdx.x * per + k)] : 0;
+    tot += cnt[k];
+  }
+  int all;
+  int before = mb_block_scan(tot, sh, all);
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    if (k < per && before < remaining && remaining <= before + cnt[k]) {
+      sh[4] = nb - 1 - (threadIdx.x * per + k);
+      sh[5] = remaining - before;
+    }
+    before += cnt[k];
+  }
+  __syncthreads();
+  remaining = sh[5];
+  return sh[4];
+}
+
+// Digits chosen by the first `passes` passes for one slot: key prefix and what remains.
+__device__ __forceinline__ uint32_t mb_prefix(const MbArgs& a, int c, int slot, int passes, int& remaining,
+                                              int* sh, int* last_digit) {
+  uint32_t prefix = 0;
+  for (int p = 0; p < passes; ++p) {
+    const int* h = a.hist + (((int64_t)c * 3 + p) * 2 + slot) * kMbBins;
+    const int d = mb_pick(h, p == 2 ? 1024 : kMbBins, remaining, sh);
+    prefix |= (uint32_t)d << (p == 0 ? 21 : p == 1 ? 10 : 0);
+    if (last_digit) *last_digit = d;
+  }
+  return prefix;
+}
+
+__global__ void mb_zero_kernel(int* __restrict__ p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+template <int PASS>
+__global__ __launch_bounds__(kMbThreads) void mb_hist_kernel(MbArgs a) {
+  __shared__ int lh[kMbBins];
+  __shared__ int sh[8];
+  const int c = blockIdx.y, chunk = blockIdx.x;
+  const int len = a.fill[c];
+  const int64_t i0 = (int64_t)chunk * kMbChunk + threadIdx.x * kMbItems;
+  constexpr int NB = PASS == 2 ? 1024 : kMbBins;
+  for (int slot = 0; slot < 2; ++slot) {
+    const MbSel s = mb_sel(a, c, slot, len);
+    int* bh = PASS == 2 ? a.blk_hist2 + (((int64_t)c * a.n_chunks + chunk) * 2 + slot) * 1024 : nullptr;
+    if (!s.partial || (int64_t)chunk * kMbChunk >= len) {  // uniform
+      if (PASS == 2)
+        for (int b = threadIdx.x; b < 1024; b += kMbThreads) bh[b] = 0;
+      continue;
+    }
+    int remaining = s.m;
+    const uint32_t prefix = mb_prefix(a, c, slot, PASS, remaining, sh, nullptr);
+    const uint32_t pmask = mb_mask(PASS);
+    for (int b = threadIdx.x; b < NB; b += kMbThreads) lh[b] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kMbItems; ++j) {
+      if (i0 + j < len) {
+        const uint32_t key = order_key(s.v[i0 + j], s.smallest);
+        if ((key & pmask) == prefix) atomicAdd(&lh[mb_digit(key, PASS)], 1);
+      }
+    }
+    __syncthreads();
+    int* gh = a.hist + (((int64_t)c * 3 + PASS) * 2 + slot) * kMbBins;
+    for (int b = threadIdx.x; b < NB; b += kMbThreads) {
+      const int n = lh[b];
+      if (PASS == 2) bh[b] = n;
+      if (n) atomicAdd(&gh[b], n);
+    }
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(kMbThreads) void mb_mark_kernel(MbArgs a) {
+  __shared__ int sh[8];
+  const int c = blockIdx.y, chunk = blockIdx.x;
+  const int len = a.fill[c];
+  const int64_t i0 = (int64_t)chunk * kMbChunk + threadIdx.x * kMbItems;
+  if ((int64_t)chunk * kMbChunk >= len) {  // uniform
+    if (threadIdx.x == 0) a.blk_kept[(int64_t)c * a.n_chunks + chunk] = 0;
+    return;
+  }
+  uint32_t selbits[2] = {0u, 0u};  // bit j: row i0+j is taken by the slot's selection
+  for (int slot = 0; slot < 2; ++slot) {
+    const MbSel s = mb_sel(a, c, slot, len);
+    if (!s.used || s.m <= 0) continue;  // uniform
+    if (s.m >= len) {
+      selbits[slot] = 0xffffu;
+      continue;
+    }
+    int remaining = s.m, d2 = 0;
+    const uint32_t kstar = mb_prefix(a, c, slot, 3, remaining, sh, &d2);
+    // rows equal to the threshold key in earlier chunks
+    int part = 0;
+    for (int b = threadIdx.x; b < chunk; b += kMbThreads)
+      part += a.blk_hist2[(((int64_t)c * a.n_chunks + b) * 2 + slot) * 1024 + d2];
+    int eq_before;
+    mb_block_scan(part, sh, eq_before);
+    uint32_t gt = 0, eq = 0;
+#pragma unroll
+    for (int j = 0; j < kMbItems; ++j) {
+      if (i0 + j < len) {
+        const uint32_t key = order_key(s.v[i0 + j], s.smallest);
+        gt |= (key > kstar ? 1u : 0u) << j;
+        eq |= (key == kstar ? 1u : 0u) << j;
+      }
+    }
+    int tot;
+    int rank = eq_before + mb_block_scan(__popc(eq), sh, tot);
+    uint32_t take = gt;
+#pragma unroll
+    for (int j = 0; j < kMbItems; ++j) {
+      if ((eq >> j) & 1u) {
+        if (rank < remaining) take |= 1u << j;
+        ++rank;
+      }
+    }
+    selbits[slot] = take;
+  }
+  uint32_t valid = 0;
+#pragma unroll
+  for (int j = 0; j < kMbItems; ++j) valid |= (i0 + j < len ? 1u : 0u) << j;
+  const uint32_t keep = (a.policy == PIKV_EVICT_H2O ? (selbits[0] | selbits[1]) : ~selbits[0]) & valid;
+  uint8_t* flag = a.keep_flag + a.row_base[c];
+#pragma unroll
+  for (int j = 0; j < kMbItems; ++j)
+    if ((valid >> j) & 1u) flag[i0 + j] = (keep >> j) & 1u;
+  int kept;
+  mb_block_scan(__popc(keep), sh, kept);
+  if (threadIdx.x == 0) a.blk_kept[(int64_t)c * a.n_chunks + chunk] = kept;
+}
+
+__global__ __launch_bounds__(kMbThreads) void mb_list_kernel(MbArgs a) {
+  __shared__ int sh[8];
+  const int c = blockIdx.y, chunk = blockIdx.x;
+  const int len = a.fill[c];
+  // survivors in the earlier chunks, and (chunk 0) in all of them
+  int before = 0, all = 0;
+  const int lim = chunk == 0 ? a.n_chunks : chunk;
+  for (int b = threadIdx.x; b < lim; b += kMbThreads) before += a.blk_kept[(int64_t)c * a.n_chunks + b];
+  mb_block_scan(before, sh, all);
+  if (chunk == 0) {
+    if (threadIdx.x == 0) a.new_len[c] = len > 0 ? all : 0;
+    all = 0;
+  }
+  if ((int64_t)chunk * kMbChunk >= len) return;  // uniform
+  const int64_t i0 = (int64_t)chunk * kMbChunk + threadIdx.x * kMbItems;
+  const uint8_t* flag = a.keep_flag + a.row_base[c];
+  uint32_t keep = 0;
+#pragma unroll
+  for (int j = 0; j < kMbItems; ++j)
+    if (i0 + j < len && flag[i0 + j]) keep |= 1u << j;
+  int tot;
+  int pos = all + mb_block_scan(__popc(keep), sh, tot);
+  int32_t* out = a.keep_index + a.row_base[c];
+#pragma unroll
+  for (int j = 0; j < kMbItems; ++j)
+    if ((keep >> j) & 1u) out[pos++] = (int32_t)(i0 + j);
+}
+
 __global__ void h2o_budget_kernel(const int32_t* __restrict__ fill, int n, double heavy_ratio,
                                   double recent_ratio, int32_t* __restrict__ n_heavy,
                                   int32_t* __restrict__ n_recent) {
@@ -346,19 +605,52 @@ __global__ void set_fill_kernel(int32_t* __restrict__ fill, const int32_t* __res
 
 using namespace pikv;
 
+static int64_t mb_chunks(int64_t max_len) { return (max_len + kMbChunk - 1) / kMbChunk; }
+
+extern "C" int64_t pikv_evict_workspace_bytes(int n_caches, int64_t max_len) {
+  if (n_caches < 1 || max_len < 0) return 0;
+  const int64_t nch = mb_chunks(max_len);
+  return (int64_t)n_caches * (3 * 2 * kMbBins + nch * 2 * 1024 + nch) * (int64_t)sizeof(int);
+}
+
 extern "C" int pikv_evict_select(int policy, const float* row_acc, const float* row_ts,
                                  const int64_t* cache_row_base, const int32_t* cache_fill,
                                  const int32_t* n_heavy, const int32_t* n_recent, int n_caches,
-                                 uint8_t* keep_flag, int32_t* keep_index, int32_t* new_len,
+                                 int64_t max_len, uint8_t* keep_flag, int32_t* keep_index,
+                                 int32_t* new_len, void* workspace, int64_t workspace_bytes,
                                  void* stream) {
   if (!row_ts || !cache_row_base || !cache_fill || !n_heavy || !keep_flag || !keep_index || !new_len)
     return PIKV_ERR_NULL;
   if (policy != PIKV_EVICT_H2O && policy != PIKV_EVICT_LRU) return PIKV_ERR_UNSUPPORTED;
   if (policy == PIKV_EVICT_H2O && (!row_acc || !n_recent)) return PIKV_ERR_NULL;
-  if (n_caches < 1) return PIKV_ERR_SHAPE;
-  hipLaunchKernelGGL(evict_select_kernel, dim3((unsigned)n_caches), dim3(kSelThreads), 0,
-                     (hipStream_t)stream, policy, row_acc, row_ts, cache_row_base, cache_fill,
-                     n_heavy, n_recent, keep_flag, keep_index, new_len);
+  if (n_caches < 1 || max_len < 0) return PIKV_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  // caches of more than two chunks are worth several blocks each, when the caller
+  // brought the tables
+  if (workspace && max_len > 2 * kMbChunk) {
+    if (n_caches > 65535) return PIKV_ERR_SHAPE;
+    if (workspace_bytes < pikv_evict_workspace_bytes(n_caches, max_len)) return PIKV_ERR_WORKSPACE;
+    const int64_t nch = mb_chunks(max_len);
+    if (nch > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+    MbArgs a{policy, row_acc, row_ts, cache_row_base, cache_fill, n_heavy, n_recent, keep_flag,
+             keep_index, new_len, nullptr, nullptr, nullptr, (int)nch};
+    a.hist = reinterpret_cast<int*>(workspace);
+    a.blk_hist2 = a.hist + (int64_t)n_caches * 3 * 2 * kMbBins;
+    a.blk_kept = a.blk_hist2 + (int64_t)n_caches * nch * 2 * 1024;
+    const int64_t nz = (int64_t)n_caches * 3 * 2 * kMbBins;
+    hipLaunchKernelGGL(mb_zero_kernel, dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, st, a.hist, nz);
+    const dim3 grid((unsigned)nch, (unsigned)n_caches);
+    hipLaunchKernelGGL(mb_hist_kernel<0>, grid, dim3(kMbThreads), 0, st, a);
+    hipLaunchKernelGGL(mb_hist_kernel<1>, grid, dim3(kMbThreads), 0, st, a);
+    hipLaunchKernelGGL(mb_hist_kernel<2>, grid, dim3(kMbThreads), 0, st, a);
+    hipLaunchKernelGGL(mb_mark_kernel, grid, dim3(kMbThreads), 0, st, a);
+    hipLaunchKernelGGL(mb_list_kernel, grid, dim3(kMbThreads), 0, st, a);
+    PIKV_CHECK_LAUNCH();
+    return PIKV_OK;
+  }
+  hipLaunchKernelGGL(evict_select_kernel, dim3((unsigned)n_caches), dim3(kSelThreads), 0, st, policy,
+                     row_acc, row_ts, cache_row_base, cache_fill, n_heavy, n_recent, keep_flag,
+                     keep_index, new_len);
   PIKV_CHECK_LAUNCH();
   return PIKV_OK;
 }

@@ -312,7 +312,12 @@ def fakequant_colblocks(x, group: int, bits: int = 8, symmetric: bool = False):
 # cache pool
 # --------------------------------------------------------------------------
 
-def select_top_rows(score, seg_base, seg_len, n_keep):
+def _evict_workspace(n_caches: int, max_len: int, device):
+    nbytes = int(N.lib().pikv_evict_workspace_bytes(n_caches, max_len))
+    return torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device), nbytes
+
+
+def select_top_rows(score, seg_base, seg_len, n_keep, max_len: Optional[int] = None):
     """Per segment c of a flat score array (rows seg_base[c] .. +seg_len[c]): keep
     the n_keep[c] largest scores, ties to the lower index.  Returns (keep_flag
     uint8 [rows], keep_index int32 [rows], n_kept int32 [segments]); segment c's
@@ -331,9 +336,13 @@ def select_top_rows(score, seg_base, seg_len, n_keep):
     if n == 0 or score.numel() == 0:
         return flag, index, kept
     zero = torch.zeros(n, dtype=torch.int32, device=dev)
+    if max_len is None:   # an upper bound of every segment length that needs no device read
+        max_len = score.numel()
+    ws, ws_bytes = _evict_workspace(n, int(max_len), dev)
     # H2O selection with an empty "recent" budget; the score doubles as the (unused) timestamp
     N.call("pikv_evict_select", EVICT_H2O, _ptr(score), _ptr(score), _ptr(seg_base), _ptr(seg_len),
-           _ptr(n_keep), _ptr(zero), n, _ptr(flag), _ptr(index), _ptr(kept), _stream())
+           _ptr(n_keep), _ptr(zero), n, int(max_len), _ptr(flag), _ptr(index), _ptr(kept), _ptr(ws),
+           ws_bytes, _stream())
     return flag, index, kept
 
 
@@ -605,10 +614,11 @@ class CachePool:
 
     # ---- eviction ----
     def evict_select(self, policy: int, *, heavy_ratio=0.1, recent_ratio=0.1,
-                     n_heavy=None, n_recent=None, n_evict=None):
+                     n_heavy=None, n_recent=None, n_evict=None, multi_block: bool = True):
         """Fill keep_flag / keep_index / new_len.  H2O: budgets from the
         ratios (per cache, from its current fill) or explicit int32 tensors;
-        LRU: n_evict int32 [n_caches]."""
+        LRU: n_evict int32 [n_caches].  multi_block=False withholds the workspace, so
+        that one block selects each cache whatever its length (same result)."""
         if policy == EVICT_H2O:
             if n_heavy is None:
                 N.call("pikv_h2o_budget", _ptr(self.fill), self.n_caches, float(heavy_ratio),
@@ -624,9 +634,14 @@ class CachePool:
             raise ValueError(f"unknown eviction policy {policy}")
         if nh.numel() != self.n_caches or (nr is not None and nr.numel() != self.n_caches):
             raise ValueError("budgets must have one entry per cache")
+        ws, ws_bytes = None, 0
+        if multi_block:
+            if getattr(self, "_evict_ws", None) is None:
+                self._evict_ws = _evict_workspace(self.n_caches, self.max_cap, self.device)
+            ws, ws_bytes = self._evict_ws
         N.call("pikv_evict_select", policy, _ptr(self.acc), _ptr(self.ts), _ptr(self.row_base),
-               _ptr(self.fill), _ptr(nh), _ptr(nr), self.n_caches, _ptr(self.keep_flag),
-               _ptr(self.keep_index), _ptr(self.new_len), _stream())
+               _ptr(self.fill), _ptr(nh), _ptr(nr), self.n_caches, self.max_cap, _ptr(self.keep_flag),
+               _ptr(self.keep_index), _ptr(self.new_len), _ptr(ws), ws_bytes, _stream())
 
     def planes(self):
         ps = [self.k_codes, self.k_scale, self.k_zero, self.v_codes, self.v_scale, self.v_zero,

@@ -59,7 +59,7 @@ class PyramidCache:
         seg_base = torch.arange(L, dtype=torch.int64, device=dev) * n
         seg_len = torch.full((L,), n, dtype=torch.int32, device=dev)
         flat = scores.contiguous().reshape(-1)
-        _, index, kept = ops.select_top_rows(flat, seg_base, seg_len, self._n_keep)
+        _, index, kept = ops.select_top_rows(flat, seg_base, seg_len, self._n_keep, max_len=n)
         self.pool.fill.zero_()
         self.pool.quant_gather(keys, values if self.pool.with_v else None, seg_base, index, kept,
                                max(self.keep), src_score=flat, now=now)

@@ -105,8 +105,8 @@ def _one_cache_select(policy: int, acc: Optional[torch.Tensor], ts: torch.Tensor
     else:
         nh.fill_(int(n_evict))
     N.call("pikv_evict_select", policy, None if acc is None else acc.data_ptr(), ts.data_ptr(),
-           row_base.data_ptr(), fill.data_ptr(), nh.data_ptr(), nr.data_ptr(), 1, flag.data_ptr(),
-           kidx.data_ptr(), new_len.data_ptr(), st)
+           row_base.data_ptr(), fill.data_ptr(), nh.data_ptr(), nr.data_ptr(), 1, length, flag.data_ptr(),
+           kidx.data_ptr(), new_len.data_ptr(), None, 0, st)
     return flag == 0
 
 

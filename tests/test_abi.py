@@ -30,7 +30,7 @@ def test_header_declares_expected_surface():
                  "pikv_h2o_budget", "pikv_compact_rows", "pikv_fakequant_colblocks",
                  "pikv_router_workspace_bytes", "pikv_fakequant_workspace_bytes",
                  "pikv_router_fused_workspace_bytes", "pikv_quant_gather", "pikv_attend_values",
-                 "pikv_attend_workspace_bytes",
+                 "pikv_attend_workspace_bytes", "pikv_evict_workspace_bytes",
                  "pikv_status_string", "pikv_abi_version"]:
         assert need in d
 
@@ -66,7 +66,9 @@ def test_pure_host_entry_points():
                                  None, None, 1, 1, None, None, None, 0, None) == -3
     assert lib.pikv_router_fused(1, 1, 7, None, None, None, 1.0, 0.0, 4, 64, 4, 2, 0,
                                  None, None, 1, 1, None, None, None, 0, None) == -3
-    assert lib.pikv_evict_select(9, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, None) == -3
+    assert lib.pikv_evict_select(9, 1, 1, 1, 1, 1, 1, 1, 64, 1, 1, 1, None, 0, None) == -3
+    assert lib.pikv_evict_workspace_bytes(2, 4097) == 2 * (3 * 2 * 2048 + 2 * 2 * 1024 + 2) * 4
+    assert lib.pikv_evict_select(0, 1, 1, 1, 1, 1, 1, 2, 10000, 1, 1, 1, 1, 100, None) == -4
     # bf16 router needs its workspace (re-laid gate weights): too small -> workspace status
     need = lib.pikv_router_fused_workspace_bytes(64, 128, 8, 2)
     assert need >= 128 * 16 * 2

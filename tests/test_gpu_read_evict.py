@@ -195,10 +195,13 @@ def test_select_brute_force_small(dev):
             assert bool(flags[rows[i]]) == want, (c, i)
 
 
+@pytest.mark.parametrize("multi_block", [False, True])
 @pytest.mark.parametrize("ties", [False, True])
-def test_h2o_select_long_cache(dev, ties):
-    """Caches longer than 32768 rows take the selection path that re-reads its keys
-    from memory in every pass; one shorter cache rides along on the register path."""
+def test_h2o_select_long_cache(dev, ties, multi_block):
+    """Long caches.  One block per cache (no workspace): caches longer than 32768 rows
+    take the selection path that re-reads its keys from memory in every pass, a shorter
+    one rides along on the register path.  With the workspace every cache is cut into
+    4096-row chunks; budgets of 1, of everything and lengths one off a chunk edge."""
     r = rng(77 + ties)
     caps = [70000, 33000, 32768]
     lens = [69999, 32769, 32768]
@@ -206,7 +209,7 @@ def test_h2o_select_long_cache(dev, ties):
     _set_state(pool, ref, r, ties)
     nh = np.array([4375, 1, 2048], dtype=np.int32)
     nr = np.array([546, 32769, 256], dtype=np.int32)
-    pool.evict_select(0, n_heavy=to_dev(nh, dev), n_recent=to_dev(nr, dev))
+    pool.evict_select(0, n_heavy=to_dev(nh, dev), n_recent=to_dev(nr, dev), multi_block=multi_block)
     keeps = []
     for c, L in enumerate(lens):
         rows = ref.valid_rows(c)
@@ -219,3 +222,36 @@ def test_h2o_select_long_cache(dev, ties):
         assert np.array_equal(np_of(pool.keep_index)[rows[0]:rows[0] + m], np.nonzero(keep)[0])
     pool.compact()
     _check_compacted(pool, ref, O.Q_I8_SYM, keeps)
+
+
+@pytest.mark.parametrize("ties", [False, True])
+def test_select_chunked_edges(dev, ties):
+    """Several blocks per cache: empty cache, lengths around the 4096-row chunk edge,
+    zero and full budgets, both policies; twice in a row on the same workspace."""
+    r = rng(91 + ties)
+    caps = [20000] * 6
+    lens = [0, 1, 4095, 4096, 4097, 20000]
+    pool, ref = _fill_pool(dev, r, caps, lens, 1, 32, 32, O.Q_I8_SYM, dtype="f32")
+    _set_state(pool, ref, r, ties)
+    for rep in range(2):
+        nh = np.array([3, 1, 0, 4096, 17, 1250 + rep], dtype=np.int32)
+        nr = np.array([2, 0, 100, 0, 4097, 156], dtype=np.int32)
+        pool.evict_select(0, n_heavy=to_dev(nh, dev), n_recent=to_dev(nr, dev))
+        for c, L in enumerate(lens):
+            rows = ref.valid_rows(c)
+            keep = O.h2o_keep(ref.acc[rows], ref.ts[rows], int(nh[c]), int(nr[c]))
+            m = int(np_of(pool.new_len)[c])
+            assert m == keep.sum(), (c, m, keep.sum())
+            if L:
+                assert np.array_equal(np_of(pool.keep_flag)[rows].astype(bool), keep), c
+                assert np.array_equal(np_of(pool.keep_index)[rows[0]:rows[0] + m], np.nonzero(keep)[0])
+        ne = np.array([1, 1, 4000, 0, 4097, 9999 - rep], dtype=np.int32)
+        pool.evict_select(1, n_evict=to_dev(ne, dev))
+        for c, L in enumerate(lens):
+            rows = ref.valid_rows(c)
+            keep = O.lru_keep(ref.ts[rows], int(ne[c]))
+            m = int(np_of(pool.new_len)[c])
+            assert m == keep.sum(), (c, m, keep.sum())
+            if L:
+                assert np.array_equal(np_of(pool.keep_flag)[rows].astype(bool), keep), c
+                assert np.array_equal(np_of(pool.keep_index)[rows[0]:rows[0] + m], np.nonzero(keep)[0])
