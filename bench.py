@@ -152,9 +152,10 @@ def decode_read_workload(torch, ops, dev, iters):
         pool.quant_scatter(new_k, new_v, seq_id, zero_slot, 1, now=2.0)
         pool.advance(one)
         s_, m_, z_ = pool.scores(q, hq)
-        pool.h2o_accumulate(s_, m_, z_, now=2.0)
-        return pool.attend_values(s_, pool.head_stats)
+        pool.h2o_accumulate(s_, m_, z_, now=2.0, stats_only=True)
+        return pool.attend_values(s_, pool.head_stats, accumulate=True, now=2.0)
     t_step = _median_ms(torch, decode_step, iters)
+    t_att_acc = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats, accumulate=True, now=1.0), iters)
     pool.fill.fill_(N)
     t_sel = _median_ms(torch, lambda: pool.evict_select(0, heavy_ratio=1 / 16, recent_ratio=1 / 128), iters)
 
@@ -172,7 +173,9 @@ def decode_read_workload(torch, ops, dev, iters):
                                         bytes_with_score_store=k_bytes + rows * hq * 4),
         "h2o_accumulate": _entry(t_h2o, rows * hq * 4 + rows * 12),
         "attend_values": _entry(t_att, k_bytes + rows * hq * 4),
-        "decode_step": {"ms": t_step, "what": "append 1 token per sequence + scores + H2O accumulate + attention output",
+        "attend_values_with_h2o": _entry(t_att_acc, k_bytes + rows * hq * 4 + rows * 12),
+        "decode_step": {"ms": t_step, "what": "append 1 token per sequence + scores + head statistics + attention "
+                                              "output with the H2O accumulate in the same pass",
                         "cached_tokens_per_s": rows / (t_step * 1e-3),
                         "algorithmic_bytes": 2 * k_bytes + 2 * rows * hq * 4 + rows * 12,
                         "GBps": (2 * k_bytes + 2 * rows * hq * 4 + rows * 12) / (t_step * 1e-3) / 1e9},

@@ -283,7 +283,9 @@ int pikv_gather_dequant_scores(const void* k_codes, const void* k_scale,
  *   If write_probs != 0 scores is overwritten with the probabilities.
  *   importance_out [n_caches, score_stride] float or NULL receives the summed
  *   probabilities.  head_stats [n_caches, n_q_heads, 2] float receives the final
- *   (max, sum of exp(score - max)) of every head; pikv_attend_values takes it. */
+ *   (max, sum of exp(score - max)) of every head; pikv_attend_values takes it.
+ *   With write_probs == 0 and row_acc, row_ts, importance_out all NULL only the
+ *   statistics are computed (for a pikv_attend_values call that accumulates itself). */
 int pikv_h2o_accumulate(float* scores, const float* tile_max,
                         const float* tile_sum, int n_q_heads,
                         const int64_t* cache_row_base,
@@ -305,7 +307,11 @@ int pikv_h2o_accumulate(float* scores, const float* tile_max,
  *   out [n_caches, n_q_heads, head_dim] float; V planes as in the pool layout;
  *   workspace: pikv_attend_workspace_bytes(...) bytes (partial sums of token
  *   ranges, added in a fixed order), 256-byte aligned.  Shape limits as for
- *   pikv_gather_dequant_scores. */
+ *   pikv_gather_dequant_scores.
+ *   row_acc / row_ts (each may be NULL): the H2O bookkeeping of pikv_h2o_accumulate
+ *   on the same probabilities, done in the same pass over the scores:
+ *   acc[row] = acc[row]*decay + sum_h p[c,h,n], ts[row] = now
+ *   (core/single/cache_scheduling.py:69-73). */
 int pikv_attend_values(const float* scores, const float* head_stats,
                        int64_t score_stride,
                        const void* v_codes, const void* v_scale, const void* v_zero,
@@ -313,6 +319,7 @@ int pikv_attend_values(const float* scores, const float* head_stats,
                        int n_kv_heads, int n_q_heads, int head_dim,
                        const int64_t* cache_row_base, const int32_t* cache_fill,
                        int n_caches, int64_t max_len,
+                       float decay, float now, float* row_acc, float* row_ts,
                        float* out, void* workspace, int64_t workspace_bytes,
                        void* stream);
 int64_t pikv_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim,

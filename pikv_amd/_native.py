@@ -48,7 +48,7 @@ SIGNATURES = {
     "pikv_h2o_accumulate": (_i, [_p, _p, _p, _i, _p, _p, _i, _l, _l, _f, _f, _i,
                                  _p, _p, _p, _p, _p]),
     "pikv_attend_values": (_i, [_p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _i, _l,
-                                _p, _p, _l, _p]),
+                                _f, _f, _p, _p, _p, _p, _l, _p]),
     "pikv_attend_workspace_bytes": (_l, [_i, _i, _i, _l]),
     "pikv_evict_select": (_i, [_i, _p, _p, _p, _p, _p, _p, _i, _l, _p, _p, _p, _p, _l, _p]),
     "pikv_evict_workspace_bytes": (_l, [_i, _l]),

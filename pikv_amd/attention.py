@@ -9,8 +9,9 @@ kernel), and a single-token call - the decode step - attends over the WHOLE cach
 context natively:
 
     scores   = pikv_gather_dequant_scores   (QK^T over the compressed K rows, :123)
-    softmax  = pikv_h2o_accumulate          (:163; also feeds the H2O importance)
-    context  = pikv_attend_values           (probabilities x compressed V rows, :188)
+    softmax  = pikv_h2o_accumulate          (:163; here only the per-head max and sum)
+    context  = pikv_attend_values           (probabilities x compressed V rows, :188; the same
+                                             pass adds the probabilities to the H2O importance)
 
 Multi-token calls (prefill) compute their attention in torch exactly as the reference
 does and write their K/V rows into the cache.  When a cache would overflow, the
@@ -171,8 +172,9 @@ class PiKVAttention(nn.Module):
         pool = self.pool
         qq = q.to(torch.bfloat16) if q.dtype == torch.bfloat16 else q.float()
         scores, tmax, tsum = pool.scores(qq.contiguous(), self.num_heads, 1.0 / math.sqrt(self.head_dim))
-        pool.h2o_accumulate(scores, tmax, tsum, now=float(self.clock))
-        return pool.attend_values(scores, pool.head_stats)          # [B, heads, head_dim]
+        pool.h2o_accumulate(scores, tmax, tsum, now=float(self.clock), stats_only=True)
+        # probabilities x V rows and the H2O importance of the same probabilities in one pass
+        return pool.attend_values(scores, pool.head_stats, accumulate=True, now=float(self.clock))
 
     def _dense_attention(self, q, k, v, attention_mask, causal_mask):
         """core/single/pikv_attention.py:104-191 on the K/V of this call."""

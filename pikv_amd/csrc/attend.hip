@@ -45,6 +45,11 @@ struct AttendArgs {
   int n_q_heads;
   int head_dim;
   int n_caches;
+  // optional H2O bookkeeping of the same probabilities: acc = acc*decay + sum over heads, ts = now
+  float* row_acc;
+  float* row_ts;
+  float decay;
+  float now;
 };
 
 __device__ __forceinline__ float prob_of(float s, float mx, float rz, bool normalise) {
@@ -131,6 +136,29 @@ __global__ __launch_bounds__(256) void attend_valu_kernel(AttendArgs a) {
   }
 }
 
+// Importance of every cached token (sum of its probabilities over the query heads, in
+// head order) for callers of the vector-unit form.
+__global__ __launch_bounds__(256) void attend_importance_kernel(AttendArgs a) {
+  const int c = blockIdx.y;
+  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (n >= a.fill[c]) return;
+  const bool normalise = a.head_stats != nullptr;
+  float imp = 0.f;
+  for (int hq = 0; hq < a.n_q_heads; ++hq) {
+    const int64_t hi = (int64_t)c * a.n_q_heads + hq;
+    const float mx = normalise ? a.head_stats[hi * 2] : 0.f;
+    const float rz = normalise ? 1.0f / a.head_stats[hi * 2 + 1] : 1.f;
+    imp = imp + prob_of(a.scores[hi * a.score_stride + n], mx, rz, normalise);
+  }
+  const int64_t row = a.row_base[c] + n;
+  if (a.row_acc) {
+    float acc = a.row_acc[row];
+    if (a.decay != 1.0f) acc = acc * a.decay;
+    a.row_acc[row] = acc + imp;
+  }
+  if (a.row_ts) a.row_ts[row] = a.now;
+}
+
 // ---- matrix-core form -----------------------------------------------------------------
 typedef int pikv_i32x2 __attribute__((ext_vector_type(2)));
 
@@ -144,10 +172,14 @@ __device__ __forceinline__ int att_meta_off(int tok, int g, int hk) {
   return tok * (hk * 16 + 16) + (tok >> 4) * 64 + g * 16;
 }
 
-static size_t attend_mfma_lds_bytes(int n_kv_heads) {
+constexpr int kAttPRow = 68;  // floats per query head of staged probabilities: 64 tokens + 4 (bank spread)
+
+static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads) {
   // codes [64 tokens][n_kv_heads*64 + 8 bytes]; scale and zero + bias as float4 (4 groups)
-  // [64 tokens][kv head] in padded token rows; A operands per wavefront [4 groups][8 rows][kAttARow]
-  return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * att_meta_bytes(n_kv_heads) + 4 * (size_t)4 * 8 * kAttARow;
+  // [64 tokens][kv head] in padded token rows; A operands per wavefront [4 groups][8 rows][kAttARow];
+  // probabilities [query head][kAttPRow]
+  return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * att_meta_bytes(n_kv_heads) + 4 * (size_t)4 * 8 * kAttARow +
+         (size_t)n_q_heads * kAttPRow * 4;
 }
 
 // HKS = log2(n_kv_heads); at most 4 query heads per kv head.
@@ -168,6 +200,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   unsigned char* abuf = lzterm + att_meta_bytes(HK) + wave * (4 * 8 * kAttARow);
+  float* lprob = reinterpret_cast<float*>(lzterm + att_meta_bytes(HK) + 4 * (4 * 8 * kAttARow));
 
   const int c = blockIdx.y;
   const int64_t len = a.fill[c];
@@ -193,29 +226,48 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
   pikv_f32x4 C[NH][8];
   float zacc[NH][4];
-  float mx[NH], rz[NH];
-  const float* srow[NH];
 #pragma unroll
   for (int hs = 0; hs < NH; ++hs) {
-    const int g = wave + 4 * hs;
-    const int hq = (g < HK && row_on) ? g * rep + r : 0;
-    srow[hs] = a.scores + ((int64_t)c * a.n_q_heads + hq) * a.score_stride;
-    mx[hs] = 0.f;
-    rz[hs] = 1.f;
-    if (normalise) {
-      mx[hs] = a.head_stats[((int64_t)c * a.n_q_heads + hq) * 2];
-      rz[hs] = 1.0f / a.head_stats[((int64_t)c * a.n_q_heads + hq) * 2 + 1];
-    }
 #pragma unroll
     for (int d = 0; d < 8; ++d) C[hs][d] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int sg = 0; sg < 4; ++sg) zacc[hs][sg] = 0.f;
   }
+  // score-staging role: query head sh, tokens st8..st8+7 of the tile (32 heads x 8 runs)
+  const int sh = threadIdx.x >> 3;
+  const int st8 = (threadIdx.x & 7) * 8;
+  const bool s_on = sh < a.n_q_heads;
+  const float* srow = a.scores + ((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * a.score_stride;
+  float smx = 0.f, srz = 1.f;
+  if (normalise) {
+    smx = a.head_stats[((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * 2];
+    srz = 1.0f / a.head_stats[((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * 2 + 1];
+  }
+  const bool s_vec = (a.score_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(a.scores) & 15) == 0;
+  const float s_off = normalise ? -INFINITY : 0.f;  // what a token past the end contributes: p = 0
 
   // registers that carry the next tile from HBM to LDS
   uint4 pc[NCH];
   uint2 ps[NMC], pz[NMC];
+  float psc[8];
+  // importance role: wavefront w owns tokens 16w..16w+15 of a tile, lanes 0..15 hold their accumulators
+  const int it = wave * 16 + (lane & 15);
+  const int igrp = lane >> 4;
+  float pacc = 0.f;
   auto fetch = [&](int64_t n0) {
+    if (a.row_acc && igrp == 0 && n0 + it < t1) pacc = a.row_acc[base_row + n0 + it];
+    if (s_on) {
+      const int64_t n = n0 + st8;
+      if (s_vec && n + 8 <= t1) {
+        const float4 lo4 = *reinterpret_cast<const float4*>(srow + n);
+        const float4 hi4 = *reinterpret_cast<const float4*>(srow + n + 4);
+        psc[0] = lo4.x, psc[1] = lo4.y, psc[2] = lo4.z, psc[3] = lo4.w;
+        psc[4] = hi4.x, psc[5] = hi4.y, psc[6] = hi4.z, psc[7] = hi4.w;
+      } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) psc[k] = n + k < t1 ? srow[n + k] : s_off;
+      }
+    }
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
       const int ch = k * 256 + threadIdx.x;
@@ -239,6 +291,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   };
   auto h2f = [](uint32_t w, int hi) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> (16 * hi))); };
   auto stage = [&]() {
+    if (s_on) {
+      // tokens {l, l+4, l+8, l+12} of a 16-token group go side by side: one float4 per reader
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int t = st8 + k;
+        lprob[sh * kAttPRow + (t & ~15) + (t & 3) * 4 + ((t >> 2) & 3)] = prob_of(psc[k], smx, srz, normalise);
+      }
+    }
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
       const int ch = k * 256 + threadIdx.x;
@@ -268,21 +328,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     __syncthreads();  // the previous tile has been consumed
     stage();
     __syncthreads();
+    float acc = pacc;
     if (n0 + kAttTile < t1) fetch(n0 + kAttTile);  // in flight while this tile is multiplied
+    if (a.row_acc || a.row_ts) {  // uniform
+      // importance of the tile's tokens: four lanes per token add every fourth head, and two
+      // exchanges add the four partial sums
+      const int t = it;
+      const int grp = igrp;
+      const bool mine = grp == 0 && n0 + t < t1;
+      const int64_t row = base_row + n0 + t;
+      const float* lp = lprob + (t & ~15) + (t & 3) * 4 + ((t >> 2) & 3);
+      float imp = 0.f;
+      for (int hq = grp; hq < a.n_q_heads; hq += 4) imp = imp + lp[hq * kAttPRow];
+      imp = imp + __shfl_xor(imp, 16, 64);
+      imp = imp + __shfl_xor(imp, 32, 64);
+      if (mine) {
+        if (a.row_acc) {
+          if (a.decay != 1.0f) acc = acc * a.decay;
+          a.row_acc[row] = acc + imp;
+        }
+        if (a.row_ts) a.row_ts[row] = a.now;
+      }
+    }
 
 #pragma unroll
     for (int hs = 0; hs < NH; ++hs) {
       const int g = wave + 4 * hs;
       if (g >= HK) continue;  // uniform
       // ---- weights: this lane prepares head r for four tokens, all four groups ----
-      float p4[4];
       float4 s4[4], z4[4];
+      const float4 pv = *reinterpret_cast<const float4*>(lprob + (row_on ? g * rep + r : 0) * kAttPRow + wkg * 16 +
+                                                         (lane & 3) * 4);
+      const float p4[4] = {row_on ? pv.x : 0.f, row_on ? pv.y : 0.f, row_on ? pv.z : 0.f, row_on ? pv.w : 0.f};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int64_t n = n0 + tk + 4 * j;
-        const bool ok = row_on && n < t1;
-        const float sv = ok ? srow[hs][n] : 0.f;
-        p4[j] = ok ? prob_of(sv, mx[hs], rz[hs], normalise) : 0.f;
         s4[j] = *reinterpret_cast<const float4*>(lscale + att_meta_off(tk + 4 * j, g, HK));
         z4[j] = *reinterpret_cast<const float4*>(lzterm + att_meta_off(tk + 4 * j, g, HK));
       }
@@ -382,7 +461,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
 template <int SCHEME>
 static void launch_attend_mfma(int n_kv_heads, dim3 grid, hipStream_t st, const AttendArgs& a) {
-  const size_t lds = attend_mfma_lds_bytes(n_kv_heads);
+  const size_t lds = attend_mfma_lds_bytes(n_kv_heads, a.n_q_heads);
   switch (n_kv_heads) {
     case 1: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 0>), grid, dim3(256), lds, st, a); break;
     case 2: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 1>), grid, dim3(256), lds, st, a); break;
@@ -424,7 +503,8 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
                                   const void* v_codes, const void* v_scale, const void* v_zero,
                                   int scheme, int group, int n_kv_heads, int n_q_heads, int head_dim,
                                   const int64_t* cache_row_base, const int32_t* cache_fill,
-                                  int n_caches, int64_t max_len, float* out, void* workspace,
+                                  int n_caches, int64_t max_len, float decay, float now,
+                                  float* row_acc, float* row_ts, float* out, void* workspace,
                                   int64_t workspace_bytes, void* stream) {
   if (!scores || !v_codes || !v_scale || !cache_row_base || !cache_fill || !out) return PIKV_ERR_NULL;
   if (scheme < 0 || scheme > 3) return PIKV_ERR_UNSUPPORTED;
@@ -451,7 +531,8 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
       return PIKV_ERR_WORKSPACE;
   }
   AttendArgs a{scores, head_stats, v_codes, v_scale, v_zero, cache_row_base, cache_fill,
-               (float*)workspace, score_stride, group, n_kv_heads, n_q_heads, head_dim, n_caches};
+               (float*)workspace, score_stride, group, n_kv_heads, n_q_heads, head_dim, n_caches,
+               row_acc, row_ts, decay, now};
   const int rep = n_q_heads / n_kv_heads;
   if (max_len > 0) {
     const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;
@@ -460,6 +541,9 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
       if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(n_kv_heads, grid, st, a);
       else launch_attend_mfma<PIKV_Q_I4_SYM>(n_kv_heads, grid, st, a);
     } else {
+      if (row_acc || row_ts)
+        hipLaunchKernelGGL(attend_importance_kernel, dim3((unsigned)((max_len + 255) / 256), (unsigned)n_caches),
+                           dim3(256), 0, st, a);
       // heads of a kv group per pass: the float accumulators of one lane must fit
       const int rp = eight ? (rep >= 4 ? 4 : rep >= 2 ? 2 : 1) : (rep >= 2 ? 2 : 1);
       const dim3 grid((unsigned)splits, (unsigned)n_caches, (unsigned)((rep + rp - 1) / rp));

@@ -834,6 +834,11 @@ extern "C" int pikv_h2o_accumulate(float* scores, const float* tile_max, const f
   hipStream_t st = (hipStream_t)stream;
   hipLaunchKernelGGL(head_stats_kernel, dim3((unsigned)n_q_heads, (unsigned)n_caches), dim3(64), 0,
                      st, tile_max, tile_sum, cache_fill, n_q_heads, n_tiles, head_stats);
+  // nothing to normalise or accumulate: the caller only wanted the statistics
+  if (!write_probs && !row_acc && !row_ts && !importance_out) {
+    PIKV_CHECK_LAUNCH();
+    return PIKV_OK;
+  }
   // 16-byte accesses need every score row to start on a 16-byte boundary
   const bool vec4 = (score_stride % 4 == 0) && ((reinterpret_cast<uintptr_t>(scores) & 15) == 0);
   const int per_block = 256 * (vec4 ? 4 : 1);

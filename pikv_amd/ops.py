@@ -564,8 +564,11 @@ class CachePool:
         return scores, tmax, tsum
 
     def h2o_accumulate(self, scores, tile_max, tile_sum, now: float, decay: float = 1.0,
-                       write_probs: bool = False, return_importance: bool = False):
-        """Normalise, sum over heads, acc += importance, ts = now."""
+                       write_probs: bool = False, return_importance: bool = False,
+                       stats_only: bool = False):
+        """Normalise, sum over heads, acc += importance, ts = now.  stats_only=True
+        leaves acc and ts alone and only fills self.head_stats (for an attend_values
+        call that accumulates itself)."""
         scores = _need(scores, "scores", dtype=torch.float32, ndim=3)
         tile_max = _need(tile_max, "tile_max", dtype=torch.float32, ndim=3)
         tile_sum = _need(tile_sum, "tile_sum", dtype=torch.float32, ndim=3)
@@ -580,16 +583,19 @@ class CachePool:
         head_stats = torch.empty(nc, hq, 2, dtype=torch.float32, device=dev)
         N.call("pikv_h2o_accumulate", _ptr(scores), _ptr(tile_max), _ptr(tile_sum), hq,
                _ptr(self.row_base), _ptr(self.fill), nc, stride, stride, float(decay), float(now),
-               int(bool(write_probs)), _ptr(self.acc), _ptr(self.ts), _ptr(imp), _ptr(head_stats),
-               _stream())
+               int(bool(write_probs)), None if stats_only else _ptr(self.acc),
+               None if stats_only else _ptr(self.ts), _ptr(imp), _ptr(head_stats), _stream())
         self.head_stats = head_stats   # (max, sum) per (cache, head): what attend_values normalises with
         return imp
 
-    def attend_values(self, scores, head_stats=None):
+    def attend_values(self, scores, head_stats=None, accumulate: bool = False, now: float = 0.0,
+                      decay: float = 1.0):
         """out[c,h,:] = sum_n p[c,h,n] * dequant(V[c,n,h/rep,:]) over the valid rows.
         scores [n_caches, n_q_heads, stride] float32: raw scores together with
         head_stats [n_caches, n_q_heads, 2] (as left in self.head_stats by
-        h2o_accumulate), or probabilities when head_stats is None."""
+        h2o_accumulate), or probabilities when head_stats is None.
+        accumulate=True also does h2o_accumulate's bookkeeping (acc = acc*decay + sum of
+        the probabilities over the heads, ts = now) in the same pass."""
         if not self.with_v:
             raise ValueError("this pool stores no V rows")
         scores = _need(scores, "scores", dtype=torch.float32, ndim=3)
@@ -608,8 +614,9 @@ class CachePool:
         ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
         N.call("pikv_attend_values", _ptr(scores), _ptr(head_stats), stride, _ptr(self.v_codes),
                _ptr(self.v_scale), _ptr(self.v_zero), self.scheme, self.group, self.n_heads, hq,
-               self.head_dim, _ptr(self.row_base), _ptr(self.fill), nc, stride, _ptr(out), _ptr(ws),
-               ws_bytes, _stream())
+               self.head_dim, _ptr(self.row_base), _ptr(self.fill), nc, stride, float(decay), float(now),
+               _ptr(self.acc) if accumulate else None, _ptr(self.ts) if accumulate else None,
+               _ptr(out), _ptr(ws), ws_bytes, _stream())
         return out
 
     # ---- eviction ----

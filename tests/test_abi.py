@@ -77,10 +77,12 @@ def test_pure_host_entry_points():
     # pyramid gather: NULL index list; attention output: heads must divide, workspace must fit
     assert lib.pikv_quant_gather(1, None, 1, 128, 128, 0, 1, None, 1, 4, None, 1, 1, 1, 1,
                                  1, None, 1, None, None, None, None, None, 0.0, None) == -1
-    assert lib.pikv_attend_values(1, None, 64, 1, 1, None, 0, 128, 3, 4, 128, 1, 1, 1, 64, 1, 1, 1 << 20, None) == -2
+    assert lib.pikv_attend_values(1, None, 64, 1, 1, None, 0, 128, 3, 4, 128, 1, 1, 1, 64, 1.0, 0.0, None, None,
+                                  1, 1, 1 << 20, None) == -2
     ws = lib.pikv_attend_workspace_bytes(2, 4, 128, 5000)
     assert ws == 3 * 2 * 4 * 128 * 4
-    assert lib.pikv_attend_values(1, None, 5000, 1, 1, None, 0, 128, 4, 4, 128, 1, 1, 2, 5000, 1, 1, ws - 1, None) == -4
+    assert lib.pikv_attend_values(1, None, 5000, 1, 1, None, 0, 128, 4, 4, 128, 1, 1, 2, 5000, 1.0, 0.0, None, None,
+                                  1, 1, ws - 1, None) == -4
 
 
 def test_ops_reject_cpu_tensors():

@@ -54,6 +54,47 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
         assert err <= 1e-3 * rms, (c, err, rms)
 
 
+@pytest.mark.parametrize("scheme,group,heads,hq,dh", [
+    (O.Q_I4_ASYM, 32, 8, 32, 128),     # matrix-core form: importance summed from the staged tile
+    (O.Q_I4_ASYM, 32, 2, 4, 128),
+    (O.Q_I8_SYM, 128, 4, 8, 128),      # vector form: importance in a kernel of its own
+])
+@pytest.mark.parametrize("decay", [1.0, 0.95])
+def test_attend_accumulates_importance(dev, scheme, group, heads, hq, dh, decay):
+    """attend_values(accumulate=True) after a statistics-only h2o_accumulate leaves the
+    same accumulators and timestamps as the separate h2o_accumulate pass, and the same
+    output as without the bookkeeping."""
+    import torch
+    r = rng(scheme * 7 + hq)
+    caps = [4200, 64, 130, 10]
+    lens = [4100, 64, 1, 0]
+    pool, ref = _fill_pool(dev, r, caps, lens, heads, dh, group, scheme)
+    pool.acc.copy_(to_dev(r.random(pool.rows).astype(np.float32), dev))
+    pool.ts.fill_(-3.0)
+    acc0 = pool.acc.clone()
+    q = O.bf16_round(r.standard_normal((len(caps), hq, dh)).astype(np.float32) * 3)
+    scores, tmax, tsum = pool.scores(to_dev(q, dev, "bf16"), hq)
+    pool.h2o_accumulate(scores, tmax, tsum, now=9.0, decay=decay)
+    acc_sep, ts_sep = np_of(pool.acc), np_of(pool.ts)
+    out_sep = np_of(pool.attend_values(scores, pool.head_stats))
+    pool.acc.copy_(acc0)
+    pool.ts.fill_(-3.0)
+    pool.h2o_accumulate(scores, tmax, tsum, now=9.0, stats_only=True)
+    assert torch.equal(pool.acc, acc0) and bool((pool.ts == -3.0).all())
+    out = np_of(pool.attend_values(scores, pool.head_stats, accumulate=True, now=9.0, decay=decay))
+    assert np.array_equal(out, out_sep)
+    assert np.array_equal(np_of(pool.ts), ts_sep)
+    np.testing.assert_allclose(np_of(pool.acc), acc_sep, rtol=1e-5, atol=1e-6)
+    # against the numpy restatement as well
+    for c, L in enumerate(lens):
+        if L:
+            rows = ref.valid_rows(c)
+            _, imp = O.h2o_importance(np_of(scores)[c, :, :L])
+            want = np_of(acc0)[rows] * np.float32(decay) + imp
+            np.testing.assert_allclose(np_of(pool.acc)[rows], want, rtol=1e-3, atol=1e-5)
+            assert (np_of(pool.ts)[rows] == 9.0).all()
+
+
 def test_attend_peaked_distribution(dev):
     """One token carries almost all the weight: the output must equal that row of V to
     float32 accuracy, which a bf16-only weight operand would miss by 2^-9."""
