@@ -100,7 +100,7 @@ template <int SCHEME, int REP, int Q_DT>
 __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   using Q = QScheme<SCHEME>;
   constexpr int EPL = Q::epl;
-  __shared__ float stage[kMaxQHeads * kTile];  // [q head of this block][token in tile]
+  extern __shared__ float stage[];  // [q head of this block][token in tile]
 
   const int c = blockIdx.y;
   const int64_t tile = blockIdx.x;
@@ -232,8 +232,9 @@ template <int SCHEME>
 __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
-  __shared__ float stage[kMaxQHeads * kTile];  // [q head][token in tile]
-  __shared__ float qs[kMaxQHeads * 4];         // sum of q over each 32-wide group
+  extern __shared__ float mfma_lds[];
+  float* stage = mfma_lds;                      // [q head][token in tile]
+  float* qs = mfma_lds + a.n_q_heads * kTile;   // sum of q over each 32-wide group
 
   const int c = blockIdx.y;
   const int64_t tile = blockIdx.x;
@@ -695,10 +696,12 @@ static void launch_gather(unsigned blocks, hipStream_t st, const void* codes, co
 
 template <int SCHEME, int REP>
 static void launch_scores_q(dim3 grid, hipStream_t st, int q_dtype, const ScoreArgs& a) {
+  // staged scores of the block's query heads: the fewer, the more blocks share a compute unit
+  const size_t lds = (size_t)(a.n_q_heads / a.head_split) * kTile * sizeof(float);
   if (q_dtype == PIKV_BF16)
-    hipLaunchKernelGGL((scores_kernel<SCHEME, REP, PIKV_BF16>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((scores_kernel<SCHEME, REP, PIKV_BF16>), grid, dim3(256), lds, st, a);
   else
-    hipLaunchKernelGGL((scores_kernel<SCHEME, REP, PIKV_F32>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((scores_kernel<SCHEME, REP, PIKV_F32>), grid, dim3(256), lds, st, a);
 }
 
 template <int SCHEME>
@@ -790,15 +793,16 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   // grouped 4-bit caches read with bf16 queries go to the matrix-core kernel
   if (!eight && group == 32 && head_dim == 128 && q_dtype == PIKV_BF16 && rep <= 16) {
     int grc = PIKV_ERR_UNSUPPORTED;
+    const size_t mlds = (size_t)n_q_heads * (kTile + 4) * sizeof(float);
     if (rep <= 4)
       grc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(a, n_caches, n_tiles, st)
                                        : launch_gqa<PIKV_Q_I4_SYM>(a, n_caches, n_tiles, st);
     if (grc == PIKV_OK) {
       // launched above
     } else if (scheme == PIKV_Q_I4_ASYM) {
-      hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_ASYM>), grid, dim3(256), 0, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_ASYM>), grid, dim3(256), mlds, st, a);
     } else {
-      hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_SYM>), grid, dim3(256), 0, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_SYM>), grid, dim3(256), mlds, st, a);
     }
     PIKV_CHECK_LAUNCH();
     return PIKV_OK;
