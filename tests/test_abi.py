@@ -85,6 +85,18 @@ def test_pure_host_entry_points():
                                   1, 1, ws - 1, None) == -4
 
 
+def test_header_is_plain_c(tmp_path):
+    """include/pikv_hip.h compiles as C99 and as C++ with nothing but <stdint.h>."""
+    import subprocess
+    src = tmp_path / "use.c"
+    src.write_text('#include "pikv_hip.h"\nint main(void) { return pikv_abi_version() > 0 ? 0 : 1; }\n')
+    inc = os.path.join(ROOT, "include")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, "-fsyntax-only", str(src)],
+                   check=True)
+    subprocess.run(["g++", "-std=c++11", "-Wall", "-Werror", "-I", inc, "-fsyntax-only", "-x", "c++", str(src)],
+                   check=True)
+
+
 def test_ops_reject_cpu_tensors():
     """The product path has no CPU fallback."""
     import torch
