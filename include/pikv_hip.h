@@ -368,8 +368,9 @@ int pikv_h2o_budget(const int32_t* cache_fill, int n_caches,
  * order, for up to PIKV_MAX_PLANES planes (codes, scales, zeros, acc, ts ...),
  * then set cache_fill[c] = new_len[c].
  *   plane_ptrs_host  [n_planes] device pointers (the ARRAY itself is on the
- *                    host); plane_row_bytes_host [n_planes] bytes per row,
- *                    each a multiple of 4. */
+ *                    host); plane_row_bytes_host [n_planes] bytes per row
+ *                    (any positive width; rows are moved in the widest units
+ *                    their width is a multiple of, up to 16 bytes). */
 #define PIKV_MAX_PLANES 10
 int pikv_compact_rows(void* const* plane_ptrs_host,
                       const int64_t* plane_row_bytes_host, int n_planes,

@@ -590,10 +590,15 @@ __global__ __launch_bounds__(256) void compact_rows_kernel(CompactPlanes pl,
   const int m = new_len[c];
   const int32_t* keep = keep_index + base;
   char* plane = reinterpret_cast<char*>(pl.ptr[p]);
+  // widest element that every row start is aligned to
   if (rb % 16 == 0)
     compact_slab<uint4>(plane, rb, base, col0, slab_bytes, keep, m);
-  else
+  else if (rb % 4 == 0)
     compact_slab<uint32_t>(plane, rb, base, col0, slab_bytes, keep, m);
+  else if (rb % 2 == 0)
+    compact_slab<uint16_t>(plane, rb, base, col0, slab_bytes, keep, m);
+  else
+    compact_slab<uint8_t>(plane, rb, base, col0, slab_bytes, keep, m);
 }
 
 __global__ void set_fill_kernel(int32_t* __restrict__ fill, const int32_t* __restrict__ new_len, int n) {
@@ -682,7 +687,7 @@ extern "C" int pikv_compact_rows(void* const* plane_ptrs_host, const int64_t* pl
     for (int p = 0; p < n_planes; ++p) {
       if (!plane_ptrs_host[p]) return PIKV_ERR_NULL;
       const int64_t rb = plane_row_bytes_host[p];
-      if (rb <= 0 || rb % 4 != 0 || rb > (1 << 24)) return PIKV_ERR_SHAPE;
+      if (rb <= 0 || rb > (1 << 24)) return PIKV_ERR_SHAPE;
       pl.ptr[p] = plane_ptrs_host[p];
       pl.row_bytes[p] = rb;
       pl.slab_begin[p] = slabs;

@@ -780,7 +780,6 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   if (!is_pow2(head_dim) || head_dim < epl || group % epl != 0) return PIKV_ERR_UNSUPPORTED;
   const int lanes_per_row = D / epl;
   if (lanes_per_row > 256 || 256 % lanes_per_row != 0) return PIKV_ERR_UNSUPPORTED;
-  if (kTile % (256 / lanes_per_row) != 0) return PIKV_ERR_UNSUPPORTED;
   if (n_q_heads > kMaxQHeads) return PIKV_ERR_UNSUPPORTED;
   if (max_len == 0) return PIKV_OK;
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
