@@ -111,3 +111,120 @@ def test_random_shape_chain(dev, seed):
         keeps = [O.h2o_keep(ref.acc[ref.valid_rows(c)], ref.ts[ref.valid_rows(c)], int(nh[c]), int(nr[c]))
                  if L else np.zeros(0, dtype=bool) for c, L in enumerate(lens)]
     _check_compacted(pool, ref, scheme, keeps)
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_shape_router(dev, seed):
+    """Fused gate projection + tail over random T, H (multiples of 8), E <= 64, k <= 8, both
+    dtypes, with and without bias / scaling / mask / capacity."""
+    from pikv_amd import ops
+    r = rng(2000 + seed)
+    T = int(r.integers(1, 700))
+    H = 8 * int(r.integers(1, 200))
+    E = int(r.integers(1, 65))
+    k = int(r.integers(1, min(E, 8) + 1))
+    dtype = "bf16" if seed % 2 else "f32"
+    print(f"seed {seed}: T {T} H {H} E {E} k {k} {dtype}", flush=True)
+    x = r.standard_normal((T, H)).astype(np.float32)
+    w = (r.standard_normal((E, H)) / np.sqrt(H)).astype(np.float32)
+    if dtype == "bf16":
+        x, w = O.bf16_round(x), O.bf16_round(w)
+    b = (0.1 * r.standard_normal(E)).astype(np.float32) if seed % 3 else None
+    kw, okw = {}, {}
+    if seed % 4 == 1:
+        scale = (0.5 + r.random(E)).astype(np.float32)
+        kw.update(temperature=0.8, expert_scale=to_dev(scale, dev))
+        okw.update(temperature=0.8, expert_scale=scale)
+    if seed % 4 == 2:
+        mask = (r.random(E) > 0.3).astype(np.float32)
+        if mask.sum() < k:
+            mask[:] = 1
+        kw.update(expert_mask=to_dev(mask, dev))
+        okw.update(expert_mask=mask)
+    cap = int(r.integers(1, 2 * T + 2)) if seed % 5 else None
+    out = ops.router_fused(to_dev(x, dev, dtype), to_dev(w, dev, dtype), None if b is None else to_dev(b, dev),
+                           top_k=k, capacity=cap, return_logits=True, **kw)
+    lg = (x.astype(np.float64) @ w.astype(np.float64).T + (0 if b is None else b)).astype(np.float32)
+    # the returned logits are the scaled / masked ones (what the softmax sees)
+    if "temperature" in okw:
+        lg = lg / np.float32(okw["temperature"]) * okw["expert_scale"]
+    if "expert_mask" in okw:
+        lg = lg + (np.float32(1) - okw["expert_mask"]) * np.float32(-1e9)
+    assert np.allclose(np_of(out.logits), lg, atol=4e-5 * np.sqrt(H), rtol=1e-5)
+    # everything after the projection is exact arithmetic on the logits the GPU produced
+    probs, idx, wts, _ = O.router_tail(np_of(out.logits), k)
+    assert np.array_equal(np_of(out.topk_idx), idx)
+    assert np.allclose(np_of(out.probs), probs, atol=2e-6, rtol=1e-5)
+    assert np.allclose(np_of(out.topk_w), wts, atol=2e-6, rtol=1e-5)
+    if cap is not None:
+        slot, count = O.capacity_slots(idx, E, cap)
+        assert np.array_equal(np_of(out.slot), slot)
+        assert np.array_equal(np_of(out.count), count)
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_shape_quantize_dequantize(dev, seed):
+    """quantize_rows / dequantize_rows (plain and through a row list) for random widths and groups."""
+    import torch
+    from pikv_amd import ops
+    r = rng(3000 + seed)
+    scheme = int(r.integers(0, 4))
+    four = scheme in (O.Q_I4_ASYM, O.Q_I4_SYM)
+    group = int(r.choice([32, 64, 128, 256, 512, 1024, 2048] if four else [16, 32, 64, 128, 256, 512, 1024]))
+    D = group * int(r.integers(1, 9))
+    n = int(r.integers(1, 400))
+    dtype = "bf16" if seed % 2 else "f32"
+    print(f"seed {seed}: scheme {scheme} D {D} group {group} n {n} {dtype}", flush=True)
+    x = kv_like(r, n, D, dtype=dtype)
+    try:
+        codes, scale, zero = ops.quantize_rows(to_dev(x, dev, dtype), group, scheme)
+    except ValueError as e:      # widths the entry point states it does not take
+        pytest.skip(str(e))
+    q_ref, s_ref, z_ref = O.quantize_groups(x, group, scheme)
+    assert np.array_equal(codes_np(codes, scheme), q_ref)
+    assert np.array_equal(np_of(scale).astype(np.float32), s_ref)
+    if zero is not None:
+        assert np.array_equal(np_of(zero).astype(np.float32), z_ref)
+    dq_ref = O.dequantize_groups(q_ref, s_ref, z_ref, group)
+    assert np.array_equal(np_of(ops.dequantize_rows(codes, scale, zero, group, scheme)), dq_ref, equal_nan=True)
+    rows = r.integers(0, n, size=int(r.integers(1, 50))).astype(np.int64)
+    got = ops.dequantize_rows(codes, scale, zero, group, scheme, out_dtype=torch.bfloat16, rows=to_dev(rows, dev))
+    assert np.array_equal(np_of(got), O.bf16_round(dq_ref[rows]), equal_nan=True)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_shape_select_and_gather(dev, seed):
+    """select_top_rows + quant_gather (the pyramid path) over random segment lengths and budgets."""
+    from pikv_amd import ops
+    r = rng(4000 + seed)
+    L = int(r.integers(1, 7))
+    n = int(r.integers(1, 9000 if seed % 4 == 3 else 300))
+    heads, dh = int(r.choice([1, 2, 4])), int(r.choice([64, 128]))
+    D = heads * dh
+    scheme = int(r.integers(0, 4))
+    group = dh if scheme in (O.Q_I8_SYM, O.Q_I8_ASYM) else 32
+    lens = np.array([int(r.integers(0, n + 1)) for _ in range(L)], dtype=np.int32)
+    keep = np.array([int(r.integers(0, l + 2)) for l in lens], dtype=np.int32)
+    print(f"seed {seed}: L {L} n {n} D {D} scheme {scheme} lens {lens} keep {keep}", flush=True)
+    sc = (np.round(r.random((L, n)) * 16) / 16).astype(np.float32)
+    seg_base = np.arange(L, dtype=np.int64) * n
+    flag, index, kept = ops.select_top_rows(to_dev(sc.reshape(-1), dev), to_dev(seg_base, dev), to_dev(lens, dev),
+                                            to_dev(keep, dev), max_len=n)
+    want_kept = np.minimum(keep, lens)
+    assert np.array_equal(np_of(kept), want_kept)
+    ks, vs = kv_like(r, L * n, D, dtype="bf16"), kv_like(r, L * n, D, dtype="bf16")
+    caps = [int(max(1, k_ - (1 if seed % 2 else 0))) for k_ in want_kept]     # some caches one row short
+    pool = ops.CachePool(caps, heads, dh, group, scheme, dev, with_v=True)
+    pool.quant_gather(to_dev(ks, dev, "bf16"), to_dev(vs, dev, "bf16"), to_dev(seg_base, dev), index, kept,
+                      int(n), src_score=to_dev(sc.reshape(-1), dev), now=2.0)
+    base = np_of(pool.row_base)
+    for l in range(L):
+        want = np.nonzero(O.h2o_keep(sc[l, :lens[l]], sc[l, :lens[l]], int(keep[l]), 0))[0]
+        assert np.array_equal(np_of(index)[l * n:l * n + want.size], want), l
+        m = min(want.size, caps[l])
+        rows = slice(int(base[l]), int(base[l]) + m)
+        for src, codes, scale in ((ks, pool.k_codes, pool.k_scale), (vs, pool.v_codes, pool.v_scale)):
+            q, s, _ = O.quantize_groups(src[l * n + want[:m]], group, scheme)
+            assert np.array_equal(codes_np(codes, scheme)[rows], q), l
+            assert np.array_equal(np_of(scale)[rows].astype(np.float32), s), l
+        assert np.array_equal(np_of(pool.acc)[rows], sc[l, want[:m]])
