@@ -61,68 +61,106 @@ __device__ __forceinline__ float wave_transpose_reduce(float (&v)[64], int lane)
 
 // Lane holds the raw logit of (token t, expert e); groups of EPAD adjacent lanes
 // form one token.  Writes probs / top-k for the token.
-template <int EPAD>
-__device__ __forceinline__ void router_tail_lanes(float lg, int64_t t, int e, int lane,
+// NTOK independent token groups go through the steps side by side: every step is a
+// chain of dependent cross-lane operations, and the chains of different tokens fill each
+// other's wait states.
+template <int EPAD, int NTOK>
+__device__ __forceinline__ void router_tail_multi(float (&lg)[NTOK], const int64_t (&t)[NTOK], int e, int lane,
                                                   const TailParams& p) {
-  const bool valid = (t < p.T) && (e < p.E);
-  if (valid) {
-    if (p.bias) lg = lg + p.bias[e];
-    if (p.temperature != 1.0f) lg = lg / p.temperature;
-    if (p.expert_scale) lg = lg * p.expert_scale[e];
-    if (p.expert_mask) {
-      const float pen = (1.0f - p.expert_mask[e]) * -1e9f;
-      lg = lg + pen;
+  bool valid[NTOK];
+#pragma unroll
+  for (int n = 0; n < NTOK; ++n) {
+    valid[n] = (t[n] < p.T) && (e < p.E);
+    if (valid[n]) {
+      if (p.bias) lg[n] = lg[n] + p.bias[e];
+      if (p.temperature != 1.0f) lg[n] = lg[n] / p.temperature;
+      if (p.expert_scale) lg[n] = lg[n] * p.expert_scale[e];
+      if (p.expert_mask) {
+        const float pen = (1.0f - p.expert_mask[e]) * -1e9f;
+        lg[n] = lg[n] + pen;
+      }
+      if (p.logits_out) p.logits_out[t[n] * p.E + e] = lg[n];
+    } else {
+      lg[n] = -__builtin_inff();
     }
-    if (p.logits_out) p.logits_out[t * p.E + e] = lg;
-  } else {
-    lg = -__builtin_inff();
   }
-  float prob = 0.f;
+  float carried[NTOK];
+#pragma unroll
+  for (int n = 0; n < NTOK; ++n) carried[n] = lg[n];
   if (p.use_softmax) {
-    const float m = group_max_dpp(lg, EPAD);
-    const float ex = valid ? expf(lg - m) : 0.f;
-    const float sum = group_sum_dpp(ex, EPAD);
-    prob = ex / sum;
-    if (valid && p.probs) p.probs[t * p.E + e] = prob;
+    float m[NTOK], ex[NTOK], sum[NTOK];
+#pragma unroll
+    for (int n = 0; n < NTOK; ++n) m[n] = group_max_dpp(lg[n], EPAD);
+#pragma unroll
+    for (int n = 0; n < NTOK; ++n) ex[n] = valid[n] ? expf(lg[n] - m[n]) : 0.f;
+#pragma unroll
+    for (int n = 0; n < NTOK; ++n) sum[n] = group_sum_dpp(ex[n], EPAD);
+#pragma unroll
+    for (int n = 0; n < NTOK; ++n) {
+      carried[n] = ex[n] / sum[n];
+      if (valid[n] && p.probs) p.probs[t[n] * p.E + e] = carried[n];
+    }
   }
-  const float carried = p.use_softmax ? prob : lg;
 
   const int gstart = lane & ~(EPAD - 1);
   const uint64_t gmask = (EPAD == 64) ? ~0ull : (((1ull << EPAD) - 1ull) << gstart);
-  bool remaining = valid;
-  int my_idx = 0;
-  float my_val = 0.f;
-  float wsum = 0.f;  // sum of the selected values, in selection order
+  bool remaining[NTOK];
+  int my_idx[NTOK];
+  float my_val[NTOK], wsum[NTOK];  // wsum: sum of the selected values, in selection order
+#pragma unroll
+  for (int n = 0; n < NTOK; ++n) {
+    remaining[n] = valid[n];
+    my_idx[n] = 0;
+    my_val[n] = 0.f;
+    wsum[n] = 0.f;
+  }
   for (int j = 0; j < p.k; ++j) {
-    const float key = remaining ? lg : -__builtin_inff();
-    const float mx = group_max_dpp(key, EPAD);
-    uint64_t cand = __ballot(remaining && key == mx) & gmask;
-    if (cand == 0) cand = __ballot(remaining) & gmask;  // only NaNs left
-    int win = e;  // padding tokens (no candidates at all) stay harmless
-    if (cand != 0) win = (int)__builtin_ctzll(cand) - gstart;
-    float wv;
-    if constexpr (EPAD == 64) {
-      // one token per wavefront: the winner is wave-uniform
-      wv = read_lane_f(carried, __builtin_amdgcn_readfirstlane(win));
-    } else {
-      wv = __shfl(carried, gstart + win, PIKV_WAVE);
+    float key[NTOK], mx[NTOK];
+#pragma unroll
+    for (int n = 0; n < NTOK; ++n) key[n] = remaining[n] ? lg[n] : -__builtin_inff();
+#pragma unroll
+    for (int n = 0; n < NTOK; ++n) mx[n] = group_max_dpp(key[n], EPAD);
+#pragma unroll
+    for (int n = 0; n < NTOK; ++n) {
+      uint64_t cand = __ballot(remaining[n] && key[n] == mx[n]) & gmask;
+      if (cand == 0) cand = __ballot(remaining[n]) & gmask;  // only NaNs left
+      int win = e;  // padding tokens (no candidates at all) stay harmless
+      if (cand != 0) win = (int)__builtin_ctzll(cand) - gstart;
+      float wv;
+      if constexpr (EPAD == 64) {
+        // one token per wavefront: the winner is wave-uniform
+        wv = read_lane_f(carried[n], __builtin_amdgcn_readfirstlane(win));
+      } else {
+        wv = __shfl(carried[n], gstart + win, PIKV_WAVE);
+      }
+      wsum[n] = wsum[n] + wv;
+      if (e == j) {
+        my_idx[n] = win;
+        my_val[n] = wv;
+      }
+      if (e == win) remaining[n] = false;
     }
-    wsum = wsum + wv;
-    if (e == j) {
-      my_idx = win;
-      my_val = wv;
+  }
+#pragma unroll
+  for (int n = 0; n < NTOK; ++n) {
+    if (p.use_softmax) {
+      float sden = wsum[n];
+      if (p.renorm_eps != 0.f) sden = sden + p.renorm_eps;
+      my_val[n] = my_val[n] / sden;
     }
-    if (e == win) remaining = false;
+    if (t[n] < p.T && e < p.k) {
+      p.topk_idx[t[n] * p.k + e] = my_idx[n];
+      p.topk_w[t[n] * p.k + e] = my_val[n];
+    }
   }
-  if (p.use_softmax) {
-    float s = wsum;
-    if (p.renorm_eps != 0.f) s = s + p.renorm_eps;
-    my_val = my_val / s;
-  }
-  if (t < p.T && e < p.k) {
-    p.topk_idx[t * p.k + e] = my_idx;
-    p.topk_w[t * p.k + e] = my_val;
-  }
+}
+
+template <int EPAD>
+__device__ __forceinline__ void router_tail_lanes(float lg, int64_t t, int e, int lane,
+                                                  const TailParams& p) {
+  float lgs[1] = {lg};
+  const int64_t ts[1] = {t};
+  router_tail_multi<EPAD, 1>(lgs, ts, e, lane, p);
 }
 
 template <int EPAD, int DT>
@@ -223,11 +261,15 @@ __global__ __launch_bounds__(256) void gate_weight_relayout_kernel(const uint16_
 
 // NT 16-expert tiles (1, 2 or 4) x MT 16-token tiles per block; WAVES wavefronts share the k-steps
 template <int NT, int MT, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void router_gate_mfma_kernel(
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2))) void router_gate_mfma_kernel(
     const void* __restrict__ x, const void* __restrict__ wb, int H, TailParams p) {
   constexpr int EP = 16 * NT;
   constexpr int TB = 16 * MT;  // tokens per block
-  __shared__ float red[WAVES][TB][EP];
+  // Partial sums of the wavefronts: one slab each, or - when those would not leave room
+  // for two blocks per compute unit - a single slab that the wavefronts add to in turn
+  // (same order of additions either way).
+  constexpr bool SEQ = WAVES * TB * EP * 4 > 32 * 1024;
+  __shared__ float red[SEQ ? 1 : WAVES][TB][EP];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int64_t tok0 = (int64_t)blockIdx.x * TB;
@@ -250,7 +292,7 @@ __global__ __launch_bounds__(WAVES * 64) void router_gate_mfma_kernel(
 
   // the k-steps are dealt round-robin to the wavefronts; each keeps UN steps in flight
   const int steps = H / 32;
-  constexpr int UN = (MT + NT > 4) ? 2 : 4;
+  constexpr int UN = (MT >= 8) ? 1 : (MT + NT > 4) ? 2 : 4;  // registers: 2 wavefronts per SIMD must fit
   for (int st0 = wave; st0 < steps; st0 += WAVES * UN) {
     uint4 av[UN][MT], bv[UN][NT];
 #pragma unroll
@@ -275,30 +317,56 @@ __global__ __launch_bounds__(WAVES * 64) void router_gate_mfma_kernel(
               acc[mt][t], 0, 0, 0);
   }
   // C layout: lane holds rows 4*(lane/16)+i, column lane%16 of each tile.
+  if constexpr (SEQ) {
+    for (int w2 = 0; w2 < WAVES; ++w2) {
+      if (wave == w2) {
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+          for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) red[wave][mt * 16 + 4 * kg + i][t * 16 + m] = acc[mt][t][i];
-  __syncthreads();
+            for (int i = 0; i < 4; ++i) {
+              float* cell = &red[0][mt * 16 + 4 * kg + i][t * 16 + m];
+              *cell = (w2 == 0 ? 0.f : *cell) + acc[mt][t][i];
+            }
+      }
+      __syncthreads();
+    }
+  } else {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[wave][mt * 16 + 4 * kg + i][t * 16 + m] = acc[mt][t][i];
+    __syncthreads();
+  }
   // Wavefront w finishes tokens TW*w .. TW*w+TW-1: lane -> (token, expert) with the
   // experts of a token in EP adjacent lanes, as the tail expects.
   constexpr int TW = TB / WAVES;  // tokens finished by one wavefront
   constexpr int TPC = 64 / EP;         // tokens per tail call
+  constexpr int CALLS = (TW + TPC - 1) / TPC;
+  constexpr int NTOK = CALLS >= 4 ? 4 : CALLS >= 2 ? 2 : 1;  // token groups finished side by side
+  static_assert(CALLS % NTOK == 0, "calls come in whole bundles");
 #pragma unroll
-  for (int c = 0; c < (TW + TPC - 1) / TPC; ++c) {
-    const int tw = c * TPC + lane / EP;
-    const int tl = TW * wave + tw;
+  for (int c0 = 0; c0 < CALLS; c0 += NTOK) {
+    float lg[NTOK];
+    int64_t tt[NTOK];
     const int e = lane % EP;
-    const bool in_range = tw < TW;
-    float lg = 0.f;
-    if (in_range) {
 #pragma unroll
-      for (int w2 = 0; w2 < WAVES; ++w2) lg += red[w2][tl][e];
+    for (int n = 0; n < NTOK; ++n) {
+      const int tw = (c0 + n) * TPC + lane / EP;
+      const int tl = TW * wave + tw;
+      const bool in_range = tw < TW;
+      lg[n] = 0.f;
+      if (in_range) {
+#pragma unroll
+        for (int w2 = 0; w2 < (SEQ ? 1 : WAVES); ++w2) lg[n] += red[w2][tl][e];
+      }
+      // lanes beyond this wavefront's tokens present an out-of-range token
+      tt[n] = in_range ? tok0 + tl : p.T;
     }
-    // lanes beyond this wavefront's tokens present an out-of-range token
-    router_tail_lanes<EP>(lg, in_range ? tok0 + tl : p.T, e, lane, p);
+    router_tail_multi<EP, NTOK>(lg, tt, e, lane, p);
   }
 }
 
@@ -510,7 +578,12 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
       const int64_t mb = (T + 63) / 64;
       if (mb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
       const dim3 grid((unsigned)mb);
-      if (ep == 16)
+      if (ep == 64 && T >= 32768)
+        // enough tokens to fill the chip with 128-token blocks: the weights are re-read
+        // from L2 once per block, so twice the tokens per block halves that traffic
+        hipLaunchKernelGGL((router_gate_mfma_kernel<4, 8, 4>), dim3((unsigned)((T + 127) / 128)), dim3(256), 0, st,
+                           x, wb, H, p);
+      else if (ep == 16)
         hipLaunchKernelGGL((router_gate_mfma_kernel<1, 4, 8>), grid, dim3(512), 0, st, x, wb, H, p);
       else if (ep == 32)
         hipLaunchKernelGGL((router_gate_mfma_kernel<2, 4, 4>), grid, dim3(256), 0, st, x, wb, H, p);
