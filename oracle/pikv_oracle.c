@@ -178,6 +178,11 @@ static void quant_domain(const float* x, int g, int scheme, int* q, float* scale
   if (bits == 4) {
     scale = half_to_f32(f32_to_half_sat(scale));
     if (scale == 0.0f) scale = 5.9604644775390625e-08f; /* 2^-24 */
+    if (!sym && fabsf(mn) > 2032.0f * scale) {
+      /* the half-precision zero point must stay an exact integer: widen the scale */
+      scale = half_to_f32(f32_to_half_sat(fabsf(mn) / 2032.0f));
+      if (scale == 0.0f) scale = 5.9604644775390625e-08f;
+    }
   }
   if (sym) zero = 0.f;
   else {

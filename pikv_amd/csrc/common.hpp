@@ -143,6 +143,16 @@ __device__ __forceinline__ void quant_params(float mn, float mx, float& scale, f
     // positive half (2^-24) so that encoder and decoder never divide by zero
     scale = (float)float_to_half_sat(scale);
     if (scale == 0.0f) scale = 5.9604644775390625e-08f;
+    if constexpr (!Q::sym) {
+      // The zero point is stored as half as well and must stay an integer that half
+      // holds exactly (|zero| <= 2048).  A group whose spread is tiny next to its offset
+      // (a constant non-zero group, with the 1e-5 range above) would need a far larger
+      // one: its scale is widened until the zero point fits.  Error <= |min| / 4064.
+      if (fabsf(mn) > 2032.0f * scale) {
+        scale = (float)float_to_half_sat(fabsf(mn) / 2032.0f);
+        if (scale == 0.0f) scale = 5.9604644775390625e-08f;
+      }
+    }
   }
   if constexpr (Q::sym) {
     zero = 0.0f;

@@ -26,6 +26,9 @@ def _edge_rows(D):
     rows.append(np.full(D, 1e-30)); rows[-1][0] = -1e-30
     rows.append(np.linspace(1e4, 3e4, D))
     rows.append(-np.abs(np.linspace(0.1, 5.0, D)))
+    # spread tiny next to the offset: the 4-bit zero point would not fit half precision
+    rows += [np.full(D, 1.0), np.full(D, 1000.0), 1.0 + 1e-4 * np.linspace(0, 1, D), -200.0 - 1e-3 * np.arange(D) / D,
+             np.full(D, 0.04)]
     return np.stack(rows).astype(np.float32)
 
 
