@@ -65,9 +65,9 @@ extern "C" {
 #define PIKV_Q_I4_ASYM   2   /* codes 0..15,     half scale + half zero      */
 #define PIKV_Q_I4_SYM    3   /* codes -8..7,     half scale                  */
 /* 4-bit metadata is rounded to half BEFORE the codes are computed, so encoder and
- * decoders share the same two numbers.  PIKV_Q_I4_ASYM only: when |min| > 2032*scale
+ * decoders share the same two numbers.  PIKV_Q_I4_ASYM only: when |min| > 1024*scale
  * (a spread that is tiny next to the offset, e.g. a constant group) the scale becomes
- * half(|min|/2032), which keeps the zero point an integer that half represents exactly. */
+ * half(|min|/1024), which keeps the zero point an integer that half represents exactly. */
 
 /* ---- eviction policies (core/single/cache_scheduling.py:9-17) ----------- */
 #define PIKV_EVICT_H2O   0

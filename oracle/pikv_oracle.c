@@ -178,9 +178,9 @@ static void quant_domain(const float* x, int g, int scheme, int* q, float* scale
   if (bits == 4) {
     scale = half_to_f32(f32_to_half_sat(scale));
     if (scale == 0.0f) scale = 5.9604644775390625e-08f; /* 2^-24 */
-    if (!sym && fabsf(mn) > 2032.0f * scale) {
+    if (!sym && fabsf(mn) > 1024.0f * scale) {
       /* the half-precision zero point must stay an exact integer: widen the scale */
-      scale = half_to_f32(f32_to_half_sat(fabsf(mn) / 2032.0f));
+      scale = half_to_f32(f32_to_half_sat(fabsf(mn) * 0.0009765625f));
       if (scale == 0.0f) scale = 5.9604644775390625e-08f;
     }
   }

@@ -242,8 +242,8 @@ def quant_params(x_min: np.ndarray, x_max: np.ndarray, scheme: int):
     For the 4-bit schemes the stored metadata is float16: the scale is rounded
     to float16 first, and the zero point is computed from that rounded scale
     and itself rounded (saturating) to float16, so that the encoder and every
-    decoder use the same two numbers.  4-bit asymmetric only: when |x_min| > 2032*scale
-    the scale becomes float16(|x_min|/2032), which keeps the zero point an integer that
+    decoder use the same two numbers.  4-bit asymmetric only: when |x_min| > 1024*scale
+    the scale becomes float16(|x_min|/1024), which keeps the zero point an integer that
     float16 represents exactly (a build rule; the reference keeps float32 metadata)."""
     bits, sym, qmin, qmax = scheme_info(scheme)
     x_min = np.asarray(x_min, dtype=F32)
@@ -263,11 +263,11 @@ def quant_params(x_min: np.ndarray, x_max: np.ndarray, scheme: int):
             scale = np.where(scale == 0, F32(2.0 ** -24), scale).astype(F32)
             if not sym:
                 # the zero point is float16 too and must stay an integer float16 holds
-                # exactly (|zero| <= 2048): a group whose spread is tiny next to its offset
+                # exactly (here |zero| <= 1025): a group whose spread is tiny next to its offset
                 # (a constant non-zero group and its 1e-5 range) gets a wider scale
-                wide = _to_half_sat((np.abs(x_min) / F32(2032.0)).astype(F32)).astype(F32)
+                wide = _to_half_sat((np.abs(x_min) * F32(2.0 ** -10)).astype(F32)).astype(F32)
                 wide = np.where(wide == 0, F32(2.0 ** -24), wide).astype(F32)
-                scale = np.where(np.abs(x_min) > (F32(2032.0) * scale).astype(F32), wide, scale).astype(F32)
+                scale = np.where(np.abs(x_min) > (F32(1024.0) * scale).astype(F32), wide, scale).astype(F32)
         if sym:
             zero = np.zeros_like(scale)
         else:

@@ -145,13 +145,15 @@ __device__ __forceinline__ void quant_params(float mn, float mx, float& scale, f
     if (scale == 0.0f) scale = 5.9604644775390625e-08f;
     if constexpr (!Q::sym) {
       // The zero point is stored as half as well and must stay an integer that half
-      // holds exactly (|zero| <= 2048).  A group whose spread is tiny next to its offset
-      // (a constant non-zero group, with the 1e-5 range above) would need a far larger
-      // one: its scale is widened until the zero point fits.  Error <= |min| / 4064.
-      if (fabsf(mn) > 2032.0f * scale) {
-        scale = (float)float_to_half_sat(fabsf(mn) / 2032.0f);
+      // holds exactly.  A group whose spread is tiny next to its offset (a constant
+      // non-zero group, with the 1e-5 range above) would need a far larger one: its
+      // scale is widened to |min| / 1024 (|zero| <= 1025).  Error <= |min| / 2048.
+#ifndef PIKV_AB_NO_WIDEN
+      if (fabsf(mn) > 1024.0f * scale) {
+        scale = (float)float_to_half_sat(fabsf(mn) * 0.0009765625f);
         if (scale == 0.0f) scale = 5.9604644775390625e-08f;
       }
+#endif
     }
   }
   if constexpr (Q::sym) {
