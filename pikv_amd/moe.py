@@ -221,14 +221,14 @@ class PiKVMoE(nn.Module):
         return F.softmax(scores, dim=-1).sum(dim=1)
 
     def _cached_means(self, pool):
-        """Mean dequantised cached value of every expert, [E, H] (zeros when empty)."""
+        """Mean dequantised cached value of every expert, [E, H] (zeros when empty).  Plain
+        masked sums per cache: the result does not depend on scheduling."""
         v = pool.gather_dequant("v")                                   # [rows, H]
-        rows = torch.arange(pool.rows, device=pool.device)
-        owner = torch.bucketize(rows, pool.row_base, right=True) - 1
-        valid = (rows - pool.row_base[owner]) < pool.fill[owner]
-        sums = torch.zeros(pool.n_caches, v.shape[1], device=pool.device)
-        sums.index_add_(0, owner[valid], v[valid])
-        return sums / pool.fill.clamp_min(1).unsqueeze(1).float()
+        means = []
+        for c, (b, cap) in enumerate(zip(pool.base_host, pool.caps_host)):
+            live = (torch.arange(cap, device=pool.device) < pool.fill[c]).unsqueeze(1)
+            means.append((v[b:b + cap] * live).sum(dim=0))
+        return torch.stack(means) / pool.fill.clamp_min(1).unsqueeze(1).float()
 
     def update_cache(self, expert_idx, key, value, importance):
         """Single-expert update (core/single/pikv_moe.py:249-261); the forward pass
@@ -324,3 +324,65 @@ class PiKVMoE(nn.Module):
 
     def get_cache_stats(self):
         return {f'expert_{i}': cache.get_cache_stats() for i, cache in enumerate(self.kv_caches)}
+
+    def print_cache_stats(self):
+        """core/single/pikv_moe.py:388-402."""
+        if not self.use_cache_scheduling:
+            print("Cache scheduling is not enabled.")
+            return
+        print("\n===== Cache Scheduling Statistics =====")
+        for expert_name, expert_stats in self.get_cache_stats().items():
+            print(f"\n{expert_name.upper()}:")
+            for stat_name, value in expert_stats.items():
+                print(f"  {stat_name}: {value:.4f}" if isinstance(value, float) else f"  {stat_name}: {value}")
+        print("\n======================================")
+
+    # ---- distillation (core/single/pikv_moe.py:404-454): outside the cache data path ----
+    def enable_distillation(self, teacher_model_path=None):
+        raise NotImplementedError("knowledge distillation is not part of the cache data path")
+
+    def disable_distillation(self):
+        self.use_distillation = False
+
+    def load_teacher_model(self, model_path):
+        raise NotImplementedError("knowledge distillation is not part of the cache data path")
+
+    def distillation_step(self, input_data, targets=None, optimizer=None):
+        raise NotImplementedError("knowledge distillation is not part of the cache data path")
+
+    # ---- checkpoint (core/single/pikv_moe.py:456-505) -----------------------------------
+    def save_checkpoint(self, path):
+        """The reference stores the module weights, the write pointers and one MEAN vector
+        per expert cache (get_all).  Here 'kv_pool' holds the caches themselves - codes,
+        scales, zero points, accumulators, timestamps and fill of the shared pool - so a
+        resumed model continues with the very rows it had; 'kv_caches' keeps the
+        reference's mean vectors for readers of that key.  Tensors and plain values only:
+        the file loads with torch.load(weights_only=True)."""
+        checkpoint = {
+            'model_state_dict': self.state_dict(),
+            'cache_ptrs': self.cache_ptrs,
+            'kv_caches': [cache.get_all() for cache in self.kv_caches],
+            'kv_pool': None if self.pool is None else self.pool.state_dict(),
+            'clock': self.clock,
+            'use_distillation': False,
+            'use_cache_scheduling': self.use_cache_scheduling,
+            'cache_scheduling_policy': self.cache_scheduling_policy.value if self.use_cache_scheduling else None,
+        }
+        if self.use_cache_scheduling:
+            checkpoint['cache_stats'] = self.get_cache_stats()
+        torch.save(checkpoint, path)
+
+    def load_checkpoint(self, path):
+        checkpoint = torch.load(path, weights_only=True)
+        self.load_state_dict(checkpoint['model_state_dict'])
+        self.cache_ptrs.copy_(checkpoint['cache_ptrs'])
+        self.clock = int(checkpoint.get('clock', 0))
+        if checkpoint.get('kv_pool') is not None:
+            device = self.cache_ptrs.device
+            self._ensure_pool(device).load_state_dict(checkpoint['kv_pool'])
+        if checkpoint.get('use_cache_scheduling', False):
+            policy_name = checkpoint.get('cache_scheduling_policy', 'none')
+            try:
+                self.enable_cache_scheduling(SchedulingPolicy(policy_name))
+            except ValueError:
+                print(f"Unknown scheduling policy in checkpoint: {policy_name}")

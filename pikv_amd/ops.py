@@ -370,6 +370,7 @@ class CachePool:
             base.append(run)
             run += c
         self.rows = run
+        self.caps_host, self.base_host = caps, base     # the geometry, for host-side slicing
         dev = self.device
         self.cap = torch.tensor(caps, dtype=torch.int32, device=dev)
         self.row_base = torch.tensor(base, dtype=torch.int64, device=dev)

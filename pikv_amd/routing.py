@@ -8,6 +8,8 @@ capacity slots - runs in the fused HIP router.
   PiKVRouter ........... :380-549  two gates chosen per token by an importance
                                    mask, cache-usage correction factor, 5-tuple
   EPLBRouter ........... :551-735  /temperature then *expert_weights, KL + z loss
+  HierarchicalRouter ... :737-860  group softmax x in-group softmax, top-k of the
+                                   products (the per-group MLPs stay in torch)
 
 The hidden layers of the gate MLPs and the auxiliary losses stay in torch (dense
 GEMMs and scalar reductions); everything after the last hidden activation goes
@@ -247,3 +249,51 @@ class PiKVRouter(AdaptiveRouter):
         if return_compact:
             return out, probs, aux, importance
         return out[0], out[1], probs, aux, importance
+
+
+class HierarchicalRouter(BaseRouter):
+    """core/single/pikv_routing.py:737-860: router_probs[t, e] = softmax(group logits)[group of e]
+    * softmax(logits of e's group router)[e], optionally times the expert mask; the k largest
+    products are renormalised.  The two small softmaxes are torch; the top-k (ties to the lower
+    expert index) and the capacity slots are the native tail on the products.  The reference
+    writes every selected expert to slot 0 of its dense tensors (:838-846, marked "simplified");
+    here the slots follow the token-major capacity rule like every other router."""
+
+    def __init__(self, hidden_size: int, num_experts: int, top_k: int = 2, capacity_factor: float = 1.5,
+                 expert_backend: str = "fairscale", num_groups: int = 4, group_top_k: int = 1):
+        super().__init__(hidden_size, num_experts, top_k, capacity_factor, expert_backend)
+        if num_experts % num_groups:
+            raise ValueError("num_experts must be a multiple of num_groups")
+        self.num_groups = num_groups
+        self.group_top_k = group_top_k
+        self.experts_per_group = num_experts // num_groups
+        self.group_router = nn.Sequential(nn.Linear(hidden_size, hidden_size), nn.ReLU(),
+                                          nn.Linear(hidden_size, num_groups))
+        self.expert_routers = nn.ModuleList([
+            nn.Sequential(nn.Linear(hidden_size, hidden_size // 2), nn.ReLU(),
+                          nn.Linear(hidden_size // 2, self.experts_per_group))
+            for _ in range(num_groups)])
+
+    def router_probs(self, hidden_states: torch.Tensor, expert_mask: Optional[torch.Tensor] = None):
+        group_probs = F.softmax(self.group_router(hidden_states), dim=-1)              # [B,S,G]
+        parts = [group_probs[..., g:g + 1] * F.softmax(r(hidden_states), dim=-1)
+                 for g, r in enumerate(self.expert_routers)]
+        probs = torch.cat(parts, dim=-1)                                                 # [B,S,E]
+        if expert_mask is not None:
+            probs = probs * expert_mask.view(1, 1, -1)
+        return probs
+
+    def forward(self, hidden_states: torch.Tensor, expert_mask: Optional[torch.Tensor] = None,
+                return_compact: bool = False):
+        B, S, _ = hidden_states.shape
+        probs = self.router_probs(hidden_states, expert_mask)
+        flat = probs.detach().reshape(B * S, self.num_experts).float().contiguous()
+        r = ops.router_tail(flat, top_k=self.top_k, capacity=self._compute_capacity(B, S), use_softmax=False)
+        r.topk_w = r.topk_w / r.topk_w.sum(dim=-1, keepdim=True)
+        r.probs = flat
+        p = probs.mean(dim=[0, 1])
+        aux = torch.sum(p * torch.log(p * self.num_experts + 1e-9))
+        if return_compact:
+            return r, probs, aux
+        disp, comb = _dense_dispatch_combine(r, B, S, self.num_experts, r.capacity)
+        return disp, comb, probs, aux

@@ -96,6 +96,41 @@ def test_eplb_and_pikv_router(dev):
     assert int(p.update_counter) == 1
 
 
+def test_hierarchical_router(dev):
+    """core/single/pikv_routing.py:737-860: probabilities as the reference forms them (torch
+    float64 evaluation of the same graph), top-k of the products with ties to the lower index,
+    renormalised weights, token-major capacity slots, dense tensors of the reference's shape."""
+    import torch
+    from pikv_amd.routing import HierarchicalRouter
+    torch.manual_seed(3)
+    B, S, H, E, k = 2, 48, 128, 16, 2
+    r = HierarchicalRouter(H, E, top_k=k, capacity_factor=1.5, num_groups=4).to(dev)
+    x = torch.randn(B, S, H, device=dev)
+    mask = torch.ones(E, device=dev)
+    mask[5] = 0
+    disp, comb, probs, aux = r(x, expert_mask=mask)
+    cap = O.compute_capacity(B, S, 1.5, k, E)
+    assert disp.shape == (B, S, E, cap) and comb.shape == disp.shape and probs.shape == (B, S, E)
+    r64 = HierarchicalRouter(H, E, top_k=k, num_groups=4).double()
+    r64.load_state_dict({n: v.double().cpu() for n, v in r.state_dict().items()})
+    want = r64.router_probs(x.double().cpu(), mask.double().cpu()).detach().numpy()
+    assert np.allclose(np_of(probs), want, atol=1e-6)
+    assert (np_of(probs)[..., 5] == 0).all()
+    out, _, _ = r(x, expert_mask=mask, return_compact=True)
+    p = np_of(out.probs)
+    idx = O.topk_desc(p, k)
+    assert np.array_equal(np_of(out.topk_idx), idx)
+    vals = np.take_along_axis(p, idx.astype(np.int64), 1)
+    assert np.allclose(np_of(out.topk_w), vals / vals.sum(1, keepdims=True), rtol=1e-6)
+    slot, count = O.capacity_slots(idx, E, cap)
+    assert np.array_equal(np_of(out.slot), slot) and np.array_equal(np_of(out.count), count)
+    # the dense tensors carry exactly the kept assignments
+    assert int(disp.sum().item()) == int((slot >= 0).sum())
+    assert np.isclose(float(comb.sum().item()), float(np_of(out.topk_w)[slot >= 0].sum()), rtol=1e-5)
+    p_mean = want.mean(axis=(0, 1))
+    assert np.isclose(float(aux.detach()), float((p_mean * np.log(p_mean * E + 1e-9)).sum()), atol=1e-5)
+
+
 def test_quantized_compressor(dev):
     import torch
     from pikv_amd.compression import QuantizedCompressor

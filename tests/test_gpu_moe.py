@@ -174,3 +174,37 @@ def test_kvcache_standalone(dev, small_config):
         assert np.array_equal(np_of(cache.pool.v_codes)[rows], ref.v_codes[rows])
         want = O.dequantize_groups(ref.v_codes[rows], ref.v_scale[rows], ref.v_zero[rows], 256).mean(0)
         assert np.allclose(np_of(cache.get_all()), want, rtol=1e-5, atol=1e-6)
+
+
+def test_pikvmoe_checkpoint_resumes_caches(dev, small_config, tmp_path, capsys):
+    """save_checkpoint / load_checkpoint (core/single/pikv_moe.py:456-505): a fresh model that
+    loads the file holds the same quantised rows and continues with identical outputs."""
+    import torch
+    from pikv_amd import moe
+    from pikv_amd.scheduling import SchedulingPolicy
+    torch.manual_seed(1)
+    model = moe.PiKVMoE(use_cache_scheduling=True, cache_scheduling_policy=SchedulingPolicy.H2O).to(dev).eval()
+    ids = [torch.randint(0, 512, (2, 64), device=dev) for _ in range(4)]
+    with torch.no_grad():
+        for x in ids[:3]:
+            model(x)
+    path = str(tmp_path / "moe.pt")
+    model.save_checkpoint(path)
+    torch.manual_seed(2)
+    other = moe.PiKVMoE(use_cache_scheduling=False).to(dev).eval()
+    other.load_checkpoint(path)
+    assert other.use_cache_scheduling and other.cache_scheduling_policy == SchedulingPolicy.H2O
+    assert other.clock == model.clock
+    a, b = model.pool, other.pool
+    assert torch.equal(a.fill, b.fill)
+    base, fill = a.row_base.cpu(), a.fill.cpu()
+    rows = torch.cat([torch.arange(int(base[c]), int(base[c]) + int(fill[c])) for c in range(a.n_caches)]).to(dev)
+    for name in ("k_codes", "v_codes", "k_scale", "v_scale", "acc", "ts"):
+        assert torch.equal(getattr(a, name)[rows], getattr(b, name)[rows]), name
+    with torch.no_grad():
+        assert torch.equal(model(ids[3]), other(ids[3]))
+    assert torch.equal(a.fill, b.fill)
+    other.print_cache_stats()
+    assert "Cache Scheduling Statistics" in capsys.readouterr().out
+    with pytest.raises(NotImplementedError):
+        other.enable_distillation()
