@@ -69,6 +69,15 @@ extern "C" {
  * (a spread that is tiny next to the offset, e.g. a constant group) the scale becomes
  * half(|min|/1024), which keeps the zero point an integer that half represents exactly. */
 
+/* ---- router arithmetic: the reference holds two copies of its routers --------
+ * SINGLE (core/single/pikv_routing.py:653-656, :68-70):  logits / temperature, then
+ *        * expert_scale, mask penalty (1-mask)*-1e9.
+ * MODULE (core/single/module/pikv_routing.py:596-600, :133-134): * expert_scale, then
+ *        / temperature, mask penalty (1-mask)*finfo(float32).min; its renormalisation
+ *        adds 1e-8 to the sum (:143) - pass renorm_eps = 1e-8. */
+#define PIKV_ROUTER_SINGLE 0
+#define PIKV_ROUTER_MODULE 1
+
 /* ---- eviction policies (core/single/cache_scheduling.py:9-17) ----------- */
 #define PIKV_EVICT_H2O   0
 #define PIKV_EVICT_LRU   1
@@ -92,6 +101,7 @@ int pikv_abi_version(void);
  *   logits     /= temperature            (if temperature != 1; true division)
  *   logits     *= expert_scale[e]        (if expert_scale != NULL)
  *   logits     += (1-expert_mask[e])*-1e9 (if expert_mask != NULL)
+ *                 (order and penalty of arithmetic = PIKV_ROUTER_SINGLE; see above)
  *   probs       = softmax_e(logits)
  *   topk_idx    = k largest logits, (value desc, index asc)
  *   topk_w      = probs[topk_idx] / (sum_j probs[topk_idx[j]] + renorm_eps)
@@ -114,7 +124,7 @@ int pikv_abi_version(void);
 int pikv_router_fused(const void* x, const void* w, int x_dtype,
                       const float* bias, const float* expert_scale,
                       const float* expert_mask, float temperature,
-                      float renorm_eps,
+                      float renorm_eps, int arithmetic,
                       int64_t T, int H, int E, int k, int64_t capacity,
                       float* probs, float* logits_out,
                       int32_t* topk_idx, float* topk_w,
@@ -137,6 +147,7 @@ int pikv_router_tail(const float* logits_a, const float* logits_b,
                      const uint8_t* select,
                      const float* expert_scale, const float* expert_mask,
                      float temperature, float renorm_eps, int use_softmax,
+                     int arithmetic,
                      int64_t T, int E, int k, int64_t capacity,
                      float* probs, int32_t* topk_idx, float* topk_w,
                      int32_t* slot, int32_t* count,

@@ -77,18 +77,30 @@ def gate_logits(x: np.ndarray, w: np.ndarray, bias=None) -> np.ndarray:
 
 
 def scale_logits(logits, temperature=1.0, expert_scale=None, expert_mask=None,
-                 logits_b=None, select=None) -> np.ndarray:
+                 logits_b=None, select=None, module_arithmetic=False) -> np.ndarray:
     """Logit post-processing in float32, in the order of
     core/single/pikv_routing.py:
       PiKV  (:450-460)  row-wise choice between two gates by the importance
                         mask, then * cache_correction_factor[e];
       EPLB  (:653-656)  / temperature, then * expert_weights[e];
       mask  (:68-70)    + (1 - mask[e]) * -1e9.
+    module_arithmetic=True follows core/single/module/pikv_routing.py instead:
+    * expert_weights before / temperature (:596-600), penalty finfo(float32).min (:133-134).
     """
     lg = np.asarray(logits, dtype=F32)
     if logits_b is not None and select is not None:
         sel = np.asarray(select).astype(bool)[:, None]
         lg = np.where(sel, lg, np.asarray(logits_b, dtype=F32))
+    if module_arithmetic:
+        if expert_scale is not None:
+            lg = lg * np.asarray(expert_scale, dtype=F32)[None, :]
+        if temperature != 1.0:
+            lg = lg / F32(temperature)
+        if expert_mask is not None:
+            m = np.asarray(expert_mask, dtype=F32)[None, :]
+            with np.errstate(over="ignore"):
+                lg = (lg + (F32(1.0) - m) * np.finfo(F32).min).astype(F32)
+        return lg.astype(F32)
     if temperature != 1.0:
         lg = lg / F32(temperature)
     if expert_scale is not None:
@@ -125,7 +137,7 @@ def topk_asc(v: np.ndarray, k: int) -> np.ndarray:
 
 def router_tail(logits, top_k, temperature=1.0, expert_scale=None,
                 expert_mask=None, logits_b=None, select=None,
-                renorm_eps=0.0, use_softmax=True):
+                renorm_eps=0.0, use_softmax=True, module_arithmetic=False):
     """softmax -> top-k -> renormalise (core/single/pikv_routing.py:73-79;
     the +1e-8 variant is core/single/module/pikv_routing.py:143).
     Returns (probs [T,E] f32, idx [T,k] i32, w [T,k] f32, final logits).
@@ -133,7 +145,7 @@ def router_tail(logits, top_k, temperature=1.0, expert_scale=None,
     torch.topk on the raw logits (core/single/pikv_kernels.py:97): w holds
     the selected logits."""
     lg = scale_logits(logits, temperature, expert_scale, expert_mask,
-                      logits_b, select)
+                      logits_b, select, module_arithmetic)
     k = min(int(top_k), lg.shape[-1])
     idx = topk_desc(lg, k)
     if not use_softmax:

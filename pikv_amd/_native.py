@@ -29,9 +29,9 @@ _p, _i, _l, _f, _d = C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_double
 SIGNATURES = {
     "pikv_status_string": (C.c_char_p, [_i]),
     "pikv_abi_version": (_i, []),
-    "pikv_router_fused": (_i, [_p, _p, _i, _p, _p, _p, _f, _f, _l, _i, _i, _i, _l,
+    "pikv_router_fused": (_i, [_p, _p, _i, _p, _p, _p, _f, _f, _i, _l, _i, _i, _i, _l,
                                _p, _p, _p, _p, _p, _p, _p, _l, _p]),
-    "pikv_router_tail": (_i, [_p, _p, _p, _p, _p, _f, _f, _i, _l, _i, _i, _l,
+    "pikv_router_tail": (_i, [_p, _p, _p, _p, _p, _f, _f, _i, _i, _l, _i, _i, _l,
                               _p, _p, _p, _p, _p, _p, _l, _p]),
     "pikv_capacity_slots": (_i, [_p, _l, _i, _l, _p, _p, _p, _l, _p]),
     "pikv_router_workspace_bytes": (_l, [_l, _i, _i]),

@@ -27,6 +27,7 @@ struct TailParams {
   float temperature;
   float renorm_eps;
   int use_softmax;
+  int arithmetic;  // PIKV_ROUTER_SINGLE | PIKV_ROUTER_MODULE
   int E;
   int k;
   int64_t T;
@@ -73,11 +74,21 @@ __device__ __forceinline__ void router_tail_multi(float (&lg)[NTOK], const int64
     valid[n] = (t[n] < p.T) && (e < p.E);
     if (valid[n]) {
       if (p.bias) lg[n] = lg[n] + p.bias[e];
-      if (p.temperature != 1.0f) lg[n] = lg[n] / p.temperature;
-      if (p.expert_scale) lg[n] = lg[n] * p.expert_scale[e];
-      if (p.expert_mask) {
-        const float pen = (1.0f - p.expert_mask[e]) * -1e9f;
-        lg[n] = lg[n] + pen;
+      if (p.arithmetic == PIKV_ROUTER_MODULE) {
+        // core/single/module/pikv_routing.py:596-600, :133-134
+        if (p.expert_scale) lg[n] = lg[n] * p.expert_scale[e];
+        if (p.temperature != 1.0f) lg[n] = lg[n] / p.temperature;
+        if (p.expert_mask) {
+          const float pen = (1.0f - p.expert_mask[e]) * -3.4028234663852886e38f;  // finfo(float32).min
+          lg[n] = lg[n] + pen;
+        }
+      } else {
+        if (p.temperature != 1.0f) lg[n] = lg[n] / p.temperature;
+        if (p.expert_scale) lg[n] = lg[n] * p.expert_scale[e];
+        if (p.expert_mask) {
+          const float pen = (1.0f - p.expert_mask[e]) * -1e9f;
+          lg[n] = lg[n] + pen;
+        }
       }
       if (p.logits_out) p.logits_out[t[n] * p.E + e] = lg[n];
     } else {
@@ -540,12 +551,13 @@ static int check_router_dims(int64_t T, int E, int k, int64_t capacity) {
 
 extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, const float* bias,
                                  const float* expert_scale, const float* expert_mask,
-                                 float temperature, float renorm_eps, int64_t T, int H, int E,
-                                 int k, int64_t capacity, float* probs, float* logits_out,
+                                 float temperature, float renorm_eps, int arithmetic, int64_t T,
+                                 int H, int E, int k, int64_t capacity, float* probs, float* logits_out,
                                  int32_t* topk_idx, float* topk_w, int32_t* slot, int32_t* count,
                                  void* workspace, int64_t workspace_bytes, void* stream) {
   if (!x || !w || !topk_idx || !topk_w) return PIKV_ERR_NULL;
   if (x_dtype != PIKV_F32 && x_dtype != PIKV_BF16) return PIKV_ERR_UNSUPPORTED;
+  if (arithmetic != PIKV_ROUTER_SINGLE && arithmetic != PIKV_ROUTER_MODULE) return PIKV_ERR_UNSUPPORTED;
   int rc = check_router_dims(T, E, k, capacity);
   if (rc != PIKV_OK) return rc;
   if (H < 8) return PIKV_ERR_SHAPE;
@@ -561,7 +573,7 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
   char* wb = reinterpret_cast<char*>(workspace) + (slot ? slot_ws : 0);
   hipStream_t st = (hipStream_t)stream;
   if (T > 0) {
-    TailParams p{bias, expert_scale, expert_mask, temperature, renorm_eps, 1, E, k, T,
+    TailParams p{bias, expert_scale, expert_mask, temperature, renorm_eps, 1, arithmetic, E, k, T,
                  probs, logits_out, topk_idx, topk_w};
     const int epad = epad_of(E);
     const int64_t tiles = (T + (64 / epad) - 1) / (64 / epad);
@@ -602,11 +614,13 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
 
 extern "C" int pikv_router_tail(const float* logits_a, const float* logits_b, const uint8_t* select,
                                 const float* expert_scale, const float* expert_mask,
-                                float temperature, float renorm_eps, int use_softmax, int64_t T,
-                                int E, int k, int64_t capacity, float* probs, int32_t* topk_idx,
+                                float temperature, float renorm_eps, int use_softmax,
+                                int arithmetic, int64_t T, int E, int k, int64_t capacity,
+                                float* probs, int32_t* topk_idx,
                                 float* topk_w, int32_t* slot, int32_t* count, void* workspace,
                                 int64_t workspace_bytes, void* stream) {
   if (!logits_a || !topk_idx || !topk_w) return PIKV_ERR_NULL;
+  if (arithmetic != PIKV_ROUTER_SINGLE && arithmetic != PIKV_ROUTER_MODULE) return PIKV_ERR_UNSUPPORTED;
   int rc = check_router_dims(T, E, k, capacity);
   if (rc != PIKV_OK) return rc;
   if (slot) {
@@ -616,7 +630,7 @@ extern "C" int pikv_router_tail(const float* logits_a, const float* logits_b, co
   hipStream_t st = (hipStream_t)stream;
   if (T > 0) {
     TailParams p{nullptr, expert_scale, expert_mask, temperature, renorm_eps, use_softmax ? 1 : 0,
-                 E, k, T, use_softmax ? probs : nullptr, nullptr, topk_idx, topk_w};
+                 arithmetic, E, k, T, use_softmax ? probs : nullptr, nullptr, topk_idx, topk_w};
     const int epad = epad_of(E);
     const int64_t tiles = (T + (64 / epad) - 1) / (64 / epad);
     const int64_t blocks = (tiles + 3) / 4;

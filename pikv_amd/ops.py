@@ -150,11 +150,21 @@ def _router_common(T, E, k, capacity, device, want_probs=True, want_logits=False
     return probs, logits, idx, w, slot, count, ws, ws_bytes
 
 
+ROUTER_SINGLE, ROUTER_MODULE = 0, 1
+
+
+def _arith(module_arithmetic: bool) -> int:
+    return ROUTER_MODULE if module_arithmetic else ROUTER_SINGLE
+
+
 def router_fused(x, weight, bias=None, *, top_k=2, capacity=None, expert_scale=None,
                  expert_mask=None, temperature=1.0, renorm_eps=0.0,
-                 return_logits=False) -> RouterOut:
+                 return_logits=False, module_arithmetic=False) -> RouterOut:
     """Gate projection + softmax + top-k + renormalise (+ capacity slots).
-    x [T,H] f32|bf16, weight [E,H] same dtype (nn.Linear layout)."""
+    x [T,H] f32|bf16, weight [E,H] same dtype (nn.Linear layout).
+    module_arithmetic=True: the operation order and mask penalty of the reference's
+    module/ copy (* expert_scale before / temperature, finfo.min instead of -1e9;
+    core/single/module/pikv_routing.py:596-600, :133-134)."""
     x = _need(x, "x", ndim=2)
     weight = _need(weight, "weight", ndim=2)
     if x.dtype != weight.dtype:
@@ -179,7 +189,8 @@ def router_fused(x, weight, bias=None, *, top_k=2, capacity=None, expert_scale=N
             count.zero_()
         return RouterOut(probs, idx, w, slot, count, logits, capacity)
     N.call("pikv_router_fused", _ptr(x), _ptr(weight), dt, _ptr(bias), _ptr(expert_scale),
-           _ptr(expert_mask), float(temperature), float(renorm_eps), T, H, E, top_k,
+           _ptr(expert_mask), float(temperature), float(renorm_eps), _arith(module_arithmetic),
+           T, H, E, top_k,
            int(capacity or 0), _ptr(probs), _ptr(logits), _ptr(idx), _ptr(w), _ptr(slot),
            _ptr(count), _ptr(ws), ws_bytes, _stream())
     return RouterOut(probs, idx, w, slot, count, logits, capacity)
@@ -187,7 +198,7 @@ def router_fused(x, weight, bias=None, *, top_k=2, capacity=None, expert_scale=N
 
 def router_tail(logits, *, top_k=2, capacity=None, logits_b=None, select=None,
                 expert_scale=None, expert_mask=None, temperature=1.0, renorm_eps=0.0,
-                use_softmax=True) -> RouterOut:
+                use_softmax=True, module_arithmetic=False) -> RouterOut:
     """Router tail on precomputed float32 logits [T,E]."""
     logits = _need(logits, "logits", dtype=torch.float32, ndim=2)
     T, E = logits.shape
@@ -211,7 +222,7 @@ def router_tail(logits, *, top_k=2, capacity=None, logits_b=None, select=None,
         return RouterOut(probs, idx, w, slot, count, None, capacity)
     N.call("pikv_router_tail", _ptr(logits), _ptr(logits_b), _ptr(select), _ptr(expert_scale),
            _ptr(expert_mask), float(temperature), float(renorm_eps), int(bool(use_softmax)),
-           T, E, top_k, int(capacity or 0), _ptr(probs), _ptr(idx), _ptr(w), _ptr(slot),
+           _arith(module_arithmetic), T, E, top_k, int(capacity or 0), _ptr(probs), _ptr(idx), _ptr(w), _ptr(slot),
            _ptr(count), _ptr(ws), ws_bytes, _stream())
     return RouterOut(probs, idx, w, slot, count, None, capacity)
 

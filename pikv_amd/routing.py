@@ -66,6 +66,15 @@ def _gate_tail(hidden: torch.Tensor, linear: nn.Linear, **kw) -> ops.RouterOut:
 
 
 class BaseRouter(nn.Module):
+    # The reference has a second copy of its routers (core/single/module/pikv_routing.py) whose
+    # arithmetic differs in three places: * expert weights BEFORE / temperature (:596-600), mask
+    # penalty finfo.min instead of -1e9 (:133-134), and + 1e-8 in the renormalisation (:143).
+    # Set router.module_arithmetic = True to get that copy's numbers.
+    module_arithmetic = False
+
+    def _arith_kw(self):
+        return dict(module_arithmetic=True, renorm_eps=1e-8) if self.module_arithmetic else {}
+
     def __init__(self, hidden_size: int, num_experts: int, top_k: int = 2,
                  capacity_factor: float = 1.5, expert_backend: str = "fairscale"):
         super().__init__()
@@ -92,7 +101,8 @@ class BaseRouter(nn.Module):
         with torch.no_grad():
             h = self._hidden_before_gate(seq, hidden_states.reshape(B * S, H))
         cap = self._compute_capacity(B, S)
-        return _gate_tail(h, seq[-1], top_k=self.top_k, capacity=cap, expert_mask=expert_mask, **scale_kw)
+        return _gate_tail(h, seq[-1], top_k=self.top_k, capacity=cap, expert_mask=expert_mask,
+                          **self._arith_kw(), **scale_kw)
 
     def _aux_loss(self, router_probs: torch.Tensor) -> torch.Tensor:
         p = router_probs.mean(dim=[0, 1])
@@ -171,7 +181,7 @@ class EPLBRouter(BaseRouter):
         r = ops.router_fused(h.contiguous(), seq[-1].weight.detach().to(h.dtype).contiguous(),
                              seq[-1].bias.detach().float(), top_k=self.top_k, capacity=cap,
                              expert_scale=self.expert_weights, expert_mask=expert_mask,
-                             temperature=self.temperature, return_logits=True)
+                             temperature=self.temperature, return_logits=True, **self._arith_kw())
         out, probs = self._finish(r, B, S, return_compact)
         aux = torch.zeros((), device=probs.device)
         usage = r.count.float()
@@ -211,7 +221,7 @@ class AdaptiveRouter(BaseRouter):
         sel = (importance.reshape(-1) > self.imp_threshold)
         cap = self._compute_capacity(B, S)
         return ops.router_tail(la, top_k=self.top_k, capacity=cap, logits_b=lb, select=sel,
-                               expert_scale=expert_scale, expert_mask=expert_mask)
+                               expert_scale=expert_scale, expert_mask=expert_mask, **self._arith_kw())
 
 
 class PiKVRouter(AdaptiveRouter):

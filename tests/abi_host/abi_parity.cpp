@@ -124,7 +124,8 @@ int main() {
   Dev<int32_t> d_idx((size_t)A), d_slot((size_t)A), d_count(E);
   const int64_t ws_bytes = pikv_router_workspace_bytes(T, E, K);
   Dev<uint8_t> d_ws((size_t)ws_bytes);
-  PIKV_CALL(pikv_router_tail(d_logits.p, nullptr, nullptr, nullptr, nullptr, 1.0f, 0.0f, 1, T, E, K, capacity,
+  PIKV_CALL(pikv_router_tail(d_logits.p, nullptr, nullptr, nullptr, nullptr, 1.0f, 0.0f, 1, PIKV_ROUTER_SINGLE, T, E, K,
+                             capacity,
                              d_probs.p, d_idx.p, d_w.p, d_slot.p, d_count.p, d_ws.p, ws_bytes, nullptr));
   HIP_OK(hipDeviceSynchronize());
   expect(d_idx.down() == idx_ref, "router: expert indices (ties to the lower index)");

@@ -62,17 +62,19 @@ def test_pure_host_entry_points():
     assert lib.pikv_quant_scatter(None, None, 0, 1, 1, 128, 128, 0, None, None, None, None, None, 1,
                                   None, None, None, None, None, None, None, None, 0.0, None) == -1
     assert lib.pikv_capacity_slots(1, 10, 100, 5, 1, None, None, 0, None) == -2
-    assert lib.pikv_router_fused(1, 1, 0, None, None, None, 1.0, 0.0, 4, 63, 4, 2, 0,
+    assert lib.pikv_router_fused(1, 1, 0, None, None, None, 1.0, 0.0, 0, 4, 63, 4, 2, 0,
                                  None, None, 1, 1, None, None, None, 0, None) == -3
-    assert lib.pikv_router_fused(1, 1, 7, None, None, None, 1.0, 0.0, 4, 64, 4, 2, 0,
+    assert lib.pikv_router_fused(1, 1, 7, None, None, None, 1.0, 0.0, 0, 4, 64, 4, 2, 0,
                                  None, None, 1, 1, None, None, None, 0, None) == -3
+    assert lib.pikv_router_fused(1, 1, 0, None, None, None, 1.0, 0.0, 5, 4, 64, 4, 2, 0,
+                                 None, None, 1, 1, None, None, None, 0, None) == -3   # unknown arithmetic
     assert lib.pikv_evict_select(9, 1, 1, 1, 1, 1, 1, 1, 64, 1, 1, 1, None, 0, None) == -3
     assert lib.pikv_evict_workspace_bytes(2, 4097) == 2 * (3 * 2 * 2048 + 2 * 2 * 1024 + 2) * 4
     assert lib.pikv_evict_select(0, 1, 1, 1, 1, 1, 1, 2, 10000, 1, 1, 1, 1, 100, None) == -4
     # bf16 router needs its workspace (re-laid gate weights): too small -> workspace status
     need = lib.pikv_router_fused_workspace_bytes(64, 128, 8, 2)
     assert need >= 128 * 16 * 2
-    assert lib.pikv_router_fused(1, 1, 1, None, None, None, 1.0, 0.0, 64, 128, 8, 2, 0,
+    assert lib.pikv_router_fused(1, 1, 1, None, None, None, 1.0, 0.0, 0, 64, 128, 8, 2, 0,
                                  None, None, 1, 1, None, None, 1, 128 * 16 * 2 - 1, None) == -4
     # pyramid gather: NULL index list; attention output: heads must divide, workspace must fit
     assert lib.pikv_quant_gather(1, None, 1, 128, 128, 0, 1, None, 1, 4, None, 1, 1, 1, 1,

@@ -109,6 +109,43 @@ def test_router_fused(dev, dtype, T, H, E, k):
     assert np.array_equal(np_of(out.count), count)
 
 
+def test_router_module_arithmetic(dev):
+    """The arithmetic of the reference's module/ copy (core/single/module/pikv_routing.py:596-600,
+    :133-134, :143): scale before temperature, finfo.min penalty, + 1e-8 in the renormalisation -
+    bit-exact indices against the restatement, on logits chosen so that the order of the two
+    roundings matters for some rows."""
+    from pikv_amd import ops
+    r = rng(77)
+    T, E, k = 3000, 12, 3
+    lg = (r.standard_normal((T, E)) * 3).astype(np.float32)
+    lg[::4, 2] = lg[::4, 7]
+    scale = (0.5 + r.random(E)).astype(np.float32)
+    mask = np.ones(E, dtype=np.float32)
+    mask[[1, 9]] = 0
+    kw = dict(temperature=0.7, expert_scale=scale, expert_mask=mask, renorm_eps=1e-8)
+    out = ops.router_tail(to_dev(lg, dev), top_k=k, capacity=900, temperature=0.7, expert_scale=to_dev(scale, dev),
+                          expert_mask=to_dev(mask, dev), renorm_eps=1e-8, module_arithmetic=True)
+    probs, idx, w, final = O.router_tail(lg, k, module_arithmetic=True, **kw)
+    assert np.array_equal(np_of(out.topk_idx), idx)
+    assert np.allclose(np_of(out.probs), probs, atol=2e-6, rtol=1e-5)
+    assert np.allclose(np_of(out.topk_w), w, atol=2e-6, rtol=1e-5)
+    assert not np.isin(np_of(out.topk_idx), [1, 9]).any()
+    # the two orders really differ in the last bit for some logits
+    other = O.scale_logits(lg, 0.7, scale, None)
+    assert (other != O.scale_logits(lg, 0.7, scale, None, module_arithmetic=True)).any()
+    # fused projection: same flag
+    x = O.bf16_round(r.standard_normal((500, 256)).astype(np.float32))
+    wg = O.bf16_round((0.05 * r.standard_normal((E, 256))).astype(np.float32))
+    out = ops.router_fused(to_dev(x, dev, "bf16"), to_dev(wg, dev, "bf16"), top_k=k, temperature=0.7,
+                           expert_scale=to_dev(scale, dev), expert_mask=to_dev(mask, dev), renorm_eps=1e-8,
+                           module_arithmetic=True, return_logits=True)
+    fin = np_of(out.logits)
+    assert (fin[:, [1, 9]] < -1e38).all()
+    _, idx2, w2, _ = O.router_tail(fin, k, renorm_eps=1e-8)
+    assert np.array_equal(np_of(out.topk_idx), idx2)
+    assert np.allclose(np_of(out.topk_w), w2, atol=2e-6, rtol=1e-5)
+
+
 def test_router_empty_and_errors(dev):
     import torch
     from pikv_amd import ops
