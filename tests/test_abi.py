@@ -87,6 +87,16 @@ def test_pure_host_entry_points():
                                   1, 1, ws - 1, None) == -4
 
 
+def test_integration_stub_matches_header():
+    """The ctypes stub shown to maintainers binds the declared number of arguments."""
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    d = _declared()
+    found = re.findall(r"_lib\.(pikv_\w+)\.argtypes\s*=\s*\[(.*?)\]", doc, flags=re.S)
+    assert found
+    for name, args in found:
+        assert len([a for a in args.split(",") if a.strip()]) == d[name], name
+
+
 def test_header_is_plain_c(tmp_path):
     """include/pikv_hip.h compiles as C99 and as C++ with nothing but <stdint.h>."""
     import subprocess
