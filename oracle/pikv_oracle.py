@@ -23,7 +23,14 @@ Pinning status (what, besides this file, fixes each function's output):
   select / compact ................... brute force on tiny inputs, invariants
   streaming / quest / flexgen / lru+ . hand-computed known answers, brute-force
                                        ranking on tiny inputs
-The reference's own tests hold no golden vectors for any of these.
+  adakv / duo / attend_values ........ hand-computed known answers, float64
+                                       closed forms
+  all of the above ................... property tests (ranges, error bounds, total
+                                       orders, conservation, monotone budgets) and the
+                                       frozen digests of tests/golden
+The reference's own tests hold no golden vectors for any of these.  Parity
+unpinned: none of the functions here; the end-to-end logits of the reference's
+PiKVMoE module graph are not restated in this file.
 """
 from __future__ import annotations
 
