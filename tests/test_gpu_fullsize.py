@@ -230,3 +230,66 @@ def test_pyramid_full(dev):
         assert torch.equal(pool.v_codes[base:base + kl], codes1)
         assert torch.equal(pool.v_scale[base:base + kl], scale1)
         assert torch.equal(pool.acc[base:base + kl], sc[l][sel])
+
+
+def test_planes_beyond_4_gib(dev):
+    """A pool whose second cache starts more than 4 GiB into every code plane and 2^31 score
+    elements away: scatter, dequantise, scores, attention output, H2O, eviction and compaction on
+    that cache (the big first cache is never touched, so the check is cheap) against the numpy
+    restatement of the same small cache - every byte offset has to be 64-bit."""
+    import torch
+    import pikv_oracle as O
+    from util import codes_np, kv_like, np_of, rng, to_dev
+    from pikv_amd import ops
+    heads, dh, group, scheme = 32, 128, 128, ops.Q_I8_SYM
+    D = heads * dh
+    big, small = 1_100_000, 300                       # 1.1 M rows x 4096 B = 4.5 GB per code plane
+    pool = ops.CachePool([big, small], heads, dh, group, scheme, dev, with_v=True)
+    assert int(pool.row_base[1]) * D > (1 << 32)
+    r = rng(12)
+    n = 257
+    ks, vs = kv_like(r, n, D), kv_like(r, n, D)
+    cid = np.full(n, 1, dtype=np.int32)
+    slot = np.arange(n, dtype=np.int32)
+    pool.quant_scatter(to_dev(ks, dev, "bf16"), to_dev(vs, dev, "bf16"), to_dev(cid, dev), to_dev(slot, dev), 1, now=1.0)
+    pool.advance(to_dev(np.array([0, n], dtype=np.int32), dev))
+    ref = O.CachePool([small], D, group, scheme)
+    ref.quant_scatter(ks, vs, np.zeros(n, dtype=np.int32), slot, 1, now=1.0)
+    ref.advance(np.array([n], dtype=np.int32))
+    rows = slice(big, big + n)
+    assert np.array_equal(codes_np(pool.k_codes[rows], scheme), ref.k_codes[:n])
+    assert np.array_equal(codes_np(pool.v_codes[rows], scheme), ref.v_codes[:n])
+    assert np.array_equal(np_of(pool.k_scale[rows]), ref.k_scale[:n])
+    assert not pool.k_codes[big - 1000:big].any() and not pool.k_codes[big + n:].any()
+    dq = pool.gather_dequant("k", row0=big, n=n)
+    assert np.array_equal(np_of(dq), O.dequantize_groups(ref.k_codes[:n], ref.k_scale[:n], ref.k_zero[:n], group))
+    # read path on the far cache (the first cache is empty: fill 0)
+    q = O.bf16_round(r.standard_normal((2, heads, dh)).astype(np.float32))
+    scores, tmax, tsum = pool.scores(to_dev(q, dev, "bf16"), heads, max_len=small)
+    pool.h2o_accumulate(scores, tmax, tsum, now=2.0, stats_only=True)
+    out = np_of(pool.attend_values(scores, pool.head_stats, accumulate=True, now=2.0))
+    k_hat = O.dequantize_groups(ref.k_codes[:n], ref.k_scale[:n], ref.k_zero[:n], group)
+    v_hat = O.dequantize_groups(ref.v_codes[:n], ref.v_scale[:n], ref.v_zero[:n], group)
+    s_ref = O.attention_scores(q[1], k_hat, heads, 1.0 / math.sqrt(dh))
+    rms = np.sqrt((s_ref.astype(np.float64) ** 2).mean())
+    assert np.abs(np_of(scores)[1, :, :n] - s_ref).max() <= 1e-3 * rms
+    p_ref, imp = O.h2o_importance(s_ref)
+    want = O.attend_values(p_ref, v_hat, heads)
+    assert np.abs(out[1] - want).max() <= 2e-3 * np.sqrt((want.astype(np.float64) ** 2).mean())
+    assert not out[0].any()
+    assert np.allclose(np_of(pool.acc[rows]), imp, rtol=1e-3, atol=1e-6)
+    assert bool((pool.ts[rows] == 2.0).all()) and not pool.ts[:big].any()
+    # eviction + compaction of the far cache
+    acc = (np.round(r.random(n) * 8) / 8).astype(np.float32)
+    pool.acc[rows] = to_dev(acc, dev)
+    ts = np_of(pool.ts[rows])
+    nh, nr = np.array([1, 40], dtype=np.int32), np.array([1, 10], dtype=np.int32)
+    pool.evict(ops.EVICT_H2O, n_heavy=to_dev(nh, dev), n_recent=to_dev(nr, dev))
+    keep = O.h2o_keep(acc, ts, 40, 10)
+    m = int(keep.sum())
+    assert np_of(pool.fill).tolist() == [0, m]
+    assert np.array_equal(codes_np(pool.k_codes[big:big + m], scheme), ref.k_codes[:n][keep])
+    assert np.array_equal(np_of(pool.v_scale[big:big + m]), ref.v_scale[:n][keep])
+    assert np.array_equal(np_of(pool.acc[big:big + m]), acc[keep])
+    del pool
+    torch.cuda.empty_cache()
