@@ -4,6 +4,8 @@ restatement.  The shapes are drawn from everything the entry points accept (all 
 schemes, 1-8 kv heads, 1-4 query heads per kv head, head sizes 64/128, every legal
 group, fp32 and bf16 sources and queries, ragged and empty caches), so that indexing
 that only holds for the benchmark shapes shows up here."""
+import os
+
 import numpy as np
 import pytest
 
@@ -12,6 +14,9 @@ from test_gpu_read_evict import _check_compacted
 from util import codes_np, kv_like, np_of, rng, to_dev
 
 pytestmark = pytest.mark.gpu
+
+# number of seeds of the widest sweep (the others scale with it); raise it for a longer soak
+SEEDS = int(os.environ.get("PIKV_SWEEP_SEEDS", "64"))
 
 
 def _draw(r, big):
@@ -31,7 +36,7 @@ def _draw(r, big):
     return scheme, heads, dh, rep, group, caps
 
 
-@pytest.mark.parametrize("seed", range(64))
+@pytest.mark.parametrize("seed", range(SEEDS))
 def test_random_shape_chain(dev, seed):
     from pikv_amd import ops
     r = rng(1000 + seed)
@@ -113,7 +118,7 @@ def test_random_shape_chain(dev, seed):
     _check_compacted(pool, ref, scheme, keeps)
 
 
-@pytest.mark.parametrize("seed", range(32))
+@pytest.mark.parametrize("seed", range(SEEDS // 2))
 def test_random_shape_router(dev, seed):
     """Fused gate projection + tail over random T, H (multiples of 8), E <= 64, k <= 8, both
     dtypes, with and without bias / scaling / mask / capacity."""
@@ -162,7 +167,7 @@ def test_random_shape_router(dev, seed):
         assert np.array_equal(np_of(out.count), count)
 
 
-@pytest.mark.parametrize("seed", range(32))
+@pytest.mark.parametrize("seed", range(SEEDS // 2))
 def test_random_shape_quantize_dequantize(dev, seed):
     """quantize_rows / dequantize_rows (plain and through a row list) for random widths and groups."""
     import torch
@@ -192,7 +197,7 @@ def test_random_shape_quantize_dequantize(dev, seed):
     assert np.array_equal(np_of(got), O.bf16_round(dq_ref[rows]), equal_nan=True)
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(SEEDS // 4))
 def test_random_shape_select_and_gather(dev, seed):
     """select_top_rows + quant_gather (the pyramid path) over random segment lengths and budgets."""
     from pikv_amd import ops
