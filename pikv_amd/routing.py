@@ -57,6 +57,43 @@ def _dense_dispatch_combine(r: ops.RouterOut, batch_size, seq_len, num_experts, 
             comb.view(batch_size, seq_len, num_experts, capacity))
 
 
+def _dense_legacy_fairscale(r: ops.RouterOut, batch_size, seq_len, num_experts, capacity):
+    """Dense tensors the way the fairscale branch of core/single/pikv_routing.py:102-128 fills
+    them: round j of the top-k is handled for all tokens at once, every token of the round that
+    picked expert e lands on position used[e], and used[e] grows by ONE per round however many
+    tokens picked e (an indexed += does not accumulate duplicates).  Small shapes only."""
+    T = batch_size * seq_len
+    dev = r.topk_idx.device
+    disp = torch.zeros(T, num_experts, capacity, device=dev)
+    comb = torch.zeros(T, num_experts, capacity, device=dev)
+    used = torch.zeros(num_experts, dtype=torch.long, device=dev)
+    tok = torch.arange(T, device=dev)
+    for j in range(r.topk_idx.shape[1]):
+        e = r.topk_idx[:, j].long()
+        room = used[e] < capacity
+        e_in, t_in = e[room], tok[room]
+        pos = used[e_in]
+        picked = torch.zeros(num_experts, dtype=torch.bool, device=dev)
+        picked[e_in] = True
+        used = used + picked.long()
+        disp[t_in, e_in, pos] = 1.0
+        comb[t_in, e_in, pos] = r.topk_w[:, j][room]
+    return (disp.view(batch_size, seq_len, num_experts, capacity),
+            comb.view(batch_size, seq_len, num_experts, capacity))
+
+
+def _dense_basic(r: ops.RouterOut, batch_size, seq_len, num_experts):
+    """The non-fairscale branch (core/single/pikv_routing.py:133-153): one position per expert."""
+    T = batch_size * seq_len
+    dev = r.topk_idx.device
+    disp = torch.zeros(T, num_experts, 1, device=dev)
+    comb = torch.zeros(T, num_experts, 1, device=dev)
+    t_idx = torch.arange(T, device=dev).unsqueeze(1).expand_as(r.topk_idx)
+    disp[t_idx, r.topk_idx.long(), 0] = 1.0
+    comb[t_idx, r.topk_idx.long(), 0] = r.topk_w
+    return disp.view(batch_size, seq_len, num_experts, 1), comb.view(batch_size, seq_len, num_experts, 1)
+
+
 def _gate_tail(hidden: torch.Tensor, linear: nn.Linear, **kw) -> ops.RouterOut:
     """hidden [T,H'] (activation before the last Linear) -> fused router."""
     x = hidden.contiguous()
@@ -71,6 +108,10 @@ class BaseRouter(nn.Module):
     # penalty finfo.min instead of -1e9 (:133-134), and + 1e-8 in the renormalisation (:143).
     # Set router.module_arithmetic = True to get that copy's numbers.
     module_arithmetic = False
+    # Dense dispatch/combine tensors follow the token-major capacity rule.  legacy_fairscale = True
+    # reproduces the vectorised fill of core/single/pikv_routing.py:102-128 instead (all tokens of
+    # a round share a position); expert_backend != "fairscale" gives the [B,S,E,1] tensors of :133-153.
+    legacy_fairscale = False
 
     def _arith_kw(self):
         return dict(module_arithmetic=True, renorm_eps=1e-8) if self.module_arithmetic else {}
@@ -112,6 +153,10 @@ class BaseRouter(nn.Module):
         probs = r.probs.view(B, S, self.num_experts)
         if return_compact:
             return r, probs
+        if self.expert_backend != "fairscale":
+            return _dense_basic(r, B, S, self.num_experts), probs
+        if self.legacy_fairscale:
+            return _dense_legacy_fairscale(r, B, S, self.num_experts, r.capacity), probs
         disp, comb = _dense_dispatch_combine(r, B, S, self.num_experts, r.capacity)
         return (disp, comb), probs
 

@@ -96,6 +96,44 @@ def test_eplb_and_pikv_router(dev):
     assert int(p.update_counter) == 1
 
 
+def test_router_legacy_dense_layouts(dev):
+    """legacy_fairscale: the round-wise fill of core/single/pikv_routing.py:102-128 (every token of
+    a round that picked expert e shares position used[e]; used[e] += 1 per round), against a literal
+    loop; expert_backend='basic': [B,S,E,1] tensors (:133-153)."""
+    import torch
+    from pikv_amd.routing import BaseRouter
+    torch.manual_seed(5)
+    B, S, H, E, k = 2, 16, 64, 4, 2
+    r = BaseRouter(H, E, top_k=k, capacity_factor=1.5).to(dev)
+    x = torch.randn(B, S, H, device=dev)
+    out, _, _ = r(x, return_compact=True)
+    idx, w = np_of(out.topk_idx), np_of(out.topk_w)
+    r.legacy_fairscale = True
+    disp, comb, _, _ = r(x)
+    cap = O.compute_capacity(B, S, 1.5, k, E)
+    want_d = np.zeros((B * S, E, cap), np.float32)
+    want_c = np.zeros_like(want_d)
+    used = np.zeros(E, np.int64)
+    for j in range(k):
+        snapshot = used.copy()
+        for t in range(B * S):
+            e = idx[t, j]
+            if snapshot[e] < cap:
+                want_d[t, e, snapshot[e]] = 1.0
+                want_c[t, e, snapshot[e]] = w[t, j]
+        for e in set(idx[:, j][snapshot[idx[:, j]] < cap]):
+            used[e] += 1
+    assert np.array_equal(np_of(disp).reshape(B * S, E, cap), want_d)
+    assert np.array_equal(np_of(comb).reshape(B * S, E, cap), want_c)
+    assert want_d[:, :, 2:].sum() == 0          # two rounds: only positions 0 and 1 are ever used
+    basic = BaseRouter(H, E, top_k=k, expert_backend="basic").to(dev)
+    basic.load_state_dict(r.state_dict())
+    d1, c1, _, _ = basic(x)
+    assert d1.shape == (B, S, E, 1)
+    assert np.array_equal(np_of(d1).reshape(B * S, E).sum(1), np.full(B * S, k, np.float32))
+    assert np.allclose(np_of(c1).reshape(B * S, E).sum(1), 1.0, atol=1e-5)
+
+
 def test_hierarchical_router(dev):
     """core/single/pikv_routing.py:737-860: probabilities as the reference forms them (torch
     float64 evaluation of the same graph), top-k of the products with ties to the lower index,
