@@ -157,12 +157,26 @@ def decode_read_workload(torch, ops, dev, iters):
     t_step = _median_ms(torch, decode_step, iters)
     t_att_acc = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats, accumulate=True, now=1.0), iters)
     pool.fill.fill_(N)
-    t_sel = _median_ms(torch, lambda: pool.evict_select(0, heavy_ratio=1 / 16, recent_ratio=1 / 128), iters)
+
+    # Eviction with a realistic state every time: importance as accumulated above, timestamps =
+    # token positions (the recent rows are the tail).  Without the restore the second call would
+    # find its survivors already compacted at the front and move nothing.
+    acc0 = pool.acc.clone()
+    ts0 = torch.arange(N, device=dev, dtype=torch.float32).repeat(B)
+
+    def restore():
+        pool.fill.fill_(N)
+        pool.acc.copy_(acc0)
+        pool.ts.copy_(ts0)
 
     def evict():
-        pool.fill.fill_(N)
+        restore()
         pool.evict(0, heavy_ratio=1 / 16, recent_ratio=1 / 128)
-    t_evict = _median_ms(torch, evict, iters)
+    t_restore = _median_ms(torch, restore, iters)
+    restore()
+    t_sel = _median_ms(torch, lambda: pool.evict_select(0, heavy_ratio=1 / 16, recent_ratio=1 / 128), iters)
+    t_evict = _median_ms(torch, evict, iters) - t_restore
+    kept_rows = int(pool.fill.sum())
     rows = B * N
     k_bytes = rows * (D // 2 + (D // 32) * 4)
     return {
@@ -180,7 +194,8 @@ def decode_read_workload(torch, ops, dev, iters):
                         "algorithmic_bytes": 2 * k_bytes + 2 * rows * hq * 4 + rows * 12,
                         "GBps": (2 * k_bytes + 2 * rows * hq * 4 + rows * 12) / (t_step * 1e-3) / 1e9},
         "evict_select": _entry(t_sel, rows * 8 + rows * 5),
-        "evict_select_plus_compact": {"ms": t_evict},
+        "evict_select_plus_compact": {"ms": t_evict, "kept_rows": kept_rows,
+                                      "moved_bytes": 2 * kept_rows * (2 * (D // 2 + (D // 32) * 4) + 8)},
     }
 
 

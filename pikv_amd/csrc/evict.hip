@@ -538,10 +538,20 @@ struct CompactPlanes {
 constexpr int kSlabBytes = 256;
 constexpr int kRowsUnroll = 16;
 
-template <typename V>
+// Survivor j of a cache moves from row keep[j] to row j (keep ascending, keep[j] >= j).
+// The m survivors split at j* = first j with keep[j] >= m:
+//   head (j < j*): sources lie inside the final region [0, m) and are themselves
+//     destinations of other survivors, so the moves are ordered - one block walks them in
+//     ascending passes, every pass reads all its rows before it writes any;
+//   tail (j >= j*): sources lie beyond the final region, nobody writes them, and their
+//     destinations [j*, m) are read by the head only - once the head is done they can move
+//     in any order, by as many blocks as there are.
+// After an eviction that keeps a small fraction nearly every survivor is in the tail.
+template <typename V, bool TAIL>
 __device__ __forceinline__ void compact_slab(char* plane, int64_t row_bytes, int64_t base_row,
                                              int64_t col0, int slab_bytes,
-                                             const int32_t* __restrict__ keep, int m) {
+                                             const int32_t* __restrict__ keep, int j_begin, int j_end,
+                                             int chunk, int n_chunks) {
   const int lanes_per_row = slab_bytes / (int)sizeof(V);
   const int rows_per_pass = 256 / lanes_per_row;
   const int lane_in_row = threadIdx.x % lanes_per_row;
@@ -549,7 +559,7 @@ __device__ __forceinline__ void compact_slab(char* plane, int64_t row_bytes, int
   const bool active = row_in_pass < rows_per_pass;  // 256 % lanes_per_row may be non-zero
   const int step_rows = rows_per_pass * kRowsUnroll;
   const int64_t col = col0 + (int64_t)lane_in_row * sizeof(V);
-  for (int j0 = 0; j0 < m; j0 += step_rows) {
+  for (int j0 = j_begin + chunk * step_rows; j0 < j_end; j0 += n_chunks * step_rows) {
     V val[kRowsUnroll];
     int src[kRowsUnroll];
 #pragma unroll
@@ -557,23 +567,25 @@ __device__ __forceinline__ void compact_slab(char* plane, int64_t row_bytes, int
       const int j = j0 + u * rows_per_pass + row_in_pass;
       src[u] = -1;
       val[u] = V{};
-      if (active && j < m) {
+      if (active && j < j_end) {
         const int s = keep[j];
         if (s != j) src[u] = s;
       }
       if (src[u] >= 0)
         val[u] = *reinterpret_cast<const V*>(plane + (base_row + src[u]) * row_bytes + col);
     }
-    __syncthreads();
+    if (!TAIL) __syncthreads();
 #pragma unroll
     for (int u = 0; u < kRowsUnroll; ++u) {
       const int j = j0 + u * rows_per_pass + row_in_pass;
       if (src[u] >= 0) *reinterpret_cast<V*>(plane + (base_row + j) * row_bytes + col) = val[u];
     }
-    __syncthreads();
+    if (!TAIL) __syncthreads();
   }
 }
 
+// grid (slabs of all planes, caches, chunks).  TAIL = false: chunks == 1.
+template <bool TAIL>
 __global__ __launch_bounds__(256) void compact_rows_kernel(CompactPlanes pl,
                                                            const int64_t* __restrict__ row_base,
                                                            const int32_t* __restrict__ keep_index,
@@ -589,16 +601,27 @@ __global__ __launch_bounds__(256) void compact_rows_kernel(CompactPlanes pl,
   const int64_t base = row_base[c];
   const int m = new_len[c];
   const int32_t* keep = keep_index + base;
+  // j* = first survivor whose source lies beyond the final region (binary search, uniform)
+  int lo = 0, hi = m;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (keep[mid] >= m) hi = mid; else lo = mid + 1;
+  }
+  const int j_begin = TAIL ? lo : 0;
+  const int j_end = TAIL ? m : lo;
+  if (j_begin >= j_end) return;  // uniform
   char* plane = reinterpret_cast<char*>(pl.ptr[p]);
+  const int chunk = TAIL ? (int)blockIdx.z : 0;
+  const int n_chunks = TAIL ? (int)gridDim.z : 1;
   // widest element that every row start is aligned to
   if (rb % 16 == 0)
-    compact_slab<uint4>(plane, rb, base, col0, slab_bytes, keep, m);
+    compact_slab<uint4, TAIL>(plane, rb, base, col0, slab_bytes, keep, j_begin, j_end, chunk, n_chunks);
   else if (rb % 4 == 0)
-    compact_slab<uint32_t>(plane, rb, base, col0, slab_bytes, keep, m);
+    compact_slab<uint32_t, TAIL>(plane, rb, base, col0, slab_bytes, keep, j_begin, j_end, chunk, n_chunks);
   else if (rb % 2 == 0)
-    compact_slab<uint16_t>(plane, rb, base, col0, slab_bytes, keep, m);
+    compact_slab<uint16_t, TAIL>(plane, rb, base, col0, slab_bytes, keep, j_begin, j_end, chunk, n_chunks);
   else
-    compact_slab<uint8_t>(plane, rb, base, col0, slab_bytes, keep, m);
+    compact_slab<uint8_t, TAIL>(plane, rb, base, col0, slab_bytes, keep, j_begin, j_end, chunk, n_chunks);
 }
 
 __global__ void set_fill_kernel(int32_t* __restrict__ fill, const int32_t* __restrict__ new_len, int n) {
@@ -694,8 +717,13 @@ extern "C" int pikv_compact_rows(void* const* plane_ptrs_host, const int64_t* pl
       slabs += (int)((rb + kSlabBytes - 1) / kSlabBytes);
     }
     pl.slab_begin[n_planes] = slabs;
-    hipLaunchKernelGGL(compact_rows_kernel, dim3((unsigned)slabs, (unsigned)n_caches), dim3(256), 0,
+    // ordered head first, then the free-moving tail spread over enough blocks to fill the chip
+    hipLaunchKernelGGL(compact_rows_kernel<false>, dim3((unsigned)slabs, (unsigned)n_caches), dim3(256), 0,
                        st, pl, cache_row_base, keep_index, new_len);
+    int64_t chunks = 4096 / ((int64_t)slabs * n_caches);
+    chunks = chunks < 1 ? 1 : (chunks > 64 ? 64 : chunks);
+    hipLaunchKernelGGL(compact_rows_kernel<true>, dim3((unsigned)slabs, (unsigned)n_caches, (unsigned)chunks),
+                       dim3(256), 0, st, pl, cache_row_base, keep_index, new_len);
   }
   if (cache_fill)
     hipLaunchKernelGGL(set_fill_kernel, dim3((n_caches + 63) / 64), dim3(64), 0, st, cache_fill,
