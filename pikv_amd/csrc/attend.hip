@@ -459,6 +459,296 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   }
 }
 
+// ---- matrix-core form, 8-bit codes ------------------------------------------------------
+// Per-head (or coarser) scales, head_dim 128, 2..8 query heads per kv head.  Same plan as
+// the 4-bit kernel - contraction over tokens, codes staged in LDS as stored and read back
+// transposed - with two differences.  An 8-bit code is not exact as one bf16, so a stored
+// byte u is fed as its nibbles, u = 16*hi + lo, each exact as 128 + nibble, against two
+// copies of the weights, w and 16*w (a power of two: exact).  And ds_read_b64_tr_b8 hands
+// result lane i byte q = byte i%8 of source lane 2q + i/8 (per 16 lanes): source lane j
+// therefore points at token T[j/2], dims d0 + 8*(j%2) .. +7, which makes result lane i
+// hold dimension d0 + i of tokens T[0..7] - the B operand layout, tokens in natural order.
+// With nibbles fed as 16 + nibble (0x4180 | nibble << 3):
+//   sum_n w_n*(16 + lo) + 16*w_n*(16 + hi) = sum_n w_n*u_n + 272*sum_n w_n
+// and the value wanted is sum_n w_n*(u_n - zz_n), zz = 128 (symmetric) or the zero point.
+// The offset term is many times the result, and taken off at the end it would cost the
+// float32 sum its low bits over thousands of tokens; a third product per tile, the weights
+// against the constant column -(272 + zz_n), removes it inside the accumulation instead.
+constexpr int kAtt8Tile = 32;    // cached tokens per step
+constexpr int kAtt8ARow = 80;    // bytes per staged A row: 32 tokens x bf16 + 16 (bank spread)
+constexpr int kAtt8PRow = 36;    // floats per query head of staged probabilities: 32 tokens + 4
+
+static size_t attend_mfma8_lds_bytes(int n_kv_heads, int n_q_heads) {
+  // codes [32 tokens][n_kv_heads*128 + 8]; scale and zero term [32][n_kv_heads] float; A rows per
+  // wavefront [2 copies][16 rows][kAtt8ARow]; probabilities [query head][kAtt8PRow]
+  return (size_t)kAtt8Tile * (n_kv_heads * 128 + 8) + 2 * (size_t)kAtt8Tile * n_kv_heads * 4 +
+         4 * (size_t)2 * 16 * kAtt8ARow + (size_t)n_q_heads * kAtt8PRow * 4;
+}
+
+// HKS = log2(n_kv_heads) <= 3; 2..8 query heads per kv head, at most 64 query heads.
+template <int SCHEME, int HKS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i8_kernel(AttendArgs a) {
+  using Q = QScheme<SCHEME>;
+  static_assert(Q::bits == 8, "8-bit schemes only");
+  constexpr int HK = 1 << HKS;
+  constexpr int NH = (HK + 3) / 4;   // kv heads per wavefront
+  constexpr int RS = HK * 128 + 8;   // bytes per token row of staged codes
+  constexpr int LPR = HK * 8;        // 16-byte chunks per cached row
+  constexpr int NCH = kAtt8Tile * LPR / 256;  // code chunks per thread (= HK)
+  extern __shared__ __align__(16) unsigned char att8_lds[];
+  unsigned char* lcodes = att8_lds;
+  float* lscale = reinterpret_cast<float*>(att8_lds + kAtt8Tile * RS);
+  float* lzterm = lscale + kAtt8Tile * HK;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  unsigned char* abuf = reinterpret_cast<unsigned char*>(lzterm + kAtt8Tile * HK) + wave * (2 * 16 * kAtt8ARow);
+  float* lprob = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(lzterm + kAtt8Tile * HK) +
+                                          4 * (2 * 16 * kAtt8ARow));
+
+  const int c = blockIdx.y;
+  const int64_t len = a.fill[c];
+  const int64_t t0 = (int64_t)blockIdx.x * kAttTokensPerBlock;
+  const int64_t t1 = (t0 + kAttTokensPerBlock < len) ? t0 + kAttTokensPerBlock : len;
+  if (t0 >= t1) {  // nothing cached in this range: the partial is zero
+    for (int idx = threadIdx.x; idx < a.n_q_heads * 128; idx += 256)
+      a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * 128 + idx] = 0.f;
+    return;
+  }
+  const int rep = a.n_q_heads / HK;  // 2..8
+  const int groups_per_row = (HK * 128) / a.group;
+  // matrix-core roles: A row / B,C column i, token group kg (tokens 8*kg .. 8*kg+7 of the tile)
+  const int i = lane & 15;
+  const int kg = lane >> 4;
+  // weight-preparation roles: head r of the kv group, tokens t4 .. t4+3 of the tile
+  const int r = lane >> 3;
+  const int t4 = (lane & 7) * 4;
+  const bool row_on = r < rep;
+  const bool normalise = a.head_stats != nullptr;
+  const int64_t base_row = a.row_base[c];
+
+  pikv_f32x4 C[NH][8];
+#pragma unroll
+  for (int hs = 0; hs < NH; ++hs)
+#pragma unroll
+    for (int d = 0; d < 8; ++d) C[hs][d] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
+  // score-staging role: query head sh, tokens st8..st8+7 of the tile (64 heads x 4 runs)
+  const int sh = threadIdx.x >> 2;
+  const int st8 = (threadIdx.x & 3) * 8;
+  const bool s_on = sh < a.n_q_heads;
+  const float* srow = a.scores + ((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * a.score_stride;
+  float smx = 0.f, srz = 1.f;
+  if (normalise) {
+    smx = a.head_stats[((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * 2];
+    srz = 1.0f / a.head_stats[((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * 2 + 1];
+  }
+  const bool s_vec = (a.score_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(a.scores) & 15) == 0;
+  const float s_off = normalise ? -INFINITY : 0.f;  // what a token past the end contributes: p = 0
+  // importance role: wavefront w owns tokens 8w..8w+7 of a tile, eight lanes per token
+  const int it = wave * 8 + (lane & 7);
+  const int igrp = lane >> 3;
+
+  // registers that carry the next tile from HBM to LDS
+  uint4 pc[NCH];
+  float ps = 0.f, pz = 0.f, pacc = 0.f;
+  float psc[8];
+  auto fetch = [&](int64_t n0) {
+    if (a.row_acc && igrp == 0 && n0 + it < t1) pacc = a.row_acc[base_row + n0 + it];
+    if (s_on) {
+      const int64_t n = n0 + st8;
+      if (s_vec && n + 8 <= t1) {
+        const float4 lo4 = *reinterpret_cast<const float4*>(srow + n);
+        const float4 hi4 = *reinterpret_cast<const float4*>(srow + n + 4);
+        psc[0] = lo4.x, psc[1] = lo4.y, psc[2] = lo4.z, psc[3] = lo4.w;
+        psc[4] = hi4.x, psc[5] = hi4.y, psc[6] = hi4.z, psc[7] = hi4.w;
+      } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) psc[k] = n + k < t1 ? srow[n + k] : s_off;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+      const int ch = k * 256 + threadIdx.x;
+      const int tok = ch >> (HKS + 3), off = ch & (LPR - 1);
+      pc[k] = make_uint4(0, 0, 0, 0);
+      if (n0 + tok < t1)
+        pc[k] = ld16(reinterpret_cast<const char*>(a.codes) + ((base_row + n0 + tok) * LPR + off) * 16);
+    }
+    {  // one (token, kv head) metadata pair per thread
+      const int tok = threadIdx.x >> HKS, hd = threadIdx.x & (HK - 1);
+      ps = 0.f;
+      pz = 0.f;
+      if (tok < kAtt8Tile && n0 + tok < t1) {
+        const int64_t mi = (base_row + n0 + tok) * groups_per_row + (hd * 128) / a.group;
+        ps = reinterpret_cast<const float*>(a.scale)[mi];
+        if constexpr (!Q::sym) pz = reinterpret_cast<const float*>(a.zero)[mi];
+      }
+    }
+  };
+  auto stage = [&]() {
+    if (s_on) {
+      float4 v0, v1;
+      v0.x = prob_of(psc[0], smx, srz, normalise), v0.y = prob_of(psc[1], smx, srz, normalise);
+      v0.z = prob_of(psc[2], smx, srz, normalise), v0.w = prob_of(psc[3], smx, srz, normalise);
+      v1.x = prob_of(psc[4], smx, srz, normalise), v1.y = prob_of(psc[5], smx, srz, normalise);
+      v1.z = prob_of(psc[6], smx, srz, normalise), v1.w = prob_of(psc[7], smx, srz, normalise);
+      *reinterpret_cast<float4*>(lprob + sh * kAtt8PRow + st8) = v0;
+      *reinterpret_cast<float4*>(lprob + sh * kAtt8PRow + st8 + 4) = v1;
+    }
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+      const int ch = k * 256 + threadIdx.x;
+      const int tok = ch >> (HKS + 3), off = ch & (LPR - 1);
+      uint2* dst = reinterpret_cast<uint2*>(lcodes + tok * RS + off * 16);  // rows are 8-byte aligned only
+      dst[0] = make_uint2(pc[k].x, pc[k].y);
+      dst[1] = make_uint2(pc[k].z, pc[k].w);
+    }
+    {
+      const int tok = threadIdx.x >> HKS, hd = threadIdx.x & (HK - 1);
+      if (tok < kAtt8Tile) {
+        lscale[tok * HK + hd] = ps;
+        lzterm[tok * HK + hd] = -(272.0f + (Q::sym ? 128.0f : pz));
+      }
+    }
+  };
+  auto bf16_hi = [](float v) { return __float_as_uint(v) & 0xffff0000u; };
+
+  fetch(t0);
+  for (int64_t n0 = t0; n0 < t1; n0 += kAtt8Tile) {
+    __syncthreads();  // the previous tile has been consumed
+    stage();
+    __syncthreads();
+    float acc = pacc;
+    if (n0 + kAtt8Tile < t1) fetch(n0 + kAtt8Tile);  // in flight while this tile is multiplied
+    if (a.row_acc || a.row_ts) {  // uniform
+      const bool mine = igrp == 0 && n0 + it < t1;
+      const int64_t row = base_row + n0 + it;
+      float imp = 0.f;
+      for (int hq = igrp; hq < a.n_q_heads; hq += 8) imp = imp + lprob[hq * kAtt8PRow + it];
+      imp = imp + __shfl_xor(imp, 8, 64);
+      imp = imp + __shfl_xor(imp, 16, 64);
+      imp = imp + __shfl_xor(imp, 32, 64);
+      if (mine) {
+        if (a.row_acc) {
+          if (a.decay != 1.0f) acc = acc * a.decay;
+          a.row_acc[row] = acc + imp;
+        }
+        if (a.row_ts) a.row_ts[row] = a.now;
+      }
+    }
+
+#pragma unroll
+    for (int hs = 0; hs < NH; ++hs) {
+      const int g = wave + 4 * hs;
+      if (g >= HK) continue;  // uniform
+      // ---- weights: head r, tokens t4..t4+3: w = p * scale as bf16 high part + remainder,
+      // both also times 16; the bias sum uses the same two-part value ----
+      const float4 pv = *reinterpret_cast<const float4*>(lprob + (row_on ? g * rep + r : 0) * kAtt8PRow + t4);
+      const float p4[4] = {row_on ? pv.x : 0.f, row_on ? pv.y : 0.f, row_on ? pv.z : 0.f, row_on ? pv.w : 0.f};
+      uint32_t hi[4], lo[4], hi16[4], lo16[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float w = p4[j] * lscale[(t4 + j) * HK + g];
+        const float wh = __uint_as_float(bf16_hi(w));
+        const float wl = __uint_as_float(bf16_hi(w - wh));
+        hi[j] = __float_as_uint(wh) >> 16;
+        lo[j] = __float_as_uint(wl) >> 16;
+        hi16[j] = __float_as_uint(wh * 16.0f) >> 16;
+        lo16[j] = __float_as_uint(wl * 16.0f) >> 16;
+      }
+      if (row_on) {
+        unsigned char* rowp = abuf + (2 * r) * kAtt8ARow + t4 * 2;
+        *reinterpret_cast<uint2*>(rowp) = make_uint2(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16));
+        *reinterpret_cast<uint2*>(rowp + kAtt8ARow) = make_uint2(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16));
+        *reinterpret_cast<uint2*>(rowp + 16 * kAtt8ARow) = make_uint2(hi16[0] | (hi16[1] << 16), hi16[2] | (hi16[3] << 16));
+        *reinterpret_cast<uint2*>(rowp + 17 * kAtt8ARow) = make_uint2(lo16[0] | (lo16[1] << 16), lo16[2] | (lo16[3] << 16));
+      }
+      // the rows were written by other lanes of this wavefront
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      // ---- products: rows 2r / 2r+1 of A against 16 dimensions of 32 tokens ----
+      uint4 a1 = make_uint4(0, 0, 0, 0), a16 = make_uint4(0, 0, 0, 0);
+      if (i < 2 * rep) {
+        a1 = *reinterpret_cast<const uint4*>(abuf + i * kAtt8ARow + kg * 16);
+        a16 = *reinterpret_cast<const uint4*>(abuf + (16 + i) * kAtt8ARow + kg * 16);
+      }
+      // the offset column of tokens 8*kg .. 8*kg+7 (the same for every dimension), as a bf16
+      // high part and - asymmetric schemes, whose zero points are arbitrary floats - a remainder
+      uint4 bz = make_uint4(0, 0, 0, 0), bzl = make_uint4(0, 0, 0, 0);
+      {
+        uint32_t zh[8], zlw[8];
+#pragma unroll
+        for (int q8 = 0; q8 < 8; ++q8) {
+          const float zt = lzterm[(kg * 8 + q8) * HK + g];
+          const float zhf = __uint_as_float(bf16_hi(zt));
+          zh[q8] = __float_as_uint(zhf) >> 16;
+          zlw[q8] = bf16_hi(zt - zhf) >> 16;
+        }
+        bz = make_uint4(zh[0] | (zh[1] << 16), zh[2] | (zh[3] << 16), zh[4] | (zh[5] << 16), zh[6] | (zh[7] << 16));
+        bzl = make_uint4(zlw[0] | (zlw[1] << 16), zlw[2] | (zlw[3] << 16), zlw[4] | (zlw[5] << 16), zlw[6] | (zlw[7] << 16));
+      }
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+        // source lane i points at token 8*kg + i/2, dims 16*db + 8*(i%2) .. +7; result lane i
+        // holds dimension 16*db + i of tokens 8*kg .. 8*kg+7
+        const pikv_i32x2 tr = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+            (pikv_i32x2 __attribute__((address_space(3)))*)(lcodes + (kg * 8 + (i >> 1)) * RS + g * 128 + db * 16 +
+                                                            8 * (i & 1)));
+        const uint32_t x0 = Q::sym ? ((uint32_t)tr[0] ^ 0x80808080u) : (uint32_t)tr[0];
+        const uint32_t x1 = Q::sym ? ((uint32_t)tr[1] ^ 0x80808080u) : (uint32_t)tr[1];
+        // nibble n -> bf16 16 + n = 0x4180 | n << 3: bytes {0x80 | n << 3, 0x41}
+        const uint32_t l0 = ((x0 << 3) & 0x78787878u) | 0x80808080u, l1 = ((x1 << 3) & 0x78787878u) | 0x80808080u;
+        const uint32_t h0 = ((x0 >> 1) & 0x78787878u) | 0x80808080u, h1 = ((x1 >> 1) & 0x78787878u) | 0x80808080u;
+        const uint32_t k43 = 0x41414141u;
+        const uint4 blo = make_uint4(__builtin_amdgcn_perm(k43, l0, 0x05010400u), __builtin_amdgcn_perm(k43, l0, 0x05030402u),
+                                     __builtin_amdgcn_perm(k43, l1, 0x05010400u), __builtin_amdgcn_perm(k43, l1, 0x05030402u));
+        const uint4 bhi = make_uint4(__builtin_amdgcn_perm(k43, h0, 0x05010400u), __builtin_amdgcn_perm(k43, h0, 0x05030402u),
+                                     __builtin_amdgcn_perm(k43, h1, 0x05010400u), __builtin_amdgcn_perm(k43, h1, 0x05030402u));
+        C[hs][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, a1),
+                                                            __builtin_bit_cast(pikv_bf16x8, blo), C[hs][db], 0, 0, 0);
+        C[hs][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, a16),
+                                                            __builtin_bit_cast(pikv_bf16x8, bhi), C[hs][db], 0, 0, 0);
+        C[hs][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, a1),
+                                                            __builtin_bit_cast(pikv_bf16x8, bz), C[hs][db], 0, 0, 0);
+        if constexpr (!Q::sym)
+          C[hs][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, a1),
+                                                              __builtin_bit_cast(pikv_bf16x8, bzl), C[hs][db], 0, 0, 0);
+      }
+      // the next head's rows go into the same buffer
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+  }
+
+  // Epilogue.  C: lane (dimension i, rows 4*kg + q): rows 2r / 2r+1 are the two parts of head r,
+  // so head 2*kg is q = 0,1 and head 2*kg+1 is q = 2,3.
+#pragma unroll
+  for (int hs = 0; hs < NH; ++hs) {
+    const int g = wave + 4 * hs;
+    if (g >= HK) continue;
+#pragma unroll
+    for (int rr = 0; rr < 2; ++rr) {
+      const int ro = 2 * kg + rr;  // head (inside the kv group) held by this lane
+      if (ro >= rep) continue;
+      float* o = a.partial + (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep + ro) * 128;
+#pragma unroll
+      for (int db = 0; db < 8; ++db) o[db * 16 + i] = C[hs][db][2 * rr] + C[hs][db][2 * rr + 1];
+    }
+  }
+}
+
+template <int SCHEME>
+static void launch_attend_mfma8(int n_kv_heads, dim3 grid, hipStream_t st, const AttendArgs& a) {
+  const size_t lds = attend_mfma8_lds_bytes(n_kv_heads, a.n_q_heads);
+  switch (n_kv_heads) {
+    case 1: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 0>), grid, dim3(256), lds, st, a); break;
+    case 2: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 1>), grid, dim3(256), lds, st, a); break;
+    case 4: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 2>), grid, dim3(256), lds, st, a); break;
+    default: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 3>), grid, dim3(256), lds, st, a); break;
+  }
+}
+
 template <int SCHEME>
 static void launch_attend_mfma(int n_kv_heads, dim3 grid, hipStream_t st, const AttendArgs& a) {
   const size_t lds = attend_mfma_lds_bytes(n_kv_heads, a.n_q_heads);
@@ -540,16 +830,21 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(n_kv_heads, grid, st, a);
       else launch_attend_mfma<PIKV_Q_I4_SYM>(n_kv_heads, grid, st, a);
+    } else if (eight && group % 128 == 0 && head_dim == 128 && rep >= 2 && rep <= 8 && hk_ok) {
+      const dim3 grid((unsigned)splits, (unsigned)n_caches);
+      if (scheme == PIKV_Q_I8_SYM) launch_attend_mfma8<PIKV_Q_I8_SYM>(n_kv_heads, grid, st, a);
+      else launch_attend_mfma8<PIKV_Q_I8_ASYM>(n_kv_heads, grid, st, a);
     } else {
       if (row_acc || row_ts)
         hipLaunchKernelGGL(attend_importance_kernel, dim3((unsigned)((max_len + 255) / 256), (unsigned)n_caches),
                            dim3(256), 0, st, a);
       // heads of a kv group per pass: the float accumulators of one lane must fit
-      const int rp = eight ? (rep >= 4 ? 4 : rep >= 2 ? 2 : 1) : (rep >= 2 ? 2 : 1);
+      const int rp = eight ? (rep >= 8 ? 8 : rep >= 4 ? 4 : rep >= 2 ? 2 : 1) : (rep >= 2 ? 2 : 1);
       const dim3 grid((unsigned)splits, (unsigned)n_caches, (unsigned)((rep + rp - 1) / rp));
 #define PIKV_ATTEND_CASE(S)                                                                        \
   case S:                                                                                          \
-    if (rp == 4) hipLaunchKernelGGL((attend_valu_kernel<S, 4>), grid, dim3(256), 0, st, a);        \
+    if (rp == 8) hipLaunchKernelGGL((attend_valu_kernel<S, 8>), grid, dim3(256), 0, st, a);        \
+    else if (rp == 4) hipLaunchKernelGGL((attend_valu_kernel<S, 4>), grid, dim3(256), 0, st, a);   \
     else if (rp == 2) hipLaunchKernelGGL((attend_valu_kernel<S, 2>), grid, dim3(256), 0, st, a);   \
     else hipLaunchKernelGGL((attend_valu_kernel<S, 1>), grid, dim3(256), 0, st, a);                \
     break;

@@ -361,6 +361,48 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 // hazard handling between vector and matrix-core instructions.
 __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) { return (x & m) | o; }
 
+// Tile statistics and score rows from the staged scores [q head][token in tile], four
+// heads per wavefront pass: lane (rg, nl) owns tokens nl, nl+16, nl+32, nl+48 of head
+// h4 + rg; the 16 lanes of a row reduce with DPP.
+__device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float* stage, int c, int64_t tile,
+                                                 int64_t n0, int len, int wave, int rg, int nl) {
+  for (int h4 = wave * 4; h4 < a.n_q_heads; h4 += 16) {
+    const int hq = h4 + rg;
+    const bool hok = hq < a.n_q_heads;
+    float x[4];
+    bool okk[4];
+    float m = -__builtin_inff();
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      okk[k] = hok && (n0 + nl + 16 * k < len);
+      x[k] = okk[k] ? stage[hq * kTile + nl + 16 * k] : -__builtin_inff();
+      m = fmaxf(m, x[k]);
+    }
+    PIKV_DPP_INPLACE("v_max_f32_dpp", m, "quad_perm:[1,0,3,2]");
+    PIKV_DPP_INPLACE("v_max_f32_dpp", m, "quad_perm:[2,3,0,1]");
+    PIKV_DPP_INPLACE("v_max_f32_dpp", m, "row_half_mirror");
+    PIKV_DPP_INPLACE("v_max_f32_dpp", m, "row_mirror");
+    float sum = 0.f;
+    float* out = a.scores + ((int64_t)c * a.n_q_heads + (hok ? hq : 0)) * a.score_stride + n0 + nl;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (okk[k]) {
+        sum += __builtin_amdgcn_exp2f((x[k] - m) * 1.4426950408889634f);
+        out[16 * k] = x[k];
+      }
+    }
+    PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "quad_perm:[1,0,3,2]");
+    PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "quad_perm:[2,3,0,1]");
+    PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "row_half_mirror");
+    PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "row_mirror");
+    if (nl == 0 && hok) {
+      const int64_t ti = ((int64_t)c * a.n_q_heads + hq) * a.n_tiles + tile;
+      a.tile_max[ti] = m;
+      a.tile_sum[ti] = sum;
+    }
+  }
+}
+
 constexpr int kGqaTilesPerBlock = 4;   // consecutive 64-token tiles handled by one block
 constexpr int kGqaMaxKvHeads = 16;     // code vectors of one 16-token slice kept in registers
 
@@ -521,44 +563,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 
     }
     __syncthreads();
 
-    // Tile statistics and score rows, four heads per wavefront pass: lane (rg, nl)
-    // owns tokens nl, nl+16, nl+32, nl+48 of head h4 + rg; the 16 lanes of a row
-    // reduce with DPP.
-    for (int h4 = wave * 4; h4 < a.n_q_heads; h4 += 16) {
-      const int hq = h4 + rg;
-      const bool hok = hq < a.n_q_heads;
-      float x[4];
-      bool okk[4];
-      float m = -__builtin_inff();
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        okk[k] = hok && (n0 + nl + 16 * k < len);
-        x[k] = okk[k] ? stage[hq * kTile + nl + 16 * k] : -__builtin_inff();
-        m = fmaxf(m, x[k]);
-      }
-      PIKV_DPP_INPLACE("v_max_f32_dpp", m, "quad_perm:[1,0,3,2]");
-      PIKV_DPP_INPLACE("v_max_f32_dpp", m, "quad_perm:[2,3,0,1]");
-      PIKV_DPP_INPLACE("v_max_f32_dpp", m, "row_half_mirror");
-      PIKV_DPP_INPLACE("v_max_f32_dpp", m, "row_mirror");
-      float sum = 0.f;
-      float* out = a.scores + ((int64_t)c * a.n_q_heads + (hok ? hq : 0)) * a.score_stride + n0 + nl;
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        if (okk[k]) {
-          sum += __builtin_amdgcn_exp2f((x[k] - m) * 1.4426950408889634f);
-          out[16 * k] = x[k];
-        }
-      }
-      PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "quad_perm:[1,0,3,2]");
-      PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "quad_perm:[2,3,0,1]");
-      PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "row_half_mirror");
-      PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "row_mirror");
-      if (nl == 0 && hok) {
-        const int64_t ti = ((int64_t)c * a.n_q_heads + hq) * a.n_tiles + tile;
-        a.tile_max[ti] = m;
-        a.tile_sum[ti] = sum;
-      }
-    }
+    tile_stats_store(a, stage, c, tile, n0, len, wave, rg, nl);
     __syncthreads();  // stage and the metadata rows are reused by the next tile
     return true;
   };
@@ -567,6 +572,150 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 
     if (!do_tile(tt, ra, rb)) break;
     if (!do_tile(tt + 1, rb, ra)) break;
   }
+}
+
+// ---- 8-bit scores on the matrix cores ------------------------------------------------
+// Per-head (or coarser) scales, head_dim 128, bf16 queries, up to 16 query heads per kv
+// head.  The vector form above is instruction-bound as soon as several query heads share
+// a kv head (measured at 64 x 32768 cached tokens, 8 kv heads: 793 us for 4 heads per kv
+// head, 2143 us for 8, where HBM allows about 440 us).  An 8-bit code does not fit one
+// bf16 exactly, so a stored byte u (the code itself, or code + 128 for the symmetric
+// scheme) is fed as its two nibbles: u = 16*hi + lo, both exact as bf16 16 + nibble,
+// against A operands that hold q for the low nibble and 16*q (exact,
+// a power of two) for the high one:
+//   C[head][token] = sum_d q_d*(16 + lo_d) + 16*q_d*(16 + hi_d) = sum_d q_d*u_d + 272*Qs
+// with Qs = sum_d q_d, which comes out of the same matrix cores from a constant B operand
+// (1 at the low-nibble positions).  score = scale * (C - (272 + zz)*Qs), zz = 128
+// (symmetric) or the zero point.  (16 + nibble = 0x4180 | nibble << 3 is the smallest
+// offset a single OR can give; the smaller the offset, the less the subtraction costs in
+// float32 accuracy.)
+// A wavefront owns kv heads {w, w+4, ...} and keeps their A operands in registers (8
+// k-steps of 16 dimensions per head); per 16-token slice a lane loads the two 16-byte
+// halves of its token's head row, so one load instruction fetches whole 128-byte lines.
+constexpr int kI8TilesPerBlock = 4;
+
+template <int SCHEME, int NHW>  // NHW = kv heads per wavefront: ceil(n_kv_heads / 4), 1, 2 or 4
+__global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
+  using Q = QScheme<SCHEME>;
+  static_assert(Q::bits == 8, "8-bit schemes only");
+  extern __shared__ float i8_lds[];
+  float* stage = i8_lds;  // [q head][token in tile]
+
+  const int c = blockIdx.y;
+  const int len = a.fill[c];
+  const int64_t tile0 = (int64_t)blockIdx.x * kI8TilesPerBlock;
+  if (tile0 * kTile >= len) return;  // uniform for the block
+  const int rep = a.n_q_heads / a.n_kv_heads;  // <= 16
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nl = lane & 15;   // token of a slice (B, C column) / query head (A row)
+  const int rg = lane >> 4;   // k-slice: dimensions 16*rg .. 16*rg+15 of a 64-wide half
+  const int64_t row_bytes = (int64_t)a.n_kv_heads * 128;
+  const int groups_per_row = (a.n_kv_heads * 128) / a.group;
+  const int64_t base_row = a.row_base[c];
+  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * 128;
+  const uint32_t kNib = 0x00780078u, kExp = 0x41804180u;  // two nibbles -> two bf16 values 16 + nibble
+
+  // A operands of this wavefront's kv heads: lane (row nl = query head, k-slice rg), k-step
+  // (half, b2) covers dimensions d0 = 64*half + 16*rg + 4*b2 .. +3 in the slot order
+  // {d0, d0+2, 16x d0, 16x d0+2, d0+1, d0+3, 16x d0+1, 16x d0+3} that the nibble unpack produces.
+  uint4 areg[NHW][8];
+  float qs[NHW][4];
+#pragma unroll
+  for (int hs = 0; hs < NHW; ++hs) {
+    const int g = wave + 4 * hs;
+    const bool on = g < a.n_kv_heads && nl < rep;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      uint2 qd = make_uint2(0, 0);
+      if (on) qd = *reinterpret_cast<const uint2*>(qbase + (int64_t)(g * rep + nl) * 128 + 64 * (ks >> 2) + 16 * rg + 4 * (ks & 3));
+      // bf16 x 16: through float, exact (zero stays zero)
+      auto x16 = [](uint32_t h) { return __float_as_uint(__uint_as_float(h << 16) * 16.0f) >> 16; };
+      const uint32_t q0 = qd.x & 0xffffu, q1 = qd.x >> 16, q2 = qd.y & 0xffffu, q3 = qd.y >> 16;
+      areg[hs][ks] = make_uint4(q0 | (q2 << 16), x16(q0) | (x16(q2) << 16), q1 | (q3 << 16), x16(q1) | (x16(q3) << 16));
+    }
+    // Qs of heads 4*rg .. 4*rg+3 (C rows) from a B operand that is 1 at the low-nibble slots
+    const uint4 ones = make_uint4(0x3f803f80u, 0u, 0x3f803f80u, 0u);
+    pikv_f32x4 sumq = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+      sumq = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, areg[hs][ks]),
+                                                     __builtin_bit_cast(pikv_bf16x8, ones), sumq, 0, 0, 0);
+#pragma unroll
+    for (int qq = 0; qq < 4; ++qq) qs[hs][qq] = sumq[qq];
+  }
+
+  for (int tt = 0; tt < kI8TilesPerBlock; ++tt) {
+    const int64_t tile = tile0 + tt;
+    const int64_t n0 = tile * kTile;
+    if (n0 >= len) break;  // uniform
+#pragma unroll
+    for (int hs = 0; hs < NHW; ++hs) {
+      const int g = wave + 4 * hs;
+      if (g >= a.n_kv_heads) continue;  // uniform
+      // the four 16-token slices of the tile: two 16-byte halves and the metadata of each
+      uint4 cv[4][2];
+      float sc[4], zr[4];
+      bool ok[4];
+#pragma unroll
+      for (int sl = 0; sl < 4; ++sl) {
+        const int64_t n = n0 + 16 * sl + nl;
+        ok[sl] = n < len;
+        cv[sl][0] = cv[sl][1] = make_uint4(0, 0, 0, 0);
+        sc[sl] = 0.f;
+        zr[sl] = 0.f;
+        if (ok[sl]) {
+          const char* rowp = reinterpret_cast<const char*>(a.codes) + (base_row + n) * row_bytes + g * 128 + 16 * rg;
+          cv[sl][0] = ld16(rowp);
+          cv[sl][1] = ld16(rowp + 64);
+          const int64_t mi = (base_row + n) * groups_per_row + (g * 128) / a.group;
+          sc[sl] = reinterpret_cast<const float*>(a.scale)[mi];
+          if constexpr (!Q::sym) zr[sl] = reinterpret_cast<const float*>(a.zero)[mi];
+        }
+      }
+#pragma unroll
+      for (int sl = 0; sl < 4; ++sl) {
+        pikv_f32x4 pc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const uint32_t wv[4] = {cv[sl][half].x, cv[sl][half].y, cv[sl][half].z, cv[sl][half].w};
+#pragma unroll
+          for (int b2 = 0; b2 < 4; ++b2) {
+            const uint32_t w = Q::sym ? (wv[b2] ^ 0x80808080u) : wv[b2];
+            const uint4 bb = make_uint4(and_or(w << 3, kNib, kExp), and_or(w >> 1, kNib, kExp),
+                                        and_or(w >> 5, kNib, kExp), and_or(w >> 9, kNib, kExp));
+            pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, areg[hs][half * 4 + b2]),
+                                                         __builtin_bit_cast(pikv_bf16x8, bb), pc, 0, 0, 0);
+          }
+        }
+        const float zz = 272.0f + (Q::sym ? 128.0f : zr[sl]);
+#pragma unroll
+        for (int qq = 0; qq < 4; ++qq) {
+          const int r = 4 * rg + qq;
+          if (r < rep) {
+            const float score = sc[sl] * fmaf(-zz, qs[hs][qq], pc[qq]) * a.scale_qk;
+            stage[(g * rep + r) * kTile + 16 * sl + nl] = ok[sl] ? score : -__builtin_inff();
+          }
+        }
+      }
+    }
+    __syncthreads();
+    tile_stats_store(a, stage, c, tile, n0, len, wave, rg, nl);
+    __syncthreads();  // stage is reused by the next tile
+  }
+}
+
+template <int SCHEME>
+static int launch_i8_mfma(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
+  const size_t lds = (size_t)a.n_q_heads * kTile * sizeof(float);
+  const dim3 grid((unsigned)((n_tiles + kI8TilesPerBlock - 1) / kI8TilesPerBlock), (unsigned)n_caches);
+  if (a.n_kv_heads <= 4)
+    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 1>), grid, dim3(256), lds, st, a);
+  else if (a.n_kv_heads <= 8)
+    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 2>), grid, dim3(256), lds, st, a);
+  else
+    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 4>), grid, dim3(256), lds, st, a);
+  return PIKV_OK;
 }
 
 template <int SCHEME>
@@ -803,6 +952,14 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
     } else {
       hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_SYM>), grid, dim3(256), mlds, st, a);
     }
+    PIKV_CHECK_LAUNCH();
+    return PIKV_OK;
+  }
+  // 8-bit caches with per-head (or coarser) scales, several bf16 query heads per kv head
+  if (eight && head_dim == 128 && group % 128 == 0 && q_dtype == PIKV_BF16 && rep >= 2 && rep <= 16 &&
+      n_kv_heads <= 16) {
+    if (scheme == PIKV_Q_I8_SYM) launch_i8_mfma<PIKV_Q_I8_SYM>(a, n_caches, n_tiles, st);
+    else launch_i8_mfma<PIKV_Q_I8_ASYM>(a, n_caches, n_tiles, st);
     PIKV_CHECK_LAUNCH();
     return PIKV_OK;
   }

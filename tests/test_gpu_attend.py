@@ -21,7 +21,12 @@ pytestmark = pytest.mark.gpu
     (O.Q_I4_ASYM, 32, 16, 16, 128),    # more kv heads than the matrix-core form takes: vector form
     (O.Q_I8_SYM, 128, 4, 4, 128),      # int8 per token per head
     (O.Q_I8_SYM, 256, 4, 8, 64),       # one scale per token
-    (O.Q_I8_ASYM, 64, 2, 16, 64),      # 8 q heads per kv head: two passes of 4
+    (O.Q_I8_ASYM, 64, 2, 16, 64),      # 8 q heads per kv head in one pass
+    (O.Q_I8_SYM, 128, 2, 24, 128),     # 12 q heads per kv head: passes of 8 and 4
+    (O.Q_I8_SYM, 128, 8, 32, 128),     # 8-bit matrix-core form: 4 q heads per kv head
+    (O.Q_I8_ASYM, 128, 2, 16, 128),    # ... 8 q heads per kv head, zero points
+    (O.Q_I8_SYM, 256, 4, 8, 128),      # ... one scale per two heads
+    (O.Q_I8_ASYM, 128, 1, 6, 128),     # ... one kv head, 6 q heads
     (O.Q_I4_SYM, 64, 4, 4, 64),
 ])
 @pytest.mark.parametrize("form", ["stats", "probs"])
@@ -57,7 +62,9 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
 @pytest.mark.parametrize("scheme,group,heads,hq,dh", [
     (O.Q_I4_ASYM, 32, 8, 32, 128),     # matrix-core form: importance summed from the staged tile
     (O.Q_I4_ASYM, 32, 2, 4, 128),
-    (O.Q_I8_SYM, 128, 4, 8, 128),      # vector form: importance in a kernel of its own
+    (O.Q_I8_SYM, 128, 4, 8, 128),      # 8-bit matrix-core form
+    (O.Q_I8_ASYM, 128, 8, 64, 128),    # ... 64 query heads
+    (O.Q_I8_SYM, 64, 4, 8, 64),        # vector form: importance in a kernel of its own
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.95])
 def test_attend_accumulates_importance(dev, scheme, group, heads, hq, dh, decay):

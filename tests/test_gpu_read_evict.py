@@ -46,6 +46,11 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I4_SYM, 32, 2, 4, 128),       # matrix-core kernel, symmetric codes, 2 q heads per kv head
     (O.Q_I4_ASYM, 32, 1, 16, 128),     # matrix-core kernel, all 16 rows of the tile in use
     (O.Q_I4_ASYM, 32, 16, 16, 128),    # more kv heads than wavefronts, one q head each
+    (O.Q_I8_SYM, 128, 8, 32, 128),     # 8-bit matrix-core kernel: 4 q heads per kv head, scale per head
+    (O.Q_I8_ASYM, 128, 2, 16, 128),    # ... 8 q heads per kv head, zero points
+    (O.Q_I8_SYM, 256, 4, 64, 128),     # ... 16 q heads per kv head, one scale per two heads
+    (O.Q_I8_ASYM, 128, 16, 32, 128),   # ... 16 kv heads (four per wavefront)
+    (O.Q_I8_SYM, 1024, 8, 16, 128),    # ... one scale per token
 ])
 @pytest.mark.parametrize("qdtype", ["f32", "bf16"])
 def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
