@@ -1,7 +1,7 @@
 """GPU: seeded sweep over small random shapes of the whole chain - scatter two
 batches, scores, attention output, H2O accumulate, evict, compact - against the numpy
 restatement.  The shapes are drawn from everything the entry points accept (all four
-schemes, 1-8 kv heads, 1-4 query heads per kv head, head sizes 64/128, every legal
+schemes, 1-8 kv heads, 1-8 query heads per kv head, head sizes 64/128, every legal
 group, fp32 and bf16 sources and queries, ragged and empty caches), so that indexing
 that only holds for the benchmark shapes shows up here."""
 import os
@@ -24,7 +24,7 @@ def _draw(r, big):
     four = scheme in (O.Q_I4_ASYM, O.Q_I4_SYM)
     heads = int(r.choice([1, 2, 4, 8]))
     dh = int(r.choice([64, 128]))
-    rep = int(r.choice([1, 2, 4]))
+    rep = int(r.choice([1, 2, 4, 8]))
     D = heads * dh
     groups = [g for g in (32, 64, 128, 256, 512, 1024) if (g >= (32 if four else 16)) and
               ((g <= dh and dh % g == 0) or g == D)]
