@@ -50,6 +50,7 @@ struct AttendArgs {
   float* row_ts;
   float decay;
   float now;
+  int head_off;  // attend_mfma_i4_kernel: first query head of every kv group handled by this launch
 };
 
 __device__ __forceinline__ float prob_of(float s, float mx, float rz, bool normalise) {
@@ -179,7 +180,7 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads) {
   // [64 tokens][kv head] in padded token rows; A operands per wavefront [4 groups][8 rows][kAttARow];
   // probabilities [query head][kAttPRow]
   return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * att_meta_bytes(n_kv_heads) + 4 * (size_t)4 * 8 * kAttARow +
-         (size_t)n_q_heads * kAttPRow * 4;
+         (size_t)4 * n_kv_heads * kAttPRow * 4;
 }
 
 // HKS = log2(n_kv_heads); at most 4 query heads per kv head.
@@ -211,7 +212,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * 128 + idx] = 0.f;
     return;
   }
-  const int rep = a.n_q_heads / HK;  // <= 4
+  // A launch covers up to 4 query heads of every kv group: heads head_off .. head_off+nr-1.
+  // More than 4 heads per kv head are served by a second launch over the same codes.
+  const int rep_all = a.n_q_heads / HK;
+  const int rep = rep_all - a.head_off < 4 ? rep_all - a.head_off : 4;  // heads of a group in this launch
   // matrix-core roles: A row / B,C column i, token group kg
   const int i = lane & 15;
   const int kg = lane >> 4;
@@ -233,15 +237,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 #pragma unroll
     for (int sg = 0; sg < 4; ++sg) zacc[hs][sg] = 0.f;
   }
-  // score-staging role: query head sh, tokens st8..st8+7 of the tile (32 heads x 8 runs)
+  // score-staging role: staged row sh = 4 * kv head + head of this launch, tokens st8..st8+7 of
+  // the tile (32 rows x 8 runs); rows without a head stage zeros
   const int sh = threadIdx.x >> 3;
   const int st8 = (threadIdx.x & 7) * 8;
-  const bool s_on = sh < a.n_q_heads;
-  const float* srow = a.scores + ((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * a.score_stride;
+  const bool s_on = (sh >> 2) < HK && (sh & 3) < rep;
+  const int s_hq = s_on ? (sh >> 2) * rep_all + a.head_off + (sh & 3) : 0;
+  const float* srow = a.scores + ((int64_t)c * a.n_q_heads + s_hq) * a.score_stride;
   float smx = 0.f, srz = 1.f;
   if (normalise) {
-    smx = a.head_stats[((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * 2];
-    srz = 1.0f / a.head_stats[((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * 2 + 1];
+    smx = a.head_stats[((int64_t)c * a.n_q_heads + s_hq) * 2];
+    srz = 1.0f / a.head_stats[((int64_t)c * a.n_q_heads + s_hq) * 2 + 1];
   }
   const bool s_vec = (a.score_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(a.scores) & 15) == 0;
   const float s_off = normalise ? -INFINITY : 0.f;  // what a token past the end contributes: p = 0
@@ -291,12 +297,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   };
   auto h2f = [](uint32_t w, int hi) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> (16 * hi))); };
   auto stage = [&]() {
-    if (s_on) {
+    {
       // tokens {l, l+4, l+8, l+12} of a 16-token group go side by side: one float4 per reader
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
         const int t = st8 + k;
-        lprob[sh * kAttPRow + (t & ~15) + (t & 3) * 4 + ((t >> 2) & 3)] = prob_of(psc[k], smx, srz, normalise);
+        lprob[sh * kAttPRow + (t & ~15) + (t & 3) * 4 + ((t >> 2) & 3)] =
+            s_on ? prob_of(psc[k], smx, srz, normalise) : 0.f;
       }
     }
 #pragma unroll
@@ -339,7 +346,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       const int64_t row = base_row + n0 + t;
       const float* lp = lprob + (t & ~15) + (t & 3) * 4 + ((t >> 2) & 3);
       float imp = 0.f;
-      for (int hq = grp; hq < a.n_q_heads; hq += 4) imp = imp + lp[hq * kAttPRow];
+      for (int hq = grp; hq < 4 * HK; hq += 4) imp = imp + lp[hq * kAttPRow];
       imp = imp + __shfl_xor(imp, 16, 64);
       imp = imp + __shfl_xor(imp, 32, 64);
       if (mine) {
@@ -357,7 +364,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       if (g >= HK) continue;  // uniform
       // ---- weights: this lane prepares head r for four tokens, all four groups ----
       float4 s4[4], z4[4];
-      const float4 pv = *reinterpret_cast<const float4*>(lprob + (row_on ? g * rep + r : 0) * kAttPRow + wkg * 16 +
+      const float4 pv = *reinterpret_cast<const float4*>(lprob + (row_on ? g * 4 + r : 0) * kAttPRow + wkg * 16 +
                                                          (lane & 3) * 4);
       const float p4[4] = {row_on ? pv.x : 0.f, row_on ? pv.y : 0.f, row_on ? pv.z : 0.f, row_on ? pv.w : 0.f};
 #pragma unroll
@@ -451,7 +458,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     for (int rr = 0; rr < 2; ++rr) {
       const int ro = 2 * kg + rr;  // head (inside the kv group) held by this lane
       if (ro >= rep) continue;
-      float* o = a.partial + (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep + ro) * 128;
+      float* o = a.partial + (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + ro) * 128;
 #pragma unroll
       for (int db = 0; db < 8; ++db)
         o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NH + hs) * 4 + ro) * 4 + (db >> 1)];
@@ -822,14 +829,20 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
   }
   AttendArgs a{scores, head_stats, v_codes, v_scale, v_zero, cache_row_base, cache_fill,
                (float*)workspace, score_stride, group, n_kv_heads, n_q_heads, head_dim, n_caches,
-               row_acc, row_ts, decay, now};
+               row_acc, row_ts, decay, now, 0};
   const int rep = n_q_heads / n_kv_heads;
   if (max_len > 0) {
     const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;
-    if (!eight && group == 32 && head_dim == 128 && rep <= 4 && hk_ok) {
+    if (!eight && group == 32 && head_dim == 128 && rep <= 8 && hk_ok) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
-      if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(n_kv_heads, grid, st, a);
-      else launch_attend_mfma<PIKV_Q_I4_SYM>(n_kv_heads, grid, st, a);
+      // four query heads of every kv group per launch; a second launch (same codes, next four
+      // heads) adds its share to the accumulators that the first one has already decayed
+      for (int off = 0; off < rep; off += 4) {
+        a.head_off = off;
+        if (off > 0) a.decay = 1.0f;
+        if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(n_kv_heads, grid, st, a);
+        else launch_attend_mfma<PIKV_Q_I4_SYM>(n_kv_heads, grid, st, a);
+      }
     } else if (eight && group % 128 == 0 && head_dim == 128 && rep >= 2 && rep <= 8 && hk_ok) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       if (scheme == PIKV_Q_I8_SYM) launch_attend_mfma8<PIKV_Q_I8_SYM>(n_kv_heads, grid, st, a);

@@ -45,6 +45,8 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I4_SYM, 64, 4, 4, 64),
     (O.Q_I4_SYM, 32, 2, 4, 128),       # matrix-core kernel, symmetric codes, 2 q heads per kv head
     (O.Q_I4_ASYM, 32, 1, 16, 128),     # matrix-core kernel, all 16 rows of the tile in use
+    (O.Q_I4_ASYM, 32, 8, 64, 128),     # 8 q heads per kv head: two sets of A rows against the same codes
+    (O.Q_I4_SYM, 32, 2, 12, 128),      # 6 q heads per kv head: the second set half empty
     (O.Q_I4_ASYM, 32, 16, 16, 128),    # more kv heads than wavefronts, one q head each
     (O.Q_I8_SYM, 128, 8, 32, 128),     # 8-bit matrix-core kernel: 4 q heads per kv head, scale per head
     (O.Q_I8_ASYM, 128, 2, 16, 128),    # ... 8 q heads per kv head, zero points
@@ -54,8 +56,8 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
 ])
 @pytest.mark.parametrize("qdtype", ["f32", "bf16"])
 def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
-    if qdtype == "f32" and hq // heads > 8:
-        pytest.skip("more than 8 query heads per kv head is served by the bf16 matrix-core kernel only")
+    if qdtype == "f32" and hq // heads not in (1, 2, 4, 8):
+        pytest.skip("float32 queries: 1, 2, 4 or 8 query heads per kv head (others go through the bf16 matrix-core kernels)")
     r = rng(scheme * 7 + heads)
     caps = [300, 64, 130, 10]
     lens = [257, 64, 1, 0]            # ragged: partial tile, full tile, single row, empty
