@@ -199,6 +199,37 @@ def decode_read_workload(torch, ops, dev, iters):
     }
 
 
+def decode_read_int8_workload(torch, ops, dev, iters):
+    """Not one of the listed configurations: the decode read of the same 64 x 32768 cached
+    tokens with the int8 per-token-per-head format of the write-side workloads, read by 8
+    query heads per kv head (8 kv heads, 64 query heads) - the shape that takes the 8-bit
+    matrix-core kernels."""
+    B, N, hkv, hq, dh = 64, 32768, 8, 64, 128
+    D = hkv * dh
+    g = torch.Generator(device=dev).manual_seed(5)
+    pool = ops.CachePool([N] * B, hkv, dh, dh, ops.Q_I8_SYM, dev, with_v=True)
+    chunk = 4
+    slot = torch.arange(N, device=dev, dtype=torch.int32).repeat(chunk)
+    for b0 in range(0, B, chunk):
+        ks = torch.randn(chunk * N, D, generator=g, device=dev).to(torch.bfloat16)
+        vs = torch.randn(chunk * N, D, generator=g, device=dev).to(torch.bfloat16)
+        cid = torch.arange(b0, b0 + chunk, device=dev, dtype=torch.int32).repeat_interleave(N)
+        pool.quant_scatter(ks, vs, cid, slot, 1)
+    pool.fill.fill_(N)
+    q = torch.randn(B, hq, dh, generator=g, device=dev).to(torch.bfloat16)
+    t_scores = _median_ms(torch, lambda: pool.scores(q, hq), iters)
+    sc, tm, tsu = pool.scores(q, hq)
+    pool.h2o_accumulate(sc, tm, tsu, now=1.0, stats_only=True)
+    t_att = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats, accumulate=True, now=1.0), iters)
+    rows = B * N
+    k_bytes = rows * (D + hkv * 4)
+    return {
+        "workload": "decode read, int8 per token per head: 64 seq x 32768 cached tokens, 8 KV heads x 128 (64 q heads)",
+        "gather_dequant_scores": _entry(t_scores, k_bytes, bytes_with_score_store=k_bytes + rows * hq * 4),
+        "attend_values_with_h2o": _entry(t_att, k_bytes + rows * hq * 4 + rows * 12),
+    }
+
+
 def wide_routing_workload(torch, ops, dev, iters):
     """Wide MoE routing: 65536 tokens, hidden 7168, 64 experts top-8, Zipf(1.2) expert
     popularity, EPLB-style per-expert logit scale; int8 KV of 8 heads x 128 scattered
@@ -380,8 +411,8 @@ def main():
     if not args.only_headline:
         it = max(5, min(args.steps, 20))
         out["other_workloads"] = {}
-        for name, fn in (("decode_read", decode_read_workload), ("wide_routing", wide_routing_workload),
-                         ("pyramid", pyramid_workload)):
+        for name, fn in (("decode_read", decode_read_workload), ("decode_read_int8_gqa8", decode_read_int8_workload),
+                         ("wide_routing", wide_routing_workload), ("pyramid", pyramid_workload)):
             out["other_workloads"][name] = fn(torch, ops, dev, it)
             torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
