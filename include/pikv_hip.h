@@ -272,7 +272,7 @@ int pikv_gather_dequant(const void* codes, const void* scale, const void* zero,
  *   for n < cache_fill[c]; entries n >= cache_fill[c] are not written.
  *   q       [n_caches, n_q_heads, head_dim] q_dtype
  *   scores  [n_caches, n_q_heads, score_stride] float
- *   tile_max, tile_sum [n_caches, n_q_heads, n_tiles] float: per tile of
+ *   tile_max, tile_sum [n_caches, n_tiles, n_q_heads] float: per tile of
  *   PIKV_SCORE_TILE cached tokens, max score and sum of exp(score - max);
  *   n_tiles = ceil(max_len / PIKV_SCORE_TILE) with max_len <= score_stride
  *   the largest cache_fill the caller wants covered.

@@ -194,7 +194,7 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
     const float e = ok ? __builtin_amdgcn_exp2f((s - m) * 1.4426950408889634f) : 0.f;
     const float sum = group_sum_dpp(e, 64);
     if (lane == 0) {
-      const int64_t ti = ((int64_t)c * a.n_q_heads + hq) * a.n_tiles + tile;
+      const int64_t ti = ((int64_t)c * a.n_tiles + tile) * a.n_q_heads + hq;  // heads of a tile side by side
       a.tile_max[ti] = m;
       a.tile_sum[ti] = sum;
     }
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
     const float e = ok ? expf(sv - m) : 0.f;
     const float sum = group_sum<64>(e);
     if (lane == 0) {
-      const int64_t ti = ((int64_t)c * a.n_q_heads + hq) * a.n_tiles + tile;
+      const int64_t ti = ((int64_t)c * a.n_tiles + tile) * a.n_q_heads + hq;  // heads of a tile side by side
       a.tile_max[ti] = m;
       a.tile_sum[ti] = sum;
     }
@@ -396,7 +396,7 @@ __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float
     PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "row_half_mirror");
     PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "row_mirror");
     if (nl == 0 && hok) {
-      const int64_t ti = ((int64_t)c * a.n_q_heads + hq) * a.n_tiles + tile;
+      const int64_t ti = ((int64_t)c * a.n_tiles + tile) * a.n_q_heads + hq;  // heads of a tile side by side
       a.tile_max[ti] = m;
       a.tile_sum[ti] = sum;
     }
@@ -732,28 +732,57 @@ static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStre
   return PIKV_OK;
 }
 
-// Final max and sum per (cache, q head) from the tile statistics.
-__global__ __launch_bounds__(64) void head_stats_kernel(const float* __restrict__ tile_max,
-                                                        const float* __restrict__ tile_sum,
-                                                        const int32_t* __restrict__ fill,
-                                                        int n_q_heads, int64_t n_tiles,
-                                                        float* __restrict__ head_stats) {
+// Final max and sum per (cache, q head) from the tile statistics [cache][tile][head].
+// A block takes 16 heads of one cache: thread (head hl, tile lane tl) folds tiles
+// tl, tl+16, ... into a running (max, sum) pair - neighbouring threads read neighbouring
+// heads - and the 16 pairs of a head are merged in tile-lane order.
+__global__ __launch_bounds__(256) void head_stats_kernel(const float* __restrict__ tile_max,
+                                                         const float* __restrict__ tile_sum,
+                                                         const int32_t* __restrict__ fill,
+                                                         int n_q_heads, int64_t n_tiles,
+                                                         float* __restrict__ head_stats) {
+  __shared__ float sm[16][17], sz[16][17];
   const int c = blockIdx.y;
-  const int hq = blockIdx.x;
-  const int lane = threadIdx.x;
+  const int hl = threadIdx.x & 15, tl = threadIdx.x >> 4;
+  const int hq = blockIdx.x * 16 + hl;
   const int64_t used = ((int64_t)fill[c] + kTile - 1) / kTile;
   const int64_t lim = used < n_tiles ? used : n_tiles;
-  const float* tm = tile_max + ((int64_t)c * n_q_heads + hq) * n_tiles;
-  const float* tsum = tile_sum + ((int64_t)c * n_q_heads + hq) * n_tiles;
-  float m = -__builtin_inff();
-  for (int64_t t = lane; t < lim; t += 64) m = fmaxf(m, tm[t]);
-  m = group_max<64>(m);
-  float z = 0.f;
-  for (int64_t t = lane; t < lim; t += 64) z += tsum[t] * expf(tm[t] - m);
-  z = group_sum<64>(z);
-  if (lane == 0) {
-    head_stats[((int64_t)c * n_q_heads + hq) * 2] = m;
-    head_stats[((int64_t)c * n_q_heads + hq) * 2 + 1] = z;
+  const float ninf = -__builtin_inff();
+  float m = ninf, z = 0.f;
+  if (hq < n_q_heads) {
+    const float* tm = tile_max + (int64_t)c * n_tiles * n_q_heads + hq;
+    const float* ts = tile_sum + (int64_t)c * n_tiles * n_q_heads + hq;
+    for (int64_t t0 = tl; t0 < lim; t0 += 16 * 8) {
+      float tmx[8], tsm[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {  // eight tiles in flight per thread
+        const int64_t t = t0 + 16 * u;
+        tmx[u] = t < lim ? tm[t * n_q_heads] : ninf;
+        tsm[u] = t < lim ? ts[t * n_q_heads] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (tmx[u] == ninf) continue;
+        if (tmx[u] > m) {
+          z = z * expf(m - tmx[u]) + tsm[u];  // expf(-inf) = 0 for the first tile
+          m = tmx[u];
+        } else {
+          z += tsm[u] * expf(tmx[u] - m);
+        }
+      }
+    }
+  }
+  sm[tl][hl] = m;
+  sz[tl][hl] = z;
+  __syncthreads();
+  if (tl == 0 && hq < n_q_heads) {
+    float mm = ninf;
+    for (int k = 0; k < 16; ++k) mm = fmaxf(mm, sm[k][hl]);
+    float zz = 0.f;
+    for (int k = 0; k < 16; ++k)
+      if (sm[k][hl] != ninf) zz += sz[k][hl] * expf(sm[k][hl] - mm);
+    head_stats[((int64_t)c * n_q_heads + hq) * 2] = mm;
+    head_stats[((int64_t)c * n_q_heads + hq) * 2 + 1] = zz;
   }
 }
 
@@ -992,7 +1021,7 @@ extern "C" int pikv_h2o_accumulate(float* scores, const float* tile_max, const f
   if (max_len == 0) return PIKV_OK;
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(head_stats_kernel, dim3((unsigned)n_q_heads, (unsigned)n_caches), dim3(64), 0,
+  hipLaunchKernelGGL(head_stats_kernel, dim3((unsigned)((n_q_heads + 15) / 16), (unsigned)n_caches), dim3(256), 0,
                      st, tile_max, tile_sum, cache_fill, n_q_heads, n_tiles, head_stats);
   // nothing to normalise or accumulate: the caller only wanted the statistics
   if (!write_probs && !row_acc && !row_ts && !importance_out) {

@@ -565,7 +565,7 @@ class CachePool:
         n_tiles = (max_len + SCORE_TILE - 1) // SCORE_TILE
         dev = self.device
         scores = torch.empty(self.n_caches, n_q_heads, stride, dtype=torch.float32, device=dev)
-        tmax = torch.empty(self.n_caches, n_q_heads, max(n_tiles, 1), dtype=torch.float32, device=dev)
+        tmax = torch.empty(self.n_caches, max(n_tiles, 1), n_q_heads, dtype=torch.float32, device=dev)
         tsum = torch.empty_like(tmax)
         if scale_qk is None:
             scale_qk = 1.0 / (self.head_dim ** 0.5)
@@ -588,7 +588,7 @@ class CachePool:
         if nc != self.n_caches:
             raise ValueError("scores must have one slab per cache")
         n_tiles = (stride + SCORE_TILE - 1) // SCORE_TILE
-        if tile_max.shape != (nc, hq, max(n_tiles, 1)) or tile_sum.shape != tile_max.shape:
+        if tile_max.shape != (nc, max(n_tiles, 1), hq) or tile_sum.shape != tile_max.shape:
             raise ValueError("tile statistics do not match scores")
         dev = self.device
         imp = torch.zeros(nc, stride, dtype=torch.float32, device=dev) if return_importance else None
