@@ -381,6 +381,106 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
   }
 }
 
+// 64 experts and a long token stream: the classic tiled form.  A block owns 128 tokens
+// x 64 experts; its 256 threads bring KS k-values of every token row (256 contiguous
+// bytes per row, four whole rows per load instruction) through registers into one of two
+// LDS buffers while the matrix cores work on the other, one barrier per stage.  Wavefront
+// w owns expert tile w for all eight token tiles, so its B operands (the re-laid weights,
+// L2 hits) are 4 KB per stage and no partial sums have to meet at the end.  Rows are
+// padded by 16 bytes: the 16 rows that one ds_read_b128 phase touches then start 4 banks
+// apart.  Two blocks per compute unit (2 x 68 KB of LDS).  Requires H % KS == 0.  KS = 64
+// (four blocks of 36 KB per compute unit) measured slower at 65536 tokens: 512 blocks are
+// two per compute unit either way, and the narrower stage only halves the bytes each has
+// in flight.
+template <int KS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KS == 128 ? 2 : 4))) void router_gate_lds_kernel(
+    const void* __restrict__ x, const void* __restrict__ wb, int H, TailParams p) {
+  constexpr int EP = 64, TB = 128, WAVES = 4;
+  constexpr int ROW = KS * 2 + 16;  // bytes of one staged token row
+  constexpr int BUF = TB * ROW;
+  constexpr int CPR = KS / 8;        // 16-byte chunks per row
+  constexpr int RPP = 256 / CPR;     // rows per staging pass
+  constexpr int NP = TB / RPP;       // staging passes
+  constexpr int NK = KS / 32;        // k-steps per stage
+  constexpr int LDS_BYTES = 2 * BUF > TB * EP * 4 ? 2 * BUF : TB * EP * 4;
+  __shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];  // staging, then the block's logits
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 15, kg = lane >> 4;
+  const int64_t tok0 = (int64_t)blockIdx.x * TB;
+  // staging: thread -> 16-byte chunk (tid % CPR) of rows tid/CPR + RPP i
+  const int srow = tid / CPR, schunk = tid % CPR;
+  const char* xsrc[NP];
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    int64_t t = tok0 + srow + RPP * i;
+    if (t >= p.T) t = p.T - 1;  // rows past the end repeat the last token; the tail drops them
+    xsrc[i] = reinterpret_cast<const char*>(x) + (t * (int64_t)H) * 2 + schunk * 16;
+  }
+  char* swrite = lds + srow * ROW + schunk * 16;
+  const char* aread = lds + m * ROW + kg * 16;
+  const char* wlane = reinterpret_cast<const char*>(wb) + ((wave * 16 + m) * 32 + kg * 8) * 2;
+  pikv_f32x4 acc[8];
+#pragma unroll
+  for (int mt = 0; mt < 8; ++mt) acc[mt] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
+  uint4 areg[NP], bcur[NK], bnext[NK];
+  const int stages = H / KS;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) areg[i] = ld16(xsrc[i]);
+#pragma unroll
+  for (int ks = 0; ks < NK; ++ks) bcur[ks] = ld16(wlane + (int64_t)ks * EP * 64);
+#pragma unroll
+  for (int i = 0; i < NP; ++i) *reinterpret_cast<uint4*>(swrite + i * RPP * ROW) = areg[i];
+  __syncthreads();
+  for (int s = 0; s < stages; ++s) {
+    const int buf = (s & 1) * BUF;
+    const bool more = s + 1 < stages;
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < NP; ++i) areg[i] = ld16(xsrc[i] + (int64_t)(s + 1) * (KS * 2));
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) bnext[ks] = ld16(wlane + (int64_t)(NK * (s + 1) + ks) * EP * 64);
+    }
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks)
+#pragma unroll
+      for (int mt = 0; mt < 8; ++mt) {
+        const uint4 a = *reinterpret_cast<const uint4*>(aread + buf + mt * 16 * ROW + ks * 64);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, a),
+                                                          __builtin_bit_cast(pikv_bf16x8, bcur[ks]),
+                                                          acc[mt], 0, 0, 0);
+      }
+    if (more) {
+      // the other buffer was last read before the barrier that ended the previous stage
+#pragma unroll
+      for (int i = 0; i < NP; ++i) *reinterpret_cast<uint4*>(swrite + (BUF - buf) + i * RPP * ROW) = areg[i];
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) bcur[ks] = bnext[ks];
+    }
+    __syncthreads();
+  }
+  float (*red)[EP] = reinterpret_cast<float (*)[EP]>(lds);
+#pragma unroll
+  for (int mt = 0; mt < 8; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[mt * 16 + 4 * kg + i][wave * 16 + m] = acc[mt][i];
+  __syncthreads();
+  // wavefront w finishes tokens 32 w .. 32 w + 31, one token per 64 lanes, four side by side
+  // (eight side by side measured slower)
+  constexpr int TW = TB / WAVES;
+#pragma unroll 1
+  for (int c0 = 0; c0 < TW; c0 += 4) {
+    float lg[4];
+    int64_t tt[4];
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const int tl = TW * wave + c0 + n;
+      lg[n] = red[tl][lane];
+      tt[n] = tok0 + tl;
+    }
+    router_tail_multi<EP, 4>(lg, tt, lane, lane, p);
+  }
+}
+
 // ---- capacity slots -------------------------------------------------------------
 __global__ __launch_bounds__(256) void slot_hist_kernel(const int32_t* __restrict__ idx, int64_t A,
                                                         int E, int32_t* __restrict__ ws) {
@@ -590,9 +690,13 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
       const int64_t mb = (T + 63) / 64;
       if (mb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
       const dim3 grid((unsigned)mb);
-      if (ep == 64 && T >= 32768)
-        // enough tokens to fill the chip with 128-token blocks: the weights are re-read
-        // from L2 once per block, so twice the tokens per block halves that traffic
+      if (ep == 64 && T >= 32768 && H % 128 == 0)
+        // enough tokens to fill the chip with 128-token blocks, staged through LDS
+        hipLaunchKernelGGL(router_gate_lds_kernel<128>, dim3((unsigned)((T + 127) / 128)), dim3(256), 0, st, x,
+                           wb, H, p);
+      else if (ep == 64 && T >= 32768)
+        // 128-token blocks: the weights are re-read from L2 once per block, so twice the
+        // tokens per block halves that traffic
         hipLaunchKernelGGL((router_gate_mfma_kernel<4, 8, 4>), dim3((unsigned)((T + 127) / 128)), dim3(256), 0, st,
                            x, wb, H, p);
       else if (ep == 16)

@@ -109,6 +109,31 @@ def test_router_fused(dev, dtype, T, H, E, k):
     assert np.array_equal(np_of(out.count), count)
 
 
+@pytest.mark.parametrize("T,H,E,k", [(32768 + 37, 256, 64, 8), (32768, 128, 40, 3), (32768 + 5, 416, 64, 8),
+                                      (40000, 1152, 33, 1)])
+def test_router_many_experts_long_stream(dev, T, H, E, k):
+    """More than 32 experts and at least 32768 tokens take the 128-token block kernels (LDS-staged
+    when H % 128 == 0): ragged last block, one and several stages, padded expert columns."""
+    import torch
+    from pikv_amd import ops
+    g = torch.Generator(device=dev).manual_seed(T + H + E)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    w = (0.05 * torch.randn(E, H, generator=g, device=dev)).to(torch.bfloat16)
+    b = 0.1 * torch.randn(E, generator=g, device=dev)
+    cap = int(T * 1.25 * k / E)
+    out = ops.router_fused(x, w, b, top_k=k, capacity=cap, return_logits=True)
+    lg = x.double() @ w.double().T + b.double()
+    assert torch.allclose(out.logits.double(), lg, atol=1e-5 * H ** 0.5, rtol=1e-5)
+    assert torch.allclose(out.probs, torch.softmax(out.logits, dim=1), atol=1e-6)
+    order = torch.sort(out.logits, dim=1, descending=True, stable=True).indices[:, :k]
+    assert torch.equal(out.topk_idx.long(), order)
+    sel = torch.gather(out.probs, 1, order)
+    assert torch.allclose(out.topk_w, sel / sel.sum(1, keepdim=True), atol=1e-6)
+    slot, count = O.capacity_slots(np_of(out.topk_idx), E, cap)
+    assert np.array_equal(np_of(out.slot), slot)
+    assert np.array_equal(np_of(out.count), count)
+
+
 def test_router_module_arithmetic(dev):
     """The arithmetic of the reference's module/ copy (core/single/module/pikv_routing.py:596-600,
     :133-134, :143): scale before temperature, finfo.min penalty, + 1e-8 in the renormalisation -
