@@ -60,6 +60,29 @@ __device__ __forceinline__ float wave_transpose_reduce(float (&v)[64], int lane)
   return v[0];
 }
 
+// Bias, temperature, per-expert scale and mask penalty of expert e, in the order of the
+// chosen copy of the reference's routers.
+__device__ __forceinline__ float final_logit(float lg, int e, const TailParams& p) {
+  if (p.bias) lg = lg + p.bias[e];
+  if (p.arithmetic == PIKV_ROUTER_MODULE) {
+    // core/single/module/pikv_routing.py:596-600, :133-134
+    if (p.expert_scale) lg = lg * p.expert_scale[e];
+    if (p.temperature != 1.0f) lg = lg / p.temperature;
+    if (p.expert_mask) {
+      const float pen = (1.0f - p.expert_mask[e]) * -3.4028234663852886e38f;  // finfo(float32).min
+      lg = lg + pen;
+    }
+  } else {
+    if (p.temperature != 1.0f) lg = lg / p.temperature;
+    if (p.expert_scale) lg = lg * p.expert_scale[e];
+    if (p.expert_mask) {
+      const float pen = (1.0f - p.expert_mask[e]) * -1e9f;
+      lg = lg + pen;
+    }
+  }
+  return lg;
+}
+
 // Lane holds the raw logit of (token t, expert e); groups of EPAD adjacent lanes
 // form one token.  Writes probs / top-k for the token.
 // NTOK independent token groups go through the steps side by side: every step is a
@@ -73,23 +96,7 @@ __device__ __forceinline__ void router_tail_multi(float (&lg)[NTOK], const int64
   for (int n = 0; n < NTOK; ++n) {
     valid[n] = (t[n] < p.T) && (e < p.E);
     if (valid[n]) {
-      if (p.bias) lg[n] = lg[n] + p.bias[e];
-      if (p.arithmetic == PIKV_ROUTER_MODULE) {
-        // core/single/module/pikv_routing.py:596-600, :133-134
-        if (p.expert_scale) lg[n] = lg[n] * p.expert_scale[e];
-        if (p.temperature != 1.0f) lg[n] = lg[n] / p.temperature;
-        if (p.expert_mask) {
-          const float pen = (1.0f - p.expert_mask[e]) * -3.4028234663852886e38f;  // finfo(float32).min
-          lg[n] = lg[n] + pen;
-        }
-      } else {
-        if (p.temperature != 1.0f) lg[n] = lg[n] / p.temperature;
-        if (p.expert_scale) lg[n] = lg[n] * p.expert_scale[e];
-        if (p.expert_mask) {
-          const float pen = (1.0f - p.expert_mask[e]) * -1e9f;
-          lg[n] = lg[n] + pen;
-        }
-      }
+      lg[n] = final_logit(lg[n], e, p);
       if (p.logits_out) p.logits_out[t[n] * p.E + e] = lg[n];
     } else {
       lg[n] = -__builtin_inff();
@@ -381,6 +388,112 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
   }
 }
 
+// ---- one token per LANE: softmax and top-k of 64 logits held in LDS ------------------
+// A cross-lane arg-max round costs ~27 instructions per token and round; with a token per
+// lane the same work is compare-exchanges on registers, 64 tokens per instruction.
+// Order key: (float order with -0 = +0 and NaN below -inf, then the LOWER expert first)
+// packed as one 64-bit integer, larger = earlier.  0 marks a padding column.
+__device__ __forceinline__ uint64_t lane_topk_key(float v, int e) {
+  uint32_t k;
+  if (v != v) {
+    k = 1u;
+  } else {
+    const uint32_t u = __float_as_uint(v + 0.0f);  // -0 + 0 = +0
+    k = (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // >= 0x007fffff (-inf)
+  }
+  return ((uint64_t)k << 32) | (uint32_t)(63 - e);
+}
+__device__ __forceinline__ void ce_desc(uint64_t& a, uint64_t& b) {
+  const bool sw = b > a;
+  const uint64_t hi = sw ? b : a;
+  b = sw ? a : b;
+  a = hi;
+}
+// 19-comparator network for eight keys, descending
+__device__ __forceinline__ void sort8_desc(uint64_t (&v)[8]) {
+  ce_desc(v[0], v[2]); ce_desc(v[1], v[3]); ce_desc(v[4], v[6]); ce_desc(v[5], v[7]);
+  ce_desc(v[0], v[4]); ce_desc(v[1], v[5]); ce_desc(v[2], v[6]); ce_desc(v[3], v[7]);
+  ce_desc(v[0], v[1]); ce_desc(v[2], v[3]); ce_desc(v[4], v[5]); ce_desc(v[6], v[7]);
+  ce_desc(v[2], v[4]); ce_desc(v[3], v[5]);
+  ce_desc(v[1], v[4]); ce_desc(v[3], v[6]);
+  ce_desc(v[1], v[2]); ce_desc(v[3], v[4]); ce_desc(v[5], v[6]);
+}
+// top = the eight largest of two descending lists: max(top[i], other[7-i]) is that set as a
+// bitonic sequence, three half-cleaner stages sort it
+__device__ __forceinline__ void merge_top8(uint64_t (&top)[8], const uint64_t (&other)[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) top[i] = top[i] > other[7 - i] ? top[i] : other[7 - i];
+  ce_desc(top[0], top[4]); ce_desc(top[1], top[5]); ce_desc(top[2], top[6]); ce_desc(top[3], top[7]);
+  ce_desc(top[0], top[2]); ce_desc(top[1], top[3]); ce_desc(top[4], top[6]); ce_desc(top[5], top[7]);
+  ce_desc(top[0], top[1]); ce_desc(top[2], top[3]); ce_desc(top[4], top[5]); ce_desc(top[6], top[7]);
+}
+// Sum of 16 values in the order of the DPP row reduction (pairs, quads, halves, row)
+__device__ __forceinline__ float tree16(const float* a) {
+  const float q0 = (a[0] + a[1]) + (a[2] + a[3]), q1 = (a[4] + a[5]) + (a[6] + a[7]);
+  const float q2 = (a[8] + a[9]) + (a[10] + a[11]), q3 = (a[12] + a[13]) + (a[14] + a[15]);
+  return (q0 + q1) + (q2 + q3);
+}
+
+// Row `row` (stride RS floats) holds the final logits of one token, -inf in the padding
+// columns e >= E.  Leaves the probabilities in the row and writes the token's top-k.
+// Same arithmetic, in the same order, as the lane-per-expert tail: max, expf(l - max), the
+// balanced sum, one division per expert; weights = p / (sum of the selected p, largest first).
+template <int RS>
+__device__ __forceinline__ void lane_token_tail(float* row, int64_t t, const TailParams& p) {
+  uint64_t top[8];
+#pragma unroll
+  for (int g = 0; g < 8; ++g) {
+    uint64_t cur[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int e = 8 * g + i;
+      cur[i] = e < p.E ? lane_topk_key(row[e], e) : 0ull;
+    }
+    sort8_desc(cur);
+    if (g == 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) top[i] = cur[i];
+    } else {
+      merge_top8(top, cur);
+    }
+  }
+  int idx[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) idx[j] = 63 - (int)(uint32_t)top[j];
+  const float m = row[idx[0]];
+  float ex[64];
+#pragma unroll
+  for (int e = 0; e < 64; ++e) ex[e] = e < p.E ? expf(row[e] - m) : 0.f;
+  const float sum = (tree16(ex) + tree16(ex + 16)) + (tree16(ex + 32) + tree16(ex + 48));
+#pragma unroll
+  for (int e = 0; e < 64; ++e) row[e] = ex[e] / sum;
+  float pv[8], wsum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    pv[j] = j < p.k ? row[idx[j]] : 0.f;
+    if (j < p.k) wsum = wsum + pv[j];
+  }
+  if (p.renorm_eps != 0.f) wsum = wsum + p.renorm_eps;
+  if (t < p.T) {
+    if (p.k == 8) {
+      // 32 contiguous, 16-byte aligned bytes per token
+      int4* oi = reinterpret_cast<int4*>(p.topk_idx + t * 8);
+      float4* ow = reinterpret_cast<float4*>(p.topk_w + t * 8);
+      oi[0] = make_int4(idx[0], idx[1], idx[2], idx[3]);
+      oi[1] = make_int4(idx[4], idx[5], idx[6], idx[7]);
+      ow[0] = make_float4(pv[0] / wsum, pv[1] / wsum, pv[2] / wsum, pv[3] / wsum);
+      ow[1] = make_float4(pv[4] / wsum, pv[5] / wsum, pv[6] / wsum, pv[7] / wsum);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (j < p.k) {
+          p.topk_idx[t * p.k + j] = idx[j];
+          p.topk_w[t * p.k + j] = pv[j] / wsum;
+        }
+    }
+  }
+}
+
 // 64 experts and a long token stream: the classic tiled form.  A block owns 128 tokens
 // x 64 experts; its 256 threads bring KS k-values of every token row (256 contiguous
 // bytes per row, four whole rows per load instruction) through registers into one of two
@@ -388,7 +501,8 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
 // w owns expert tile w for all eight token tiles, so its B operands (the re-laid weights,
 // L2 hits) are 4 KB per stage and no partial sums have to meet at the end.  Rows are
 // padded by 16 bytes: the 16 rows that one ds_read_b128 phase touches then start 4 banks
-// apart.  Two blocks per compute unit (2 x 68 KB of LDS).  Requires H % KS == 0.  KS = 64
+// apart.  Two blocks per compute unit (2 x 68 KB of LDS).  Requires H % KS == 0 and the
+// softmax form of the tail.  KS = 64
 // (four blocks of 36 KB per compute unit) measured slower at 65536 tokens: 512 blocks are
 // two per compute unit either way, and the narrower stage only halves the bytes each has
 // in flight.
@@ -458,26 +572,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KS == 128 ?
     }
     __syncthreads();
   }
-  float (*red)[EP] = reinterpret_cast<float (*)[EP]>(lds);
+  // The block's logits, one row of RS floats per token (RS odd: a lane per token and a lane
+  // per expert both walk the banks without conflicts).
+  constexpr int RS = EP + 1;
+  static_assert(TB * RS * 4 <= LDS_BYTES, "the logits of the block reuse the staging buffers");
+  float* red = reinterpret_cast<float*>(lds);
 #pragma unroll
   for (int mt = 0; mt < 8; ++mt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[mt * 16 + 4 * kg + i][wave * 16 + m] = acc[mt][i];
+    for (int i = 0; i < 4; ++i) red[(mt * 16 + 4 * kg + i) * RS + wave * 16 + m] = acc[mt][i];
   __syncthreads();
-  // wavefront w finishes tokens 32 w .. 32 w + 31, one token per 64 lanes, four side by side
-  // (eight side by side measured slower)
+  // lane = expert: bias / temperature / scale / mask, the logits output
   constexpr int TW = TB / WAVES;
-#pragma unroll 1
-  for (int c0 = 0; c0 < TW; c0 += 4) {
-    float lg[4];
-    int64_t tt[4];
-#pragma unroll
-    for (int n = 0; n < 4; ++n) {
-      const int tl = TW * wave + c0 + n;
-      lg[n] = red[tl][lane];
-      tt[n] = tok0 + tl;
+  for (int i = 0; i < TW; ++i) {
+    const int tl = TW * wave + i;
+    const int64_t t = tok0 + tl;
+    float lg = -__builtin_inff();
+    if (lane < p.E) {
+      lg = final_logit(red[tl * RS + lane], lane, p);
+      if (p.logits_out && t < p.T) p.logits_out[t * p.E + lane] = lg;
     }
-    router_tail_multi<EP, 4>(lg, tt, lane, lane, p);
+    red[tl * RS + lane] = lg;
+  }
+  __syncthreads();
+  // lane = token: softmax and top-k of a whole row on registers (two of the four wavefronts)
+  if (tid < TB) lane_token_tail<RS>(red + tid * RS, tok0 + tid, p);
+  __syncthreads();
+  if (p.probs) {
+    for (int i = 0; i < TW; ++i) {
+      const int tl = TW * wave + i;
+      const int64_t t = tok0 + tl;
+      if (lane < p.E && t < p.T) p.probs[t * p.E + lane] = red[tl * RS + lane];
+    }
   }
 }
 
