@@ -19,6 +19,7 @@
 namespace pikv {
 
 constexpr int kSlotChunk = 512;  // assignments per block in the slot pass
+constexpr int kRowsTailMinK = 5;  // standalone tail, 33-64 experts: a token per lane from this k on
 
 struct TailParams {
   const float* bias;
@@ -61,26 +62,53 @@ __device__ __forceinline__ float wave_transpose_reduce(float (&v)[64], int lane)
 }
 
 // Bias, temperature, per-expert scale and mask penalty of expert e, in the order of the
-// chosen copy of the reference's routers.
-__device__ __forceinline__ float final_logit(float lg, int e, const TailParams& p) {
-  if (p.bias) lg = lg + p.bias[e];
+// chosen copy of the reference's routers.  The per-expert numbers are loaded once per lane.
+struct ExpertConsts {
+  float bias, scale, penalty;
+};
+// Absent vectors load as the neutral elements -0 (x + -0 == x bit for bit), 1 and -0.
+__device__ __forceinline__ ExpertConsts load_expert_consts(int e, const TailParams& p) {
+  ExpertConsts c{-0.f, 1.f, -0.f};
+  if (e < p.E) {
+    if (p.bias) c.bias = p.bias[e];
+    if (p.expert_scale) c.scale = p.expert_scale[e];
+    if (p.expert_mask)
+      c.penalty = (1.0f - p.expert_mask[e]) * (p.arithmetic == PIKV_ROUTER_MODULE
+                                                    ? -3.4028234663852886e38f  // finfo(float32).min
+                                                    : -1e9f);
+  }
+  return c;
+}
+__device__ __forceinline__ float final_logit(float lg, const ExpertConsts& c, const TailParams& p) {
+  if (p.bias) lg = lg + c.bias;
   if (p.arithmetic == PIKV_ROUTER_MODULE) {
     // core/single/module/pikv_routing.py:596-600, :133-134
-    if (p.expert_scale) lg = lg * p.expert_scale[e];
+    if (p.expert_scale) lg = lg * c.scale;
     if (p.temperature != 1.0f) lg = lg / p.temperature;
-    if (p.expert_mask) {
-      const float pen = (1.0f - p.expert_mask[e]) * -3.4028234663852886e38f;  // finfo(float32).min
-      lg = lg + pen;
-    }
+    if (p.expert_mask) lg = lg + c.penalty;
   } else {
+    // core/single/pikv_routing.py:653-656, :68-70
     if (p.temperature != 1.0f) lg = lg / p.temperature;
-    if (p.expert_scale) lg = lg * p.expert_scale[e];
-    if (p.expert_mask) {
-      const float pen = (1.0f - p.expert_mask[e]) * -1e9f;
-      lg = lg + pen;
-    }
+    if (p.expert_scale) lg = lg * c.scale;
+    if (p.expert_mask) lg = lg + c.penalty;
   }
   return lg;
+}
+// The same without branches, for loops over many rows: MODE 0 = temperature 1 (both orders
+// coincide), 1 = divide then scale (single/), 2 = scale then divide (module/).
+template <int MODE>
+__device__ __forceinline__ float final_logit_rows(float lg, const ExpertConsts& c, float temperature) {
+  lg = lg + c.bias;
+  if (MODE == 1) lg = lg / temperature;
+  lg = lg * c.scale;
+  if (MODE == 2) lg = lg / temperature;
+  return lg + c.penalty;
+}
+__device__ __forceinline__ int final_logit_mode(const TailParams& p) {
+  return p.temperature == 1.0f ? 0 : (p.arithmetic == PIKV_ROUTER_MODULE ? 2 : 1);
+}
+__device__ __forceinline__ float final_logit(float lg, int e, const TailParams& p) {
+  return final_logit(lg, load_expert_consts(e, p), p);
 }
 
 // Lane holds the raw logit of (token t, expert e); groups of EPAD adjacent lanes
@@ -392,7 +420,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
 // A cross-lane arg-max round costs ~27 instructions per token and round; with a token per
 // lane the same work is compare-exchanges on registers, 64 tokens per instruction.
 // Order key: (float order with -0 = +0 and NaN below -inf, then the LOWER expert first)
-// packed as one 64-bit integer, larger = earlier.  0 marks a padding column.
+// packed as one 64-bit integer, larger = earlier.  0 marks a padding column (below NaN).
 __device__ __forceinline__ uint64_t lane_topk_key(float v, int e) {
   uint32_t k;
   if (v != v) {
@@ -435,7 +463,8 @@ __device__ __forceinline__ float tree16(const float* a) {
 }
 
 // Row `row` (stride RS floats) holds the final logits of one token, -inf in the padding
-// columns e >= E.  Leaves the probabilities in the row and writes the token's top-k.
+// columns e >= E.  Leaves the probabilities in the row and writes the token's top-k
+// (without the softmax: the top-k of the logits, nothing else).
 // Same arithmetic, in the same order, as the lane-per-expert tail: max, expf(l - max), the
 // balanced sum, one division per expert; weights = p / (sum of the selected p, largest first).
 template <int RS>
@@ -460,10 +489,21 @@ __device__ __forceinline__ void lane_token_tail(float* row, int64_t t, const Tai
   int idx[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) idx[j] = 63 - (int)(uint32_t)top[j];
+  if (!p.use_softmax) {  // raw top-k: the selected logits themselves
+    if (t < p.T) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (j < p.k) {
+          p.topk_idx[t * p.k + j] = idx[j];
+          p.topk_w[t * p.k + j] = row[idx[j]];
+        }
+    }
+    return;
+  }
   const float m = row[idx[0]];
   float ex[64];
 #pragma unroll
-  for (int e = 0; e < 64; ++e) ex[e] = e < p.E ? expf(row[e] - m) : 0.f;
+  for (int e = 0; e < 64; ++e) ex[e] = expf(row[e] - m);  // padding: expf(-inf) = 0
   const float sum = (tree16(ex) + tree16(ex + 16)) + (tree16(ex + 32) + tree16(ex + 48));
 #pragma unroll
   for (int e = 0; e < 64; ++e) row[e] = ex[e] / sum;
@@ -518,7 +558,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KS == 128 ?
   constexpr int NK = KS / 32;        // k-steps per stage
   constexpr int LDS_BYTES = 2 * BUF > TB * EP * 4 ? 2 * BUF : TB * EP * 4;
   __shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];  // staging, then the block's logits
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform
   const int m = lane & 15, kg = lane >> 4;
   const int64_t tok0 = (int64_t)blockIdx.x * TB;
   // staging: thread -> 16-byte chunk (tid % CPR) of rows tid/CPR + RPP i
@@ -584,15 +625,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KS == 128 ?
   __syncthreads();
   // lane = expert: bias / temperature / scale / mask, the logits output
   constexpr int TW = TB / WAVES;
-  for (int i = 0; i < TW; ++i) {
-    const int tl = TW * wave + i;
-    const int64_t t = tok0 + tl;
-    float lg = -__builtin_inff();
-    if (lane < p.E) {
-      lg = final_logit(red[tl * RS + lane], lane, p);
-      if (p.logits_out && t < p.T) p.logits_out[t * p.E + lane] = lg;
+  {
+    const ExpertConsts ec = load_expert_consts(lane, p);
+    const int mode = final_logit_mode(p);
+    const bool col = lane < p.E;
+    for (int i = 0; i < TW; ++i) {
+      const int tl = TW * wave + i;
+      const int64_t t = tok0 + tl;
+      const float raw = red[tl * RS + lane];
+      float lg = mode == 0 ? final_logit_rows<0>(raw, ec, p.temperature)
+                 : mode == 1 ? final_logit_rows<1>(raw, ec, p.temperature)
+                             : final_logit_rows<2>(raw, ec, p.temperature);
+      if (!col) lg = -__builtin_inff();
+      if (p.logits_out && col && t < p.T) p.logits_out[t * p.E + lane] = lg;
+      red[tl * RS + lane] = lg;
     }
-    red[tl * RS + lane] = lg;
   }
   __syncthreads();
   // lane = token: softmax and top-k of a whole row on registers (two of the four wavefronts)
@@ -603,6 +650,63 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KS == 128 ?
       const int tl = TW * wave + i;
       const int64_t t = tok0 + tl;
       if (lane < p.E && t < p.T) p.probs[t * p.E + lane] = red[tl * RS + lane];
+    }
+  }
+}
+
+// Router tail on precomputed logits, 33-64 experts: 128 tokens per block go through LDS as
+// [token][65] - read and written with a lane per expert (coalesced), finished with a lane
+// per token.
+template <int MODE>
+__device__ __forceinline__ void tail_rows_stage(const float* __restrict__ la, const float* __restrict__ lb,
+                                                uint64_t from_a, int64_t tbase, int wave, int lane,
+                                                float* red, const TailParams& p) {
+  constexpr int RS = 65;
+  const ExpertConsts ec = load_expert_consts(lane, p);
+  const bool col = lane < p.E;
+  for (int i0 = 0; i0 < 64; i0 += 16) {
+    float v[16];  // sixteen rows in flight per wavefront
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int64_t t = tbase + i0 + u;
+      const float* src = ((from_a >> (i0 + u)) & 1ull) ? la : lb;
+      v[u] = (t < p.T && col) ? src[t * p.E + lane] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int tl = 64 * wave + i0 + u;
+      const float lg = final_logit_rows<MODE>(v[u], ec, p.temperature);
+      red[tl * RS + lane] = (tbase + i0 + u < p.T && col) ? lg : -__builtin_inff();
+    }
+  }
+}
+
+__global__ __launch_bounds__(128) void router_tail_rows_kernel(const float* __restrict__ la,
+                                                               const float* __restrict__ lb,
+                                                               const uint8_t* __restrict__ select,
+                                                               TailParams p) {
+  constexpr int TB = 128, RS = 65;
+  __shared__ float red[TB * RS];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: row addresses stay scalar
+  const int64_t tok0 = (int64_t)blockIdx.x * TB;
+  const int64_t tbase = tok0 + 64 * wave;  // first token of this wavefront
+  uint64_t from_a = ~0ull;                 // bit i: token tbase + i reads logits_a
+  if (lb != nullptr && select != nullptr) {
+    const int64_t t = tbase + lane;
+    from_a = __ballot(t < p.T ? select[t] != 0 : true);
+  }
+  const int mode = final_logit_mode(p);
+  if (mode == 0) tail_rows_stage<0>(la, lb, from_a, tbase, wave, lane, red, p);
+  else if (mode == 1) tail_rows_stage<1>(la, lb, from_a, tbase, wave, lane, red, p);
+  else tail_rows_stage<2>(la, lb, from_a, tbase, wave, lane, red, p);
+  __syncthreads();
+  lane_token_tail<RS>(red + tid * RS, tok0 + tid, p);
+  __syncthreads();
+  if (p.probs) {
+    for (int i = 0; i < 64; ++i) {
+      const int64_t t = tbase + i;
+      if (t < p.T && lane < p.E) p.probs[t * p.E + lane] = red[(64 * wave + i) * RS + lane];
     }
   }
 }
@@ -869,7 +973,14 @@ extern "C" int pikv_router_tail(const float* logits_a, const float* logits_b, co
       case 8: hipLaunchKernelGGL((router_tail_kernel<8>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p); break;
       case 16: hipLaunchKernelGGL((router_tail_kernel<16>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p); break;
       case 32: hipLaunchKernelGGL((router_tail_kernel<32>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p); break;
-      default: hipLaunchKernelGGL((router_tail_kernel<64>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p); break;
+      default:
+        // 33-64 experts: an arg-max round over 64 lanes costs ~2.9 us per round at 65536 tokens
+        // (20 us at k = 1), a token per lane 31 us whatever k
+        if (k >= kRowsTailMinK)
+          hipLaunchKernelGGL(router_tail_rows_kernel, dim3((unsigned)((T + 127) / 128)), dim3(128), 0, st, logits_a, logits_b, select, p);
+        else
+          hipLaunchKernelGGL((router_tail_kernel<64>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p);
+        break;
     }
     PIKV_CHECK_LAUNCH();
   }

@@ -18,7 +18,7 @@ from util import np_of, rng, to_dev
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("E,k", [(4, 2), (8, 2), (6, 3), (16, 4), (64, 8), (33, 1), (1, 1)])
+@pytest.mark.parametrize("E,k", [(4, 2), (8, 2), (6, 3), (16, 4), (64, 8), (33, 1), (1, 1), (48, 5), (40, 8), (64, 2), (64, 5), (33, 6)])
 def test_router_tail_bit_exact(dev, E, k):
     from pikv_amd import ops
     r = rng(E * 10 + k)
