@@ -58,6 +58,47 @@ def test_router_tail_bit_exact(dev, E, k):
     assert np.array_equal(np_of(out.topk_w), vals)
 
 
+@pytest.mark.parametrize("E", [40, 64])
+def test_router_tail_special_values_both_forms(dev, E):
+    """33-64 experts are served by arg-max rounds below k = 5 and by the token-per-lane sort from
+    k = 5 on: on rows with NaN, +-inf, signed zeros and many ties the top-4 of one must be the
+    first four of the other's top-8, and NaN is picked last, lowest index first."""
+    from pikv_amd import ops
+    r = rng(E)
+    T = 512
+    lg = r.standard_normal((T, E)).astype(np.float32)
+    lg[0] = 0.0
+    lg[1, ::2] = -0.0
+    lg[1, 1::2] = 0.0
+    lg[2] = np.nan
+    lg[3, : E - 3] = np.nan                      # three numbers, the rest NaN
+    lg[4] = -np.inf
+    lg[4, 7] = 1.0
+    lg[5, ::3] = np.inf
+    lg[6, 5] = np.nan
+    lg[7] = np.round(lg[7])
+    lg[8:64] = np.round(lg[8:64] * 2) / 2
+    lg[64:80, 3] = np.nan
+    lg[64:80, 9] = -np.inf
+    d = to_dev(lg, dev)
+    a = np_of(ops.router_tail(d, top_k=4, use_softmax=False).topk_idx)
+    b = np_of(ops.router_tail(d, top_k=8, use_softmax=False).topk_idx)
+    assert np.array_equal(a, b[:, :4])
+    assert ((b >= 0) & (b < E)).all()
+    assert all(len(set(row)) == 8 for row in b)
+    assert list(b[0]) == list(range(8)) and list(b[1]) == list(range(8)) and list(b[2]) == list(range(8))
+    assert sorted(b[3][:3]) == [E - 3, E - 2, E - 1] and list(b[3][3:]) == [0, 1, 2, 3, 4]
+    assert b[4][0] == 7 and list(b[4][1:]) == [0, 1, 2, 3, 4, 5, 6]
+    assert list(b[5]) == [0, 3, 6, 9, 12, 15, 18, 21]
+    assert 5 not in b[6]
+    # with the softmax: same selection, probabilities of the two forms bit-identical on finite rows
+    fin = np.isfinite(lg).all(axis=1)
+    oa = ops.router_tail(d, top_k=4)
+    ob = ops.router_tail(d, top_k=8)
+    assert np.array_equal(np_of(oa.topk_idx)[fin], np_of(ob.topk_idx)[fin][:, :4])
+    assert np.array_equal(np_of(oa.probs)[fin], np_of(ob.probs)[fin])
+
+
 @pytest.mark.parametrize("A,E,cap", [(1, 4, 1), (2047, 8, 100), (2049, 8, 3), (100000, 64, 1500),
                                       (65536, 8, 10240), (5000, 3, 0)])
 def test_capacity_slots_exact(dev, A, E, cap):
