@@ -467,11 +467,12 @@ __device__ __forceinline__ float tree16(const float* a) {
 // (without the softmax: the top-k of the logits, nothing else).
 // Same arithmetic, in the same order, as the lane-per-expert tail: max, expf(l - max), the
 // balanced sum, one division per expert; weights = p / (sum of the selected p, largest first).
-template <int RS>
+template <int EP, int RS>
 __device__ __forceinline__ void lane_token_tail(float* row, int64_t t, const TailParams& p) {
+  static_assert(EP == 16 || EP == 32 || EP == 64, "rows of 16, 32 or 64 columns");
   uint64_t top[8];
 #pragma unroll
-  for (int g = 0; g < 8; ++g) {
+  for (int g = 0; g < EP / 8; ++g) {
     uint64_t cur[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -489,77 +490,88 @@ __device__ __forceinline__ void lane_token_tail(float* row, int64_t t, const Tai
   int idx[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) idx[j] = 63 - (int)(uint32_t)top[j];
-  if (!p.use_softmax) {  // raw top-k: the selected logits themselves
-    if (t < p.T) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        if (j < p.k) {
-          p.topk_idx[t * p.k + j] = idx[j];
-          p.topk_w[t * p.k + j] = row[idx[j]];
-        }
-    }
-    return;
-  }
-  const float m = row[idx[0]];
-  float ex[64];
-#pragma unroll
-  for (int e = 0; e < 64; ++e) ex[e] = expf(row[e] - m);  // padding: expf(-inf) = 0
-  const float sum = (tree16(ex) + tree16(ex + 16)) + (tree16(ex + 32) + tree16(ex + 48));
-#pragma unroll
-  for (int e = 0; e < 64; ++e) row[e] = ex[e] / sum;
   float pv[8], wsum = 0.f;
+  if (p.use_softmax) {
+    const float m = row[idx[0]];
+    float ex[EP];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    pv[j] = j < p.k ? row[idx[j]] : 0.f;
-    if (j < p.k) wsum = wsum + pv[j];
-  }
-  if (p.renorm_eps != 0.f) wsum = wsum + p.renorm_eps;
-  if (t < p.T) {
-    if (p.k == 8) {
-      // 32 contiguous, 16-byte aligned bytes per token
-      int4* oi = reinterpret_cast<int4*>(p.topk_idx + t * 8);
-      float4* ow = reinterpret_cast<float4*>(p.topk_w + t * 8);
-      oi[0] = make_int4(idx[0], idx[1], idx[2], idx[3]);
-      oi[1] = make_int4(idx[4], idx[5], idx[6], idx[7]);
-      ow[0] = make_float4(pv[0] / wsum, pv[1] / wsum, pv[2] / wsum, pv[3] / wsum);
-      ow[1] = make_float4(pv[4] / wsum, pv[5] / wsum, pv[6] / wsum, pv[7] / wsum);
-    } else {
+    for (int e = 0; e < EP; ++e) ex[e] = expf(row[e] - m);  // padding: expf(-inf) = 0
+    float sum = tree16(ex);
+    if constexpr (EP == 32) sum = sum + tree16(ex + 16);
+    if constexpr (EP == 64) sum = (sum + tree16(ex + 16)) + (tree16(ex + 32) + tree16(ex + 48));
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        if (j < p.k) {
-          p.topk_idx[t * p.k + j] = idx[j];
-          p.topk_w[t * p.k + j] = pv[j] / wsum;
-        }
+    for (int e = 0; e < EP; ++e) row[e] = ex[e] / sum;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      pv[j] = j < p.k ? row[idx[j]] : 0.f;
+      if (j < p.k) wsum = wsum + pv[j];
     }
+    if (p.renorm_eps != 0.f) wsum = wsum + p.renorm_eps;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pv[j] = pv[j] / wsum;
+  } else {  // raw top-k: the selected logits themselves
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pv[j] = j < p.k ? row[idx[j]] : 0.f;
+  }
+  if (t >= p.T) return;
+  // k values per token, contiguous over the lanes
+  if (p.k == 8) {
+    int4* oi = reinterpret_cast<int4*>(p.topk_idx + t * 8);
+    float4* ow = reinterpret_cast<float4*>(p.topk_w + t * 8);
+    oi[0] = make_int4(idx[0], idx[1], idx[2], idx[3]);
+    oi[1] = make_int4(idx[4], idx[5], idx[6], idx[7]);
+    ow[0] = make_float4(pv[0], pv[1], pv[2], pv[3]);
+    ow[1] = make_float4(pv[4], pv[5], pv[6], pv[7]);
+  } else if (p.k == 4) {
+    *reinterpret_cast<int4*>(p.topk_idx + t * 4) = make_int4(idx[0], idx[1], idx[2], idx[3]);
+    *reinterpret_cast<float4*>(p.topk_w + t * 4) = make_float4(pv[0], pv[1], pv[2], pv[3]);
+  } else if (p.k == 2) {
+    *reinterpret_cast<int2*>(p.topk_idx + t * 2) = make_int2(idx[0], idx[1]);
+    *reinterpret_cast<float2*>(p.topk_w + t * 2) = make_float2(pv[0], pv[1]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < p.k) {
+        p.topk_idx[t * p.k + j] = idx[j];
+        p.topk_w[t * p.k + j] = pv[j];
+      }
   }
 }
 
-// 64 experts and a long token stream: the classic tiled form.  A block owns 128 tokens
-// x 64 experts; its 256 threads bring KS k-values of every token row (256 contiguous
-// bytes per row, four whole rows per load instruction) through registers into one of two
-// LDS buffers while the matrix cores work on the other, one barrier per stage.  Wavefront
-// w owns expert tile w for all eight token tiles, so its B operands (the re-laid weights,
-// L2 hits) are 4 KB per stage and no partial sums have to meet at the end.  Rows are
-// padded by 16 bytes: the 16 rows that one ds_read_b128 phase touches then start 4 banks
-// apart.  Two blocks per compute unit (2 x 68 KB of LDS).  Requires H % KS == 0 and the
-// softmax form of the tail.  KS = 64
-// (four blocks of 36 KB per compute unit) measured slower at 65536 tokens: 512 blocks are
-// two per compute unit either way, and the narrower stage only halves the bytes each has
-// in flight.
-template <int KS>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KS == 128 ? 2 : 4))) void router_gate_lds_kernel(
+// Long token streams: the classic tiled form.  A block owns TB tokens x EP (padded)
+// experts; its 256 threads bring KS k-values of every token row (256 or 512 contiguous
+// bytes per row, whole rows per load instruction) through registers into one of two LDS
+// buffers while the matrix cores work on the other, one barrier per stage.  The 16 x 16
+// output tiles are dealt to the four wavefronts along the experts first (64 experts:
+// wavefront w owns expert tile w for all eight token tiles), so a wavefront's B operands
+// (the re-laid weights, L2 hits) are at most 4 KB per stage and no partial sums have to
+// meet at the end.  Rows are padded by 16 bytes: the 16 rows that one ds_read_b128 phase
+// touches then start 4 banks apart.  Two blocks per compute unit (2 x 68 KB of LDS).
+// Requires H % KS == 0 and the softmax form of the tail.  128 tokens x 64-wide stages (four
+// blocks of 36 KB per compute unit) measured slower at 65536 tokens x 64 experts: 512 blocks
+// are two per compute unit either way, and the narrower stage only halves the bytes each
+// has in flight.
+template <int EP, int TB, int KS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void router_gate_lds_kernel(
     const void* __restrict__ x, const void* __restrict__ wb, int H, TailParams p) {
-  constexpr int EP = 64, TB = 128, WAVES = 4;
+  constexpr int WAVES = 4;
+  constexpr int NT = EP / 16, MT = TB / 16;  // expert and token tiles of the block
+  constexpr int WE = NT < WAVES ? NT : WAVES;  // wavefronts along the experts
+  constexpr int WT = WAVES / WE;               // ... and along the tokens
+  constexpr int MTW = MT / WT;                 // token tiles per wavefront (one expert tile each)
+  static_assert(NT <= WAVES && MT % WT == 0, "one expert tile per wavefront");
   constexpr int ROW = KS * 2 + 16;  // bytes of one staged token row
   constexpr int BUF = TB * ROW;
   constexpr int CPR = KS / 8;        // 16-byte chunks per row
   constexpr int RPP = 256 / CPR;     // rows per staging pass
   constexpr int NP = TB / RPP;       // staging passes
   constexpr int NK = KS / 32;        // k-steps per stage
-  constexpr int LDS_BYTES = 2 * BUF > TB * EP * 4 ? 2 * BUF : TB * EP * 4;
+  constexpr int RS = EP + 1;         // floats per token row of the block's logits
+  constexpr int LDS_BYTES = 2 * BUF > TB * RS * 4 ? 2 * BUF : TB * RS * 4;
   __shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];  // staging, then the block's logits
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform
+  const int we = wave % WE, wt = wave / WE;
   const int m = lane & 15, kg = lane >> 4;
   const int64_t tok0 = (int64_t)blockIdx.x * TB;
   // staging: thread -> 16-byte chunk (tid % CPR) of rows tid/CPR + RPP i
@@ -572,11 +584,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KS == 128 ?
     xsrc[i] = reinterpret_cast<const char*>(x) + (t * (int64_t)H) * 2 + schunk * 16;
   }
   char* swrite = lds + srow * ROW + schunk * 16;
-  const char* aread = lds + m * ROW + kg * 16;
-  const char* wlane = reinterpret_cast<const char*>(wb) + ((wave * 16 + m) * 32 + kg * 8) * 2;
-  pikv_f32x4 acc[8];
+  const char* aread = lds + (wt * MTW * 16 + m) * ROW + kg * 16;
+  const char* wlane = reinterpret_cast<const char*>(wb) + ((we * 16 + m) * 32 + kg * 8) * 2;
+  pikv_f32x4 acc[MTW];
 #pragma unroll
-  for (int mt = 0; mt < 8; ++mt) acc[mt] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int mt = 0; mt < MTW; ++mt) acc[mt] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
   uint4 areg[NP], bcur[NK], bnext[NK];
   const int stages = H / KS;
 #pragma unroll
@@ -598,7 +610,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KS == 128 ?
 #pragma unroll
     for (int ks = 0; ks < NK; ++ks)
 #pragma unroll
-      for (int mt = 0; mt < 8; ++mt) {
+      for (int mt = 0; mt < MTW; ++mt) {
         const uint4 a = *reinterpret_cast<const uint4*>(aread + buf + mt * 16 * ROW + ks * 64);
         acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, a),
                                                           __builtin_bit_cast(pikv_bf16x8, bcur[ks]),
@@ -615,41 +627,42 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KS == 128 ?
   }
   // The block's logits, one row of RS floats per token (RS odd: a lane per token and a lane
   // per expert both walk the banks without conflicts).
-  constexpr int RS = EP + 1;
-  static_assert(TB * RS * 4 <= LDS_BYTES, "the logits of the block reuse the staging buffers");
   float* red = reinterpret_cast<float*>(lds);
 #pragma unroll
-  for (int mt = 0; mt < 8; ++mt)
+  for (int mt = 0; mt < MTW; ++mt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[(mt * 16 + 4 * kg + i) * RS + wave * 16 + m] = acc[mt][i];
+    for (int i = 0; i < 4; ++i) red[((wt * MTW + mt) * 16 + 4 * kg + i) * RS + we * 16 + m] = acc[mt][i];
   __syncthreads();
-  // lane = expert: bias / temperature / scale / mask, the logits output
-  constexpr int TW = TB / WAVES;
+  // lanes = (token, expert), 64 / EP tokens side by side: bias / temperature / scale / mask,
+  // the logits output
+  constexpr int TW = TB / WAVES;  // tokens finished by one wavefront
+  constexpr int TPP = 64 / EP;    // tokens per pass
+  const int e = lane % EP, sub = lane / EP;
   {
-    const ExpertConsts ec = load_expert_consts(lane, p);
+    const ExpertConsts ec = load_expert_consts(e, p);
     const int mode = final_logit_mode(p);
-    const bool col = lane < p.E;
-    for (int i = 0; i < TW; ++i) {
-      const int tl = TW * wave + i;
+    const bool col = e < p.E;
+    for (int i = 0; i < TW; i += TPP) {
+      const int tl = TW * wave + i + sub;
       const int64_t t = tok0 + tl;
-      const float raw = red[tl * RS + lane];
+      const float raw = red[tl * RS + e];
       float lg = mode == 0 ? final_logit_rows<0>(raw, ec, p.temperature)
                  : mode == 1 ? final_logit_rows<1>(raw, ec, p.temperature)
                              : final_logit_rows<2>(raw, ec, p.temperature);
       if (!col) lg = -__builtin_inff();
-      if (p.logits_out && col && t < p.T) p.logits_out[t * p.E + lane] = lg;
-      red[tl * RS + lane] = lg;
+      if (p.logits_out && col && t < p.T) p.logits_out[t * p.E + e] = lg;
+      red[tl * RS + e] = lg;
     }
   }
   __syncthreads();
-  // lane = token: softmax and top-k of a whole row on registers (two of the four wavefronts)
-  if (tid < TB) lane_token_tail<RS>(red + tid * RS, tok0 + tid, p);
+  // lane = token: softmax and top-k of a whole row on registers
+  if (tid < TB) lane_token_tail<EP, RS>(red + tid * RS, tok0 + tid, p);
   __syncthreads();
   if (p.probs) {
-    for (int i = 0; i < TW; ++i) {
-      const int tl = TW * wave + i;
+    for (int i = 0; i < TW; i += TPP) {
+      const int tl = TW * wave + i + sub;
       const int64_t t = tok0 + tl;
-      if (lane < p.E && t < p.T) p.probs[t * p.E + lane] = red[tl * RS + lane];
+      if (e < p.E && t < p.T) p.probs[t * p.E + e] = red[tl * RS + e];
     }
   }
 }
@@ -701,7 +714,7 @@ __global__ __launch_bounds__(128) void router_tail_rows_kernel(const float* __re
   else if (mode == 1) tail_rows_stage<1>(la, lb, from_a, tbase, wave, lane, red, p);
   else tail_rows_stage<2>(la, lb, from_a, tbase, wave, lane, red, p);
   __syncthreads();
-  lane_token_tail<RS>(red + tid * RS, tok0 + tid, p);
+  lane_token_tail<64, RS>(red + tid * RS, tok0 + tid, p);
   __syncthreads();
   if (p.probs) {
     for (int i = 0; i < 64; ++i) {
@@ -920,10 +933,16 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
       const int64_t mb = (T + 63) / 64;
       if (mb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
       const dim3 grid((unsigned)mb);
+      // long token streams: the tiled kernel (enough blocks to fill the chip twice)
       if (ep == 64 && T >= 32768 && H % 128 == 0)
-        // enough tokens to fill the chip with 128-token blocks, staged through LDS
-        hipLaunchKernelGGL(router_gate_lds_kernel<128>, dim3((unsigned)((T + 127) / 128)), dim3(256), 0, st, x,
-                           wb, H, p);
+        hipLaunchKernelGGL((router_gate_lds_kernel<64, 128, 128>), dim3((unsigned)((T + 127) / 128)), dim3(256), 0,
+                           st, x, wb, H, p);
+      else if (ep == 32 && T >= 32768 && H % 128 == 0)
+        hipLaunchKernelGGL((router_gate_lds_kernel<32, 128, 128>), dim3((unsigned)((T + 127) / 128)), dim3(256), 0,
+                           st, x, wb, H, p);
+      else if (ep == 16 && T >= 32768 && H % 256 == 0)
+        hipLaunchKernelGGL((router_gate_lds_kernel<16, 64, 256>), dim3((unsigned)((T + 63) / 64)), dim3(256), 0,
+                           st, x, wb, H, p);
       else if (ep == 64 && T >= 32768)
         // 128-token blocks: the weights are re-read from L2 once per block, so twice the
         // tokens per block halves that traffic

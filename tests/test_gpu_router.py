@@ -151,10 +151,13 @@ def test_router_fused(dev, dtype, T, H, E, k):
 
 
 @pytest.mark.parametrize("T,H,E,k", [(32768 + 37, 256, 64, 8), (32768, 128, 40, 3), (32768 + 5, 416, 64, 8),
-                                      (40000, 1152, 33, 1)])
-def test_router_many_experts_long_stream(dev, T, H, E, k):
-    """More than 32 experts and at least 32768 tokens take the 128-token block kernels (LDS-staged
-    when H % 128 == 0): ragged last block, one and several stages, padded expert columns."""
+                                      (40000, 1152, 33, 1), (32768 + 70, 512, 8, 2), (32768 + 3, 256, 16, 4),
+                                      (33000, 384, 20, 4), (32768, 768, 5, 1), (32768 + 1, 1024, 32, 8),
+                                      (32768, 384, 8, 2)])
+def test_router_long_stream(dev, T, H, E, k):
+    """At least 32768 tokens take the tiled, LDS-staged kernels (H % 128 == 0, or % 256 up to 16
+    experts; otherwise the generic ones): ragged last block, one and several stages, padded
+    expert columns, every tile split over the wavefronts."""
     import torch
     from pikv_amd import ops
     g = torch.Generator(device=dev).manual_seed(T + H + E)
