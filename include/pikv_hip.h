@@ -409,6 +409,20 @@ int pikv_fakequant_colblocks(const float* x, int64_t N, int H, int group,
                              void* stream);
 int64_t pikv_fakequant_workspace_bytes(int64_t N, int H, int group);
 
+/* The same with parameters fixed beforehand: out = (clamp(round(x/scale + zero)) - zero)*scale
+ * with ONE (scale, zero) for every element.
+ * Replaces: QuantizedCompressor._quantize with dynamic_quantization=False
+ *   (core/single/pikv_compression.py:430-472): the first tensor the module sees fixes scale
+ *   and zero_point, every later one is quantised with them.
+ *   preset [4] float (device): a (min, max, scale, zero) row as pikv_fakequant_colblocks
+ *   writes it; only scale and zero are read.  sq_err, workspace as above (group only
+ *   sets the column blocks that the errors are reported for). */
+int pikv_fakequant_preset(const float* x, int64_t N, int H, int group,
+                          int bits, int symmetric, const float* preset,
+                          float* out, float* sq_err,
+                          void* workspace, int64_t workspace_bytes,
+                          void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,9 @@ Pinning status (what, besides this file, fixes each function's output):
                                        ranking on tiny inputs
   adakv / duo / attend_values ........ hand-computed known answers, float64
                                        closed forms
+  fakequant_colblocks / _preset ...... hand-computed known answers; the preset form
+                                       given a block's own parameters must repeat
+                                       the block form bit for bit
   all of the above ................... property tests (ranges, error bounds, total
                                        orders, conservation, monotone budgets) and the
                                        frozen digests of tests/golden
@@ -379,6 +382,23 @@ def fakequant_colblocks(x: np.ndarray, group: int, bits: int = 8,
         stats.append((mn, mx, scale, zero))
         mse.append(np.mean((blk.astype(np.float64) - dq.astype(np.float64)) ** 2))
     return out, np.array(stats, dtype=F32), np.array(mse, dtype=np.float64)
+
+
+def fakequant_preset(x: np.ndarray, scale, zero, group: int, bits: int = 8,
+                     symmetric: bool = False):
+    """QuantizedCompressor._quantize with dynamic_quantization=False once calibrated
+    (core/single/pikv_compression.py:455-472): q = clamp(round(x/scale + zero_point)),
+    dq = (q - zero_point)*scale with the stored scalars.  Returns (dq [N,H] f32,
+    mse per block of `group` columns)."""
+    x = np.asarray(x, dtype=F32)
+    scale, zero = F32(scale), F32(zero)
+    qmin = -(1 << (bits - 1)) if symmetric else 0
+    qmax = (1 << (bits - 1)) - 1 if symmetric else (1 << bits) - 1
+    q = np.clip(np.rint(((x / scale).astype(F32) + zero).astype(F32)), qmin, qmax).astype(F32)
+    dq = ((q - zero).astype(F32) * scale).astype(F32)
+    mse = [np.mean((x[:, c0:c0 + group].astype(np.float64) - dq[:, c0:c0 + group].astype(np.float64)) ** 2)
+           for c0 in range(0, x.shape[1], group)]
+    return dq, np.array(mse, dtype=np.float64)
 
 
 def quant8_minshift(x: np.ndarray):

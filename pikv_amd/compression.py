@@ -4,7 +4,8 @@ Mirrors core/single/pikv_compression.py:368-516 (constructor, forward,
 _quantize, get_compression_stats) and the symmetric option of
 core/single/module/pikv_compression.py:919-1060.  forward() reproduces the
 reference's behaviour - fake quantisation with min/max taken over ALL rows of
-each block of `group_size` columns, float output.  quantize()/dequantize() are
+each block of `group_size` columns, float output; with dynamic_quantization=False
+the first block the module ever sees fixes one (scale, zero_point) for everything after.  quantize()/dequantize() are
 the additions of this build: they keep the integer codes, at per-token,
 per-token-per-head or per-group granularity (the formula is the same one).
 
@@ -53,10 +54,6 @@ class QuantizedCompressor(BaseCompressor):
         self.calibrated = False
         self.register_buffer("quantization_error", torch.zeros(1))
         self.register_buffer("sample_count", torch.tensor(0.0))
-        if not self.dynamic_quantization:
-            raise NotImplementedError(
-                "static (pre-calibrated) quantisation keeps the first batch's parameters "
-                "(core/single/pikv_compression.py:430-472); only the dynamic mode is on the GPU path")
 
     # ---- reference behaviour -------------------------------------------------
     def _fake(self, x2d: torch.Tensor, group: int):
@@ -66,11 +63,33 @@ class QuantizedCompressor(BaseCompressor):
         self.sample_count += mse.numel()
         return dq, stats
 
+    # ---- pre-calibrated mode (core/single/pikv_compression.py:430-472) ------------------
+    def _calibrate(self, x2d: torch.Tensor):
+        """The first tensor the module quantises fixes scale and zero_point for good."""
+        stats = ops.fakequant_colblocks(x2d, x2d.shape[1], self.bits, self.symmetric)[1]
+        self.scale = stats[0, 2:3].clone()
+        self.zero_point = stats[0, 3:4].clone()
+        self.calibrated = True
+
+    def _fake_static(self, x2d: torch.Tensor, group: int):
+        if not self.calibrated:
+            self._calibrate(x2d[:, :group].contiguous())
+        # (min, max, scale, zero) row as the kernel takes it; only scale and zero are read
+        preset = torch.cat([self.scale.new_zeros(2), self.scale.reshape(1).float(),
+                            self.zero_point.reshape(1).float()])
+        dq, mse = ops.fakequant_preset(x2d, preset, group, self.bits, self.symmetric)
+        self.quantization_error = mse[-1:].clone()
+        self.sample_count += mse.numel()
+        return dq
+
     def _quantize(self, x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         """One reduction domain = the whole tensor x (as the reference's
         _quantize: x.min()/x.max()).  Returns (q_x, dq_x, scale); q_x holds the
         integer codes as floats, like the reference."""
         x2 = x.reshape(-1, x.shape[-1]).float().contiguous()
+        if not self.dynamic_quantization:
+            dq = self._fake_static(x2, x2.shape[1]).reshape(x.shape)
+            return torch.round(dq / self.scale + self.zero_point), dq, self.scale
         # one column block as wide as the tensor: min/max over every element
         dq, stats = self._fake(x2, x2.shape[1])
         scale, zero = stats[0, 2], stats[0, 3]
@@ -85,6 +104,11 @@ class QuantizedCompressor(BaseCompressor):
         shape = keys.shape
         k2 = keys.reshape(-1, shape[-1]).float().contiguous()
         v2 = values.reshape(-1, shape[-1]).float().contiguous()
+        if not self.dynamic_quantization:
+            # the first column block of the first keys calibrates; everything else reuses it
+            dqk = self._fake_static(k2, self.group_size)
+            dqv = self._fake_static(v2, self.group_size)
+            return dqk.reshape(shape).to(keys.dtype), dqv.reshape(shape).to(values.dtype)
         dqk, _ = self._fake(k2, self.group_size)
         dqv, _ = self._fake(v2, self.group_size)
         return dqk.reshape(shape).to(keys.dtype), dqv.reshape(shape).to(values.dtype)

@@ -6,6 +6,8 @@
 // Four small launches: partial min/max per (column block, row chunk); reduce to
 // (min, max, scale, zero) per column block; apply + partial squared error in
 // double; fixed-order sum of the partials.  Everything is order-deterministic.
+// The pre-calibrated mode of the same class (core/single/pikv_compression.py:430-472)
+// skips the first two launches and applies one given (scale, zero) to every element.
 #include "common.hpp"
 
 namespace pikv {
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(256) void fq_params_kernel(const float* __restrict_
 __global__ __launch_bounds__(256) void fq_apply_kernel(const float* __restrict__ x, int64_t N, int H,
                                                        int group, int64_t n_chunks, int bits,
                                                        int symmetric, const float* __restrict__ stats,
-                                                       float* __restrict__ out,
+                                                       int stats_stride, float* __restrict__ out,
                                                        double* __restrict__ err_part) {
   __shared__ double shd[256];
   const int cb = blockIdx.x;
@@ -97,8 +99,9 @@ __global__ __launch_bounds__(256) void fq_apply_kernel(const float* __restrict__
   const int gw = (H - c0) < group ? (H - c0) : group;
   const int64_t r0 = chunk * kFqRows;
   const int64_t rows = (N - r0) < kFqRows ? (N - r0) : kFqRows;
-  const float scale = stats[cb * 4 + 2];
-  const float zero = stats[cb * 4 + 3];
+  // stats_stride 4: one (min, max, scale, zero) row per column block; 0: one row for all
+  const float scale = stats[cb * stats_stride + 2];
+  const float zero = stats[cb * stats_stride + 3];
   const float qmin = symmetric ? -(float)(1 << (bits - 1)) : 0.f;
   const float qmax = symmetric ? (float)((1 << (bits - 1)) - 1) : (float)((1 << bits) - 1);
   double err = 0.0;
@@ -168,7 +171,30 @@ extern "C" int pikv_fakequant_colblocks(const float* x, int64_t N, int H, int gr
   hipLaunchKernelGGL(fq_params_kernel, dim3((unsigned)nblk), dim3(256), 0, st, part, nch, bits,
                      symmetric, stats);
   hipLaunchKernelGGL(fq_apply_kernel, grid, dim3(256), 0, st, x, N, H, group, nch, bits, symmetric,
-                     stats, out, err_part);
+                     stats, 4, out, err_part);
+  hipLaunchKernelGGL(fq_err_kernel, dim3((unsigned)nblk), dim3(64), 0, st, err_part, nch, N, H, group,
+                     sq_err);
+  PIKV_CHECK_LAUNCH();
+  return PIKV_OK;
+}
+
+extern "C" int pikv_fakequant_preset(const float* x, int64_t N, int H, int group, int bits,
+                                     int symmetric, const float* preset, float* out, float* sq_err,
+                                     void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!x || !out || !preset || !sq_err) return PIKV_ERR_NULL;
+  if (N < 0 || H < 1 || group < 1) return PIKV_ERR_SHAPE;
+  if (bits < 2 || bits > 16) return PIKV_ERR_UNSUPPORTED;
+  if (N == 0) return PIKV_OK;
+  if (!workspace) return PIKV_ERR_NULL;
+  if (workspace_bytes < pikv_fakequant_workspace_bytes(N, H, group)) return PIKV_ERR_WORKSPACE;
+  const int64_t nblk = (H + group - 1) / group;
+  const int64_t nch = fq_chunks(N);
+  if (nblk > 0x7fffffffLL || nch > 65535) return PIKV_ERR_SHAPE;
+  double* err_part = reinterpret_cast<double*>(workspace);
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)nblk, (unsigned)nch);
+  hipLaunchKernelGGL(fq_apply_kernel, grid, dim3(256), 0, st, x, N, H, group, nch, bits, symmetric,
+                     preset, 0, out, err_part);
   hipLaunchKernelGGL(fq_err_kernel, dim3((unsigned)nblk), dim3(64), 0, st, err_part, nch, N, H, group,
                      sq_err);
   PIKV_CHECK_LAUNCH();

@@ -27,7 +27,7 @@ from ._native import (BF16, EVICT_H2O, EVICT_LRU, F32, Q_I4_ASYM, Q_I4_SYM,
 
 __all__ = [
     "router_fused", "router_tail", "capacity_slots", "quantize_rows",
-    "dequantize_rows", "fakequant_colblocks", "CachePool", "scheme_bits",
+    "dequantize_rows", "fakequant_colblocks", "fakequant_preset", "CachePool", "scheme_bits",
     "Q_I8_SYM", "Q_I8_ASYM", "Q_I4_ASYM", "Q_I4_SYM", "EVICT_H2O", "EVICT_LRU",
 ]
 
@@ -317,6 +317,28 @@ def fakequant_colblocks(x, group: int, bits: int = 8, symmetric: bool = False):
     N.call("pikv_fakequant_colblocks", _ptr(x), Nr, H, group, bits, int(bool(symmetric)),
            _ptr(out), _ptr(stats), _ptr(mse), _ptr(ws), ws_bytes, _stream())
     return out, stats, mse
+
+
+def fakequant_preset(x, preset, group: int, bits: int = 8, symmetric: bool = False):
+    """Fake quantisation with parameters fixed beforehand: `preset` is a (min, max, scale,
+    zero) row of a fakequant_colblocks `stats` output; one (scale, zero) serves every
+    element.  x [N,H] f32 -> (dq [N,H] f32, mse [nblk] per block of `group` columns)."""
+    x = _need(x, "x", dtype=torch.float32, ndim=2)
+    preset = _need(preset, "preset", dtype=torch.float32)
+    if preset.numel() != 4:
+        raise ValueError("preset must hold (min, max, scale, zero)")
+    Nr, H = x.shape
+    if group < 1:
+        raise ValueError("group must be >= 1")
+    nblk = (H + group - 1) // group
+    dev = x.device
+    out = torch.empty_like(x)
+    mse = torch.zeros(nblk, dtype=torch.float32, device=dev)
+    ws_bytes = int(N.lib().pikv_fakequant_workspace_bytes(Nr, H, group))
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+    N.call("pikv_fakequant_preset", _ptr(x), Nr, H, group, bits, int(bool(symmetric)),
+           _ptr(preset), _ptr(out), _ptr(mse), _ptr(ws), ws_bytes, _stream())
+    return out, mse
 
 
 # --------------------------------------------------------------------------

@@ -27,7 +27,7 @@ def test_header_declares_expected_surface():
     for need in ["pikv_router_fused", "pikv_router_tail", "pikv_capacity_slots", "pikv_quant_scatter",
                  "pikv_cache_advance", "pikv_quantize_rows", "pikv_gather_dequant",
                  "pikv_gather_dequant_scores", "pikv_h2o_accumulate", "pikv_evict_select",
-                 "pikv_h2o_budget", "pikv_compact_rows", "pikv_fakequant_colblocks",
+                 "pikv_h2o_budget", "pikv_compact_rows", "pikv_fakequant_colblocks", "pikv_fakequant_preset",
                  "pikv_router_workspace_bytes", "pikv_fakequant_workspace_bytes",
                  "pikv_router_fused_workspace_bytes", "pikv_quant_gather", "pikv_attend_values",
                  "pikv_attend_workspace_bytes", "pikv_evict_workspace_bytes",

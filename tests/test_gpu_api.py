@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import pikv_oracle as O
-from util import np_of, rng
+from util import np_of, rng, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -167,6 +167,46 @@ def test_hierarchical_router(dev):
     assert np.isclose(float(comb.sum().item()), float(np_of(out.topk_w)[slot >= 0].sum()), rtol=1e-5)
     p_mean = want.mean(axis=(0, 1))
     assert np.isclose(float(aux.detach()), float((p_mean * np.log(p_mean * E + 1e-9)).sum()), atol=1e-5)
+
+
+def test_quantized_compressor_static_mode(dev):
+    """dynamic_quantization=False (core/single/pikv_compression.py:430-472): the first column
+    block of the first keys calibrates one (scale, zero_point); values, later blocks and later
+    calls reuse it."""
+    import torch
+    from pikv_amd import ops
+    from pikv_amd.compression import QuantizedCompressor
+    r = rng(4)
+    c = QuantizedCompressor(256, bits=8, group_size=128, dynamic_quantization=False).to(dev)
+    k = torch.from_numpy(r.standard_normal((3, 20, 256)).astype(np.float32)).to(dev)
+    v = torch.from_numpy((3 * r.standard_normal((3, 20, 256))).astype(np.float32)).to(dev)
+    dk, dv = c(k, v)
+    kn, vn = np_of(k).reshape(-1, 256), np_of(v).reshape(-1, 256)
+    _, st, _ = O.fakequant_colblocks(kn[:, :128], 128)
+    assert float(c.scale) == st[0, 2] and float(c.zero_point) == st[0, 3] and c.calibrated
+    ref_k, _ = O.fakequant_preset(kn, st[0, 2], st[0, 3], 128)
+    ref_v, mse_v = O.fakequant_preset(vn, st[0, 2], st[0, 3], 128)
+    assert np.array_equal(np_of(dk).reshape(-1, 256), ref_k)
+    assert np.array_equal(np_of(dv).reshape(-1, 256), ref_v)
+    assert (np.abs(np_of(dv)) <= np.abs(ref_v).max()).all()      # the wider values are clamped
+    st_ = c.get_compression_stats()
+    assert abs(st_["quantization_error"] - mse_v[-1]) < 1e-6 * max(1.0, mse_v[-1]) and st_["num_samples"] == 4
+    # a second call keeps the parameters
+    k2 = 5 * k
+    dk2, _ = c(k2, v)
+    ref_k2, _ = O.fakequant_preset(5 * kn, st[0, 2], st[0, 3], 128)
+    assert np.array_equal(np_of(dk2).reshape(-1, 256), ref_k2) and float(c.scale) == st[0, 2]
+    q, dq, scale = c._quantize(k[0])
+    assert np.array_equal(np_of(dq), O.fakequant_preset(np_of(k[0]), st[0, 2], st[0, 3], 256)[0])
+    assert float(q.min()) >= 0 and float(q.max()) <= 255 and float(scale) == st[0, 2]
+    # the raw op: ragged last block, 4-bit symmetric, errors
+    x = r.standard_normal((77, 200)).astype(np.float32)
+    preset = torch.tensor([0.0, 0.0, 0.37, 0.0], device=dev)
+    dq, mse = ops.fakequant_preset(to_dev(x, dev), preset, 128, 4, True)
+    ref, mse_ref = O.fakequant_preset(x, 0.37, 0.0, 128, 4, True)
+    assert np.array_equal(np_of(dq), ref) and np.allclose(np_of(mse), mse_ref, rtol=1e-5)
+    with pytest.raises(ValueError):
+        ops.fakequant_preset(to_dev(x, dev), preset[:3], 128)
 
 
 def test_quantized_compressor(dev):

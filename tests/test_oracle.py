@@ -397,3 +397,23 @@ def test_adakv_duo_known_answers():
         assert np.array_equal(kk, want)
     assert O.duo_keep(10, 2, 3).tolist() == [True, True] + [False] * 5 + [True] * 3
     assert O.duo_keep(4, 3, 3).all()
+
+
+def test_fakequant_preset_known_answers():
+    """Pre-calibrated fake quantisation (core/single/pikv_compression.py:455-472): hand-computed
+    values, clamping at both ends, and the identity with the block form when it is handed the
+    block's own parameters."""
+    x = np.array([[1.3, -2.0, 200.0, 0.26, 0.24]], dtype=np.float32)
+    dq, mse = O.fakequant_preset(x, 0.5, 3.0, 5)
+    # 1.3/0.5+3 = 5.6 -> 6 -> 1.5 ; -2/0.5+3 = -1 -> 0 -> -1.5 ; 403 -> 255 -> 126 ;
+    # 0.52+3 -> 4 -> 0.5 ; 0.48+3 -> 3 -> 0
+    assert dq.tolist() == [[1.5, -1.5, 126.0, 0.5, 0.0]]
+    want = np.mean((x.astype(np.float64) - dq.astype(np.float64)) ** 2)
+    assert abs(mse[0] - want) < 1e-12
+    dq, _ = O.fakequant_preset(np.array([[-3.0, 0.26, 9.0]], np.float32), 0.5, 0.0, 3, bits=4, symmetric=True)
+    assert dq.tolist() == [[-3.0, 0.5, 3.5]]          # 18 -> 7 -> 3.5; -6 stays
+    r = np.random.default_rng(5)
+    y = r.standard_normal((50, 96)).astype(np.float32)
+    ref, st, mse_ref = O.fakequant_colblocks(y, 96)
+    dq, mse = O.fakequant_preset(y, st[0, 2], st[0, 3], 96)
+    assert np.array_equal(dq, ref) and np.allclose(mse, mse_ref, rtol=0, atol=0)
