@@ -411,13 +411,24 @@ __global__ __launch_bounds__(kMbThreads) void mb_hist_kernel(MbArgs a) {
     const uint32_t pmask = mb_mask(PASS);
     for (int b = threadIdx.x; b < NB; b += kMbThreads) lh[b] = 0;
     __syncthreads();
+    // neighbouring rows often share a digit (timestamps grow along the cache, scores of a
+    // region are of one magnitude): a run of equal digits costs one LDS atomic, not one per row
+    int run_digit = -1, run = 0;
 #pragma unroll
     for (int j = 0; j < kMbItems; ++j) {
+      int d = -1;
       if (i0 + j < len) {
         const uint32_t key = order_key(s.v[i0 + j], s.smallest);
-        if ((key & pmask) == prefix) atomicAdd(&lh[mb_digit(key, PASS)], 1);
+        if ((key & pmask) == prefix) d = mb_digit(key, PASS);
       }
+      if (d != run_digit) {
+        if (run_digit >= 0) atomicAdd(&lh[run_digit], run);
+        run_digit = d;
+        run = 0;
+      }
+      ++run;
     }
+    if (run_digit >= 0) atomicAdd(&lh[run_digit], run);
     __syncthreads();
     int* gh = a.hist + (((int64_t)c * 3 + PASS) * 2 + slot) * kMbBins;
     for (int b = threadIdx.x; b < NB; b += kMbThreads) {
