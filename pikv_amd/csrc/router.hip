@@ -1,7 +1,12 @@
 // K1: fused router - gate projection, logit scaling/mask, softmax, top-k,
 // renormalisation - and the capacity-slot pass.
 //
-// Gate projection (skinny: E <= 64 outputs per token, HBM-bound for small E):
+// Three forms of the gate projection (skinny: E <= 64 outputs per token):
+//   bf16, >= 32768 tokens ... router_gate_lds_kernel: token rows staged through LDS in whole
+//                             256/512-byte pieces, matrix cores, one token per lane in the tail
+//   bf16, fewer tokens ...... router_gate_mfma_kernel: matrix cores, k-steps dealt to the
+//                             wavefronts, operands straight from global memory
+//   fp32, or H % 32 != 0 .... router_gate_kernel, vector ALU:
 // a wavefront owns a tile of TPW = 64/EPAD tokens (EPAD = E rounded up to
 // 8/16/32/64).  Lanes stride the hidden dimension with 128-bit loads; every lane
 // keeps TPW*EPAD = 64 partial sums, so a slice of W fetched once (from L2) is
@@ -278,10 +283,10 @@ __global__ __launch_bounds__(256) void router_tail_kernel(const float* __restric
 // Measured on the prefill workload (T=32768, H=4096, E=8) the VALU kernel above
 // issues 25.8 M wavefront instructions - 42 us of pure issue time against 34 us of
 // HBM time - and has too few wavefronts to hide latency.  For bf16 inputs the
-// contraction over H therefore runs as v_mfma_f32_16x16x32_bf16: a block owns 16
-// tokens, its 8 wavefronts interleave over 32-wide slices of H (so the block
-// reads 512 contiguous bytes of each token row per sweep), every wavefront keeps
-// one 16x16 fp32 tile per group of 16 experts, and the partial tiles meet in LDS.
+// contraction over H therefore runs as v_mfma_f32_16x16x32_bf16: a block owns 16 MT
+// tokens, its wavefronts interleave over 32-wide slices of H (so the block
+// reads 64 WAVES contiguous bytes of each token row per sweep), every wavefront keeps
+// one 16x16 fp32 tile per token tile and group of 16 experts, and the partial tiles meet in LDS.
 // The kernel stays HBM-bound up to E = 64 (the MFMA work is ~1/7 of the HBM time
 // there), which the VALU formulation cannot be.
 typedef __bf16 pikv_bf16x8 __attribute__((ext_vector_type(8)));
