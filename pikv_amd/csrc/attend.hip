@@ -260,38 +260,45 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int it = wave * 16 + (lane & 15);
   const int igrp = lane >> 4;
   float pacc = 0.f;
+  // Every address below is a wave-uniform base plus a multiple of the thread index: chunk
+  // ch = k * 256 + thread of the tile's code rows IS the (token, 16-byte piece) pair
+  // (tok * LPR + off), and 4 * ch halves the (token, kv head) pair of the metadata rows; the
+  // bounds are uniform thresholds on the thread index.  (Per-chunk 64-bit lane addresses and
+  // token indices had cost the registers whose spill reloads waited, inside the loop, for
+  // the whole prefetch.)
+  const float* const sp = srow + st8;
   auto fetch = [&](int64_t n0) {
-    if (a.row_acc && igrp == 0 && n0 + it < t1) pacc = a.row_acc[base_row + n0 + it];
+    const int64_t left = t1 - n0;
+    const int rem = left < kAttTile ? (int)left : kAttTile;  // tokens of this tile
+    const int64_t urow = base_row + n0;
+    if (a.row_acc && igrp == 0 && it < rem) pacc = (a.row_acc + urow)[it];
     if (s_on) {
-      const int64_t n = n0 + st8;
-      if (s_vec && n + 8 <= t1) {
-        const float4 lo4 = *reinterpret_cast<const float4*>(srow + n);
-        const float4 hi4 = *reinterpret_cast<const float4*>(srow + n + 4);
+      const float* spn = sp + n0;
+      if (s_vec && st8 + 8 <= rem) {
+        const float4 lo4 = *reinterpret_cast<const float4*>(spn);
+        const float4 hi4 = *reinterpret_cast<const float4*>(spn + 4);
         psc[0] = lo4.x, psc[1] = lo4.y, psc[2] = lo4.z, psc[3] = lo4.w;
         psc[4] = hi4.x, psc[5] = hi4.y, psc[6] = hi4.z, psc[7] = hi4.w;
       } else {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) psc[k] = n + k < t1 ? srow[n + k] : s_off;
+        for (int k = 0; k < 8; ++k) psc[k] = st8 + k < rem ? spn[k] : s_off;
       }
     }
+    const char* cb = reinterpret_cast<const char*>(a.codes) + urow * (LPR * 16);
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
-      const int ch = k * 256 + threadIdx.x;
-      const int tok = ch >> (HKS + 2), off = ch & (LPR - 1);
       pc[k] = make_uint4(0, 0, 0, 0);
-      if (tok < kAttTile && n0 + tok < t1)
-        pc[k] = ld16(reinterpret_cast<const char*>(a.codes) + ((base_row + n0 + tok) * LPR + off) * 16);
+      if ((int)threadIdx.x < rem * LPR - k * 256) pc[k] = ld16(cb + k * 4096 + threadIdx.x * 16);
     }
+    const uint16_t* sb = reinterpret_cast<const uint16_t*>(a.scale) + urow * LPR;
+    const uint16_t* zb = reinterpret_cast<const uint16_t*>(a.zero) + urow * LPR;
 #pragma unroll
     for (int k = 0; k < NMC; ++k) {
-      const int ch = k * 256 + threadIdx.x;
-      const int tok = ch >> HKS, hd = ch & (HK - 1);
       ps[k] = make_uint2(0, 0);
       pz[k] = make_uint2(0, 0);
-      if (tok < kAttTile && n0 + tok < t1) {
-        const int64_t mi = (base_row + n0 + tok) * LPR + hd * 4;
-        ps[k] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.scale) + mi);
-        if constexpr (!Q::sym) pz[k] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.zero) + mi);
+      if ((int)threadIdx.x < rem * HK - k * 256) {
+        ps[k] = *reinterpret_cast<const uint2*>(sb + k * 1024 + threadIdx.x * 4);
+        if constexpr (!Q::sym) pz[k] = *reinterpret_cast<const uint2*>(zb + k * 1024 + threadIdx.x * 4);
       }
     }
   };
@@ -343,18 +350,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       const int t = it;
       const int grp = igrp;
       const bool mine = grp == 0 && n0 + t < t1;
-      const int64_t row = base_row + n0 + t;
+      // wave-uniform row pointers + a 32-bit lane offset: the addresses cost no registers
+      // across the loop (a per-lane 64-bit address pair per plane had been spilled, and its
+      // reload waited for the whole prefetch of the next tile)
+      float* const acc_rows = a.row_acc ? a.row_acc + (base_row + n0) : nullptr;
+      float* const ts_rows = a.row_ts ? a.row_ts + (base_row + n0) : nullptr;
       const float* lp = lprob + (t & ~15) + (t & 3) * 4 + ((t >> 2) & 3);
       float imp = 0.f;
       for (int hq = grp; hq < 4 * HK; hq += 4) imp = imp + lp[hq * kAttPRow];
       imp = imp + __shfl_xor(imp, 16, 64);
       imp = imp + __shfl_xor(imp, 32, 64);
       if (mine) {
-        if (a.row_acc) {
+        if (acc_rows) {
           if (a.decay != 1.0f) acc = acc * a.decay;
-          a.row_acc[row] = acc + imp;
+          acc_rows[t] = acc + imp;
         }
-        if (a.row_ts) a.row_ts[row] = a.now;
+        if (ts_rows) {
+          float now = a.now;
+          asm volatile("" : "+v"(now));  // copied from its scalar register here, not kept live across the loop
+          ts_rows[t] = now;
+        }
       }
     }
 
@@ -559,7 +574,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   float ps = 0.f, pz = 0.f, pacc = 0.f;
   float psc[8];
   auto fetch = [&](int64_t n0) {
-    if (a.row_acc && igrp == 0 && n0 + it < t1) pacc = a.row_acc[base_row + n0 + it];
+    if (a.row_acc && igrp == 0 && n0 + it < t1) pacc = (a.row_acc + (base_row + n0))[it];  // uniform base + lane
     if (s_on) {
       const int64_t n = n0 + st8;
       if (s_vec && n + 8 <= t1) {
@@ -628,18 +643,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     if (n0 + kAtt8Tile < t1) fetch(n0 + kAtt8Tile);  // in flight while this tile is multiplied
     if (a.row_acc || a.row_ts) {  // uniform
       const bool mine = igrp == 0 && n0 + it < t1;
-      const int64_t row = base_row + n0 + it;
+      const int t = it;
+      // wave-uniform row pointers + a 32-bit lane offset (no per-lane address registers live
+      // across the loop)
+      float* const acc_rows = a.row_acc ? a.row_acc + (base_row + n0) : nullptr;
+      float* const ts_rows = a.row_ts ? a.row_ts + (base_row + n0) : nullptr;
       float imp = 0.f;
       for (int hq = igrp; hq < a.n_q_heads; hq += 8) imp = imp + lprob[hq * kAtt8PRow + it];
       imp = imp + __shfl_xor(imp, 8, 64);
       imp = imp + __shfl_xor(imp, 16, 64);
       imp = imp + __shfl_xor(imp, 32, 64);
       if (mine) {
-        if (a.row_acc) {
+        if (acc_rows) {
           if (a.decay != 1.0f) acc = acc * a.decay;
-          a.row_acc[row] = acc + imp;
+          acc_rows[t] = acc + imp;
         }
-        if (a.row_ts) a.row_ts[row] = a.now;
+        if (ts_rows) {
+          float now = a.now;
+          asm volatile("" : "+v"(now));  // copied from its scalar register here, not kept live across the loop
+          ts_rows[t] = now;
+        }
       }
     }
 
