@@ -364,18 +364,23 @@ __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) {
 // Tile statistics and score rows from the staged scores [q head][token in tile], four
 // heads per wavefront pass: lane (rg, nl) owns tokens nl, nl+16, nl+32, nl+48 of head
 // h4 + rg; the 16 lanes of a row reduce with DPP.
+// GROUPED: the staged rows are [kv head][4] (row 4 g + r = head g * rep + r, rows r >= rep
+// unused), so that the row of a kv head sits at a compile-time offset for the writers.
+template <bool GROUPED>
 __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float* stage, int c, int64_t tile,
-                                                 int64_t n0, int len, int wave, int rg, int nl) {
-  for (int h4 = wave * 4; h4 < a.n_q_heads; h4 += 16) {
-    const int hq = h4 + rg;
-    const bool hok = hq < a.n_q_heads;
+                                                 int64_t n0, int len, int wave, int rg, int nl, int rep = 4) {
+  const int n_pass_rows = GROUPED ? a.n_kv_heads * 4 : a.n_q_heads;
+  for (int h4 = wave * 4; h4 < n_pass_rows; h4 += 16) {
+    const int srow = h4 + rg;                                  // staged row
+    const int hq = GROUPED ? (h4 >> 2) * rep + rg : srow;      // query head
+    const bool hok = GROUPED ? rg < rep : hq < a.n_q_heads;
     float x[4];
     bool okk[4];
     float m = -__builtin_inff();
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       okk[k] = hok && (n0 + nl + 16 * k < len);
-      x[k] = okk[k] ? stage[hq * kTile + nl + 16 * k] : -__builtin_inff();
+      x[k] = okk[k] ? stage[srow * kTile + nl + 16 * k] : -__builtin_inff();
       m = fmaxf(m, x[k]);
     }
     PIKV_DPP_INPLACE("v_max_f32_dpp", m, "quad_perm:[1,0,3,2]");
@@ -409,7 +414,7 @@ constexpr int kGqaMaxKvHeads = 16;     // code vectors of one 16-token slice kep
 // LDS bytes of scores_mfma_i4_gqa_kernel: score staging, query sums, compact A
 // operands plus an all-zero twin, and the (scale, zero) rows of one tile.
 static size_t gqa_lds_bytes(int n_q_heads, int n_kv_heads) {
-  return (size_t)n_q_heads * kTile * sizeof(float) + (size_t)n_kv_heads * 16 * sizeof(float) +
+  return (size_t)n_kv_heads * 4 * kTile * sizeof(float) + (size_t)n_kv_heads * 16 * sizeof(float) +
          2 * (size_t)n_kv_heads * 4 * 16 * 16 + 2 * (size_t)kTile * (n_kv_heads * 4 + 2) * sizeof(uint16_t);
 }
 
@@ -424,8 +429,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 
   static_assert(Q::bits == 4, "4-bit schemes only");
   static_assert(kGqaTilesPerBlock % 2 == 0, "tiles are processed in pairs");
   extern __shared__ float gqa_lds[];
-  float* stage = gqa_lds;                            // [q head][token in tile]
-  float4* qs4 = reinterpret_cast<float4*>(stage + a.n_q_heads * kTile);  // [kv head][group]: q sums of its <=4 heads
+  float* stage = gqa_lds;                            // [kv head][4 head slots][token in tile]
+  float4* qs4 = reinterpret_cast<float4*>(stage + a.n_kv_heads * 4 * kTile);  // [kv head][group]: q sums of its <=4 heads
   uint4* alds = reinterpret_cast<uint4*>(qs4 + a.n_kv_heads * 4);        // [kv head][b][gq*4 + r]
   uint4* azero = alds + a.n_kv_heads * 64;                                // same shape, all zero
   const int meta_stride = a.n_kv_heads * 4 + 2;      // halves; +2 spreads the tokens over banks
@@ -454,26 +459,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 
     uint4 cv[NKV];
     uint2 sv[NM], zv[NM];
   };
+  // Addresses are a wave-uniform base plus a small lane offset: this wavefront's slice starts
+  // (wave*16 + nl) rows into the tile, and chunk ch = j*256 + thread of the tile's metadata
+  // rows is the (token, kv head) pair, 4*ch halves into the rows (lanes_per_row = 4 kv heads).
+  // (64-bit lane addresses per chunk had cost the registers whose spill reloads waited,
+  // inside the loop, for the code loads just issued.)
+  const int code_lane_off = ((wave * 16 + nl) * lanes_per_row + rg) * 16;
   auto issue = [&](int tt, TileRegs& t) {
     const int64_t t0 = tok0 + tt * kTile;
-    const int64_t n = t0 + wave * 16 + nl;
-    const bool okn = n < len;
-    const char* rowp = reinterpret_cast<const char*>(a.codes) + ((base_row + n) * lanes_per_row + rg) * 16;
+    const int64_t left = len - t0;
+    const int rem = left < kTile ? (int)left : kTile;  // tokens of the tile that exist
+    const bool okn = wave * 16 + nl < rem;
+    const char* rowp = reinterpret_cast<const char*>(a.codes) + (base_row + t0) * lanes_per_row * 16 + code_lane_off;
 #pragma unroll
     for (int g = 0; g < NKV; ++g) {
       t.cv[g] = make_uint4(0, 0, 0, 0);
       if (okn && g < a.n_kv_heads) t.cv[g] = ld16(rowp + g * 64);
     }
+    const uint16_t* sb = reinterpret_cast<const uint16_t*>(a.scale) + (base_row + t0) * lanes_per_row;
+    const uint16_t* zb = reinterpret_cast<const uint16_t*>(a.zero) + (base_row + t0) * lanes_per_row;
 #pragma unroll
     for (int j = 0; j < NM; ++j) {
-      const int ch = j * 256 + threadIdx.x;
-      const int tok = ch / a.n_kv_heads, hd = ch - tok * a.n_kv_heads;
       t.sv[j] = make_uint2(0, 0);
       t.zv[j] = make_uint2(0, 0);
-      if (tok < kTile && t0 + tok < len) {
-        const int64_t mi = (base_row + t0 + tok) * lanes_per_row + hd * 4;
-        t.sv[j] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.scale) + mi);
-        if constexpr (!Q::sym) t.zv[j] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.zero) + mi);
+      if ((int)threadIdx.x < rem * a.n_kv_heads - j * 256) {
+        t.sv[j] = *reinterpret_cast<const uint2*>(sb + j * 1024 + threadIdx.x * 4);
+        if constexpr (!Q::sym) t.zv[j] = *reinterpret_cast<const uint2*>(zb + j * 1024 + threadIdx.x * 4);
       }
     }
   };
@@ -558,12 +569,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 
         const float u23 = __uint_as_float(s23[0]) + __uint_as_float(s23[1]);
         auto sf = __builtin_amdgcn_permlane32_swap(__float_as_uint(u01), __float_as_uint(u23), false, false);
         const float score = (__uint_as_float(sf[0]) + __uint_as_float(sf[1])) * a.scale_qk;
-        if (rg < rep) stage[(g * rep + rg) * kTile + tl] = okt ? score : -__builtin_inff();
+        if (rg < rep) stage[(g * 4 + rg) * kTile + tl] = okt ? score : -__builtin_inff();
       }
     }
     __syncthreads();
 
-    tile_stats_store(a, stage, c, tile, n0, len, wave, rg, nl);
+    tile_stats_store<true>(a, stage, c, tile, n0, len, wave, rg, nl, rep);
     __syncthreads();  // stage and the metadata rows are reused by the next tile
     return true;
   };
@@ -700,7 +711,7 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
       }
     }
     __syncthreads();
-    tile_stats_store(a, stage, c, tile, n0, len, wave, rg, nl);
+    tile_stats_store<false>(a, stage, c, tile, n0, len, wave, rg, nl);
     __syncthreads();  // stage is reused by the next tile
   }
 }
