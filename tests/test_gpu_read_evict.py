@@ -48,6 +48,9 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I4_ASYM, 32, 8, 64, 128),     # 8 q heads per kv head: two sets of A rows against the same codes
     (O.Q_I4_SYM, 32, 2, 12, 128),      # 6 q heads per kv head: the second set half empty
     (O.Q_I4_ASYM, 32, 16, 16, 128),    # more kv heads than wavefronts, one q head each
+    (O.Q_I4_ASYM, 32, 8, 24, 128),     # 3 q heads per kv head: one of the four staged head slots stays empty
+    (O.Q_I4_SYM, 32, 4, 4, 128),       # one q head per kv head on the GQA kernel
+    (O.Q_I4_ASYM, 32, 16, 48, 128),    # 16 kv heads x 3
     (O.Q_I8_SYM, 128, 8, 32, 128),     # 8-bit matrix-core kernel: 4 q heads per kv head, scale per head
     (O.Q_I8_ASYM, 128, 2, 16, 128),    # ... 8 q heads per kv head, zero points
     (O.Q_I8_SYM, 256, 4, 64, 128),     # ... 16 q heads per kv head, one scale per two heads
