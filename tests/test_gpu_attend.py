@@ -19,6 +19,7 @@ pytestmark = pytest.mark.gpu
     (O.Q_I4_ASYM, 32, 1, 8, 128),      # matrix-core form, all 16 operand rows in use
     (O.Q_I4_ASYM, 32, 4, 4, 128),      # matrix-core form, one row pair per kv head
     (O.Q_I4_ASYM, 32, 16, 16, 128),    # more kv heads than the matrix-core form takes: vector form
+    (O.Q_I4_ASYM, 32, 8, 24, 128),     # 3 q heads per kv head: a row pair of every kv head stays empty
     (O.Q_I4_ASYM, 32, 8, 64, 128),     # 8 q heads per kv head: two launches of four heads each
     (O.Q_I4_SYM, 32, 2, 12, 128),      # 6 q heads per kv head: the second launch half empty
     (O.Q_I8_SYM, 128, 4, 4, 128),      # int8 per token per head
@@ -65,6 +66,8 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
     (O.Q_I4_ASYM, 32, 8, 32, 128),     # matrix-core form: importance summed from the staged tile
     (O.Q_I4_ASYM, 32, 2, 4, 128),
     (O.Q_I4_ASYM, 32, 4, 32, 128),     # two launches: the second adds to what the first decayed
+    (O.Q_I4_ASYM, 32, 8, 24, 128),     # 3 q heads per kv head
+    (O.Q_I4_SYM, 32, 8, 40, 128),      # 5 per kv head: second launch with a single head
     (O.Q_I8_SYM, 128, 4, 8, 128),      # 8-bit matrix-core form
     (O.Q_I8_ASYM, 128, 8, 64, 128),    # ... 64 query heads
     (O.Q_I8_SYM, 64, 4, 8, 64),        # vector form: importance in a kernel of its own
