@@ -117,9 +117,10 @@ int pikv_abi_version(void);
  *   count    [E] int32 or NULL
  *   1 <= E <= 64, 1 <= k <= min(E,8), H % 8 == 0
  *   workspace: pikv_router_fused_workspace_bytes(T,H,E,k) bytes, 256-byte aligned
- *              (slot scan counters, and the gate weights re-laid per 32-wide
- *              k-step for the bf16 matrix-core projection); required whenever
- *              slot != NULL or x_dtype == PIKV_BF16.
+ *              (slot scan counters, the gate weights re-laid per 32-wide k-step
+ *              for the bf16 matrix-core projection and, for short token streams,
+ *              partial logits per slice of H); required whenever slot != NULL
+ *              or x_dtype == PIKV_BF16.
  * ---------------------------------------------------------------------- */
 int pikv_router_fused(const void* x, const void* w, int x_dtype,
                       const float* bias, const float* expert_scale,

@@ -259,11 +259,13 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const void* __restrict
   router_tail_lanes<EPAD>(lg, tok0 + lane / EPAD, lane % EPAD, lane, p);
 }
 
+// n_parts > 1: logits_a holds n_parts slabs [T,E] of partial sums (the split gate
+// projection), added in slab order.
 template <int EPAD>
 __global__ __launch_bounds__(256) void router_tail_kernel(const float* __restrict__ la,
                                                           const float* __restrict__ lb,
                                                           const uint8_t* __restrict__ select,
-                                                          TailParams p) {
+                                                          TailParams p, int n_parts = 1) {
   constexpr int TPW = 64 / EPAD;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -275,6 +277,7 @@ __global__ __launch_bounds__(256) void router_tail_kernel(const float* __restric
   if (t < p.T && e < p.E) {
     const bool use_a = (lb == nullptr) || (select == nullptr) || (select[t] != 0);
     lg = use_a ? la[t * p.E + e] : lb[t * p.E + e];
+    for (int s = 1; s < n_parts; ++s) lg = lg + la[((int64_t)s * p.T + t) * p.E + e];
   }
   router_tail_lanes<EPAD>(lg, t, e, lane, p);
 }
@@ -311,9 +314,13 @@ __global__ __launch_bounds__(256) void gate_weight_relayout_kernel(const uint16_
 }
 
 // NT 16-expert tiles (1, 2 or 4) x MT 16-token tiles per block; WAVES wavefronts share the k-steps
-template <int NT, int MT, int WAVES>
+// PARTIAL (short token streams): blockIdx.y picks a slice of the k-steps, and the block
+// writes its partial logits to part[slice][T][E] instead of running the tail - with a few
+// dozen tokens a single block would walk all of H alone, one load latency per k-step.
+template <int NT, int MT, int WAVES, bool PARTIAL = false>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2))) void router_gate_mfma_kernel(
-    const void* __restrict__ x, const void* __restrict__ wb, int H, TailParams p) {
+    const void* __restrict__ x, const void* __restrict__ wb, int H, TailParams p, float* __restrict__ part = nullptr,
+    int steps_per_slice = 0) {
   constexpr int EP = 16 * NT;
   constexpr int TB = 16 * MT;  // tokens per block
   // Partial sums of the wavefronts: one slab each, or - when those would not leave room
@@ -342,9 +349,13 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
     for (int t = 0; t < NT; ++t) acc[mt][t] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
 
   // the k-steps are dealt round-robin to the wavefronts; each keeps UN steps in flight
-  const int steps = H / 32;
+  int steps = H / 32, step0 = 0;
+  if constexpr (PARTIAL) {
+    step0 = blockIdx.y * steps_per_slice;
+    steps = step0 + steps_per_slice < steps ? step0 + steps_per_slice : steps;
+  }
   constexpr int UN = (MT >= 8) ? 1 : (MT + NT > 4) ? 2 : 4;  // registers: 2 wavefronts per SIMD must fit
-  for (int st0 = wave; st0 < steps; st0 += WAVES * UN) {
+  for (int st0 = step0 + wave; st0 < steps; st0 += WAVES * UN) {
     uint4 av[UN][MT], bv[UN][NT];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
@@ -391,6 +402,20 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
 #pragma unroll
         for (int i = 0; i < 4; ++i) red[wave][mt * 16 + 4 * kg + i][t * 16 + m] = acc[mt][t][i];
     __syncthreads();
+  }
+  if constexpr (PARTIAL) {
+    float* dst = part + (int64_t)blockIdx.y * p.T * p.E;
+    for (int i = threadIdx.x; i < TB * EP; i += WAVES * 64) {
+      const int tl = i / EP, e = i % EP;
+      const int64_t t = tok0 + tl;
+      if (t < p.T && e < p.E) {
+        float v = 0.f;
+#pragma unroll
+        for (int w2 = 0; w2 < (SEQ ? 1 : WAVES); ++w2) v += red[w2][tl][e];
+        dst[t * p.E + e] = v;
+      }
+    }
+    return;
   }
   // Wavefront w finishes tokens TW*w .. TW*w+TW-1: lane -> (token, expert) with the
   // experts of a token in EP adjacent lanes, as the tail expects.
@@ -877,9 +902,25 @@ static int gate_epad(int E) { return E <= 16 ? 16 : E <= 32 ? 32 : 64; }
 static int64_t gate_weight_bytes(int H, int E) { return (int64_t)H * gate_epad(E) * 2; }
 static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
+// Short token streams split the gate projection over the hidden dimension: slices of at
+// least 16 k-steps, as many as it takes to put about a thousand blocks on the chip.
+constexpr int64_t kSplitMaxTokens = 16383;  // 256 and more token blocks keep the chip busy without
+static int gate_slices(int64_t T, int H) {
+  if (T <= 0 || T > kSplitMaxTokens || H % 32 != 0) return 1;
+  const int64_t steps = H / 32, token_blocks = (T + 63) / 64;
+  int64_t s = (steps + 15) / 16;
+  const int64_t want = (1024 + token_blocks - 1) / token_blocks;
+  if (s > want) s = want;
+  return s < 1 ? 1 : (int)s;
+}
+static int64_t gate_partial_bytes(int64_t T, int H, int E) {
+  const int s = gate_slices(T, H);
+  return s > 1 ? align256((int64_t)s * T * E * 4) : 0;
+}
+
 extern "C" int64_t pikv_router_fused_workspace_bytes(int64_t T, int H, int E, int k) {
   if (T < 0 || H < 1 || E < 1 || k < 1) return 0;
-  return align256(slot_workspace_bytes(T * k, E)) + gate_weight_bytes(H, E);
+  return align256(slot_workspace_bytes(T * k, E)) + align256(gate_weight_bytes(H, E)) + gate_partial_bytes(T, H, E);
 }
 
 extern "C" int pikv_capacity_slots(const int32_t* expert_idx, int64_t A, int E, int64_t capacity,
@@ -914,7 +955,8 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
   const int64_t slot_ws = align256(slot_workspace_bytes(T * k, E));
   if ((slot || mfma) && T > 0) {
     if (!workspace) return PIKV_ERR_NULL;
-    if (workspace_bytes < (slot ? slot_ws : 0) + (mfma ? gate_weight_bytes(H, E) : 0))
+    if (workspace_bytes < (slot ? slot_ws : 0) +
+                              (mfma ? align256(gate_weight_bytes(H, E)) + gate_partial_bytes(T, H, E) : 0))
       return PIKV_ERR_WORKSPACE;
   }
   // the re-laid gate weights sit behind the slot area when both are in use
@@ -938,6 +980,25 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
       const int64_t mb = (T + 63) / 64;
       if (mb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
       const dim3 grid((unsigned)mb);
+      const int slices = gate_slices(T, H);
+      if (slices > 1) {
+        // short token streams: partial logits per slice of H, then the tail on their sum
+        float* part = reinterpret_cast<float*>(wb + align256(gate_weight_bytes(H, E)));
+        const int sps = (int)((H / 32 + slices - 1) / slices);
+        const dim3 g2((unsigned)mb, (unsigned)slices);
+        if (ep == 16)
+          hipLaunchKernelGGL((router_gate_mfma_kernel<1, 4, 8, true>), g2, dim3(512), 0, st, x, wb, H, p, part, sps);
+        else if (ep == 32)
+          hipLaunchKernelGGL((router_gate_mfma_kernel<2, 4, 4, true>), g2, dim3(256), 0, st, x, wb, H, p, part, sps);
+        else
+          hipLaunchKernelGGL((router_gate_mfma_kernel<4, 4, 4, true>), g2, dim3(256), 0, st, x, wb, H, p, part, sps);
+        switch (epad) {
+          case 8: hipLaunchKernelGGL((router_tail_kernel<8>), dim3((unsigned)blocks), dim3(256), 0, st, part, nullptr, nullptr, p, slices); break;
+          case 16: hipLaunchKernelGGL((router_tail_kernel<16>), dim3((unsigned)blocks), dim3(256), 0, st, part, nullptr, nullptr, p, slices); break;
+          case 32: hipLaunchKernelGGL((router_tail_kernel<32>), dim3((unsigned)blocks), dim3(256), 0, st, part, nullptr, nullptr, p, slices); break;
+          default: hipLaunchKernelGGL((router_tail_kernel<64>), dim3((unsigned)blocks), dim3(256), 0, st, part, nullptr, nullptr, p, slices); break;
+        }
+      } else
       // long token streams: the tiled kernel (enough blocks to fill the chip twice)
       if (ep == 64 && T >= 32768 && H % 128 == 0)
         hipLaunchKernelGGL((router_gate_lds_kernel<64, 128, 128>), dim3((unsigned)((T + 127) / 128)), dim3(256), 0,

@@ -183,6 +183,38 @@ def test_router_long_stream(dev, T, H, E, k):
     assert np.array_equal(np_of(out.count), count)
 
 
+@pytest.mark.parametrize("T,H,E,k", [(64, 7168, 64, 8), (1, 4096, 8, 2), (700, 2048, 20, 4), (4096 + 9, 1024, 64, 6),
+                                      (8192, 512, 8, 1), (16383, 1536, 33, 2)])
+def test_router_short_stream_split(dev, T, H, E, k):
+    """Short token streams split the gate projection over the hidden dimension (partial logits
+    per slice, summed in slice order by the tail): single token, ragged blocks, slices that do
+    not divide the k-steps, every padded expert width."""
+    import torch
+    from pikv_amd import ops
+    g = torch.Generator(device=dev).manual_seed(T + H + E)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    w = (0.05 * torch.randn(E, H, generator=g, device=dev)).to(torch.bfloat16)
+    b = 0.1 * torch.randn(E, generator=g, device=dev)
+    if E >= 20:
+        w[5], w[17] = w[2], w[2]
+        b[5], b[17] = b[2], b[2]
+    cap = max(1, int(T * 1.25 * k / E))
+    out = ops.router_fused(x, w, b, top_k=k, capacity=cap, return_logits=True)
+    lg = x.double() @ w.double().T + b.double()
+    assert torch.allclose(out.logits.double(), lg, atol=1e-5 * H ** 0.5, rtol=1e-5)
+    if E >= 20:
+        assert torch.equal(out.logits[:, 2], out.logits[:, 17])
+    assert torch.allclose(out.probs, torch.softmax(out.logits, dim=1), atol=1e-6)
+    order = torch.sort(out.logits, dim=1, descending=True, stable=True).indices[:, :k]
+    assert torch.equal(out.topk_idx.long(), order)
+    slot, count = O.capacity_slots(np_of(out.topk_idx), E, cap)
+    assert np.array_equal(np_of(out.slot), slot)
+    assert np.array_equal(np_of(out.count), count)
+    # the same call twice gives the same bits (fixed order of the partial sums)
+    again = ops.router_fused(x, w, b, top_k=k, capacity=cap, return_logits=True)
+    assert torch.equal(out.logits, again.logits) and torch.equal(out.topk_w, again.topk_w)
+
+
 def test_router_module_arithmetic(dev):
     """The arithmetic of the reference's module/ copy (core/single/module/pikv_routing.py:596-600,
     :133-134, :143): scale before temperature, finfo.min penalty, + 1e-8 in the renormalisation -
