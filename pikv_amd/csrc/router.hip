@@ -904,9 +904,12 @@ static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
 // Short token streams split the gate projection over the hidden dimension: slices of at
 // least 16 k-steps, as many as it takes to put about a thousand blocks on the chip.
-constexpr int64_t kSplitMaxTokens = 16383;  // 256 and more token blocks keep the chip busy without
-static int gate_slices(int64_t T, int H) {
-  if (T <= 0 || T > kSplitMaxTokens || H % 32 != 0) return 1;
+// Measured at H = 7168, 64 experts: 71 -> 25 us (64..1024 tokens), 74 -> 35 us (4096),
+// 77 -> 67 us (16384); with 8 experts (H = 4096) nothing is gained from 16384 tokens on.
+constexpr int64_t kTiled64MinTokens = 20480;
+static int gate_slices(int64_t T, int H, int E) {
+  const int64_t max_tokens = E > 16 ? kTiled64MinTokens - 1 : 16383;
+  if (T <= 0 || T > max_tokens || H % 32 != 0) return 1;
   const int64_t steps = H / 32, token_blocks = (T + 63) / 64;
   int64_t s = (steps + 15) / 16;
   const int64_t want = (1024 + token_blocks - 1) / token_blocks;
@@ -914,7 +917,7 @@ static int gate_slices(int64_t T, int H) {
   return s < 1 ? 1 : (int)s;
 }
 static int64_t gate_partial_bytes(int64_t T, int H, int E) {
-  const int s = gate_slices(T, H);
+  const int s = gate_slices(T, H, E);
   return s > 1 ? align256((int64_t)s * T * E * 4) : 0;
 }
 
@@ -980,7 +983,18 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
       const int64_t mb = (T + 63) / 64;
       if (mb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
       const dim3 grid((unsigned)mb);
-      const int slices = gate_slices(T, H);
+      const int slices = gate_slices(T, H, E);
+      // 20480 tokens and more: the tiled kernel.  Its blocks hold 68 KB of LDS, two per compute
+      // unit = 512 on the chip: 64-token blocks while they fit in one round (<= 32768 tokens;
+      // 32768 x 7168 x 64 experts: 129 us against 155 us with half as many 128-token blocks),
+      // 128-token blocks beyond (40960 tokens: 167 us against 185 us in two uneven rounds).
+      // Up to 16 experts the untiled kernel streams as fast (8 experts, H = 4096: 81 vs 88 us
+      // at 40960 tokens) until about 65536 tokens (117 vs 110 us; H = 7168: 195 vs 178 us),
+      // always on 64-token blocks (128-token blocks: 129 us).
+      const bool tiled = T >= (ep == 16 ? 65536 : kTiled64MinTokens);
+      const bool t128 = tiled && ep != 16 && H % 128 == 0 && (T > 32768 || H % 256 != 0);
+      const bool t64 = tiled && !t128 && H % 256 == 0;
+      const dim3 g64((unsigned)((T + 63) / 64)), g128((unsigned)((T + 127) / 128));
       if (slices > 1) {
         // short token streams: partial logits per slice of H, then the tail on their sum
         float* part = reinterpret_cast<float*>(wb + align256(gate_weight_bytes(H, E)));
@@ -998,17 +1012,16 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
           case 32: hipLaunchKernelGGL((router_tail_kernel<32>), dim3((unsigned)blocks), dim3(256), 0, st, part, nullptr, nullptr, p, slices); break;
           default: hipLaunchKernelGGL((router_tail_kernel<64>), dim3((unsigned)blocks), dim3(256), 0, st, part, nullptr, nullptr, p, slices); break;
         }
-      } else
-      // long token streams: the tiled kernel (enough blocks to fill the chip twice)
-      if (ep == 64 && T >= 32768 && H % 128 == 0)
-        hipLaunchKernelGGL((router_gate_lds_kernel<64, 128, 128>), dim3((unsigned)((T + 127) / 128)), dim3(256), 0,
-                           st, x, wb, H, p);
-      else if (ep == 32 && T >= 32768 && H % 128 == 0)
-        hipLaunchKernelGGL((router_gate_lds_kernel<32, 128, 128>), dim3((unsigned)((T + 127) / 128)), dim3(256), 0,
-                           st, x, wb, H, p);
-      else if (ep == 16 && T >= 32768 && H % 256 == 0)
-        hipLaunchKernelGGL((router_gate_lds_kernel<16, 64, 256>), dim3((unsigned)((T + 63) / 64)), dim3(256), 0,
-                           st, x, wb, H, p);
+      } else if (t64 && ep == 64)
+        hipLaunchKernelGGL((router_gate_lds_kernel<64, 64, 256>), g64, dim3(256), 0, st, x, wb, H, p);
+      else if (t64 && ep == 32)
+        hipLaunchKernelGGL((router_gate_lds_kernel<32, 64, 256>), g64, dim3(256), 0, st, x, wb, H, p);
+      else if (t64)
+        hipLaunchKernelGGL((router_gate_lds_kernel<16, 64, 256>), g64, dim3(256), 0, st, x, wb, H, p);
+      else if (t128 && ep == 64)
+        hipLaunchKernelGGL((router_gate_lds_kernel<64, 128, 128>), g128, dim3(256), 0, st, x, wb, H, p);
+      else if (t128 && ep == 32)
+        hipLaunchKernelGGL((router_gate_lds_kernel<32, 128, 128>), g128, dim3(256), 0, st, x, wb, H, p);
       else if (ep == 64 && T >= 32768)
         // 128-token blocks: the weights are re-read from L2 once per block, so twice the
         // tokens per block halves that traffic

@@ -153,7 +153,7 @@ def test_router_fused(dev, dtype, T, H, E, k):
 @pytest.mark.parametrize("T,H,E,k", [(32768 + 37, 256, 64, 8), (32768, 128, 40, 3), (32768 + 5, 416, 64, 8),
                                       (40000, 1152, 33, 1), (32768 + 70, 512, 8, 2), (32768 + 3, 256, 16, 4),
                                       (33000, 384, 20, 4), (32768, 768, 5, 1), (32768 + 1, 1024, 32, 8),
-                                      (32768, 384, 8, 2)])
+                                      (32768, 384, 8, 2), (65536 + 3, 256, 8, 2), (65536, 512, 16, 8)])
 def test_router_long_stream(dev, T, H, E, k):
     """At least 32768 tokens take the tiled, LDS-staged kernels (H % 128 == 0, or % 256 up to 16
     experts; otherwise the generic ones): ragged last block, one and several stages, padded
@@ -184,7 +184,8 @@ def test_router_long_stream(dev, T, H, E, k):
 
 
 @pytest.mark.parametrize("T,H,E,k", [(64, 7168, 64, 8), (1, 4096, 8, 2), (700, 2048, 20, 4), (4096 + 9, 1024, 64, 6),
-                                      (8192, 512, 8, 1), (16383, 1536, 33, 2)])
+                                      (8192, 512, 8, 1), (16383, 1536, 33, 2), (20479, 512, 64, 8),
+                                      (20480 + 5, 512, 64, 8), (24000, 256, 8, 2), (30000, 768, 24, 3)])
 def test_router_short_stream_split(dev, T, H, E, k):
     """Short token streams split the gate projection over the hidden dimension (partial logits
     per slice, summed in slice order by the tail): single token, ragged blocks, slices that do
