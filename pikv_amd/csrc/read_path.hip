@@ -364,16 +364,17 @@ __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) {
 // Tile statistics and score rows from the staged scores [q head][token in tile], four
 // heads per wavefront pass: lane (rg, nl) owns tokens nl, nl+16, nl+32, nl+48 of head
 // h4 + rg; the 16 lanes of a row reduce with DPP.
-// GROUPED: the staged rows are [kv head][4] (row 4 g + r = head g * rep + r, rows r >= rep
-// unused), so that the row of a kv head sits at a compile-time offset for the writers.
-template <bool GROUPED>
+// GROUPED: the staged rows are [kv head][SLOTS] (row SLOTS g + r = head g * rep + r, rows
+// r >= rep unused), so that the row of a kv head sits at a compile-time offset for the writers.
+template <bool GROUPED, int SLOTS = 4>
 __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float* stage, int c, int64_t tile,
                                                  int64_t n0, int len, int wave, int rg, int nl, int rep = 4) {
-  const int n_pass_rows = GROUPED ? a.n_kv_heads * 4 : a.n_q_heads;
+  const int n_pass_rows = GROUPED ? a.n_kv_heads * SLOTS : a.n_q_heads;
   for (int h4 = wave * 4; h4 < n_pass_rows; h4 += 16) {
-    const int srow = h4 + rg;                                  // staged row
-    const int hq = GROUPED ? (h4 >> 2) * rep + rg : srow;      // query head
-    const bool hok = GROUPED ? rg < rep : hq < a.n_q_heads;
+    const int srow = h4 + rg;                                  // staged row = kv head * SLOTS + slot
+    const int slot = srow % SLOTS;
+    const int hq = GROUPED ? (srow / SLOTS) * rep + slot : srow;  // query head
+    const bool hok = GROUPED ? slot < rep : hq < a.n_q_heads;
     float x[4];
     bool okk[4];
     float m = -__builtin_inff();
@@ -413,9 +414,9 @@ constexpr int kGqaMaxKvHeads = 16;     // code vectors of one 16-token slice kep
 
 // LDS bytes of scores_mfma_i4_gqa_kernel: score staging, query sums, compact A
 // operands plus an all-zero twin, and the (scale, zero) rows of one tile.
-static size_t gqa_lds_bytes(int n_q_heads, int n_kv_heads) {
-  return (size_t)n_kv_heads * 4 * kTile * sizeof(float) + (size_t)n_kv_heads * 16 * sizeof(float) +
-         2 * (size_t)n_kv_heads * 4 * 16 * 16 + 2 * (size_t)kTile * (n_kv_heads * 4 + 2) * sizeof(uint16_t);
+static size_t gqa_lds_bytes(int n_kv_heads, int nset) {
+  return (size_t)nset * n_kv_heads * 4 * kTile * sizeof(float) + (size_t)nset * n_kv_heads * 16 * sizeof(float) +
+         (size_t)(nset + 1) * n_kv_heads * 4 * 16 * 16 + 2 * (size_t)kTile * (n_kv_heads * 4 + 2) * sizeof(uint16_t);
 }
 
 // A wavefront owns one 16-token slice of the tile and walks over ALL kv heads, so
@@ -423,16 +424,19 @@ static size_t gqa_lds_bytes(int n_q_heads, int n_kv_heads) {
 // issued back to back - HBM sees complete rows instead of 64-byte pieces that are
 // revisited later.  The next tile's rows are prefetched while the current ones are
 // multiplied (two register sets, used alternately).
-template <int SCHEME, int NKV>  // NKV = n_kv_heads rounded up to 4/8/16
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 4 : 2))) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
+// NSET sets of four query heads per kv head (1: up to 4 heads, 2: up to 8): the unpacked codes
+// of a kv head are multiplied with one block-diagonal A operand per set.
+template <int SCHEME, int NKV, int NSET = 1>  // NKV = n_kv_heads rounded up to 4/8/16
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET <= 8 ? 4 : 2))) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
+  constexpr int SL = 4 * NSET;  // head slots per kv head
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
   static_assert(kGqaTilesPerBlock % 2 == 0, "tiles are processed in pairs");
   extern __shared__ float gqa_lds[];
-  float* stage = gqa_lds;                            // [kv head][4 head slots][token in tile]
-  float4* qs4 = reinterpret_cast<float4*>(stage + a.n_kv_heads * 4 * kTile);  // [kv head][group]: q sums of its <=4 heads
-  uint4* alds = reinterpret_cast<uint4*>(qs4 + a.n_kv_heads * 4);        // [kv head][b][gq*4 + r]
-  uint4* azero = alds + a.n_kv_heads * 64;                                // same shape, all zero
+  float* stage = gqa_lds;                            // [kv head][SL head slots][token in tile]
+  float4* qs4 = reinterpret_cast<float4*>(stage + a.n_kv_heads * SL * kTile);  // [set][kv head][group]: q sums of the set's 4 heads
+  uint4* alds = reinterpret_cast<uint4*>(qs4 + NSET * a.n_kv_heads * 4);  // [set][kv head][b][gq*4 + r]
+  uint4* azero = alds + NSET * a.n_kv_heads * 64;                         // [kv head][b][gq*4 + r], all zero
   const int meta_stride = a.n_kv_heads * 4 + 2;      // halves; +2 spreads the tokens over banks
   uint16_t* smeta = reinterpret_cast<uint16_t*>(azero + a.n_kv_heads * 64);
   uint16_t* zmeta = smeta + kTile * meta_stride;
@@ -442,7 +446,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 
   const int64_t tile0 = (int64_t)blockIdx.x * kGqaTilesPerBlock;
   const int64_t tok0 = tile0 * kTile;
   if (tok0 >= len) return;  // uniform for the block
-  const int rep = a.n_q_heads / a.n_kv_heads;  // <= 4
+  const int rep = a.n_q_heads / a.n_kv_heads;  // <= 4 NSET
   const int lanes_per_row = a.n_kv_heads * 4;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -493,8 +497,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 
 
   // Prologue: group sums of q, and the non-zero part of the block-diagonal A
   // operands: entry (g, b, gq, r) = q[g*rep + r][32*gq + 8*b + {0,4,1,5,2,6,3,7}].
-  for (int i = threadIdx.x; i < a.n_kv_heads * 16; i += 256) {
-    const int g = i >> 4, gq = (i >> 2) & 3, r = i & 3;
+  // (set s holds heads g*rep + 4 s + r of kv head g)
+  for (int i = threadIdx.x; i < NSET * a.n_kv_heads * 16; i += 256) {
+    const int set = i / (a.n_kv_heads * 16), ig = i - set * a.n_kv_heads * 16;
+    const int g = ig >> 4, gq = (ig >> 2) & 3, r = (ig & 3) + 4 * set;
     float sacc = 0.f;
     if (r < rep) {
       float h32[32];
@@ -504,18 +510,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 
     }
     reinterpret_cast<float*>(qs4)[i] = sacc;
   }
-  for (int i = threadIdx.x; i < a.n_kv_heads * 64; i += 256) {
-    const int g = i >> 6, b2 = (i >> 4) & 3, gq = (i >> 2) & 3, r = i & 3;
+  for (int i = threadIdx.x; i < NSET * a.n_kv_heads * 64; i += 256) {
+    const int set = i / (a.n_kv_heads * 64), ig = i - set * a.n_kv_heads * 64;
+    const int g = ig >> 6, b2 = (ig >> 4) & 3, gq = (ig >> 2) & 3, r = (ig & 3) + 4 * set;
     uint4 d = make_uint4(0, 0, 0, 0);
     if (r < rep) d = ld16(qbase + (int64_t)(g * rep + r) * 128 + gq * 32 + b2 * 8);
     alds[i] = make_uint4((d.x & 0xffffu) | (d.z << 16), (d.x >> 16) | (d.z & 0xffff0000u),
                          (d.y & 0xffffu) | (d.w << 16), (d.y >> 16) | (d.w & 0xffff0000u));
-    azero[i] = make_uint4(0, 0, 0, 0);
+    if (set == 0) azero[ig] = make_uint4(0, 0, 0, 0);
   }
 
   const float zbias = 128.0f - (float)Q::qmin;  // 128 (asymmetric) or 136 (symmetric)
   // a lane whose k-slice does not meet its row's group reads zeros
-  const uint4* a_lane = (((nl >> 2) == rg) ? alds : azero) + nl;
+  const bool a_on = (nl >> 2) == rg;
+  const uint4* a_lane[NSET];
+#pragma unroll
+  for (int set = 0; set < NSET; ++set) a_lane[set] = (a_on ? alds + set * a.n_kv_heads * 64 : azero) + nl;
   const uint32_t kNib = 0x000f000fu, kExp = 0x43004300u;  // two nibbles -> two bf16 values 128 + code
 
   // One tile: returns false when the block has run past the cache's fill.
@@ -546,35 +556,43 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV <= 8 ? 
     for (int g = 0; g < NKV; ++g) {
       if (g < a.n_kv_heads) {
         const uint32_t wv[4] = {cur.cv[g].x, cur.cv[g].y, cur.cv[g].z, cur.cv[g].w};
-        pikv_f32x4 pc = {0.f, 0.f, 0.f, 0.f};
+        pikv_f32x4 pc[NSET];
+#pragma unroll
+        for (int set = 0; set < NSET; ++set) pc[set] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int b2 = 0; b2 < 4; ++b2) {
           const uint32_t w = Q::sym ? (wv[b2] ^ 0x88888888u) : wv[b2];
           const uint4 bb = make_uint4(and_or(w, kNib, kExp), and_or(w >> 4, kNib, kExp),
                                       and_or(w >> 8, kNib, kExp), and_or(w >> 12, kNib, kExp));
-          const uint4 av = a_lane[(g * 4 + b2) * 16];
-          pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, av),
-                                                       __builtin_bit_cast(pikv_bf16x8, bb), pc, 0, 0, 0);
+#pragma unroll
+          for (int set = 0; set < NSET; ++set) {
+            const uint4 av = a_lane[set][(g * 4 + b2) * 16];
+            pc[set] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, av),
+                                                              __builtin_bit_cast(pikv_bf16x8, bb), pc[set], 0, 0, 0);
+          }
         }
         const int mo = tl * meta_stride + g * 4 + rg;
         const float sc = (float)__builtin_bit_cast(_Float16, smeta[mo]);
         const float zq = (Q::sym ? 0.f : (float)__builtin_bit_cast(_Float16, zmeta[mo])) + zbias;
-        const float4 qv = qs4[g * 4 + rg];
-        const float t0 = sc * fmaf(-zq, qv.x, pc[0]), t1 = sc * fmaf(-zq, qv.y, pc[1]);
-        const float t2 = sc * fmaf(-zq, qv.z, pc[2]), t3 = sc * fmaf(-zq, qv.w, pc[3]);
-        // sum over the four row-groups; row-group r ends with head r
-        auto s01 = __builtin_amdgcn_permlane16_swap(__float_as_uint(t0), __float_as_uint(t1), false, false);
-        auto s23 = __builtin_amdgcn_permlane16_swap(__float_as_uint(t2), __float_as_uint(t3), false, false);
-        const float u01 = __uint_as_float(s01[0]) + __uint_as_float(s01[1]);
-        const float u23 = __uint_as_float(s23[0]) + __uint_as_float(s23[1]);
-        auto sf = __builtin_amdgcn_permlane32_swap(__float_as_uint(u01), __float_as_uint(u23), false, false);
-        const float score = (__uint_as_float(sf[0]) + __uint_as_float(sf[1])) * a.scale_qk;
-        if (rg < rep) stage[(g * 4 + rg) * kTile + tl] = okt ? score : -__builtin_inff();
+#pragma unroll
+        for (int set = 0; set < NSET; ++set) {
+          const float4 qv = qs4[(set * a.n_kv_heads + g) * 4 + rg];
+          const float t0 = sc * fmaf(-zq, qv.x, pc[set][0]), t1 = sc * fmaf(-zq, qv.y, pc[set][1]);
+          const float t2 = sc * fmaf(-zq, qv.z, pc[set][2]), t3 = sc * fmaf(-zq, qv.w, pc[set][3]);
+          // sum over the four row-groups; row-group r ends with head r of the set
+          auto s01 = __builtin_amdgcn_permlane16_swap(__float_as_uint(t0), __float_as_uint(t1), false, false);
+          auto s23 = __builtin_amdgcn_permlane16_swap(__float_as_uint(t2), __float_as_uint(t3), false, false);
+          const float u01 = __uint_as_float(s01[0]) + __uint_as_float(s01[1]);
+          const float u23 = __uint_as_float(s23[0]) + __uint_as_float(s23[1]);
+          auto sf = __builtin_amdgcn_permlane32_swap(__float_as_uint(u01), __float_as_uint(u23), false, false);
+          const float score = (__uint_as_float(sf[0]) + __uint_as_float(sf[1])) * a.scale_qk;
+          if (4 * set + rg < rep) stage[(g * SL + 4 * set + rg) * kTile + tl] = okt ? score : -__builtin_inff();
+        }
       }
     }
     __syncthreads();
 
-    tile_stats_store<true>(a, stage, c, tile, n0, len, wave, rg, nl, rep);
+    tile_stats_store<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep);
     __syncthreads();  // stage and the metadata rows are reused by the next tile
     return true;
   };
@@ -731,15 +749,25 @@ static int launch_i8_mfma(const ScoreArgs& a, int n_caches, int64_t n_tiles, hip
 
 template <int SCHEME>
 static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
-  const size_t lds = gqa_lds_bytes(a.n_q_heads, a.n_kv_heads);
-  if (lds > 64 * 1024 || a.n_kv_heads > kGqaMaxKvHeads) return PIKV_ERR_UNSUPPORTED;
+  const int rep = a.n_q_heads / a.n_kv_heads;
+  const int nset = rep <= 4 ? 1 : 2;
+  const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset);
+  if (rep > 8 || lds > 64 * 1024 || a.n_kv_heads > kGqaMaxKvHeads) return PIKV_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
-  if (a.n_kv_heads <= 4)
-    hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4>), grid, dim3(256), lds, st, a);
-  else if (a.n_kv_heads <= 8)
-    hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8>), grid, dim3(256), lds, st, a);
-  else
-    hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 16>), grid, dim3(256), lds, st, a);
+  if (nset == 1) {
+    if (a.n_kv_heads <= 4)
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1>), grid, dim3(256), lds, st, a);
+    else if (a.n_kv_heads <= 8)
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1>), grid, dim3(256), lds, st, a);
+    else
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 16, 1>), grid, dim3(256), lds, st, a);
+  } else {
+    // 5-8 query heads per kv head; 16 kv heads x 8 would need more than 64 KB of LDS
+    if (a.n_kv_heads <= 4)
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2>), grid, dim3(256), lds, st, a);
+    else
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2>), grid, dim3(256), lds, st, a);
+  }
   return PIKV_OK;
 }
 
@@ -982,7 +1010,7 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   if (!eight && group == 32 && head_dim == 128 && q_dtype == PIKV_BF16 && rep <= 16) {
     int grc = PIKV_ERR_UNSUPPORTED;
     const size_t mlds = (size_t)n_q_heads * (kTile + 4) * sizeof(float);
-    if (rep <= 4)
+    if (rep <= 8)
       grc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(a, n_caches, n_tiles, st)
                                        : launch_gqa<PIKV_Q_I4_SYM>(a, n_caches, n_tiles, st);
     if (grc == PIKV_OK) {

@@ -47,6 +47,9 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I4_ASYM, 32, 1, 16, 128),     # matrix-core kernel, all 16 rows of the tile in use
     (O.Q_I4_ASYM, 32, 8, 64, 128),     # 8 q heads per kv head: two sets of A rows against the same codes
     (O.Q_I4_SYM, 32, 2, 12, 128),      # 6 q heads per kv head: the second set half empty
+    (O.Q_I4_ASYM, 32, 4, 28, 128),     # 7 q heads per kv head
+    (O.Q_I4_SYM, 32, 8, 40, 128),      # 5 q heads per kv head, 8 kv heads
+    (O.Q_I4_ASYM, 32, 16, 128, 128),   # 16 kv heads x 8: too much LDS for two sets, generic kernel
     (O.Q_I4_ASYM, 32, 16, 16, 128),    # more kv heads than wavefronts, one q head each
     (O.Q_I4_ASYM, 32, 8, 24, 128),     # 3 q heads per kv head: one of the four staged head slots stays empty
     (O.Q_I4_SYM, 32, 4, 4, 128),       # one q head per kv head on the GQA kernel
