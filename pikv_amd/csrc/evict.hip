@@ -401,11 +401,9 @@ __global__ __launch_bounds__(kMbThreads) void mb_hist_kernel(MbArgs a) {
   for (int slot = blockIdx.z; slot <= (int)blockIdx.z; ++slot) {
     const MbSel s = mb_sel(a, c, slot, len);
     int* bh = PASS == 2 ? a.blk_hist2 + (((int64_t)c * a.n_chunks + chunk) * 2 + slot) * 1024 : nullptr;
-    if (!s.partial || (int64_t)chunk * kMbChunk >= len) {  // uniform
-      if (PASS == 2)
-        for (int b = threadIdx.x; b < 1024; b += kMbThreads) bh[b] = 0;
-      continue;
-    }
+    // (no table for such a chunk: the marking pass reads the tables of chunks before one that
+    // lies inside the cache, for selections that need a threshold)
+    if (!s.partial || (int64_t)chunk * kMbChunk >= len) continue;  // uniform
     int remaining = s.m;
     const uint32_t prefix = mb_prefix(a, c, slot, PASS, remaining, sh, nullptr);
     const uint32_t pmask = mb_mask(PASS);
