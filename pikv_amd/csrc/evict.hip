@@ -517,12 +517,16 @@ __global__ __launch_bounds__(kMbThreads) void mb_list_kernel(MbArgs a) {
 #pragma unroll
   for (int j = 0; j < kMbItems; ++j)
     if (i0 + j < len && flag[i0 + j]) keep |= 1u << j;
+  // the chunk's survivors are gathered in LDS and leave as one contiguous run
+  __shared__ int32_t run[kMbChunk];
   int tot;
-  int pos = all + mb_block_scan(__popc(keep), sh, tot);
-  int32_t* out = a.keep_index + a.row_base[c];
+  int pos = mb_block_scan(__popc(keep), sh, tot);
 #pragma unroll
   for (int j = 0; j < kMbItems; ++j)
-    if ((keep >> j) & 1u) out[pos++] = (int32_t)(i0 + j);
+    if ((keep >> j) & 1u) run[pos++] = (int32_t)(i0 + j);
+  __syncthreads();
+  int32_t* out = a.keep_index + a.row_base[c] + all;
+  for (int i = threadIdx.x; i < tot; i += kMbThreads) out[i] = run[i];
 }
 
 __global__ void h2o_budget_kernel(const int32_t* __restrict__ fill, int n, double heavy_ratio,
