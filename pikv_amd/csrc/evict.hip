@@ -489,9 +489,17 @@ __global__ __launch_bounds__(kMbThreads) void mb_mark_kernel(MbArgs a) {
   for (int j = 0; j < kMbItems; ++j) valid |= (i0 + j < len ? 1u : 0u) << j;
   const uint32_t keep = (a.policy == PIKV_EVICT_H2O ? (selbits[0] | selbits[1]) : ~selbits[0]) & valid;
   uint8_t* flag = a.keep_flag + a.row_base[c];
+  static_assert(kMbItems == 16, "sixteen flags = one 16-byte store");
+  if (valid == 0xffffu && (reinterpret_cast<uintptr_t>(flag + i0) & 15) == 0) {
+    // four bits -> four 0/1 bytes: the shifts 0, 7, 14, 21 put bit k at bit 8 k
+    auto spread = [](uint32_t nib) { return ((nib & 0xfu) * 0x00204081u) & 0x01010101u; };
+    *reinterpret_cast<uint4*>(flag + i0) =
+        make_uint4(spread(keep), spread(keep >> 4), spread(keep >> 8), spread(keep >> 12));
+  } else {
 #pragma unroll
-  for (int j = 0; j < kMbItems; ++j)
-    if ((valid >> j) & 1u) flag[i0 + j] = (keep >> j) & 1u;
+    for (int j = 0; j < kMbItems; ++j)
+      if ((valid >> j) & 1u) flag[i0 + j] = (keep >> j) & 1u;
+  }
   int kept;
   mb_block_scan(__popc(keep), sh, kept);
   if (threadIdx.x == 0) a.blk_kept[(int64_t)c * a.n_chunks + chunk] = kept;
@@ -514,9 +522,16 @@ __global__ __launch_bounds__(kMbThreads) void mb_list_kernel(MbArgs a) {
   const int64_t i0 = (int64_t)chunk * kMbChunk + threadIdx.x * kMbItems;
   const uint8_t* flag = a.keep_flag + a.row_base[c];
   uint32_t keep = 0;
+  if (i0 + kMbItems <= len && (reinterpret_cast<uintptr_t>(flag + i0) & 15) == 0) {
+    // four 0/1 bytes -> four bits: the shifts 3, 10, 17, 24 collect them in bits 24..27
+    const uint4 f = *reinterpret_cast<const uint4*>(flag + i0);
+    auto gather = [](uint32_t w) { return (((w & 0x01010101u) * 0x01020408u) >> 24) & 0xfu; };
+    keep = gather(f.x) | (gather(f.y) << 4) | (gather(f.z) << 8) | (gather(f.w) << 12);
+  } else {
 #pragma unroll
-  for (int j = 0; j < kMbItems; ++j)
-    if (i0 + j < len && flag[i0 + j]) keep |= 1u << j;
+    for (int j = 0; j < kMbItems; ++j)
+      if (i0 + j < len && flag[i0 + j]) keep |= 1u << j;
+  }
   // the chunk's survivors are gathered in LDS and leave as one contiguous run
   __shared__ int32_t run[kMbChunk];
   int tot;
