@@ -343,7 +343,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     stage();
     __syncthreads();
     float acc = pacc;
-    if (n0 + kAttTile < t1) fetch(n0 + kAttTile);  // in flight while this tile is multiplied
     if (a.row_acc || a.row_ts) {  // uniform
       // importance of the tile's tokens: four lanes per token add every fourth head, and two
       // exchanges add the four partial sums
@@ -372,6 +371,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
         }
       }
     }
+    // The next tile's loads go out AFTER the bookkeeping stores: the wait at the top of the
+    // loop covers everything outstanding, and stores issued behind the loads had been
+    // adding their latency to it (366 vs 347 us).
+    if (n0 + kAttTile < t1) fetch(n0 + kAttTile);  // in flight while this tile is multiplied
 
 #pragma unroll
     for (int hs = 0; hs < NH; ++hs) {
