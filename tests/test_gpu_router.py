@@ -216,6 +216,52 @@ def test_router_short_stream_split(dev, T, H, E, k):
     assert torch.equal(out.logits, again.logits) and torch.equal(out.topk_w, again.topk_w)
 
 
+@pytest.mark.parametrize("module", [False, True])
+def test_router_tiled_and_rows_forms_logit_arithmetic(dev, module):
+    """Temperature, per-expert scale, mask and bias through the branch-free per-row arithmetic of
+    the token-per-lane forms, in both orders of the reference's two router copies: the
+    standalone tail (bit-exact against the restatement) and the tiled gate kernel (final logits
+    against float64, top-k exact on the kernel's own logits, masked experts never chosen)."""
+    import torch
+    from pikv_amd import ops
+    r = rng(170 + module)
+    T, E, k = 3000, 64, 8
+    lg = (r.standard_normal((T, E)) * 3).astype(np.float32)
+    lg[::4, 2] = lg[::4, 7]
+    scale = (0.5 + r.random(E)).astype(np.float32)
+    mask = np.ones(E, dtype=np.float32)
+    mask[[1, 9, 33]] = 0
+    kw = dict(temperature=0.7, expert_scale=scale, expert_mask=mask, renorm_eps=1e-8 if module else 0.0)
+    out = ops.router_tail(to_dev(lg, dev), top_k=k, temperature=0.7, expert_scale=to_dev(scale, dev),
+                          expert_mask=to_dev(mask, dev), renorm_eps=kw["renorm_eps"], module_arithmetic=module)
+    probs, idx, w, final = O.router_tail(lg, k, module_arithmetic=module, **kw)
+    assert np.array_equal(np_of(out.topk_idx), idx)
+    assert np.allclose(np_of(out.probs), probs, atol=2e-6, rtol=1e-5)
+    assert np.allclose(np_of(out.topk_w), w, atol=2e-6, rtol=1e-5)
+    assert not np.isin(np_of(out.topk_idx), [1, 9, 33]).any()
+    # tiled gate kernel (more than 20480 tokens)
+    T2, H = 20480 + 77, 256
+    g = torch.Generator(device=dev).manual_seed(5 + module)
+    x = torch.randn(T2, H, generator=g, device=dev).to(torch.bfloat16)
+    wg = (0.05 * torch.randn(E, H, generator=g, device=dev)).to(torch.bfloat16)
+    b = 0.1 * torch.randn(E, generator=g, device=dev)
+    o2 = ops.router_fused(x, wg, b, top_k=k, temperature=0.7, expert_scale=to_dev(scale, dev),
+                          expert_mask=to_dev(mask, dev), renorm_eps=kw["renorm_eps"], module_arithmetic=module,
+                          return_logits=True)
+    raw = (x.double() @ wg.double().T + b.double()).float().cpu().numpy()
+    want = O.scale_logits(raw, 0.7, scale, mask, module_arithmetic=module)
+    fin = np_of(o2.logits)
+    live = mask > 0
+    assert np.allclose(fin[:, live], want[:, live], atol=2e-5 * H ** 0.5, rtol=2e-5)
+    assert (fin[:, ~live] < (-1e38 if module else -1e8)).all()
+    order = torch.sort(o2.logits, dim=1, descending=True, stable=True).indices[:, :k]
+    assert torch.equal(o2.topk_idx.long(), order)
+    assert not np.isin(np_of(o2.topk_idx), [1, 9, 33]).any()
+    _, idx2, w2, _ = O.router_tail(fin, k, renorm_eps=kw["renorm_eps"])
+    assert np.array_equal(np_of(o2.topk_idx), idx2)
+    assert np.allclose(np_of(o2.topk_w), w2, atol=2e-6, rtol=1e-5)
+
+
 def test_router_module_arithmetic(dev):
     """The arithmetic of the reference's module/ copy (core/single/module/pikv_routing.py:596-600,
     :133-134, :143): scale before temperature, finfo.min penalty, + 1e-8 in the renormalisation -
