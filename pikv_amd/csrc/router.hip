@@ -783,18 +783,31 @@ __global__ __launch_bounds__(64) void slot_scan_kernel(int32_t* __restrict__ ws,
   const int64_t per = (n_chunks + 63) / 64;
   const int64_t b0 = lane * per;
   const int64_t b1 = (b0 + per < n_chunks) ? b0 + per : n_chunks;
+  // (eight loads in flight per lane: the chunks of a lane are a chain of dependent round trips
+  // to L2 otherwise)
   int total = 0;
-  for (int64_t b = b0; b < b1; ++b) total += ws[b * E + e];
+  for (int64_t b = b0; b < b1; b += 8) {
+    int v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = (b + u < b1) ? ws[(b + u) * E + e] : 0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) total += v[u];
+  }
   int incl = total;
   for (int d = 1; d < 64; d <<= 1) {
     const int up = __shfl_up(incl, d, PIKV_WAVE);
     if (lane >= d) incl += up;
   }
   int run = incl - total;
-  for (int64_t b = b0; b < b1; ++b) {
-    const int v = ws[b * E + e];
-    ws[b * E + e] = run;
-    run += v;
+  for (int64_t b = b0; b < b1; b += 8) {
+    int v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = (b + u < b1) ? ws[(b + u) * E + e] : 0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (b + u < b1) ws[(b + u) * E + e] = run;
+      run += v[u];
+    }
   }
   if (count && lane == 63) count[e] = incl;
 }
