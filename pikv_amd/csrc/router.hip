@@ -834,16 +834,16 @@ __global__ __launch_bounds__(256) void slot_rank_kernel(const int32_t* __restric
       if ((unsigned)e >= (unsigned)E) e = -1;  // out-of-range ids get slot -1
     }
     const bool valid = e >= 0;
-    int rank = 0;
-    uint64_t todo = __ballot(valid);
-    while (todo) {
-      const int leader = (int)__builtin_ctzll(todo);
-      const int e0 = __shfl(e, leader, PIKV_WAVE);
-      const uint64_t m = __ballot(valid && e == e0);
-      if (valid && e == e0) rank = __popcll(m & lt_mask);
-      if (lane == leader) wcnt[wave][e0] = __popcll(m);
-      todo &= ~m;
+    // lanes with the same expert: one ballot per bit of the expert id, and every lane keeps
+    // the side of each ballot it is on (six ballots instead of one round per distinct expert)
+    uint64_t same = __ballot(valid);
+#pragma unroll
+    for (int bit = 0; bit < 6; ++bit) {
+      const uint64_t ones = __ballot(valid && ((e >> bit) & 1));
+      same &= ((e >> bit) & 1) ? ones : ~ones;
     }
+    const int rank = __popcll(same & lt_mask);
+    if (valid && rank == 0) wcnt[wave][e] = __popcll(same);
     __syncthreads();
     if (valid) {
       int pos = running[e] + rank;
