@@ -568,6 +568,85 @@ __device__ __forceinline__ void lane_token_tail(float* row, int64_t t, const Tai
   }
 }
 
+// The same for 64 columns with TWO lanes per token: `half` 0 takes experts 0..31, half 1 the
+// rest.  Each sorts its 32, the two top-8 lists meet in LDS and are merged by both; each takes
+// the exponentials, the partial sum (two 16-trees) and the divisions of its half - the total
+// is still (R0 + R1) + (R2 + R3) - and half 0 writes the token's top-k.  Every thread of the
+// block has to call this (three block barriers); `active` says whether it holds a token.
+// xkeys: [8][2][TB] 64-bit keys, xsum: [2][TB] floats.
+template <int RS, int TB>
+__device__ __forceinline__ void pair_token_tail(float* row, int half, int tl, bool active, int64_t t,
+                                                const TailParams& p, uint64_t* xkeys, float* xsum) {
+  uint64_t top[8];
+  if (active) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      uint64_t cur[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int e = 32 * half + 8 * g + i;
+        cur[i] = e < p.E ? lane_topk_key(row[e], e) : 0ull;
+      }
+      sort8_desc(cur);
+      if (g == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) top[i] = cur[i];
+      } else {
+        merge_top8(top, cur);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) xkeys[(j * 2 + half) * TB + tl] = top[j];
+  }
+  __syncthreads();
+  int idx[8];
+  float ex[32];
+  if (active) {
+    uint64_t other[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) other[j] = xkeys[(j * 2 + (1 - half)) * TB + tl];
+    merge_top8(top, other);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) idx[j] = 63 - (int)(uint32_t)top[j];
+    const float m = row[idx[0]];
+#pragma unroll
+    for (int e = 0; e < 32; ++e) ex[e] = expf(row[32 * half + e] - m);  // padding: expf(-inf) = 0
+    xsum[half * TB + tl] = tree16(ex) + tree16(ex + 16);
+  }
+  __syncthreads();
+  if (active) {
+    const float sum = xsum[tl] + xsum[TB + tl];
+#pragma unroll
+    for (int e = 0; e < 32; ++e) row[32 * half + e] = ex[e] / sum;
+  }
+  __syncthreads();
+  if (!active || half != 0 || t >= p.T) return;
+  float pv[8], wsum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    pv[j] = j < p.k ? row[idx[j]] : 0.f;
+    if (j < p.k) wsum = wsum + pv[j];
+  }
+  if (p.renorm_eps != 0.f) wsum = wsum + p.renorm_eps;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) pv[j] = pv[j] / wsum;
+  if (p.k == 8) {
+    int4* oi = reinterpret_cast<int4*>(p.topk_idx + t * 8);
+    float4* ow = reinterpret_cast<float4*>(p.topk_w + t * 8);
+    oi[0] = make_int4(idx[0], idx[1], idx[2], idx[3]);
+    oi[1] = make_int4(idx[4], idx[5], idx[6], idx[7]);
+    ow[0] = make_float4(pv[0], pv[1], pv[2], pv[3]);
+    ow[1] = make_float4(pv[4], pv[5], pv[6], pv[7]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < p.k) {
+        p.topk_idx[t * p.k + j] = idx[j];
+        p.topk_w[t * p.k + j] = pv[j];
+      }
+  }
+}
+
 // Long token streams: the classic tiled form.  A block owns TB tokens x EP (padded)
 // experts; its 256 threads bring KS k-values of every token row (256 or 512 contiguous
 // bytes per row, whole rows per load instruction) through registers into one of two LDS
@@ -686,7 +765,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void r
   }
   __syncthreads();
   // lane = token: softmax and top-k of a whole row on registers
-  if (tid < TB) lane_token_tail<EP, RS>(red + tid * RS, tok0 + tid, p);
+  if constexpr (EP == 64) {
+    // two lanes per token; the exchange area lies behind the logits
+    static_assert(TB * RS * 4 + 8 * 2 * TB * 8 + 2 * TB * 4 <= LDS_BYTES, "exchange area fits behind the logits");
+    uint64_t* xkeys = reinterpret_cast<uint64_t*>(lds + ((TB * RS * 4 + 7) & ~7));
+    float* xsum = reinterpret_cast<float*>(xkeys + 8 * 2 * TB);
+    const int half = tid / TB, tl = tid % TB;
+    pair_token_tail<RS, TB>(red + tl * RS, half, tl, tid < 2 * TB, tok0 + tl, p, xkeys, xsum);
+  } else {
+    if (tid < TB) lane_token_tail<EP, RS>(red + tid * RS, tok0 + tid, p);
+  }
   __syncthreads();
   if (p.probs) {
     for (int i = 0; i < TW; i += TPP) {
