@@ -24,7 +24,7 @@
 namespace pikv {
 
 constexpr int kSlotChunk = 512;  // assignments per block in the slot pass
-constexpr int kRowsTailMinK = 5;  // standalone tail, 33-64 experts: a token per lane from this k on
+constexpr int kRowsTailMinK = 2;  // standalone tail, 33-64 experts: lanes per token instead of per expert from this k on
 
 struct TailParams {
   const float* bias;
@@ -608,6 +608,19 @@ __device__ __forceinline__ void pair_token_tail(float* row, int half, int tl, bo
     merge_top8(top, other);
 #pragma unroll
     for (int j = 0; j < 8; ++j) idx[j] = 63 - (int)(uint32_t)top[j];
+  }
+  if (!p.use_softmax) {  // raw top-k: the selected logits themselves (uniform for the block)
+    if (active && half == 0 && t < p.T) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (j < p.k) {
+          p.topk_idx[t * p.k + j] = idx[j];
+          p.topk_w[t * p.k + j] = row[idx[j]];
+        }
+    }
+    return;
+  }
+  if (active) {
     const float m = row[idx[0]];
 #pragma unroll
     for (int e = 0; e < 32; ++e) ex[e] = expf(row[32 * half + e] - m);  // padding: expf(-inf) = 0
@@ -790,54 +803,57 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void r
 // per token.
 template <int MODE>
 __device__ __forceinline__ void tail_rows_stage(const float* __restrict__ la, const float* __restrict__ lb,
-                                                uint64_t from_a, int64_t tbase, int wave, int lane,
+                                                uint32_t from_a, int64_t tbase, int wave, int lane,
                                                 float* red, const TailParams& p) {
   constexpr int RS = 65;
   const ExpertConsts ec = load_expert_consts(lane, p);
   const bool col = lane < p.E;
-  for (int i0 = 0; i0 < 64; i0 += 16) {
+  for (int i0 = 0; i0 < 32; i0 += 16) {
     float v[16];  // sixteen rows in flight per wavefront
 #pragma unroll
     for (int u = 0; u < 16; ++u) {
       const int64_t t = tbase + i0 + u;
-      const float* src = ((from_a >> (i0 + u)) & 1ull) ? la : lb;
+      const float* src = ((from_a >> (i0 + u)) & 1u) ? la : lb;
       v[u] = (t < p.T && col) ? src[t * p.E + lane] : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < 16; ++u) {
-      const int tl = 64 * wave + i0 + u;
+      const int tl = 32 * wave + i0 + u;
       const float lg = final_logit_rows<MODE>(v[u], ec, p.temperature);
       red[tl * RS + lane] = (tbase + i0 + u < p.T && col) ? lg : -__builtin_inff();
     }
   }
 }
 
-__global__ __launch_bounds__(128) void router_tail_rows_kernel(const float* __restrict__ la,
+__global__ __launch_bounds__(256) void router_tail_rows_kernel(const float* __restrict__ la,
                                                                const float* __restrict__ lb,
                                                                const uint8_t* __restrict__ select,
                                                                TailParams p) {
   constexpr int TB = 128, RS = 65;
   __shared__ float red[TB * RS];
+  __shared__ uint64_t xkeys[8 * 2 * TB];
+  __shared__ float xsum[2 * TB];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: row addresses stay scalar
   const int64_t tok0 = (int64_t)blockIdx.x * TB;
-  const int64_t tbase = tok0 + 64 * wave;  // first token of this wavefront
-  uint64_t from_a = ~0ull;                 // bit i: token tbase + i reads logits_a
+  const int64_t tbase = tok0 + 32 * wave;  // first of the 32 tokens this wavefront stages
+  uint32_t from_a = ~0u;                   // bit i: token tbase + i reads logits_a
   if (lb != nullptr && select != nullptr) {
-    const int64_t t = tbase + lane;
-    from_a = __ballot(t < p.T ? select[t] != 0 : true);
+    const int64_t t = tbase + (lane & 31);
+    from_a = (uint32_t)__ballot(t < p.T ? select[t] != 0 : true);
   }
   const int mode = final_logit_mode(p);
   if (mode == 0) tail_rows_stage<0>(la, lb, from_a, tbase, wave, lane, red, p);
   else if (mode == 1) tail_rows_stage<1>(la, lb, from_a, tbase, wave, lane, red, p);
   else tail_rows_stage<2>(la, lb, from_a, tbase, wave, lane, red, p);
   __syncthreads();
-  lane_token_tail<64, RS>(red + tid * RS, tok0 + tid, p);
-  __syncthreads();
-  if (p.probs) {
-    for (int i = 0; i < 64; ++i) {
+  // two lanes per token: threads 0..127 take experts 0..31, threads 128..255 the rest
+  const int half = tid / TB, tl = tid % TB;
+  pair_token_tail<RS, TB>(red + tl * RS, half, tl, true, tok0 + tl, p, xkeys, xsum);
+  if (p.probs) {  // (not with the raw top-k, which has returned without the last barrier)
+    for (int i = 0; i < 32; ++i) {
       const int64_t t = tbase + i;
-      if (t < p.T && lane < p.E) p.probs[t * p.E + lane] = red[(64 * wave + i) * RS + lane];
+      if (t < p.T && lane < p.E) p.probs[t * p.E + lane] = red[(32 * wave + i) * RS + lane];
     }
   }
 }
@@ -1174,9 +1190,9 @@ extern "C" int pikv_router_tail(const float* logits_a, const float* logits_b, co
       case 32: hipLaunchKernelGGL((router_tail_kernel<32>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p); break;
       default:
         // 33-64 experts: an arg-max round over 64 lanes costs ~2.9 us per round at 65536 tokens
-        // (20 us at k = 1), a token per lane 31 us whatever k
+        // (21 us at k = 1, 24 at k = 2), two lanes per token 20.6 us whatever k
         if (k >= kRowsTailMinK)
-          hipLaunchKernelGGL(router_tail_rows_kernel, dim3((unsigned)((T + 127) / 128)), dim3(128), 0, st, logits_a, logits_b, select, p);
+          hipLaunchKernelGGL(router_tail_rows_kernel, dim3((unsigned)((T + 127) / 128)), dim3(256), 0, st, logits_a, logits_b, select, p);
         else
           hipLaunchKernelGGL((router_tail_kernel<64>), dim3((unsigned)blocks), dim3(256), 0, st, logits_a, logits_b, select, p);
         break;
