@@ -162,6 +162,23 @@ int pikv_capacity_slots(const int32_t* expert_idx, int64_t A, int E,
                         int64_t capacity, int32_t* slot, int32_t* count,
                         void* workspace, int64_t workspace_bytes, void* stream);
 
+/* pikv_capacity_slots for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference: there every intermediate is a fresh torch tensor.
+ * Same arguments, same kernels and bit-identical results as pikv_capacity_slots,
+ * but the per-chunk counters live in a 512 KiB device array that is part of the
+ * library image (one copy per GPU, held until the process ends) instead of a
+ * caller workspace; the call allocates and frees nothing.
+ *   A <= pikv_capacity_slots_static_max() (= 1048576 assignments), E <= 64;
+ *   a larger A returns PIKV_ERR_WORKSPACE and enqueues nothing.
+ *   All calls on one GPU share the array: calls that overlap on one GPU (two
+ *   streams, two threads) race; calls on one stream are ordered and safe.
+ *   The device that is current at the call must be the one that owns the pointers. */
+int pikv_capacity_slots_static(const int32_t* expert_idx, int64_t A, int E,
+                               int64_t capacity, int32_t* slot, int32_t* count,
+                               void* stream);
+int64_t pikv_capacity_slots_static_max(void);
+
 /* Workspace of pikv_router_tail / pikv_capacity_slots, and of pikv_router_fused. */
 int64_t pikv_router_workspace_bytes(int64_t T, int E, int k);
 int64_t pikv_router_fused_workspace_bytes(int64_t T, int H, int E, int k);

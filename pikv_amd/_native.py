@@ -34,6 +34,8 @@ SIGNATURES = {
     "pikv_router_tail": (_i, [_p, _p, _p, _p, _p, _f, _f, _i, _i, _l, _i, _i, _l,
                               _p, _p, _p, _p, _p, _p, _l, _p]),
     "pikv_capacity_slots": (_i, [_p, _l, _i, _l, _p, _p, _p, _l, _p]),
+    "pikv_capacity_slots_static": (_i, [_p, _l, _i, _l, _p, _p, _p]),
+    "pikv_capacity_slots_static_max": (_l, []),
     "pikv_router_workspace_bytes": (_l, [_l, _i, _i]),
     "pikv_router_fused_workspace_bytes": (_l, [_l, _i, _i, _i]),
     "pikv_quant_scatter": (_i, [_p, _p, _i, _l, _i, _i, _i, _i, _p, _p, _p, _p, _p, _i,

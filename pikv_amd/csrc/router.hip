@@ -19,6 +19,8 @@
 // Capacity slots: deterministic three-step histogram / scan / rank over the
 // assignments in token-major order (integer LDS atomics only feed counts, whose
 // value does not depend on arrival order).
+#include <atomic>
+
 #include "common.hpp"
 
 namespace pikv {
@@ -1046,9 +1048,51 @@ extern "C" int64_t pikv_router_fused_workspace_bytes(int64_t T, int H, int E, in
 extern "C" int pikv_capacity_slots(const int32_t* expert_idx, int64_t A, int E, int64_t capacity,
                                    int32_t* slot, int32_t* count, void* workspace,
                                    int64_t workspace_bytes, void* stream) {
-  if (!expert_idx || !slot) return PIKV_ERR_NULL;
+  if (A != 0 && (!expert_idx || !slot)) return PIKV_ERR_NULL;  // an empty stream needs no buffers
   if (A < 0 || A > 0x7fffffffLL || E < 1 || E > 64 || capacity < 0) return PIKV_ERR_SHAPE;
   return launch_slots(expert_idx, A, E, capacity, slot, count, workspace, workspace_bytes,
+                      (hipStream_t)stream);
+}
+
+// ---- capacity slots for callers that cannot allocate ------------------------------
+// The per-chunk histograms of the slot pass live in a file-scope device array instead of a
+// caller workspace.  Every GPU holds its own copy of the array at its own address; the host
+// learns that address once per device and passes it to the kernels like any workspace.
+constexpr int64_t kSlotStaticMaxAssignments = 1 << 20;
+constexpr int kSlotStaticMaxExperts = 64;
+constexpr int64_t kSlotStaticWords = (kSlotStaticMaxAssignments / kSlotChunk) * kSlotStaticMaxExperts;
+static __device__ __align__(256) int32_t scratch[kSlotStaticWords];  // 512 KiB per GPU
+
+constexpr int kMaxDevices = 64;
+static std::atomic<int32_t*> g_scratch_ptr[kMaxDevices];
+
+// Address of this device's copy of `scratch` (looked up on the first call on the device).
+static int scratch_of_current_device(int32_t** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return PIKV_ERR_LAUNCH;
+  int32_t* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || !sym) return PIKV_ERR_LAUNCH;
+    p = static_cast<int32_t*>(sym);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // every thread finds the same address
+  }
+  *out = p;
+  return PIKV_OK;
+}
+
+extern "C" int64_t pikv_capacity_slots_static_max(void) { return kSlotStaticMaxAssignments; }
+
+extern "C" int pikv_capacity_slots_static(const int32_t* expert_idx, int64_t A, int E, int64_t capacity,
+                                          int32_t* slot, int32_t* count, void* stream) {
+  if (A != 0 && (!expert_idx || !slot)) return PIKV_ERR_NULL;  // an empty stream needs no buffers
+  if (A < 0 || E < 1 || E > kSlotStaticMaxExperts || capacity < 0) return PIKV_ERR_SHAPE;
+  if (A > kSlotStaticMaxAssignments) return PIKV_ERR_WORKSPACE;
+  int32_t* ws = nullptr;
+  const int rc = scratch_of_current_device(&ws);
+  if (rc != PIKV_OK) return rc;
+  // Nothing has to start at zero: the histogram pass writes every word the later passes read.
+  return launch_slots(expert_idx, A, E, capacity, slot, count, ws, kSlotStaticWords * (int64_t)sizeof(int32_t),
                       (hipStream_t)stream);
 }
 

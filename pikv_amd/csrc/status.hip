@@ -13,4 +13,4 @@ extern "C" const char* pikv_status_string(int status) {
   return "unknown status";
 }
 
-extern "C" int pikv_abi_version(void) { return 1001; }  // 1.1: + pikv_fakequant_preset
+extern "C" int pikv_abi_version(void) { return 1002; }  // 1.2: + pikv_capacity_slots_static
