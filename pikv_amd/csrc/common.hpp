@@ -148,12 +148,10 @@ __device__ __forceinline__ void quant_params(float mn, float mx, float& scale, f
       // holds exactly.  A group whose spread is tiny next to its offset (a constant
       // non-zero group, with the 1e-5 range above) would need a far larger one: its
       // scale is widened to |min| / 1024 (|zero| <= 1025).  Error <= |min| / 2048.
-#ifndef PIKV_AB_NO_WIDEN
       if (fabsf(mn) > 1024.0f * scale) {
         scale = (float)float_to_half_sat(fabsf(mn) * 0.0009765625f);
         if (scale == 0.0f) scale = 5.9604644775390625e-08f;
       }
-#endif
     }
   }
   if constexpr (Q::sym) {
@@ -283,28 +281,37 @@ __device__ __forceinline__ uint4 quantize_lane(const float (&x)[QScheme<SCHEME>:
 // quad_perm xor-1 / xor-2, row_half_mirror and row_mirror combine disjoint halves
 // inside a 16-lane row in one instruction each; wider groups finish with two
 // cross-row shuffles.
-// v = op(v, v of the partner lane) as ONE VOP2-DPP instruction.  The s_nop covers
-// the two wait states the ISA asks for between a VALU write and a DPP read of
-// the same register, which the compiler cannot see inside inline assembly.
-#define PIKV_DPP_INPLACE(op, v, ctrl)                                                     \
-  asm("s_nop 1\n\t" op " %0, %0, %0 " ctrl " row_mask:0xf bank_mask:0xf" : "+v"(v))
+// The partner's value comes from the data-parallel-primitive builtin, so the compiler sees
+// an ordinary VALU definition: it folds the move into the min / max / add that consumes it
+// (one VOP2-DPP instruction) and places every wait state itself, before and after.
+constexpr int kDppXor1 = 0xB1;         // quad_perm:[1,0,3,2]
+constexpr int kDppXor2 = 0x4E;         // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // row_half_mirror
+constexpr int kDppMirror = 0x140;      // row_mirror
+template <int CTRL>
+__device__ __forceinline__ float dpp_partner(float v) {
+  return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL> __device__ __forceinline__ float dpp_min(float v) { return fminf(v, dpp_partner<CTRL>(v)); }
+template <int CTRL> __device__ __forceinline__ float dpp_max(float v) { return fmaxf(v, dpp_partner<CTRL>(v)); }
+template <int CTRL> __device__ __forceinline__ float dpp_add(float v) { return v + dpp_partner<CTRL>(v); }
 
 __device__ __forceinline__ void group_minmax_dpp(float& mn, float& mx, int lanes) {
   if (lanes >= 2) {
-    PIKV_DPP_INPLACE("v_min_f32_dpp", mn, "quad_perm:[1,0,3,2]");
-    PIKV_DPP_INPLACE("v_max_f32_dpp", mx, "quad_perm:[1,0,3,2]");
+    mn = dpp_min<kDppXor1>(mn);
+    mx = dpp_max<kDppXor1>(mx);
   }
   if (lanes >= 4) {
-    PIKV_DPP_INPLACE("v_min_f32_dpp", mn, "quad_perm:[2,3,0,1]");
-    PIKV_DPP_INPLACE("v_max_f32_dpp", mx, "quad_perm:[2,3,0,1]");
+    mn = dpp_min<kDppXor2>(mn);
+    mx = dpp_max<kDppXor2>(mx);
   }
   if (lanes >= 8) {
-    PIKV_DPP_INPLACE("v_min_f32_dpp", mn, "row_half_mirror");
-    PIKV_DPP_INPLACE("v_max_f32_dpp", mx, "row_half_mirror");
+    mn = dpp_min<kDppHalfMirror>(mn);
+    mx = dpp_max<kDppHalfMirror>(mx);
   }
   if (lanes >= 16) {
-    PIKV_DPP_INPLACE("v_min_f32_dpp", mn, "row_mirror");
-    PIKV_DPP_INPLACE("v_max_f32_dpp", mx, "row_mirror");
+    mn = dpp_min<kDppMirror>(mn);
+    mx = dpp_max<kDppMirror>(mx);
   }
   if (lanes >= 32) { mn = fminf(mn, __shfl_xor(mn, 16, PIKV_WAVE)); mx = fmaxf(mx, __shfl_xor(mx, 16, PIKV_WAVE)); }
   if (lanes >= 64) { mn = fminf(mn, __shfl_xor(mn, 32, PIKV_WAVE)); mx = fmaxf(mx, __shfl_xor(mx, 32, PIKV_WAVE)); }
@@ -318,10 +325,10 @@ __device__ __forceinline__ float read_lane_f(float v, int l) {
 // every lane of the group ends with the result.  Rows of 16 lanes reduce with DPP;
 // a whole wavefront then combines its four rows through scalar registers.
 __device__ __forceinline__ float group_sum_dpp(float v, int lanes) {
-  if (lanes >= 2) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "quad_perm:[1,0,3,2]");
-  if (lanes >= 4) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "quad_perm:[2,3,0,1]");
-  if (lanes >= 8) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "row_half_mirror");
-  if (lanes >= 16) PIKV_DPP_INPLACE("v_add_f32_dpp", v, "row_mirror");
+  if (lanes >= 2) v = dpp_add<kDppXor1>(v);
+  if (lanes >= 4) v = dpp_add<kDppXor2>(v);
+  if (lanes >= 8) v = dpp_add<kDppHalfMirror>(v);
+  if (lanes >= 16) v = dpp_add<kDppMirror>(v);
   if (lanes >= 64)
     v = (read_lane_f(v, 0) + read_lane_f(v, 16)) + (read_lane_f(v, 32) + read_lane_f(v, 48));
   else if (lanes >= 32)
@@ -329,10 +336,10 @@ __device__ __forceinline__ float group_sum_dpp(float v, int lanes) {
   return v;
 }
 __device__ __forceinline__ float group_max_dpp(float v, int lanes) {
-  if (lanes >= 2) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "quad_perm:[1,0,3,2]");
-  if (lanes >= 4) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "quad_perm:[2,3,0,1]");
-  if (lanes >= 8) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "row_half_mirror");
-  if (lanes >= 16) PIKV_DPP_INPLACE("v_max_f32_dpp", v, "row_mirror");
+  if (lanes >= 2) v = dpp_max<kDppXor1>(v);
+  if (lanes >= 4) v = dpp_max<kDppXor2>(v);
+  if (lanes >= 8) v = dpp_max<kDppHalfMirror>(v);
+  if (lanes >= 16) v = dpp_max<kDppMirror>(v);
   if (lanes >= 64)
     v = fmaxf(fmaxf(read_lane_f(v, 0), read_lane_f(v, 16)), fmaxf(read_lane_f(v, 32), read_lane_f(v, 48)));
   else if (lanes >= 32)

@@ -384,10 +384,10 @@ __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float
       x[k] = okk[k] ? stage[srow * kTile + nl + 16 * k] : -__builtin_inff();
       m = fmaxf(m, x[k]);
     }
-    PIKV_DPP_INPLACE("v_max_f32_dpp", m, "quad_perm:[1,0,3,2]");
-    PIKV_DPP_INPLACE("v_max_f32_dpp", m, "quad_perm:[2,3,0,1]");
-    PIKV_DPP_INPLACE("v_max_f32_dpp", m, "row_half_mirror");
-    PIKV_DPP_INPLACE("v_max_f32_dpp", m, "row_mirror");
+    m = dpp_max<kDppXor1>(m);
+    m = dpp_max<kDppXor2>(m);
+    m = dpp_max<kDppHalfMirror>(m);
+    m = dpp_max<kDppMirror>(m);
     float sum = 0.f;
     float* out = a.scores + ((int64_t)c * a.n_q_heads + (hok ? hq : 0)) * a.score_stride + n0 + nl;
 #pragma unroll
@@ -397,10 +397,10 @@ __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float
         out[16 * k] = x[k];
       }
     }
-    PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "quad_perm:[1,0,3,2]");
-    PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "quad_perm:[2,3,0,1]");
-    PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "row_half_mirror");
-    PIKV_DPP_INPLACE("v_add_f32_dpp", sum, "row_mirror");
+    sum = dpp_add<kDppXor1>(sum);
+    sum = dpp_add<kDppXor2>(sum);
+    sum = dpp_add<kDppHalfMirror>(sum);
+    sum = dpp_add<kDppMirror>(sum);
     if (nl == 0 && hok) {
       const int64_t ti = ((int64_t)c * a.n_tiles + tile) * a.n_q_heads + hq;  // heads of a tile side by side
       a.tile_max[ti] = m;
