@@ -287,15 +287,17 @@ int pikv_gather_dequant(const void* codes, const void* scale, const void* zero,
 
 /* For every cache c and query head h (kv head g = h / (n_q_heads/n_kv_heads)):
  *   scores[c,h,n] = dot(q[c,h,:], dequant(K[row_base[c]+n, g, :])) * scale_qk
- *   for n < cache_fill[c]; entries n >= cache_fill[c] are not written.
+ *   for n < min(cache_fill[c], max_len); other entries are not written.  A cache
+ *   that holds more than max_len rows is read as its first max_len rows, here and
+ *   in pikv_h2o_accumulate / pikv_attend_values (same max_len in all three).
  *   q       [n_caches, n_q_heads, head_dim] q_dtype
  *   scores  [n_caches, n_q_heads, score_stride] float
  *   tile_max, tile_sum [n_caches, n_tiles, n_q_heads] float: per tile of
  *   PIKV_SCORE_TILE cached tokens, max score and sum of exp(score - max);
  *   n_tiles = ceil(max_len / PIKV_SCORE_TILE) with max_len <= score_stride
- *   the largest cache_fill the caller wants covered.
- *   D = n_kv_heads*head_dim; head_dim in {64,128}; group divides head_dim or
- *   equals it. */
+ *   the number of rows per cache the caller wants covered.
+ *   D = n_kv_heads*head_dim; head_dim a power of two >= 16 (8-bit) / 32 (4-bit);
+ *   any n_q_heads that is a multiple of n_kv_heads, for either q_dtype. */
 #define PIKV_SCORE_TILE 64
 int pikv_gather_dequant_scores(const void* k_codes, const void* k_scale,
                                const void* k_zero, int scheme, int group,

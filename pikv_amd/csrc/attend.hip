@@ -50,6 +50,7 @@ struct AttendArgs {
   float* row_ts;
   float decay;
   float now;
+  int64_t max_len;  // rows of a cache beyond max_len are not read
   int head_off;  // attend_mfma_i4_kernel: first query head of every kv group handled by this launch
 };
 
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(256) void attend_valu_kernel(AttendArgs a) {
   constexpr int EPL = Q::epl;
   __shared__ float red[256 * EPL];
   const int c = blockIdx.y;
-  const int64_t len = a.fill[c];
+  const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
   const int64_t t0 = (int64_t)blockIdx.x * kAttTokensPerBlock;
   const int64_t t1 = (t0 + kAttTokensPerBlock < len) ? t0 + kAttTokensPerBlock : len;
   const int rep = a.n_q_heads / a.n_kv_heads;
@@ -142,7 +143,7 @@ __global__ __launch_bounds__(256) void attend_valu_kernel(AttendArgs a) {
 __global__ __launch_bounds__(256) void attend_importance_kernel(AttendArgs a) {
   const int c = blockIdx.y;
   const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (n >= a.fill[c]) return;
+  if (n >= a.fill[c] || n >= a.max_len) return;
   const bool normalise = a.head_stats != nullptr;
   float imp = 0.f;
   for (int hq = 0; hq < a.n_q_heads; ++hq) {
@@ -204,7 +205,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   float* lprob = reinterpret_cast<float*>(lzterm + att_meta_bytes(HK) + 4 * (4 * 8 * kAttARow));
 
   const int c = blockIdx.y;
-  const int64_t len = a.fill[c];
+  const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
   const int64_t t0 = (int64_t)blockIdx.x * kAttTokensPerBlock;
   const int64_t t1 = (t0 + kAttTokensPerBlock < len) ? t0 + kAttTokensPerBlock : len;
   if (t0 >= t1) {  // nothing cached in this range: the partial is zero
@@ -531,7 +532,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
                                           4 * (2 * 16 * kAtt8ARow));
 
   const int c = blockIdx.y;
-  const int64_t len = a.fill[c];
+  const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
   const int64_t t0 = (int64_t)blockIdx.x * kAttTokensPerBlock;
   const int64_t t1 = (t0 + kAttTokensPerBlock < len) ? t0 + kAttTokensPerBlock : len;
   if (t0 >= t1) {  // nothing cached in this range: the partial is zero
@@ -855,7 +856,7 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
   }
   AttendArgs a{scores, head_stats, v_codes, v_scale, v_zero, cache_row_base, cache_fill,
                (float*)workspace, score_stride, group, n_kv_heads, n_q_heads, head_dim, n_caches,
-               row_acc, row_ts, decay, now, 0};
+               row_acc, row_ts, decay, now, max_len, 0};
   const int rep = n_q_heads / n_kv_heads;
   if (max_len > 0) {
     const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;

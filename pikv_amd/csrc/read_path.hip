@@ -93,6 +93,9 @@ struct ScoreArgs {
   int n_kv_heads;
   int n_q_heads;
   int head_dim;
+  int max_len;      // rows of a cache beyond max_len are not read (a cache may hold more than the caller covers)
+  int rep;          // scores_kernel: query heads per kv head, and the first head of every kv group that
+  int head_off;     //   this launch serves (it serves REP of them; other ratios take several launches)
   int head_split;   // scores_kernel: blocks along z share a tile, each owns n_kv_heads/head_split heads
 };
 
@@ -104,7 +107,7 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
 
   const int c = blockIdx.y;
   const int64_t tile = blockIdx.x;
-  const int len = a.fill[c];
+  const int len = a.fill[c] < a.max_len ? a.fill[c] : a.max_len;
   const int64_t n0 = tile * kTile;
   if (n0 >= len) return;  // uniform for the block
   // A block owns the kv heads [kv0, kv0 + kv_blk) of its tile: wide rows are split
@@ -130,7 +133,7 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   float qsum[REP];
 #pragma unroll
   for (int r = 0; r < REP; ++r) {
-    const int hq = kvh * REP + r;
+    const int hq = kvh * a.rep + a.head_off + r;
     load_as_float<Q_DT, EPL>(a.q, ((int64_t)c * a.n_q_heads + hq) * a.head_dim + d0, qv[r]);
     float sacc = 0.f;
 #pragma unroll
@@ -186,7 +189,7 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   const int wave = threadIdx.x >> 6;
   const int hq_blk = kv_blk * REP;
   for (int hl = wave; hl < hq_blk; hl += 4) {
-    const int hq = kv0 * REP + hl;
+    const int hq = (kv0 + hl / REP) * a.rep + a.head_off + hl % REP;
     const float s = stage[hl * kTile + lane];
     const bool ok = n0 + lane < len;
     if (ok) a.scores[((int64_t)c * a.n_q_heads + hq) * a.score_stride + n0 + lane] = s;
@@ -238,7 +241,7 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 
   const int c = blockIdx.y;
   const int64_t tile = blockIdx.x;
-  const int len = a.fill[c];
+  const int len = a.fill[c] < a.max_len ? a.fill[c] : a.max_len;
   const int64_t n0 = tile * kTile;
   if (n0 >= len) return;  // uniform for the block
   const int rep = a.n_q_heads / a.n_kv_heads;
@@ -442,7 +445,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   uint16_t* zmeta = smeta + kTile * meta_stride;
 
   const int c = blockIdx.y;
-  const int len = a.fill[c];
+  const int len = a.fill[c] < a.max_len ? a.fill[c] : a.max_len;
   const int64_t tile0 = (int64_t)blockIdx.x * kGqaTilesPerBlock;
   const int64_t tok0 = tile0 * kTile;
   if (tok0 >= len) return;  // uniform for the block
@@ -631,7 +634,7 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   float* stage = i8_lds;  // [q head][token in tile]
 
   const int c = blockIdx.y;
-  const int len = a.fill[c];
+  const int len = a.fill[c] < a.max_len ? a.fill[c] : a.max_len;
   const int64_t tile0 = (int64_t)blockIdx.x * kI8TilesPerBlock;
   if (tile0 * kTile >= len) return;  // uniform for the block
   const int rep = a.n_q_heads / a.n_kv_heads;  // <= 16
@@ -830,13 +833,13 @@ __global__ __launch_bounds__(256) void head_stats_kernel(const float* __restrict
 template <int VEC, bool WRITE_PROBS>
 __global__ __launch_bounds__(256) void h2o_accumulate_kernel(
     float* __restrict__ scores, const float* __restrict__ head_stats, int n_q_heads,
-    const int64_t* __restrict__ row_base, const int32_t* __restrict__ fill, int64_t score_stride,
-    float decay, float now, float* __restrict__ row_acc, float* __restrict__ row_ts,
+    const int64_t* __restrict__ row_base, const int32_t* __restrict__ fill, int64_t max_len,
+    int64_t score_stride, float decay, float now, float* __restrict__ row_acc, float* __restrict__ row_ts,
     float* __restrict__ importance_out) {
   constexpr int UN = 4;
   const int c = blockIdx.y;
   const int64_t n0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
-  const int64_t len = fill[c];
+  const int64_t len = fill[c] < max_len ? (int64_t)fill[c] : max_len;
   if (n0 >= len) return;
   const int cnt = (len - n0 < VEC) ? (int)(len - n0) : VEC;
   const float* hs = head_stats + (int64_t)c * n_q_heads * 2;
@@ -914,7 +917,7 @@ static void launch_gather(unsigned blocks, hipStream_t st, const void* codes, co
 template <int SCHEME, int REP>
 static void launch_scores_q(dim3 grid, hipStream_t st, int q_dtype, const ScoreArgs& a) {
   // staged scores of the block's query heads: the fewer, the more blocks share a compute unit
-  const size_t lds = (size_t)(a.n_q_heads / a.head_split) * kTile * sizeof(float);
+  const size_t lds = (size_t)(a.n_kv_heads / a.head_split) * REP * kTile * sizeof(float);
   if (q_dtype == PIKV_BF16)
     hipLaunchKernelGGL((scores_kernel<SCHEME, REP, PIKV_BF16>), grid, dim3(256), lds, st, a);
   else
@@ -922,13 +925,17 @@ static void launch_scores_q(dim3 grid, hipStream_t st, int q_dtype, const ScoreA
 }
 
 template <int SCHEME>
-static int launch_scores(int rep, dim3 grid, hipStream_t st, int q_dtype, const ScoreArgs& a) {
-  switch (rep) {
-    case 1: launch_scores_q<SCHEME, 1>(grid, st, q_dtype, a); break;
-    case 2: launch_scores_q<SCHEME, 2>(grid, st, q_dtype, a); break;
-    case 4: launch_scores_q<SCHEME, 4>(grid, st, q_dtype, a); break;
-    case 8: launch_scores_q<SCHEME, 8>(grid, st, q_dtype, a); break;
-    default: return PIKV_ERR_UNSUPPORTED;
+static int launch_scores(int rep, dim3 grid, hipStream_t st, int q_dtype, ScoreArgs a) {
+  // The kernel is compiled for 8, 4, 2 and 1 query heads per kv head; any other ratio is served
+  // as the sum of those (7 = 4 + 2 + 1), one launch each over the same codes.
+  a.rep = rep;
+  for (int off = 0; off < rep;) {
+    const int left = rep - off;
+    a.head_off = off;
+    if (left >= 8) { launch_scores_q<SCHEME, 8>(grid, st, q_dtype, a); off += 8; }
+    else if (left >= 4) { launch_scores_q<SCHEME, 4>(grid, st, q_dtype, a); off += 4; }
+    else if (left >= 2) { launch_scores_q<SCHEME, 2>(grid, st, q_dtype, a); off += 2; }
+    else { launch_scores_q<SCHEME, 1>(grid, st, q_dtype, a); off += 1; }
   }
   return PIKV_OK;
 }
@@ -1002,7 +1009,8 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
   if (n_tiles > 0x7fffffffLL) return PIKV_ERR_SHAPE;
   ScoreArgs a{k_codes, k_scale, k_zero, q, cache_row_base, cache_fill, scores, tile_max, tile_sum,
-              score_stride, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim, 1};
+              score_stride, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim,
+              (int)(max_len < 0x7fffffffLL ? max_len : 0x7fffffffLL), n_q_heads / n_kv_heads, 0, 1};
   const dim3 grid((unsigned)n_tiles, (unsigned)n_caches);
   hipStream_t st = (hipStream_t)stream;
   const int rep = n_q_heads / n_kv_heads;
@@ -1075,7 +1083,7 @@ extern "C" int pikv_h2o_accumulate(float* scores, const float* tile_max, const f
   const dim3 grid((unsigned)nb, (unsigned)n_caches);
 #define PIKV_H2O_LAUNCH(V, W)                                                                       \
   hipLaunchKernelGGL((h2o_accumulate_kernel<V, W>), grid, dim3(256), 0, st, scores, head_stats,     \
-                     n_q_heads, cache_row_base, cache_fill, score_stride, decay, now, row_acc,      \
+                     n_q_heads, cache_row_base, cache_fill, max_len, score_stride, decay, now, row_acc, \
                      row_ts, importance_out)
   if (vec4) {
     if (write_probs) PIKV_H2O_LAUNCH(4, true); else PIKV_H2O_LAUNCH(4, false);

@@ -62,8 +62,6 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
 ])
 @pytest.mark.parametrize("qdtype", ["f32", "bf16"])
 def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
-    if qdtype == "f32" and hq // heads not in (1, 2, 4, 8):
-        pytest.skip("float32 queries: 1, 2, 4 or 8 query heads per kv head (others go through the bf16 matrix-core kernels)")
     r = rng(scheme * 7 + heads)
     caps = [300, 64, 130, 10]
     lens = [257, 64, 1, 0]            # ragged: partial tile, full tile, single row, empty
@@ -100,6 +98,74 @@ def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
         assert np.allclose(np_of(scores2)[c, :, :len(rows)], p_ref, rtol=1e-3, atol=1e-7)
     assert np.allclose(np_of(pool.acc), acc_ref, rtol=1e-3, atol=1e-6)
     assert np.array_equal(np_of(pool.ts), ts_ref)
+
+
+@pytest.mark.parametrize("scheme,group,heads,hq,dh,qdtype", [
+    (O.Q_I4_ASYM, 32, 8, 32, 128, "bf16"),    # matrix-core 4-bit kernels
+    (O.Q_I4_ASYM, 32, 8, 64, 128, "bf16"),    # ... two sets of query heads
+    (O.Q_I8_SYM, 128, 8, 32, 128, "bf16"),    # matrix-core 8-bit kernels
+    (O.Q_I8_SYM, 128, 4, 4, 64, "f32"),       # vector forms
+    (O.Q_I4_SYM, 64, 2, 6, 64, "f32"),
+])
+def test_cache_longer_than_max_len(dev, scheme, group, heads, hq, dh, qdtype):
+    """A cache may hold more rows than the caller covers: with max_len = 200 (not a multiple of
+    the 64-token tile) only the first 200 rows of a longer cache are read, nothing is written
+    beyond column 200 of a score row or outside the covered rows' accumulators, and the
+    statistics, importance and attention output are those of the first 200 rows."""
+    import torch
+    from pikv_amd import _native as N
+    r = rng(scheme * 13 + hq)
+    caps = [300, 100, 260]
+    lens = [300, 100, 257]
+    cover = 200
+    pool, ref = _fill_pool(dev, r, caps, lens, heads, dh, group, scheme)
+    nc = len(caps)
+    q = r.standard_normal((nc, hq, dh)).astype(np.float32)
+    if qdtype == "bf16":
+        q = O.bf16_round(q)
+    qd = to_dev(q, dev, qdtype)
+    guard = 1024
+    flat = torch.full((nc * hq * cover + guard,), 777.0, dtype=torch.float32, device=dev)
+    n_tiles = (cover + 63) // 64
+    tmax = torch.empty(nc, n_tiles, hq, dtype=torch.float32, device=dev)
+    tsum = torch.empty_like(tmax)
+    stats = torch.empty(nc, hq, 2, dtype=torch.float32, device=dev)
+    imp = torch.full((nc, cover), -5.0, dtype=torch.float32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    zero = None if pool.k_zero is None else pool.k_zero.data_ptr()
+    N.call("pikv_gather_dequant_scores", pool.k_codes.data_ptr(), pool.k_scale.data_ptr(), zero, scheme, group,
+           heads, hq, dh, qd.data_ptr(), 0 if qdtype == "f32" else 1, float(1.0 / np.sqrt(dh)),
+           pool.row_base.data_ptr(), pool.fill.data_ptr(), nc, cover, cover, flat.data_ptr(),
+           tmax.data_ptr(), tsum.data_ptr(), st)
+    pool.acc.fill_(0.25)
+    pool.ts.fill_(-1.0)
+    N.call("pikv_h2o_accumulate", flat.data_ptr(), tmax.data_ptr(), tsum.data_ptr(), hq, pool.row_base.data_ptr(),
+           pool.fill.data_ptr(), nc, cover, cover, 1.0, 9.0, 0, pool.acc.data_ptr(), pool.ts.data_ptr(),
+           imp.data_ptr(), stats.data_ptr(), st)
+    scores = flat[:nc * hq * cover].view(nc, hq, cover)
+    out = np_of(pool.attend_values(scores, stats))
+    torch.cuda.synchronize()
+    assert bool((flat[nc * hq * cover:] == 777.0).all()), "score rows were written past the covered columns"
+    sc = np_of(scores)
+    acc, ts = np_of(pool.acc), np_of(pool.ts)
+    for c, L in enumerate(lens):
+        n = min(L, cover)
+        rows = ref.valid_rows(c)[:n]
+        k_hat = O.dequantize_groups(ref.k_codes[rows], ref.k_scale[rows], ref.k_zero[rows], group)
+        v_hat = O.dequantize_groups(ref.v_codes[rows], ref.v_scale[rows], ref.v_zero[rows], group)
+        s_ref = O.attention_scores(q[c], k_hat, heads, 1.0 / np.sqrt(dh))
+        rms = np.sqrt((s_ref.astype(np.float64) ** 2).mean())
+        assert np.abs(sc[c, :, :n] - s_ref).max() <= 1e-3 * rms
+        if n < cover:
+            assert (sc[c, :, n:] == 777.0).all()
+        p_ref, i_ref = O.h2o_importance(s_ref)
+        assert np.allclose(np_of(imp)[c, :n], i_ref, rtol=1e-3, atol=1e-6)
+        assert np.allclose(acc[rows], 0.25 + i_ref, rtol=1e-3, atol=1e-6)
+        assert (ts[rows] == 9.0).all()
+        rest = ref.valid_rows(c)[n:]                      # rows of the cache that were not covered
+        assert (acc[rest] == 0.25).all() and (ts[rest] == -1.0).all()
+        want = O.attend_values(p_ref, v_hat, heads)
+        assert np.abs(out[c] - want).max() <= 2e-3 * np.sqrt((want.astype(np.float64) ** 2).mean())
 
 
 def _set_state(pool, ref, r, ties):
