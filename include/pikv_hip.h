@@ -266,6 +266,19 @@ int pikv_quantize_rows(const void* src, int src_dtype, int64_t n_rows, int D,
                        int group, int scheme, int64_t dst_row0,
                        void* codes, void* scale, void* zero, void* stream);
 
+/* Min-shift 8-bit quantisation of whole rows, the algebra of the kernel facade.
+ * Replaces: PiKVKernels.compress_kv, CompressionMode.QUANT8
+ *   (core/single/pikv_kernels.py:215-246):
+ *     mn = min(row); s = (max(row) - mn) / 255
+ *     codes = clamp(round((x - mn) / s), 0, 255); dq = codes * s + mn
+ *   float32 arithmetic in that order (bf16 sources are widened first).  A constant
+ *   row has s = 0, codes 0 and dq = mn.
+ *   src [n_rows, D] src_dtype; codes uint8 [n_rows, D]; dq float [n_rows, D] or NULL;
+ *   scale, row_min float [n_rows] (the reference's k_scale / k_min as [N,1]). */
+int pikv_quant8_minshift(const void* src, int src_dtype, int64_t n_rows, int D,
+                         uint8_t* codes, float* dq, float* scale, float* row_min,
+                         void* stream);
+
 /* ------------------------------------------------------------------------
  * K3  gather + dequantise read path, attention scores, H2O accumulation
  * Replaces: dq = (q - zero_point) * scale

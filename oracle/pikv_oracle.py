@@ -23,8 +23,13 @@ Pinning status (what, besides this file, fixes each function's output):
   select / compact ................... brute force on tiny inputs, invariants
   streaming / quest / flexgen / lru+ . hand-computed known answers, brute-force
                                        ranking on tiny inputs
-  adakv / duo / attend_values ........ hand-computed known answers, float64
+  adakv / duo / attend_values ........ hand-computed known answers (attend_values: a
+                                       2-kv-head, 4-query-head, 3-token case), float64
                                        closed forms
+  quant8_minshift / pyramid_keep_counts / dense_dispatch_combine
+                                       hand-computed known answers (tie rounding, a shifted
+                                       and a constant row; interior budgets from the integer
+                                       formula; a literal 2-token dispatch)
   fakequant_colblocks / _preset ...... hand-computed known answers; the preset form
                                        given a block's own parameters must repeat
                                        the block form bit for bit

@@ -44,6 +44,7 @@ SIGNATURES = {
     "pikv_quant_gather": (_i, [_p, _p, _i, _i, _i, _i, _p, _p, _p, _l, _p, _p, _p, _p, _i,
                                _p, _p, _p, _p, _p, _p, _p, _p, _f, _p]),
     "pikv_quantize_rows": (_i, [_p, _i, _l, _i, _i, _i, _l, _p, _p, _p, _p]),
+    "pikv_quant8_minshift": (_i, [_p, _i, _l, _i, _p, _p, _p, _p, _p]),
     "pikv_gather_dequant": (_i, [_p, _p, _p, _i, _i, _i, _p, _l, _l, _p, _i, _p]),
     "pikv_gather_dequant_scores": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _f,
                                         _p, _p, _i, _l, _l, _p, _p, _p, _p]),

@@ -6,10 +6,10 @@ order and return tuples, dispatching into libpikv_hip.so.
       the fallback there is torch.topk on the raw logits; ties go to the lower
       index here (torch's tie order is unspecified).
   compress_kv(keys, values, mode, lora_params) -> (k', v', meta)       :101-287
-      QUANT8: per-row 8-bit codes.  The facade's own algebra
-      (q = round((x-min)/s), dq = q*s+min, :215-232) is kept for the returned
-      float tensors' meaning; the codes come from the library's asymmetric 8-bit
-      formula (zero point rounded to an integer), see meta['k_codes'].
+      QUANT8: the facade's own algebra (s = (max-min)/255, q = round((x-min)/s)
+      clamped to 0..255, dq = q*s+min, :215-232) in pikv_quant8_minshift; meta holds
+      k_scale, k_min, v_scale, v_min as [N,1] like the reference, plus the uint8
+      codes (k_codes, v_codes), which the reference computes and throws away.
       NONE returns the inputs; LORA and MASK are dense/elementwise torch and not
       part of the native path.
   evict_cache(keys, values, timestamps, usage, now, policy, window, thr)
@@ -65,16 +65,12 @@ class PiKVKernels:
             return keys, values, {"compression_type": "none"}
         if mode != CompressionMode.QUANT8:
             raise NotImplementedError(f"{mode.name}: only NONE and QUANT8 run on the native path")
-        n, hidden = keys.shape
-        group = hidden
-        if group & (group - 1) or not (16 <= group <= 1024):
-            raise ValueError("QUANT8 needs a power-of-two row width in [16,1024]")
-        kc, ks, kz = ops.quantize_rows(keys.contiguous(), group, ops.Q_I8_ASYM)
-        vc, vs, vz = ops.quantize_rows(values.contiguous(), group, ops.Q_I8_ASYM)
-        ck = ops.dequantize_rows(kc, ks, kz, group, ops.Q_I8_ASYM)
-        cv = ops.dequantize_rows(vc, vs, vz, group, ops.Q_I8_ASYM)
-        meta = {"compression_type": "quant8", "k_scale": ks, "k_min": -kz * ks, "v_scale": vs,
-                "v_min": -vz * vs, "k_codes": kc, "v_codes": vc, "k_zero": kz, "v_zero": vz}
+        if keys.dim() != 2 or values.shape != keys.shape:
+            raise ValueError("keys and values must be [batch, hidden] of one shape")
+        ck, kc, ks, kmin = ops.quant8_minshift(keys)
+        cv, vc, vs, vmin = ops.quant8_minshift(values)
+        meta = {"compression_type": "quant8", "k_scale": ks, "k_min": kmin, "v_scale": vs, "v_min": vmin,
+                "k_codes": kc, "v_codes": vc}
         return ck.to(keys.dtype), cv.to(values.dtype), meta
 
     # ---- eviction ------------------------------------------------------------------

@@ -26,7 +26,7 @@ from ._native import (BF16, EVICT_H2O, EVICT_LRU, F32, Q_I4_ASYM, Q_I4_SYM,
                       Q_I8_ASYM, Q_I8_SYM, SCORE_TILE)
 
 __all__ = [
-    "router_fused", "router_tail", "capacity_slots", "quantize_rows",
+    "router_fused", "router_tail", "capacity_slots", "quantize_rows", "quant8_minshift",
     "dequantize_rows", "fakequant_colblocks", "fakequant_preset", "CachePool", "scheme_bits",
     "Q_I8_SYM", "Q_I8_ASYM", "Q_I4_ASYM", "Q_I4_SYM", "EVICT_H2O", "EVICT_LRU",
 ]
@@ -267,6 +267,25 @@ def quantize_rows(x, group: int, scheme: int):
     N.call("pikv_quantize_rows", _ptr(x), dt, n, D, group, scheme, 0, _ptr(codes), _ptr(scale),
            _ptr(zero), _stream())
     return codes, scale, zero
+
+
+def quant8_minshift(x, want_dq: bool = True):
+    """Min-shift 8-bit quantisation of whole rows (core/single/pikv_kernels.py:215-232).
+    x [n, D] float32 or bfloat16.  Returns (dq float32 [n,D] or None, codes uint8 [n,D],
+    scale [n,1], row_min [n,1])."""
+    x = _need(x, "x", ndim=2)
+    dt = _dt(x, "x")
+    n, D = x.shape
+    if D < 1:
+        raise ValueError("rows must not be empty")
+    dev = x.device
+    codes = torch.empty(n, D, dtype=torch.uint8, device=dev)
+    dq = torch.empty(n, D, dtype=torch.float32, device=dev) if want_dq else None
+    scale = torch.empty(n, 1, dtype=torch.float32, device=dev)
+    mn = torch.empty(n, 1, dtype=torch.float32, device=dev)
+    if n:
+        N.call("pikv_quant8_minshift", _ptr(x), dt, n, D, _ptr(codes), _ptr(dq), _ptr(scale), _ptr(mn), _stream())
+    return dq, codes, scale, mn
 
 
 def dequantize_rows(codes, scale, zero, group: int, scheme: int, out_dtype=torch.float32,

@@ -325,11 +325,13 @@ def test_kernels_facade(dev):
     vals = r.standard_normal((32, 512)).astype(np.float32)
     ck, cv, meta = K.compress_kv(torch.from_numpy(keys).to(dev), torch.from_numpy(vals).to(dev),
                                  CompressionMode.QUANT8)
-    q_ref, s_ref, z_ref = O.quantize_groups(keys, 512, O.Q_I8_ASYM)
     assert meta["compression_type"] == "quant8"
-    assert np.array_equal(np_of(meta["k_codes"]).astype(np.int16), q_ref)
-    assert np.array_equal(np_of(ck), O.dequantize_groups(q_ref, s_ref, z_ref, 512))
-    assert np.abs(np_of(ck) - keys).max() <= s_ref.max() * 0.51
+    for got, codes, sc, mn, src in ((ck, "k_codes", "k_scale", "k_min", keys), (cv, "v_codes", "v_scale", "v_min", vals)):
+        q_ref, dq_ref, s_ref, mn_ref = O.quant8_minshift(src)      # the facade's own algebra, :215-232
+        assert meta[sc].shape == (32, 1) and meta[mn].shape == (32, 1)
+        assert np.array_equal(np_of(meta[codes]), q_ref)
+        assert np.array_equal(np_of(meta[sc]), s_ref) and np.array_equal(np_of(meta[mn]), mn_ref)
+        assert np.array_equal(np_of(got), dq_ref)
     # eviction: sliding window, stable compaction
     n = 2048
     keys = r.standard_normal((n, 512)).astype(np.float32)
@@ -382,3 +384,30 @@ def test_cache_pool_checkpoint_round_trip(dev, trim, tmp_path):
     other = ops.CachePool(caps, 2, 64, 64, ops.Q_I4_ASYM, dev)
     with pytest.raises(ValueError):
         other.load_state_dict(sd)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("n,D", [(1, 16), (37, 512), (5, 100), (3, 7), (64, 4096), (9, 8200)])
+def test_quant8_minshift_matches_facade_algebra(dev, dtype, n, D):
+    """pikv_quant8_minshift against core/single/pikv_kernels.py:215-232: codes, scale, row
+    minimum and dequantised floats bit for bit, for row widths on and off the 16-element
+    vector path, rows with rounding ties, a constant row (scale 0 -> codes 0, dq = min),
+    a two-valued row and a row with a huge outlier."""
+    from pikv_amd import ops
+    r = rng(n * 31 + D)
+    x = r.standard_normal((n, D)).astype(np.float32)
+    x[0] = np.round(x[0] * 4) / 4                       # many exact .5 ties after the shift
+    if n > 2:
+        x[1] = 3.0                                      # constant row
+        x[2] = np.where(np.arange(D) % 2 == 0, -1.5, 2.0)
+    if n > 4:
+        x[4, D // 2] = 1e30
+    if dtype == "bf16":
+        x = O.bf16_round(x)
+    dq, codes, s, mn = ops.quant8_minshift(to_dev(x, dev, dtype))
+    q_ref, dq_ref, s_ref, mn_ref = O.quant8_minshift(x)
+    assert np.array_equal(np_of(codes), q_ref)
+    assert np.array_equal(np_of(s), s_ref) and np.array_equal(np_of(mn), mn_ref)
+    assert np.array_equal(np_of(dq), dq_ref)
+    _, codes2, _, _ = ops.quant8_minshift(to_dev(x, dev, dtype), want_dq=False)
+    assert np.array_equal(np_of(codes2), q_ref)

@@ -417,3 +417,68 @@ def test_fakequant_preset_known_answers():
     ref, st, mse_ref = O.fakequant_colblocks(y, 96)
     dq, mse = O.fakequant_preset(y, st[0, 2], st[0, 3], 96)
     assert np.array_equal(dq, ref) and np.allclose(mse, mse_ref, rtol=0, atol=0)
+
+
+# ---------------------------------------------------------------- hand-computed pins of the facade / caller helpers
+def test_quant8_minshift_known_answers():
+    """core/single/pikv_kernels.py:215-232 by hand.  Row 0: min 0, max 255, s = 1, so the
+    code is the value rounded half to even.  Row 1 is row 0 shifted by +10: same codes,
+    dq = code + 10 (a dropped '- min' or '+ min' fails here).  Row 2: min 1, max 128.5,
+    s = 0.5; (1.75-1)/0.5 = 1.5 -> 2, (2.25-1)/0.5 = 2.5 -> 2, dq = 2*0.5 + 1 = 2.  Row 3 is
+    constant: s = 0, 0/0 = NaN -> code 0, dq = min."""
+    x = np.array([[0.0, 255.0, 127.4, 127.5, 128.5, 3.0],
+                  [10.0, 265.0, 137.4, 137.5, 138.5, 13.0],
+                  [1.0, 128.5, 1.75, 2.25, 64.75, 1.0],
+                  [3.0, 3.0, 3.0, 3.0, 3.0, 3.0]], np.float32)
+    q, dq, s, mn = O.quant8_minshift(x)
+    assert q.dtype == np.uint8 and s.shape == (4, 1) and mn.shape == (4, 1)
+    assert s[:, 0].tolist() == [1.0, 1.0, 0.5, 0.0] and mn[:, 0].tolist() == [0.0, 10.0, 1.0, 3.0]
+    assert q[0].tolist() == [0, 255, 127, 128, 128, 3]
+    assert q[1].tolist() == [0, 255, 127, 128, 128, 3]
+    assert q[2].tolist() == [0, 255, 2, 2, 128, 0]          # (64.75-1)/0.5 = 127.5 -> 128
+    assert q[3].tolist() == [0] * 6
+    assert dq[0].tolist() == [0.0, 255.0, 127.0, 128.0, 128.0, 3.0]
+    assert dq[1].tolist() == [10.0, 265.0, 137.0, 138.0, 138.0, 13.0]
+    assert dq[2].tolist() == [1.0, 128.5, 2.0, 2.0, 65.0, 1.0]
+    assert dq[3].tolist() == [3.0] * 6
+
+
+def test_attend_values_known_answer():
+    """matmul(attention_probs, v) (core/single/pikv_attention.py:188) with grouped heads:
+    4 query heads over 2 kv heads (heads 0,1 read kv head 0; heads 2,3 read kv head 1),
+    3 cached tokens, head_dim 2.  V[n] = [kv0: (n+1, 10(n+1)) | kv1: (-(n+1), 100(n+1))]."""
+    v = np.array([[1, 10, -1, 100],
+                  [2, 20, -2, 200],
+                  [3, 30, -3, 300]], np.float32)
+    p = np.array([[1.0, 0.0, 0.0],          # picks token 0 of kv head 0
+                  [0.5, 0.25, 0.25],        # 0.5*1 + 0.25*2 + 0.25*3 = 1.75
+                  [0.0, 0.0, 1.0],          # token 2 of kv head 1
+                  [0.25, 0.5, 0.25]], np.float32)   # -(0.25 + 1 + 0.75) = -2
+    out = O.attend_values(p, v, 2)
+    assert out.tolist() == [[1.0, 10.0], [1.75, 17.5], [-3.0, 300.0], [-2.0, 200.0]]
+    # one kv head per query head (no grouping): head h reads columns [2h, 2h+2)
+    out = O.attend_values(p[:2], v, 2)
+    assert out.tolist() == [[1.0, 10.0], [-1.75, 175.0]]
+
+
+def test_pyramid_keep_counts_interior_values():
+    """keep_l = int(N * (1 - 0.75 * l / 31)) = floor(32768 * (124 - 3 l) / 31) for N = 131072,
+    evaluated in integers: l = 1 -> 3964928 // 31, l = 16 -> 2490368 // 31, l = 30 -> 1114112 // 31."""
+    kc = O.pyramid_keep_counts(131072, 32)
+    assert (kc[1], kc[16], kc[30]) == (127900, 80334, 35939)
+    assert kc == [(32768 * (124 - 3 * l)) // 31 for l in range(32)]
+    assert O.pyramid_keep_counts(100, 1) == [100]
+    assert O.pyramid_keep_counts(1000, 5, 0.5) == [1000, 875, 750, 625, 500]
+
+
+def test_dense_dispatch_combine_known_answer():
+    """core/single/module/pikv_routing.py:77-104 on two tokens, 3 experts, capacity 1:
+    token 0 -> experts (2, 0) in slots (0, 0); token 1 -> expert 2 is full (slot -1, dropped),
+    expert 1 slot 0."""
+    idx = np.array([[2, 0], [2, 1]], np.int32)
+    w = np.array([[0.75, 0.25], [0.5, 0.125]], np.float32)
+    slot, count = O.capacity_slots(idx, 3, 1)
+    assert slot.tolist() == [[0, 0], [-1, 0]] and count.tolist() == [1, 1, 2]
+    disp, comb = O.dense_dispatch_combine(idx, w, slot, 3, 1)
+    assert disp[:, :, 0].tolist() == [[1.0, 0.0, 1.0], [0.0, 1.0, 0.0]]
+    assert comb[:, :, 0].tolist() == [[0.25, 0.0, 0.75], [0.0, 0.125, 0.0]]
