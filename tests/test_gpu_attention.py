@@ -106,3 +106,181 @@ def test_past_key_values_round_trip_and_overflow(dev):
         assert att2.cache_ptr.tolist() == [12]
         att2(torch.randn(1, 12, 128, device=dev))
         assert att2.cache_ptr.tolist() == [12]       # 12 + 12 > 16: wiped, then the new rows
+
+
+def _dense_reference(att, x, past_k_rows, past_v_rows, key_mask=None, own_quant=None):
+    """float64 attention of the module's projections over [past rows ; own rows], causal
+    inside the call.  past_*_rows: [B, L, kv_heads, dh] float64 (already dequantised)."""
+    import torch
+    B, S, _ = x.shape
+    heads, kvh, dh = att.num_heads, att.num_kv_heads, att.head_dim
+    rep = heads // kvh
+    with torch.no_grad():
+        q = _f64(att.q_proj(x)).reshape(B, S, heads, dh)
+        k = _f64(att.k_proj(x)).reshape(B, S, kvh, dh)
+        v = _f64(att.v_proj(x)).reshape(B, S, kvh, dh)
+    if own_quant is not None:                     # the native read path sees its own row quantised too
+        group, scheme = own_quant
+        k, v = [O.dequantize_groups(*O.quantize_groups(t.astype(np.float32).reshape(B * S, kvh * dh), group, scheme),
+                                    group).astype(np.float64).reshape(B, S, kvh, dh) for t in (k, v)]
+    L = past_k_rows.shape[1]
+    out = np.zeros((B, S, heads * dh))
+    for b in range(B):
+        kk = np.concatenate([past_k_rows[b], k[b]])
+        vv = np.concatenate([past_v_rows[b], v[b]])
+        for h in range(heads):
+            s = q[b, :, h] @ kk[:, h // rep].T / math.sqrt(dh)             # [S, L+S]
+            for i in range(S):
+                s[i, L + i + 1:] = -np.inf
+            if key_mask is not None:
+                s[:, ~key_mask[b]] = -np.inf
+            p = np.exp(s - s.max(axis=1, keepdims=True))
+            p /= p.sum(axis=1, keepdims=True)
+            out[b, :, h * dh:(h + 1) * dh] = p @ vv[:, h // rep]
+    return out @ _f64(att.o_proj.weight).T + _f64(att.o_proj.bias)
+
+
+@pytest.mark.parametrize("layout", ["hf", "reference"])
+def test_forward_attends_over_past_and_current(dev, layout):
+    """core/single/pikv_attention.py:240-254: past and current K/V are concatenated along the
+    sequence and attended over together - for multi-token calls and calls with a mask too."""
+    import torch
+    from pikv_amd.attention import PiKVAttention
+    torch.manual_seed(11)
+    H, heads, kvh, dh, B, L, S = 128, 4, 2, 32, 2, 23, 5
+    att = PiKVAttention(H, heads, head_dim=dh, dropout=0.0, cache_size=64, num_kv_heads=kvh, kv_quant="int8",
+                        kv_group=32).to(dev).eval()
+    with torch.no_grad():
+        for m in (att.q_proj, att.k_proj, att.v_proj):
+            m.weight.normal_(0.0, 0.3)
+    pk = torch.randn(B, L, kvh, dh, device=dev)           # reference layout
+    pv = torch.randn(B, L, kvh, dh, device=dev)
+    past = (pk, pv) if layout == "reference" else (pk.transpose(1, 2).contiguous(), pv.transpose(1, 2).contiguous())
+    dq = []
+    for t in (pk, pv):
+        rows = np_of(t).reshape(B * L, kvh * dh)
+        q, s, z = O.quantize_groups(rows, 32, O.Q_I8_SYM)
+        dq.append(O.dequantize_groups(q, s, z, 32).astype(np.float64).reshape(B, L, kvh, dh))
+    x = torch.randn(B, S, H, device=dev)
+    with torch.no_grad():
+        out, _ = att(x, past_key_values=past)
+    want = _dense_reference(att, x, dq[0], dq[1])
+    assert np.abs(_f64(out) - want).max() <= 1e-4 * np.sqrt((want ** 2).mean()) + 1e-6
+    assert att.cache_ptr.tolist() == [L + S] * B
+    # the same with a key mask over past + current (one hidden past row, one hidden own row)
+    mask = torch.ones(B, L + S, device=dev)
+    mask[0, 3] = 0
+    mask[1, L + 1] = 0
+    with torch.no_grad():
+        out_m, _ = att(x, attention_mask=mask, past_key_values=past)
+    want_m = _dense_reference(att, x, dq[0], dq[1], key_mask=np_of(mask) != 0)
+    assert np.abs(_f64(out_m) - want_m).max() <= 1e-4 * np.sqrt((want_m ** 2).mean()) + 1e-6
+    assert np.abs(want_m - want).max() > 1e-3              # the mask mattered
+    # a masked single-token call also sees the past (through the dequantised rows)
+    x1 = torch.randn(B, 1, H, device=dev)
+    m1 = torch.ones(B, L + 1, device=dev)
+    with torch.no_grad():
+        out_1, _ = att(x1, attention_mask=m1, past_key_values=past)
+        out_n, _ = att(x1, past_key_values=past)           # native read path, same context
+    want_1 = _dense_reference(att, x1, dq[0], dq[1])
+    assert np.abs(_f64(out_1) - want_1).max() <= 1e-4 * np.sqrt((want_1 ** 2).mean()) + 1e-6
+    want_n = _dense_reference(att, x1, dq[0], dq[1], own_quant=(32, O.Q_I8_SYM))
+    assert np.abs(_f64(out_n) - want_n).max() <= 1e-3 * np.sqrt((want_n ** 2).mean())
+
+
+def test_past_key_values_shape_is_checked(dev):
+    import torch
+    from pikv_amd.attention import PiKVAttention
+    att = PiKVAttention(128, 4, head_dim=32, dropout=0.0, cache_size=64, num_kv_heads=2, kv_quant="int8",
+                        kv_group=32).to(dev).eval()
+    good = torch.randn(2, 2, 10, 32, device=dev)
+    with pytest.raises(ValueError):
+        att.load_past_key_values((torch.randn(2, 4, 10, 32, device=dev),) * 2)       # 4 query heads, not 2 kv heads
+    with pytest.raises(ValueError):
+        att.load_past_key_values((torch.randn(2, 2, 10, 16, device=dev),) * 2)       # wrong head_dim
+    with pytest.raises(ValueError):
+        att.load_past_key_values((good, good[:, :, :5]))                             # k and v differ
+    with pytest.raises(ValueError):
+        att.load_past_key_values((good, good), layout="reference")                   # [B,S,heads,dh] expected
+    with pytest.raises(ValueError):
+        att.load_past_key_values((torch.randn(2, 2, 65, 32, device=dev),) * 2)       # longer than the cache
+    with pytest.raises(ValueError):
+        att.load_past_key_values(good)                                               # not a pair
+    att.load_past_key_values((good, good))
+    assert att.cache_ptr.tolist() == [10, 10]
+    with pytest.raises(ValueError):
+        att(torch.randn(3, 2, 128, device=dev))                                      # 3 sequences, 2 caches in use
+    with pytest.raises(ValueError):
+        att(torch.randn(2, 2, 128, device=dev), attention_mask=torch.ones(2, 7, device=dev))
+    # S == kv_heads: the shape cannot tell the layouts apart, past_layout decides
+    sq = torch.randn(1, 2, 2, 32, device=dev)
+    att.load_past_key_values((sq, sq))
+    k_hf, _ = att.past_key_values()
+    att.load_past_key_values((sq, sq), layout="reference")
+    k_ref, _ = att.past_key_values()
+    assert torch.equal(k_hf.transpose(1, 2), k_ref)
+
+
+def test_hf_dynamic_cache_drives_the_adapter(dev):
+    """A randomly initialised GPT-2 (nothing is fetched) prefills 16 tokens; the per-layer K/V of
+    the cache object the installed transformers returns go into PiKVAttention, one native
+    decode step runs over them, and the result is compared with float64 attention over the
+    dequantised cache.  The legacy tuple-of-tuples form that
+    downstream_tasks/llm/next_tok_pred/s_transformers.py:85-98 loops over is accepted too."""
+    import torch
+    transformers = pytest.importorskip("transformers")
+    from transformers import GPT2Config, GPT2LMHeadModel
+    from pikv_amd.attention import PiKVAttention
+    torch.manual_seed(5)
+    cfg = GPT2Config(n_layer=2, n_head=4, n_embd=256, vocab_size=512, bos_token_id=0, eos_token_id=0)
+    model = GPT2LMHeadModel(cfg).to(dev).eval()
+    B, L = 2, 16
+    ids = torch.randint(0, 512, (B, L), device=dev)
+    with torch.no_grad():
+        pkv = model(ids, use_cache=True).past_key_values
+    if hasattr(pkv, "layers"):
+        per_layer = [(l.keys, l.values) for l in pkv.layers]
+    else:
+        per_layer = [(kv[0], kv[1]) for kv in pkv]
+    assert per_layer[0][0].shape == (B, 4, L, 64)
+    for layer_idx in range(2):
+        att = PiKVAttention(256, 4, head_dim=64, dropout=0.0, cache_size=64, kv_quant="int8", kv_group=64,
+                            layer_idx=layer_idx).to(dev).eval()
+        with torch.no_grad():
+            for m in (att.q_proj, att.k_proj, att.v_proj):
+                m.weight.normal_(0.0, 0.2)
+        hk, hv = per_layer[layer_idx]
+        dq = []
+        for t in (hk, hv):
+            rows = np_of(t.transpose(1, 2)).reshape(B * L, 256)
+            q, s, z = O.quantize_groups(rows, 64, O.Q_I8_SYM)
+            dq.append(O.dequantize_groups(q, s, z, 64).reshape(B, L, 4, 64))
+        x = torch.randn(B, 1, 256, device=dev)
+        with torch.no_grad():
+            out_obj, _ = att(x, past_key_values=pkv)                     # the cache object itself
+            k_back, v_back = att.past_key_values()
+            out_tup, _ = att(x, past_key_values=tuple(per_layer))        # legacy per-layer tuples
+        assert torch.equal(out_obj, out_tup)
+        # round trip: the cache returns the dequantised rows in the Hugging Face layout
+        assert k_back.shape == (B, 4, L + 1, 64)
+        assert np.array_equal(np_of(k_back[:, :, :L]), dq[0].transpose(0, 2, 1, 3))
+        assert np.array_equal(np_of(v_back[:, :, :L]), dq[1].transpose(0, 2, 1, 3))
+        # the decode step: float64 attention over [dequantised past ; dequantised own row]
+        with torch.no_grad():
+            own = [np_of(p(x)).reshape(B, 256) for p in (att.k_proj, att.v_proj)]
+        full = []
+        for past, rows in zip(dq, own):
+            q, s, z = O.quantize_groups(rows, 64, O.Q_I8_SYM)
+            own_dq = O.dequantize_groups(q, s, z, 64).reshape(B, 1, 4, 64)
+            full.append(np.concatenate([past, own_dq], axis=1).astype(np.float64))
+        with torch.no_grad():
+            qv = _f64(att.q_proj(x)).reshape(B, 4, 64)
+        ctx = np.zeros((B, 256))
+        for b in range(B):
+            for h in range(4):
+                s = full[0][b, :, h] @ qv[b, h] / 8.0
+                p = np.exp(s - s.max())
+                p /= p.sum()
+                ctx[b, h * 64:(h + 1) * 64] = p @ full[1][b, :, h]
+        want = ctx @ _f64(att.o_proj.weight).T + _f64(att.o_proj.bias)
+        assert np.abs(_f64(out_obj[:, 0]) - want).max() <= 1e-3 * np.sqrt((want ** 2).mean())
