@@ -19,6 +19,13 @@ vectorised loop of core/single/pikv_routing.py:107-128 gives every token of a
 round the same slot; it is not reproduced).  Ties in the top-k go to the lower
 expert index.
 
+Gradients: the integer decisions (expert indices, slots, counts) have none.  The float
+outputs (router_probs, top-k weights, logits, and the losses built on them) carry the
+native kernel's VALUES and, whenever autograd is recording and a gate parameter or the
+input requires grad, the GRADIENT of the same formula evaluated in torch on the selected
+experts (value + (torch - torch.detach())), so the gate MLPs train as in the reference.
+Under torch.no_grad() nothing is recomputed.
+
 Every forward also accepts return_compact=True and then returns the RouterOut
 (topk_idx, topk_w, slot, count, probs) instead of the dense tensors, which at
 production shapes cannot exist ([T, E, capacity] floats).
@@ -94,6 +101,44 @@ def _dense_basic(r: ops.RouterOut, batch_size, seq_len, num_experts):
     return disp.view(batch_size, seq_len, num_experts, 1), comb.view(batch_size, seq_len, num_experts, 1)
 
 
+def _wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+def _attach_grad(r: ops.RouterOut, logits: torch.Tensor, *, temperature=1.0, expert_scale=None,
+                 expert_mask=None, module_arithmetic=False, renorm_eps=0.0) -> ops.RouterOut:
+    """Give the float outputs of the native router the gradient of the reference's formula
+    (core/single/pikv_routing.py:65-82, :653-660) evaluated in torch on raw gate `logits`
+    [T,E] that are part of the autograd graph.  Values stay the kernel's."""
+    lg = logits.float()
+    if expert_scale is not None:
+        expert_scale = torch.as_tensor(expert_scale, dtype=lg.dtype, device=lg.device)
+    if expert_mask is not None:
+        expert_mask = torch.as_tensor(expert_mask, dtype=lg.dtype, device=lg.device)
+    if module_arithmetic:
+        if expert_scale is not None:
+            lg = lg * expert_scale
+        if temperature != 1.0:
+            lg = lg / temperature
+        penalty = torch.finfo(torch.float32).min
+    else:
+        if temperature != 1.0:
+            lg = lg / temperature
+        if expert_scale is not None:
+            lg = lg * expert_scale
+        penalty = -1e9
+    if expert_mask is not None:
+        lg = lg + (1.0 - expert_mask) * penalty
+    probs = F.softmax(lg, dim=-1)
+    w = probs.gather(-1, r.topk_idx.long())
+    w = w / (w.sum(dim=-1, keepdim=True) + renorm_eps)
+    r.probs = r.probs + (probs - probs.detach())
+    r.topk_w = r.topk_w + (w - w.detach())
+    if r.logits is not None:
+        r.logits = r.logits + (lg - lg.detach())
+    return r
+
+
 def _gate_tail(hidden: torch.Tensor, linear: nn.Linear, **kw) -> ops.RouterOut:
     """hidden [T,H'] (activation before the last Linear) -> fused router."""
     x = hidden.contiguous()
@@ -139,11 +184,15 @@ class BaseRouter(nn.Module):
     def _route(self, hidden_states, expert_mask=None, *, seq=None, **scale_kw) -> ops.RouterOut:
         B, S, H = hidden_states.shape
         seq = self.router if seq is None else seq
+        x2d = hidden_states.reshape(B * S, H)
         with torch.no_grad():
-            h = self._hidden_before_gate(seq, hidden_states.reshape(B * S, H))
+            h = self._hidden_before_gate(seq, x2d)
         cap = self._compute_capacity(B, S)
-        return _gate_tail(h, seq[-1], top_k=self.top_k, capacity=cap, expert_mask=expert_mask,
-                          **self._arith_kw(), **scale_kw)
+        r = _gate_tail(h, seq[-1], top_k=self.top_k, capacity=cap, expert_mask=expert_mask,
+                       **self._arith_kw(), **scale_kw)
+        if _wants_grad(hidden_states, *seq.parameters()):
+            r = _attach_grad(r, seq(x2d), expert_mask=expert_mask, **self._arith_kw(), **scale_kw)
+        return r
 
     def _aux_loss(self, router_probs: torch.Tensor) -> torch.Tensor:
         p = router_probs.mean(dim=[0, 1])
@@ -220,13 +269,19 @@ class EPLBRouter(BaseRouter):
         B_S = B * S
         # /temperature, then *expert_weights, then mask: the order of :653-660
         seq = self.router
+        x2d = hidden_states.reshape(B_S, -1)
         with torch.no_grad():
-            h = self._hidden_before_gate(seq, hidden_states.reshape(B_S, -1))
+            h = self._hidden_before_gate(seq, x2d)
         cap = self._compute_capacity(B, S)
         r = ops.router_fused(h.contiguous(), seq[-1].weight.detach().to(h.dtype).contiguous(),
                              seq[-1].bias.detach().float(), top_k=self.top_k, capacity=cap,
                              expert_scale=self.expert_weights, expert_mask=expert_mask,
                              temperature=self.temperature, return_logits=True, **self._arith_kw())
+        if _wants_grad(hidden_states, *seq.parameters()):
+            # (dropout layers: the torch pass draws its own mask; in training the values are the
+            # kernel's for the eval-mode activations only when dropout is inactive)
+            r = _attach_grad(r, seq(x2d), temperature=self.temperature, expert_scale=self.expert_weights,
+                             expert_mask=expert_mask, **self._arith_kw())
         out, probs = self._finish(r, B, S, return_compact)
         aux = torch.zeros((), device=probs.device)
         usage = r.count.float()
@@ -265,8 +320,16 @@ class AdaptiveRouter(BaseRouter):
             lb = self.router_unimportant(x2).float().contiguous()
         sel = (importance.reshape(-1) > self.imp_threshold)
         cap = self._compute_capacity(B, S)
-        return ops.router_tail(la, top_k=self.top_k, capacity=cap, logits_b=lb, select=sel,
-                               expert_scale=expert_scale, expert_mask=expert_mask, **self._arith_kw())
+        scale_v = None if expert_scale is None else expert_scale.detach()
+        r = ops.router_tail(la, top_k=self.top_k, capacity=cap, logits_b=lb, select=sel,
+                            expert_scale=scale_v, expert_mask=expert_mask, **self._arith_kw())
+        if _wants_grad(hidden_states, expert_scale, *self.router_important.parameters(),
+                       *self.router_unimportant.parameters()):
+            # the per-token choice between the two gates (core/single/pikv_routing.py:450-458)
+            lg = torch.where(sel.unsqueeze(1), self.router_important(x2).float(),
+                             self.router_unimportant(x2).float())
+            r = _attach_grad(r, lg, expert_scale=expert_scale, expert_mask=expert_mask, **self._arith_kw())
+        return r
 
 
 class PiKVRouter(AdaptiveRouter):
@@ -293,7 +356,7 @@ class PiKVRouter(AdaptiveRouter):
         if kv_states is not None:
             importance = (importance + self.kv_importance_model(kv_states)) / 2
         r = self._two_gate_route(hidden_states, importance.detach(), expert_mask,
-                                 expert_scale=self.cache_correction_factor.detach())
+                                 expert_scale=self.cache_correction_factor)
         out, probs = self._finish(r, B, S, return_compact)
         usage = probs.sum(dim=[0, 1])
         usage_norm = usage / usage.sum()
@@ -344,7 +407,8 @@ class HierarchicalRouter(BaseRouter):
         probs = self.router_probs(hidden_states, expert_mask)
         flat = probs.detach().reshape(B * S, self.num_experts).float().contiguous()
         r = ops.router_tail(flat, top_k=self.top_k, capacity=self._compute_capacity(B, S), use_softmax=False)
-        r.topk_w = r.topk_w / r.topk_w.sum(dim=-1, keepdim=True)
+        w = probs.reshape(B * S, self.num_experts).float().gather(-1, r.topk_idx.long())   # differentiable
+        r.topk_w = w / w.sum(dim=-1, keepdim=True)
         r.probs = flat
         p = probs.mean(dim=[0, 1])
         aux = torch.sum(p * torch.log(p * self.num_experts + 1e-9))

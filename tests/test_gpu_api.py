@@ -411,3 +411,67 @@ def test_quant8_minshift_matches_facade_algebra(dev, dtype, n, D):
     assert np.array_equal(np_of(dq), dq_ref)
     _, codes2, _, _ = ops.quant8_minshift(to_dev(x, dev, dtype), want_dq=False)
     assert np.array_equal(np_of(codes2), q_ref)
+
+
+def test_router_outputs_carry_gradients(dev):
+    """The gate MLPs must be trainable as in the reference (ordinary nn.Module outputs,
+    core/single/pikv_routing.py:44-161): values come from the native kernel, gradients from
+    the same formula in torch.  Checked against a pure-torch evaluation of the formula on the
+    experts the kernel selected."""
+    import torch
+    import torch.nn.functional as F
+    from pikv_amd.routing import EPLBRouter, HierarchicalRouter, PiKVRouter, TopKBalancedRouter
+    torch.manual_seed(2)
+    B, S, H, E, k = 2, 24, 64, 8, 2
+    x = torch.randn(B, S, H, device=dev, requires_grad=True)
+    router = TopKBalancedRouter(H, E, top_k=k).to(dev)
+    r, probs, aux = router(x, return_compact=True)
+    assert probs.requires_grad and r.topk_w.requires_grad and aux.requires_grad
+    loss = (r.topk_w * torch.arange(1, k + 1, device=dev)).sum() + 3.0 * aux + (probs ** 2).sum()
+    loss.backward()
+    got = {n: p.grad.clone() for n, p in router.named_parameters()}
+    got_x = x.grad.clone()
+    # the same loss in torch only, on the kernel's indices
+    router.zero_grad()
+    x2 = x.detach().clone().requires_grad_(True)
+    lg = router.router(x2.reshape(B * S, H))
+    p_t = F.softmax(lg, dim=-1)
+    w_t = p_t.gather(-1, r.topk_idx.long())
+    w_t = w_t / w_t.sum(-1, keepdim=True)
+    pm = p_t.view(B, S, E).mean(dim=[0, 1])
+    aux_t = torch.sum(pm * torch.log(pm * E + 1e-9))
+    p3 = p_t.view(B, S, E)
+    aux_t = aux_t + router._balance(p3)
+    loss_t = (w_t * torch.arange(1, k + 1, device=dev)).sum() + 3.0 * aux_t + (p_t ** 2).sum()
+    loss_t.backward()
+    for n, p in router.named_parameters():
+        assert p.grad is not None and torch.allclose(got[n], p.grad, rtol=1e-4, atol=1e-6), n
+    assert torch.allclose(got_x, x2.grad, rtol=1e-4, atol=1e-6)
+    # values are still the kernel's: identical to a no-grad call
+    with torch.no_grad():
+        r0, probs0, aux0 = router(x.detach(), return_compact=True)
+    assert torch.equal(r0.topk_idx, r.topk_idx) and torch.equal(r0.slot, r.slot)
+    assert torch.allclose(probs0, probs.detach(), rtol=0, atol=1e-7)
+    assert not probs0.requires_grad
+    # every router class: the auxiliary loss reaches the gate parameters
+    for make in (lambda: EPLBRouter(H, E, top_k=k), lambda: PiKVRouter(H, E, top_k=k),
+                 lambda: HierarchicalRouter(H, E, top_k=k, num_groups=2)):
+        rt = make().to(dev).eval()
+        res = rt(x.detach(), return_compact=True)
+        rr, aux = res[0], res[2]
+        (aux + rr.topk_w.sum() * 0.5 + (rr.topk_w ** 2).sum()).backward()
+        grads = [p.grad for p in rt.parameters() if p.grad is not None]
+        assert grads and any(float(g.abs().sum()) > 0 for g in grads), type(rt).__name__
+
+
+def test_moe_load_balance_loss_backpropagates(dev):
+    import torch
+    from pikv_amd.moe import PiKVMoE
+    torch.manual_seed(0)
+    model = PiKVMoE().to(dev)
+    from pikv_amd.config import config
+    x = torch.randn(2, 16, config['hidden_size'], device=dev)
+    logits, lb = model(x, return_loss=True)
+    (logits.float().pow(2).mean() + lb).backward()
+    g = [p.grad for p in model.router.parameters()]
+    assert all(t is not None for t in g) and any(float(t.abs().sum()) > 0 for t in g)
