@@ -76,8 +76,11 @@ def test_pikvmoe_small_config(dev, small_config, policy):
         clear = (order[:, k - 1] - order[:, k]) > 1e-5
         _, idx_ref, _, _ = O.router_tail(lg64.astype(np.float32), k)
         idx = np_of(r.topk_idx)
-        assert clear.mean() > 0.9
+        assert clear.mean() > 0.98
         assert np.array_equal(idx[clear], idx_ref[clear])
+        # rows inside the band: every chosen expert still ranks within 1e-5 of the k-th logit
+        chosen = np.take_along_axis(lg64, idx.astype(np.int64), axis=1)
+        assert (chosen.min(axis=1) >= order[:, k - 1] - 1e-5).all()
         slot_ref, count_ref = O.capacity_slots(idx, E, r.capacity)
         assert np.array_equal(np_of(r.slot), slot_ref)
         assert np.array_equal(np_of(r.count), count_ref)
