@@ -115,6 +115,32 @@ def _entry(ms, nbytes, **extra):
     return d
 
 
+def hbm_ceiling(torch, dev, iters, nbytes=2 << 30):
+    """Practical HBM rates of this machine with the library's own access pattern (16 bytes per
+    lane, 1 KiB per wavefront, 8 accesses in flight per lane): read only, write only, copy;
+    plain and non-temporal stores.  Median of `iters` launches over `nbytes` (2 GiB: eight times
+    the last-level cache), HIP events on the launch stream."""
+    from pikv_amd import _native as N
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+    def run(mode, nt):
+        st = torch.cuda.current_stream().cuda_stream
+        return lambda: N.call("pikv_stream_probe", mode, src.data_ptr(), dst.data_ptr(), nbytes, nt,
+                              sink.data_ptr(), st)
+    gb = nbytes / 1e9
+    ms = {name: _median_ms(torch, run(mode, nt), iters)
+          for name, mode, nt in (("read", 0, 0), ("write", 1, 0), ("write_nt", 1, 1), ("copy", 2, 0), ("copy_nt", 2, 1))}
+    del src, dst
+    torch.cuda.empty_cache()
+    return {"buffer_bytes": nbytes, "pattern": "16 B per lane, 1 KiB per wavefront, 8 in flight per lane",
+            "read_GBps": gb / (ms["read"] * 1e-3), "write_GBps": gb / (ms["write"] * 1e-3),
+            "write_nontemporal_GBps": gb / (ms["write_nt"] * 1e-3),
+            "copy_GBps": 2 * gb / (ms["copy"] * 1e-3), "copy_nontemporal_GBps": 2 * gb / (ms["copy_nt"] * 1e-3),
+            "ms": ms, "note": "copy rates count bytes read + bytes written"}
+
+
 def decode_read_workload(torch, ops, dev, iters):
     """Decode read path: 64 sequences x 32768 cached tokens, 8 KV heads (GQA from 32
     q heads) x 128, int4 asymmetric, group 32, fp16 scale/zero; H2O keeps 2048 heavy
@@ -310,7 +336,7 @@ def main():
     ap.add_argument("--only-headline", action="store_true",
                     help="skip the per-kernel figures of the decode, wide-routing and pyramid workloads")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="run only a plain 1 GiB device copy (a kernel of known traffic, to scale "
+                    help="run only the streaming probes over 1 GiB (kernels of known traffic, to scale "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -325,14 +351,22 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     if args.calibrate_copy:
+        # five launches each of the read, write and copy probes over 1 GiB: kernels of exactly
+        # known traffic for scaling FETCH_SIZE / WRITE_SIZE, and the ceilings as a JSON line
+        from pikv_amd import _native as N
         n = 1 << 30
         src = torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
-        for _ in range(5):
-            dst.copy_(src)
+        st = torch.cuda.current_stream().cuda_stream
+        for mode in (0, 1, 2):
+            for _ in range(5):
+                N.call("pikv_stream_probe", mode, src.data_ptr(), dst.data_ptr(), n, 0, None, st)
         torch.cuda.synchronize()
-        print(json.dumps({"calibrate_copy_bytes_read": n, "calibrate_copy_bytes_written": n,
-                          "kernel": "torch elementwise copy (5 launches)"}))
+        del src, dst
+        print(json.dumps({"calibrate_bytes_per_launch": n,
+                          "kernels": {"stream_probe_kernel<0,false>": "reads n", "stream_probe_kernel<1,false>": "writes n",
+                                      "stream_probe_kernel<2,false>": "reads n and writes n"},
+                          "hbm_ceiling": hbm_ceiling(torch, dev, 10)}))
         return
     w = WORKLOAD
     T, E, k = w["batch"] * w["seq"], w["experts"], w["top_k"]
@@ -408,6 +442,7 @@ def main():
             "h2o_accumulate": {"ms": t_h2o, "GBps": gbps(b_h2o, t_h2o)},
         },
     }
+    out["hbm_ceiling"] = hbm_ceiling(torch, dev, 10)
     if not args.only_headline:
         it = max(5, min(args.steps, 20))
         out["other_workloads"] = {}

@@ -1,0 +1,70 @@
+// Streaming probes with the access pattern every kernel of this library uses for its bulk
+// data: 16 bytes per lane, 1 KiB contiguous per wavefront, several accesses in flight per
+// lane.  They put the practical HBM rates of the machine at hand (read only, write only,
+// read + write) on record next to the kernels' own figures, and give profiler counters a
+// launch of exactly known traffic to be scaled by.  Not part of the data path.
+#include "common.hpp"
+
+namespace pikv {
+
+constexpr int kProbeUnroll = 8;                              // 16-byte accesses in flight per lane
+constexpr int64_t kProbeBlockBytes = 256 * 16 * kProbeUnroll;  // 32 KiB per block
+
+// mode 0: read src, keep a running xor; the (never true) comparison keeps the loads alive
+// mode 1: write a constant pattern to dst
+// mode 2: copy src to dst
+template <int MODE, bool STREAM_STORE>
+__global__ __launch_bounds__(256) void stream_probe_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                           int64_t n16, uint32_t* __restrict__ sink) {
+  const int64_t base = (int64_t)blockIdx.x * (256 * kProbeUnroll) + threadIdx.x;
+  uint4 v[kProbeUnroll];
+#pragma unroll
+  for (int u = 0; u < kProbeUnroll; ++u) {
+    const int64_t i = base + (int64_t)u * 256;
+    if constexpr (MODE != 1) v[u] = i < n16 ? src[i] : make_uint4(0, 0, 0, 0);
+    else v[u] = make_uint4(0x01020304u, (uint32_t)i, 0x0badc0deu, (uint32_t)u);
+  }
+  if constexpr (MODE == 0) {
+    uint32_t acc = 0;
+#pragma unroll
+    for (int u = 0; u < kProbeUnroll; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    if (acc == 0x9e3779b9u && sink) sink[0] = acc;  // practically never: the data would have to conspire
+  } else {
+#pragma unroll
+    for (int u = 0; u < kProbeUnroll; ++u) {
+      const int64_t i = base + (int64_t)u * 256;
+      if (i < n16) {
+        if constexpr (STREAM_STORE) st16_stream(dst + i, v[u]);
+        else dst[i] = v[u];
+      }
+    }
+  }
+}
+
+}  // namespace pikv
+
+using namespace pikv;
+
+extern "C" int pikv_stream_probe(int mode, const void* src, void* dst, int64_t bytes, int streaming_stores,
+                                 void* sink, void* stream) {
+  if (mode < 0 || mode > 2) return PIKV_ERR_UNSUPPORTED;
+  if ((mode != 1 && !src) || (mode != 0 && !dst)) return PIKV_ERR_NULL;
+  if (bytes < 0 || bytes % 16 != 0) return PIKV_ERR_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(src) & 15) || (reinterpret_cast<uintptr_t>(dst) & 15)) return PIKV_ERR_SHAPE;
+  if (bytes == 0) return PIKV_OK;
+  const int64_t blocks = (bytes + kProbeBlockBytes - 1) / kProbeBlockBytes;
+  if (blocks > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+  const int64_t n16 = bytes / 16;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)blocks);
+  const uint4* s = reinterpret_cast<const uint4*>(src);
+  uint4* d = reinterpret_cast<uint4*>(dst);
+  uint32_t* sk = reinterpret_cast<uint32_t*>(sink);
+  if (mode == 0) hipLaunchKernelGGL((stream_probe_kernel<0, false>), grid, dim3(256), 0, st, s, d, n16, sk);
+  else if (mode == 1 && streaming_stores) hipLaunchKernelGGL((stream_probe_kernel<1, true>), grid, dim3(256), 0, st, s, d, n16, sk);
+  else if (mode == 1) hipLaunchKernelGGL((stream_probe_kernel<1, false>), grid, dim3(256), 0, st, s, d, n16, sk);
+  else if (streaming_stores) hipLaunchKernelGGL((stream_probe_kernel<2, true>), grid, dim3(256), 0, st, s, d, n16, sk);
+  else hipLaunchKernelGGL((stream_probe_kernel<2, false>), grid, dim3(256), 0, st, s, d, n16, sk);
+  PIKV_CHECK_LAUNCH();
+  return PIKV_OK;
+}
