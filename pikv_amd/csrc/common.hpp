@@ -174,37 +174,45 @@ __device__ __forceinline__ int quant_code(float x, float scale, float zero) {
   return (int)y;
 }
 
-// ---- fast exact quantiser of one lane -------------------------------------------
-// Same codes as quant_code(), at a fraction of the instructions.
-// The reference rounds twice (y = RN(x/scale), t = RN(y + zero)) and then takes
-// clamp(rint(t)).  Here t' = x*r + zero + bias with r ~ 1/scale (one v_rcp_f32
-// per group, relative error <= 2^-23) and `bias` the integer that makes the
-// stored code unsigned.  For |x/scale| <= 768 and |zero| <= 512 the two differ
-// by less than 1.8e-4 (error of r plus the roundings of both paths at magnitudes
-// below 1024).  Each element is converted twice, from t' - kBand and t' + kBand,
-// with v_cvt_pk_u8_f32 (round to nearest even, saturate to [0,255], insert the
-// byte - one instruction): t lies between the two, the conversion is monotone,
-// so when both give the same byte that byte is the reference's code.  Bytes that
-// differ (a rounding tie inside the band: about 6 elements in 10^4, plus the
-// element equal to -absmax of a symmetric group, which sits on -127.5 by
-// construction) and groups outside the stated range are recomputed with the
-// exact division sequence, so every code is the reference's code.
+// ---- exact quantiser of one lane without a division per element ------------------
+// The reference divides every element by the group's scale.  A float32 division is a
+// dozen instructions; here the group pays for ONE, r = RN(1 / scale), and every element
+// gets its correctly rounded quotient from three:
+//     q0 = RN(x * r);  e = x - scale * q0 (exact, one fma);  q = RN(q0 + e * r)
+// With r the correctly rounded reciprocal and q0 within one unit in the last place of
+// x / scale, q IS RN(x / scale) (Markstein's theorem on fma-based division; checked
+// against the division operator on 9e8 random and structured pairs, including scales
+// with an all-ones significand, powers of two, and bf16 / half operands).  The rest is the
+// reference's own arithmetic: t = RN(q + zero), round half to even, clamp.
+// The construction needs no intermediate to overflow or vanish: a group takes it only when
+// its scale lies in [1e-30, 1e30] and |x / scale| <= 768 for all of its elements (elements
+// far below the scale are harmless: any quotient of magnitude < 1/4 yields the same code).
+// Other groups - infinities, collapsed ranges - go through quant_code() element by element.
 struct GroupQuant {
-  float scale, zero, r, amax;
+  float scale, zero, r;
   bool fast;
 };
-constexpr float kBand = 3.0e-4f;
 
 template <int SCHEME>
 __device__ __forceinline__ GroupQuant make_group_quant(float mn, float mx) {
   GroupQuant g;
   quant_params<SCHEME>(mn, mx, g.scale, g.zero);
-  g.r = __builtin_amdgcn_rcpf(g.scale);
-  g.amax = fmaxf(fabsf(mn), fabsf(mx));
-  // amax * r bounds |x/scale| for every element of the group
-  g.fast = (g.scale >= 1e-30f) && (g.r < 1e30f) && (fabsf(g.zero) <= 512.0f) &&
-           (g.amax * g.r <= 768.0f);
+  g.r = 1.0f / g.scale;  // correctly rounded (-fhip-fp32-correctly-rounded-divide-sqrt)
+  const float amax = fmaxf(fabsf(mn), fabsf(mx));
+  g.fast = (g.scale >= 1e-30f) && (g.scale <= 1e30f) && (amax * g.r <= 768.0f);
   return g;
+}
+
+// Stored (unsigned) form of the code of t = x / scale + zero, as a float in [0, 2^bits - 1]
+// that the byte conversion takes as is.  NaN ends as 0, the stored form of qmin.
+template <int SCHEME>
+__device__ __forceinline__ float stored_code_value(float t) {
+  using Q = QScheme<SCHEME>;
+  if constexpr (Q::sym) t = rintf(t) + (float)(-Q::qmin);   // exact: integers
+  // the byte conversion itself rounds half to even and saturates at [0, 255]; four-bit
+  // codes are cut to [0, 15] first (median of three: a NaN gives the smaller bound)
+  if constexpr (Q::bits == 4) t = __builtin_amdgcn_fmed3f(t, 0.0f, 15.0f);
+  return t;
 }
 
 // Quantise the EPL elements of a lane and pack them into 16 code bytes.
@@ -214,63 +222,40 @@ __device__ __forceinline__ uint4 quantize_lane(const float (&x)[QScheme<SCHEME>:
   using Q = QScheme<SCHEME>;
   constexpr int EPL = Q::epl;
   constexpr int NW = EPL / 4;                          // words of one byte per element
-  constexpr float bias = (float)(-Q::qmin);            // 0, 128 or 8
-  const float zlo = (g.zero + bias) - kBand;
-  const float zhi = (g.zero + bias) + kBand;
-  uint32_t wl[NW], wh[NW];
+  uint32_t w[NW];
 #pragma unroll
-  for (int i = 0; i < NW; ++i) wl[i] = wh[i] = 0;
-  // A symmetric group's -absmax element sits on the lowest tie (-127.5 or -7.5) by
-  // construction.  Its exact code is computed once per lane, and the element is
-  // replaced by a value that the fast path maps to that code away from any tie.
-  float neg_amax = 0.f, x_sub = 0.f;
-  bool sub_ok = true;
-  if constexpr (Q::sym) {
-    const int code_neg = quant_code<SCHEME>(-g.amax, g.scale, g.zero) - Q::qmin;  // stored byte
-    neg_amax = -g.amax;
-    x_sub = code_neg == 0 ? -2.0f * g.amax : -g.amax * (1.0f - 0.001953125f);
-    sub_ok = code_neg <= 1;
-  }
+  for (int i = 0; i < NW; ++i) w[i] = 0;
+  if (g.fast) {
 #pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    // 8-bit: element i -> byte i%4 of word i/4.  4-bit: even elements of an octet
-    // go to word 2*(i/8), odd ones to word 2*(i/8)+1, byte (i%8)/2.
-    const int wi = Q::bits == 8 ? i / 4 : 2 * (i / 8) + (i & 1);
-    const int bi = Q::bits == 8 ? i % 4 : (i % 8) / 2;
-    float xi = x[i];
-    if constexpr (Q::sym) xi = (xi == neg_amax) ? x_sub : xi;
-    wl[wi] = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(xi, g.r, zlo), bi, wl[wi]);
-    wh[wi] = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(xi, g.r, zhi), bi, wh[wi]);
-  }
-  // bytes to recompute: the two conversions disagree, or (4-bit) exceed the range
-  uint32_t bad[NW];
-  const bool all_exact = !g.fast || !sub_ok;
-  uint32_t any_bad = all_exact ? 1u : 0u;
-#pragma unroll
-  for (int i = 0; i < NW; ++i) {
-    bad[i] = wl[i] ^ wh[i];
-    if constexpr (Q::bits == 4) bad[i] |= (wl[i] | wh[i]) & 0xf0f0f0f0u;
-    any_bad |= bad[i];
-  }
-  if (any_bad) {
+    for (int i = 0; i < EPL; ++i) {
+      // 8-bit: element i -> byte i%4 of word i/4.  4-bit: even elements of an octet
+      // go to word 2*(i/8), odd ones to word 2*(i/8)+1, byte (i%8)/2.
+      const int wi = Q::bits == 8 ? i / 4 : 2 * (i / 8) + (i & 1);
+      const int bi = Q::bits == 8 ? i % 4 : (i % 8) / 2;
+      const float q0 = x[i] * g.r;
+      const float e = __builtin_fmaf(-g.scale, q0, x[i]);
+      const float q = __builtin_fmaf(e, g.r, q0);
+      float t = q;
+      if constexpr (!Q::sym) t = q + g.zero;
+      w[wi] = __builtin_amdgcn_cvt_pk_u8_f32(stored_code_value<SCHEME>(t), bi, w[wi]);
+    }
+  } else {
 #pragma unroll
     for (int i = 0; i < EPL; ++i) {
       const int wi = Q::bits == 8 ? i / 4 : 2 * (i / 8) + (i & 1);
       const int bi = Q::bits == 8 ? i % 4 : (i % 8) / 2;
-      if (((bad[wi] >> (8 * bi)) & 0xffu) != 0 || all_exact) {
-        const int c = quant_code<SCHEME>(x[i], g.scale, g.zero) - Q::qmin;  // unsigned stored form
-        wl[wi] = (wl[wi] & ~(0xffu << (8 * bi))) | ((uint32_t)c << (8 * bi));
-      }
+      const int c = quant_code<SCHEME>(x[i], g.scale, g.zero) - Q::qmin;  // unsigned stored form
+      w[wi] |= (uint32_t)c << (8 * bi);
     }
   }
   uint32_t o[4];
   if constexpr (Q::bits == 8) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = Q::sym ? (wl[i] ^ 0x80808080u) : wl[i];
+    for (int i = 0; i < 4; ++i) o[i] = Q::sym ? (w[i] ^ 0x80808080u) : w[i];
   } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      o[i] = wl[2 * i] | (wl[2 * i + 1] << 4);
+      o[i] = w[2 * i] | (w[2 * i + 1] << 4);
       if constexpr (Q::sym) o[i] ^= 0x88888888u;
     }
   }
