@@ -177,10 +177,9 @@ def decode_read_workload(torch, ops, dev, iters):
         pool.fill.fill_(N - 1)
         pool.quant_scatter(new_k, new_v, seq_id, zero_slot, 1, now=2.0)
         pool.advance(one)
-        s_, m_, z_ = pool.scores(q, hq)
-        pool.h2o_accumulate(s_, m_, z_, now=2.0, stats_only=True)
-        return pool.attend_values(s_, pool.head_stats, accumulate=True, now=2.0)
+        return pool.decode_attend(q, hq, now=2.0)     # scores + softmax + attention output + H2O accumulate
     t_step = _median_ms(torch, decode_step, iters)
+    t_fused = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=2.0), iters)
     t_att_acc = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats, accumulate=True, now=1.0), iters)
     pool.fill.fill_(N)
 
@@ -214,8 +213,9 @@ def decode_read_workload(torch, ops, dev, iters):
         "h2o_accumulate": _entry(t_h2o, rows * hq * 4 + rows * 12),
         "attend_values": _entry(t_att, k_bytes + rows * hq * 4),
         "attend_values_with_h2o": _entry(t_att_acc, k_bytes + rows * hq * 4 + rows * 12),
-        "decode_step": {"ms": t_step, "what": "append 1 token per sequence + scores + head statistics + attention "
-                                              "output with the H2O accumulate in the same pass",
+        "decode_attend": _entry(t_fused, 2 * k_bytes + 2 * rows * hq * 4 + rows * 12,
+                                what="pikv_decode_attend: scores + softmax + attention output + H2O accumulate in one call"),
+        "decode_step": {"ms": t_step, "what": "append 1 token per sequence + pikv_decode_attend",
                         "cached_tokens_per_s": rows / (t_step * 1e-3),
                         "algorithmic_bytes": 2 * k_bytes + 2 * rows * hq * 4 + rows * 12,
                         "GBps": (2 * k_bytes + 2 * rows * hq * 4 + rows * 12) / (t_step * 1e-3) / 1e9},

@@ -373,6 +373,37 @@ int pikv_attend_values(const float* scores, const float* head_stats,
 int64_t pikv_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim,
                                     int64_t max_len);
 
+/* The whole decode read in one call: scores of one query per cache against the
+ * compressed K rows, softmax over each cache's tokens, attention output over the
+ * compressed V rows, and the H2O bookkeeping of the same probabilities:
+ *   s[c,h,n]  = dot(q[c,h,:], dequant(K[c,n,h/rep,:])) * scale_qk        n < min(cache_fill[c], max_len)
+ *   p[c,h,:]  = softmax_n(s[c,h,:])
+ *   out[c,h,:] = sum_n p[c,h,n] * dequant(V[c,n,h/rep,:])
+ *   acc[row] = acc[row]*decay + sum_h p[c,h,n];  ts[row] = now          (row_acc / row_ts may be NULL)
+ * Replaces: matmul(q, k^T)/sqrt(head_dim), softmax(dim=-1), matmul(probs, v)
+ *   (core/single/pikv_attention.py:123,163,188) on dequantised copies of the cache, and
+ *   H2OScheduler.update_attention_scores (core/single/cache_scheduling.py:69-73).
+ * Same results as pikv_gather_dequant_scores + pikv_h2o_accumulate + pikv_attend_values
+ * (to the float tolerance of those), but the score matrix never leaves the library: for
+ * 4-bit caches with group 32, head_dim 128, bf16 queries and up to 8 query heads per kv
+ * head (1, 2, 4 or 8 kv heads) the two matrix-core kernels exchange exp(score - tile max)
+ * with a tile's heads side by side, so that both sides stream contiguous 8 KB runs instead
+ * of the 256-byte pieces of a [head][token] score matrix; every other format runs the three
+ * steps with float scores in the workspace.
+ *   q [n_caches, n_q_heads, head_dim] q_dtype; out [n_caches, n_q_heads, head_dim] float;
+ *   planes and shape limits as for the three entry points above;
+ *   workspace: pikv_decode_attend_workspace_bytes(...) bytes, 256-byte aligned. */
+int pikv_decode_attend(const void* k_codes, const void* k_scale, const void* k_zero,
+                       const void* v_codes, const void* v_scale, const void* v_zero,
+                       int scheme, int group, int n_kv_heads, int n_q_heads, int head_dim,
+                       const void* q, int q_dtype, float scale_qk,
+                       const int64_t* cache_row_base, const int32_t* cache_fill,
+                       int n_caches, int64_t max_len, float decay, float now,
+                       float* row_acc, float* row_ts, float* out,
+                       void* workspace, int64_t workspace_bytes, void* stream);
+int64_t pikv_decode_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim,
+                                           int64_t max_len);
+
 /* ------------------------------------------------------------------------
  * K4  eviction top-k + stable in-place compaction
  * Replaces: H2OScheduler.select_eviction_candidates

@@ -53,6 +53,9 @@ SIGNATURES = {
     "pikv_attend_values": (_i, [_p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _i, _l,
                                 _f, _f, _p, _p, _p, _p, _l, _p]),
     "pikv_attend_workspace_bytes": (_l, [_i, _i, _i, _l]),
+    "pikv_decode_attend": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _f, _p, _p, _i, _l,
+                                _f, _f, _p, _p, _p, _p, _l, _p]),
+    "pikv_decode_attend_workspace_bytes": (_l, [_i, _i, _i, _l]),
     "pikv_evict_select": (_i, [_i, _p, _p, _p, _p, _p, _p, _i, _l, _p, _p, _p, _p, _l, _p]),
     "pikv_evict_workspace_bytes": (_l, [_i, _l]),
     "pikv_h2o_budget": (_i, [_p, _i, _d, _d, _p, _p, _p]),

@@ -27,6 +27,9 @@ FLAGS = [
     "-fhip-fp32-correctly-rounded-divide-sqrt",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
+    # the SLP vectoriser turns the per-word nibble expansions into short vector AND / OR
+    # pairs, which then no longer match the three-operand and-or instruction
+    "-fno-slp-vectorize",
 ]
 
 

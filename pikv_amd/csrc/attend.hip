@@ -51,6 +51,11 @@ struct AttendArgs {
   float decay;
   float now;
   int64_t max_len;  // rows of a cache beyond max_len are not read
+  // exchange format of pikv_decode_attend (attend_mfma_i4_kernel only): when escores is set, `scores` is
+  // not read; escores [cache][tile][q head][64] floats hold exp(score - tile max), tile_max [cache][tile][q head]
+  const float* escores;
+  const float* tile_max;
+  int64_t n_tiles;
   int head_off;  // attend_mfma_i4_kernel: first query head of every kv group handled by this launch
 };
 
@@ -252,6 +257,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   }
   const bool s_vec = (a.score_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(a.scores) & 15) == 0;
   const float s_off = normalise ? -INFINITY : 0.f;  // what a token past the end contributes: p = 0
+  // exchange format: eight values exp(score - tile max) per thread and tile, and the tile's max of the head;
+  // the rows of a tile lie side by side, [tile][q head][64], so a block reads one contiguous run
+  const bool exch = a.escores != nullptr;
+  const float* const ep = exch ? a.escores + ((int64_t)c * a.n_tiles * a.n_q_heads + s_hq) * kAttTile + st8 : nullptr;
+  const float* const tmp = exch ? a.tile_max + (int64_t)c * a.n_tiles * a.n_q_heads + s_hq : nullptr;
+  float ptm = 0.f;
 
   // registers that carry the next tile from HBM to LDS
   uint4 pc[NCH];
@@ -273,7 +284,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int rem = left < kAttTile ? (int)left : kAttTile;  // tokens of this tile
     const int64_t urow = base_row + n0;
     if (a.row_acc && igrp == 0 && it < rem) pacc = (a.row_acc + urow)[it];
-    if (s_on) {
+    if (exch) {
+      if (s_on) {
+        const int64_t tile = n0 / kAttTile;
+        const float4 lo4 = *reinterpret_cast<const float4*>(ep + tile * a.n_q_heads * kAttTile);
+        const float4 hi4 = *reinterpret_cast<const float4*>(ep + tile * a.n_q_heads * kAttTile + 4);
+        psc[0] = lo4.x, psc[1] = lo4.y, psc[2] = lo4.z, psc[3] = lo4.w;
+        psc[4] = hi4.x, psc[5] = hi4.y, psc[6] = hi4.z, psc[7] = hi4.w;
+        ptm = tmp[tile * a.n_q_heads];
+      }
+    } else if (s_on) {
       const float* spn = sp + n0;
       if (s_vec && st8 + 8 <= rem) {
         const float4 lo4 = *reinterpret_cast<const float4*>(spn);
@@ -307,11 +327,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   auto stage = [&]() {
     {
       // tokens {l, l+4, l+8, l+12} of a 16-token group go side by side: one float4 per reader
+      if (exch) {
+        // p = exp(s - tile max) * exp(tile max - head max) / head sum: one exponential per thread and tile
+        const float coef = s_on ? __builtin_amdgcn_exp2f((ptm - smx) * 1.4426950408889634f) * srz : 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) psc[k] = s_on ? psc[k] * coef : 0.f;
+      }
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
         const int t = st8 + k;
         lprob[sh * kAttPRow + (t & ~15) + (t & 3) * 4 + ((t >> 2) & 3)] =
-            s_on ? prob_of(psc[k], smx, srz, normalise) : 0.f;
+            exch ? psc[k] : (s_on ? prob_of(psc[k], smx, srz, normalise) : 0.f);
       }
     }
 #pragma unroll
@@ -856,7 +882,7 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
   }
   AttendArgs a{scores, head_stats, v_codes, v_scale, v_zero, cache_row_base, cache_fill,
                (float*)workspace, score_stride, group, n_kv_heads, n_q_heads, head_dim, n_caches,
-               row_acc, row_ts, decay, now, max_len, 0};
+               row_acc, row_ts, decay, now, max_len, nullptr, nullptr, 0, 0};
   const int rep = n_q_heads / n_kv_heads;
   if (max_len > 0) {
     const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;
@@ -907,4 +933,100 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
                      (const float*)workspace, cache_fill, n_caches, n_q_heads, head_dim, (int)splits, out);
   PIKV_CHECK_LAUNCH();
   return PIKV_OK;
+}
+
+// ---- one call for the decode read: scores, softmax, attention output, H2O bookkeeping ----
+static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+
+struct DecodeWs {
+  int64_t n_tiles, stride, scores, tmax, tsum, stats, partial, total;
+};
+static DecodeWs decode_ws(int n_caches, int n_q_heads, int head_dim, int64_t max_len) {
+  DecodeWs w;
+  w.n_tiles = (max_len + PIKV_SCORE_TILE - 1) / PIKV_SCORE_TILE;
+  w.stride = w.n_tiles * PIKV_SCORE_TILE;
+  w.scores = 0;  // float scores [cache][head][stride], or the exchange rows [cache][tile][head][64] (same size)
+  w.tmax = align256((int64_t)n_caches * n_q_heads * w.stride * 4);
+  w.tsum = w.tmax + align256((int64_t)n_caches * w.n_tiles * n_q_heads * 4);
+  w.stats = w.tsum + align256((int64_t)n_caches * w.n_tiles * n_q_heads * 4);
+  w.partial = w.stats + align256((int64_t)n_caches * n_q_heads * 2 * 4);
+  w.total = w.partial + align256(pikv_attend_workspace_bytes(n_caches, n_q_heads, head_dim, max_len));
+  return w;
+}
+
+extern "C" int64_t pikv_decode_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim, int64_t max_len) {
+  if (n_caches < 1 || n_q_heads < 1 || head_dim < 1 || max_len < 0) return 0;
+  return decode_ws(n_caches, n_q_heads, head_dim, max_len).total;
+}
+
+extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, const void* k_zero,
+                                  const void* v_codes, const void* v_scale, const void* v_zero,
+                                  int scheme, int group, int n_kv_heads, int n_q_heads, int head_dim,
+                                  const void* q, int q_dtype, float scale_qk,
+                                  const int64_t* cache_row_base, const int32_t* cache_fill, int n_caches,
+                                  int64_t max_len, float decay, float now, float* row_acc, float* row_ts,
+                                  float* out, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!k_codes || !k_scale || !v_codes || !v_scale || !q || !cache_row_base || !cache_fill || !out)
+    return PIKV_ERR_NULL;
+  if (scheme < 0 || scheme > 3) return PIKV_ERR_UNSUPPORTED;
+  if (n_caches < 1 || n_q_heads < 1 || n_kv_heads < 1 || head_dim < 1 || max_len < 0) return PIKV_ERR_SHAPE;
+  const DecodeWs w = decode_ws(n_caches, n_q_heads, head_dim, max_len);
+  if (max_len > 0) {
+    if (!workspace) return PIKV_ERR_NULL;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return PIKV_ERR_SHAPE;
+    if (workspace_bytes < w.total) return PIKV_ERR_WORKSPACE;
+  }
+  char* ws = reinterpret_cast<char*>(workspace);
+  float* tmax = reinterpret_cast<float*>(ws + w.tmax);
+  float* tsum = reinterpret_cast<float*>(ws + w.tsum);
+  float* stats = reinterpret_cast<float*>(ws + w.stats);
+  void* partial = ws + w.partial;
+  const int64_t partial_bytes = w.total - w.partial;
+  hipStream_t st = (hipStream_t)stream;
+  if (max_len == 0)  // nothing cached anywhere: the output is zero (the reduction writes it)
+    return pikv_attend_values(reinterpret_cast<const float*>(out), nullptr, 0, v_codes, v_scale, v_zero, scheme, group,
+                              n_kv_heads, n_q_heads, head_dim, cache_row_base, cache_fill, n_caches, 0, decay, now,
+                              row_acc, row_ts, out, nullptr, 0, stream);
+  // fast form: the 4-bit matrix-core kernels meet in the exchange format
+  const bool asym = scheme == PIKV_Q_I4_ASYM;
+  const int rep = n_q_heads % n_kv_heads == 0 ? n_q_heads / n_kv_heads : 0;
+  const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;
+  const int64_t splits = attend_splits(max_len);
+  if ((scheme == PIKV_Q_I4_ASYM || scheme == PIKV_Q_I4_SYM) && group == 32 && head_dim == 128 && rep >= 1 &&
+      rep <= 8 && hk_ok && q_dtype == PIKV_BF16 && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {
+    float* esc = reinterpret_cast<float*>(ws + w.scores);
+    const int rc = scores_exchange_launch(k_codes, k_scale, k_zero, scheme, group, n_kv_heads, n_q_heads, head_dim, q,
+                                          q_dtype, scale_qk, cache_row_base, cache_fill, n_caches, max_len, esc, tmax,
+                                          tsum, stats, st);
+    if (rc == PIKV_OK) {
+      AttendArgs a{nullptr, stats, v_codes, v_scale, v_zero, cache_row_base, cache_fill,
+                   (float*)partial, 0, group, n_kv_heads, n_q_heads, head_dim, n_caches,
+                   row_acc, row_ts, decay, now, max_len, esc, tmax, w.n_tiles, 0};
+      const dim3 grid((unsigned)splits, (unsigned)n_caches);
+      for (int off = 0; off < rep; off += 4) {   // four query heads of every kv group per launch
+        a.head_off = off;
+        if (off > 0) a.decay = 1.0f;
+        if (asym) launch_attend_mfma<PIKV_Q_I4_ASYM>(n_kv_heads, grid, st, a);
+        else launch_attend_mfma<PIKV_Q_I4_SYM>(n_kv_heads, grid, st, a);
+      }
+      const int64_t total = (int64_t)n_caches * n_q_heads * head_dim;
+      hipLaunchKernelGGL(attend_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                         (const float*)partial, cache_fill, n_caches, n_q_heads, head_dim, (int)splits, out);
+      PIKV_CHECK_LAUNCH();
+      return PIKV_OK;
+    }
+    if (rc != PIKV_ERR_UNSUPPORTED) return rc;
+  }
+  // every other cache format: the three public steps, with float scores in the workspace
+  float* scores = reinterpret_cast<float*>(ws + w.scores);
+  int rc = pikv_gather_dequant_scores(k_codes, k_scale, k_zero, scheme, group, n_kv_heads, n_q_heads, head_dim, q,
+                                      q_dtype, scale_qk, cache_row_base, cache_fill, n_caches, max_len, w.stride,
+                                      scores, tmax, tsum, stream);
+  if (rc != PIKV_OK) return rc;
+  rc = pikv_h2o_accumulate(scores, tmax, tsum, n_q_heads, cache_row_base, cache_fill, n_caches, max_len, w.stride,
+                           1.0f, now, 0, nullptr, nullptr, nullptr, stats, stream);
+  if (rc != PIKV_OK) return rc;
+  return pikv_attend_values(scores, stats, w.stride, v_codes, v_scale, v_zero, scheme, group, n_kv_heads, n_q_heads,
+                            head_dim, cache_row_base, cache_fill, n_caches, max_len, decay, now, row_acc, row_ts, out,
+                            partial, partial_bytes, stream);
 }

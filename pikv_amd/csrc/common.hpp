@@ -424,4 +424,13 @@ __device__ __forceinline__ float load_meta(const void* plane, int64_t idx) {
 
 __host__ __device__ inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 
+// read_path.hip, for pikv_decode_attend in attend.hip: the 4-bit matrix-core score kernel writing the
+// exchange format (escores [cache][tile][q head][64] floats = exp(score - tile max); tile_max, tile_sum
+// [cache][tile][q head]) followed by the merge of the tile statistics into head_stats [cache][q head][2].
+// Returns PIKV_ERR_UNSUPPORTED, with nothing enqueued, for cache formats that kernel does not serve.
+int scores_exchange_launch(const void* k_codes, const void* k_scale, const void* k_zero, int scheme, int group,
+                           int n_kv_heads, int n_q_heads, int head_dim, const void* q, int q_dtype, float scale_qk,
+                           const int64_t* cache_row_base, const int32_t* cache_fill, int n_caches, int64_t max_len,
+                           float* escores, float* tile_max, float* tile_sum, float* head_stats, hipStream_t st);
+
 }  // namespace pikv

@@ -93,6 +93,9 @@ struct ScoreArgs {
   int n_kv_heads;
   int n_q_heads;
   int head_dim;
+  float* escores;    // when set (4-bit GQA kernel only), written INSTEAD of scores: [cache][tile][q head][64] floats,
+                     // exp(score - tile max) of every token - the exchange format of pikv_decode_attend
+  int score_vec;    // score rows start on 16-byte boundaries (stride % 4 == 0, aligned base)
   int max_len;      // rows of a cache beyond max_len are not read (a cache may hold more than the caller covers)
   int rep;          // scores_kernel: query heads per kv head, and the first head of every kv group that
   int head_off;     //   this launch serves (it serves REP of them; other ratios take several launches)
@@ -365,41 +368,57 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) { return (x & m) | o; }
 
 // Tile statistics and score rows from the staged scores [q head][token in tile], four
-// heads per wavefront pass: lane (rg, nl) owns tokens nl, nl+16, nl+32, nl+48 of head
-// h4 + rg; the 16 lanes of a row reduce with DPP.
+// heads per wavefront pass: lane (rg, nl) owns the four consecutive tokens 4 nl .. 4 nl + 3 of
+// head h4 + rg, so that a score row leaves as one 16-byte store per lane (256 contiguous
+// bytes per head and instruction; a quarter of the store instructions of a token-strided
+// map); the 16 lanes of a row reduce with DPP.  Rows that are not 16-byte aligned
+// (a.score_vec == 0) are stored element by element.
 // GROUPED: the staged rows are [kv head][SLOTS] (row SLOTS g + r = head g * rep + r, rows
 // r >= rep unused), so that the row of a kv head sits at a compile-time offset for the writers.
 template <bool GROUPED, int SLOTS = 4>
 __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float* stage, int c, int64_t tile,
                                                  int64_t n0, int len, int wave, int rg, int nl, int rep = 4) {
   const int n_pass_rows = GROUPED ? a.n_kv_heads * SLOTS : a.n_q_heads;
+  const int left = len - (int)n0 - 4 * nl;                     // tokens of this lane's run that exist
   for (int h4 = wave * 4; h4 < n_pass_rows; h4 += 16) {
     const int srow = h4 + rg;                                  // staged row = kv head * SLOTS + slot
     const int slot = srow % SLOTS;
     const int hq = GROUPED ? (srow / SLOTS) * rep + slot : srow;  // query head
     const bool hok = GROUPED ? slot < rep : hq < a.n_q_heads;
-    float x[4];
-    bool okk[4];
-    float m = -__builtin_inff();
+    const float4 sv = hok ? *reinterpret_cast<const float4*>(stage + srow * kTile + 4 * nl)
+                          : make_float4(0.f, 0.f, 0.f, 0.f);
+    const float ninf = -__builtin_inff();
+    float x[4] = {sv.x, sv.y, sv.z, sv.w};
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      okk[k] = hok && (n0 + nl + 16 * k < len);
-      x[k] = okk[k] ? stage[srow * kTile + nl + 16 * k] : -__builtin_inff();
-      m = fmaxf(m, x[k]);
-    }
+    for (int k = 0; k < 4; ++k) x[k] = (hok && k < left) ? x[k] : ninf;
+    float m = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
     m = dpp_max<kDppXor1>(m);
     m = dpp_max<kDppXor2>(m);
     m = dpp_max<kDppHalfMirror>(m);
     m = dpp_max<kDppMirror>(m);
-    float sum = 0.f;
-    float* out = a.scores + ((int64_t)c * a.n_q_heads + (hok ? hq : 0)) * a.score_stride + n0 + nl;
+    float e[4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      if (okk[k]) {
-        sum += __builtin_amdgcn_exp2f((x[k] - m) * 1.4426950408889634f);
-        out[16 * k] = x[k];
+    for (int k = 0; k < 4; ++k)   // exp2(-inf) = 0 for the tokens that do not exist
+      e[k] = (m > ninf) ? __builtin_amdgcn_exp2f((x[k] - m) * 1.4426950408889634f) : 0.f;  // (a row without tokens: -inf - -inf)
+    if (a.escores) {
+      // whole tiles, heads of a tile side by side: the block's output is one contiguous run
+      if (hok) {
+        *reinterpret_cast<float4*>(a.escores + (((int64_t)c * a.n_tiles + tile) * a.n_q_heads + hq) * kTile + 4 * nl) =
+            make_float4(e[0], e[1], e[2], e[3]);
+      }
+    } else {
+      float* out = a.scores + ((int64_t)c * a.n_q_heads + (hok ? hq : 0)) * a.score_stride + n0 + 4 * nl;
+      if (hok && left > 0) {
+        if (a.score_vec && left >= 4) {
+          *reinterpret_cast<float4*>(out) = sv;
+        } else {
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+            if (k < left) out[k] = x[k];
+        }
       }
     }
+    float sum = (e[0] + e[1]) + (e[2] + e[3]);
     sum = dpp_add<kDppXor1>(sum);
     sum = dpp_add<kDppXor2>(sum);
     sum = dpp_add<kDppHalfMirror>(sum);
@@ -529,7 +548,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   const uint4* a_lane[NSET];
 #pragma unroll
   for (int set = 0; set < NSET; ++set) a_lane[set] = (a_on ? alds + set * a.n_kv_heads * 64 : azero) + nl;
-  const uint32_t kNib = 0x000f000fu, kExp = 0x43004300u;  // two nibbles -> two bf16 values 128 + code
+  // two nibbles -> two bf16 values 128 + code.  Both constants are kept in vector registers
+  // (the empty statement hides their values from the compiler, it emits no instruction): with
+  // a literal or scalar operand the three-operand and-or instruction cannot be encoded and
+  // every expansion falls apart into an AND and an OR.
+  uint32_t kNib = 0x000f000fu, kExp = 0x43004300u;
+  asm volatile("" : "+v"(kNib), "+v"(kExp));
 
   // One tile: returns false when the block has run past the cache's fill.
   auto do_tile = [&](int tt, TileRegs& cur, TileRegs& nxt) -> bool {
@@ -940,6 +964,25 @@ static int launch_scores(int rep, dim3 grid, hipStream_t st, int q_dtype, ScoreA
   return PIKV_OK;
 }
 
+int scores_exchange_launch(const void* k_codes, const void* k_scale, const void* k_zero, int scheme, int group,
+                           int n_kv_heads, int n_q_heads, int head_dim, const void* q, int q_dtype, float scale_qk,
+                           const int64_t* cache_row_base, const int32_t* cache_fill, int n_caches, int64_t max_len,
+                           float* escores, float* tile_max, float* tile_sum, float* head_stats, hipStream_t st) {
+  if (scheme != PIKV_Q_I4_ASYM && scheme != PIKV_Q_I4_SYM) return PIKV_ERR_UNSUPPORTED;
+  if (group != 32 || head_dim != 128 || q_dtype != PIKV_BF16 || n_q_heads % n_kv_heads != 0) return PIKV_ERR_UNSUPPORTED;
+  if (n_q_heads / n_kv_heads > 8 || n_q_heads > kMaxQHeads || max_len < 1) return PIKV_ERR_UNSUPPORTED;
+  const int64_t n_tiles = (max_len + kTile - 1) / kTile;
+  ScoreArgs a{k_codes, k_scale, k_zero, q, cache_row_base, cache_fill, nullptr, tile_max, tile_sum,
+              0, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim, escores, 0,
+              (int)(max_len < 0x7fffffffLL ? max_len : 0x7fffffffLL), n_q_heads / n_kv_heads, 0, 1};
+  const int rc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(a, n_caches, n_tiles, st)
+                                            : launch_gqa<PIKV_Q_I4_SYM>(a, n_caches, n_tiles, st);
+  if (rc != PIKV_OK) return rc;
+  hipLaunchKernelGGL(head_stats_kernel, dim3((unsigned)((n_q_heads + 15) / 16), (unsigned)n_caches), dim3(256), 0,
+                     st, tile_max, tile_sum, cache_fill, n_q_heads, n_tiles, head_stats);
+  return PIKV_OK;
+}
+
 }  // namespace pikv
 
 using namespace pikv;
@@ -1009,7 +1052,8 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
   if (n_tiles > 0x7fffffffLL) return PIKV_ERR_SHAPE;
   ScoreArgs a{k_codes, k_scale, k_zero, q, cache_row_base, cache_fill, scores, tile_max, tile_sum,
-              score_stride, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim,
+              score_stride, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim, nullptr,
+              (score_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(scores) & 15) == 0) ? 1 : 0,
               (int)(max_len < 0x7fffffffLL ? max_len : 0x7fffffffLL), n_q_heads / n_kv_heads, 0, 1};
   const dim3 grid((unsigned)n_tiles, (unsigned)n_caches);
   hipStream_t st = (hipStream_t)stream;

@@ -672,6 +672,40 @@ class CachePool:
                _ptr(out), _ptr(ws), ws_bytes, _stream())
         return out
 
+    def decode_attend(self, q, n_q_heads: int, now: float = 0.0, scale_qk: Optional[float] = None,
+                      max_len: Optional[int] = None, accumulate: bool = True, decay: float = 1.0):
+        """The whole decode read in one native call (pikv_decode_attend): scores of q
+        [n_caches, n_q_heads, head_dim] against the compressed K rows, softmax over each cache's
+        rows, attention output over the compressed V rows -> out [n_caches, n_q_heads, head_dim]
+        float32; accumulate=True adds the probabilities to the H2O accumulators (acc = acc*decay +
+        sum over the heads, ts = now).  The score matrix stays inside the library's workspace."""
+        if not self.with_v:
+            raise ValueError("this pool stores no V rows")
+        q = _need(q, "q", ndim=3)
+        dt = _dt(q, "q")
+        if q.shape != (self.n_caches, n_q_heads, self.head_dim):
+            raise ValueError(f"q must be [{self.n_caches},{n_q_heads},{self.head_dim}], got {tuple(q.shape)}")
+        if n_q_heads % self.n_heads:
+            raise ValueError("n_q_heads must be a multiple of the kv heads")
+        if scale_qk is None:
+            scale_qk = 1.0 / math.sqrt(self.head_dim)
+        max_len = self.max_cap if max_len is None else int(max_len)
+        dev = self.device
+        out = torch.empty(self.n_caches, n_q_heads, self.head_dim, dtype=torch.float32, device=dev)
+        key = (n_q_heads, max_len)
+        if getattr(self, "_decode_ws_key", None) != key:
+            nb = int(N.lib().pikv_decode_attend_workspace_bytes(self.n_caches, n_q_heads, self.head_dim, max_len))
+            self._decode_ws = torch.empty(max(nb, 256), dtype=torch.uint8, device=dev)
+            self._decode_ws_key = key
+        ws = self._decode_ws
+        N.call("pikv_decode_attend", _ptr(self.k_codes), _ptr(self.k_scale), _ptr(self.k_zero),
+               _ptr(self.v_codes), _ptr(self.v_scale), _ptr(self.v_zero), self.scheme, self.group,
+               self.n_heads, n_q_heads, self.head_dim, _ptr(q), dt, float(scale_qk), _ptr(self.row_base),
+               _ptr(self.fill), self.n_caches, max_len, float(decay), float(now),
+               _ptr(self.acc) if accumulate else None, _ptr(self.ts) if accumulate else None,
+               _ptr(out), _ptr(ws), ws.numel(), _stream())
+        return out
+
     # ---- eviction ----
     def evict_select(self, policy: int, *, heavy_ratio=0.1, recent_ratio=0.1,
                      n_heavy=None, n_recent=None, n_evict=None, multi_block: bool = True):

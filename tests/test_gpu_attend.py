@@ -123,3 +123,90 @@ def test_attend_peaked_distribution(dev):
     v_hat = O.dequantize_groups(ref.v_codes[rows], ref.v_scale[rows], ref.v_zero[rows], 32)
     want = O.attend_values(probs[0, :, :L], v_hat, heads)
     assert np.abs(out[0] - want).max() <= 2e-5 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("scheme,group,heads,hq,dh,qdtype", [
+    (O.Q_I4_ASYM, 32, 8, 32, 128, "bf16"),   # decode shape: exchange format between the matrix-core kernels
+    (O.Q_I4_SYM, 32, 2, 4, 128, "bf16"),     # ... symmetric codes
+    (O.Q_I4_ASYM, 32, 1, 8, 128, "bf16"),    # ... 8 q heads per kv head: two sets, two attention launches
+    (O.Q_I4_ASYM, 32, 8, 24, 128, "bf16"),   # ... 3 q heads per kv head
+    (O.Q_I4_SYM, 32, 4, 28, 128, "bf16"),    # ... 7 q heads per kv head
+    (O.Q_I4_ASYM, 32, 16, 16, 128, "bf16"),  # 16 kv heads: the three public steps inside the call
+    (O.Q_I4_ASYM, 32, 8, 32, 128, "f32"),    # float32 queries: same
+    (O.Q_I8_SYM, 128, 8, 32, 128, "bf16"),   # 8-bit matrix-core kernels
+    (O.Q_I8_ASYM, 64, 2, 16, 64, "f32"),     # vector forms
+    (O.Q_I4_SYM, 64, 4, 12, 64, "bf16"),
+])
+@pytest.mark.parametrize("decay", [1.0, 0.9])
+def test_decode_attend_one_call(dev, scheme, group, heads, hq, dh, qdtype, decay):
+    """pikv_decode_attend against core/single/pikv_attention.py:123,163,188 and
+    cache_scheduling.py:69-73 evaluated in float64 on the restatement's dequantised K and V
+    rows: attention output within 1e-3 of its root-mean-square, accumulators within 1e-3
+    relative, timestamps exact; rows outside the caches' fill untouched.  Two calls in a row
+    (the second after an append) reuse the pool's workspace."""
+    import torch
+    r = rng(scheme * 5 + heads + hq)
+    caps = [4300, 64, 130, 10]
+    lens = [4100, 64, 1, 0]           # spans three token ranges, full tile, single row, empty
+    pool, ref = _fill_pool(dev, r, caps, lens, heads, dh, group, scheme)
+    acc0 = r.random(pool.rows).astype(np.float32)
+    pool.acc.copy_(to_dev(acc0, dev))
+    pool.ts.fill_(-3.0)
+    scale_qk = 1.0 / np.sqrt(dh)
+
+    def reference(q, lens_now, acc_before):
+        outs, accs = [], acc_before.copy()
+        for c, L in enumerate(lens_now):
+            if L == 0:
+                outs.append(np.zeros((hq, dh), np.float32))
+                continue
+            rows = ref.valid_rows(c)[:L]
+            k_hat = O.dequantize_groups(ref.k_codes[rows], ref.k_scale[rows], ref.k_zero[rows], group)
+            v_hat = O.dequantize_groups(ref.v_codes[rows], ref.v_scale[rows], ref.v_zero[rows], group)
+            s = O.attention_scores(q[c], k_hat, heads, scale_qk)
+            p, imp = O.h2o_importance(s)
+            outs.append(O.attend_values(p, v_hat, heads))
+            accs[rows] = accs[rows] * np.float32(decay) + imp
+        return np.stack(outs), accs
+
+    q = r.standard_normal((len(caps), hq, dh)).astype(np.float32) * 2
+    if qdtype == "bf16":
+        q = O.bf16_round(q)
+    out = np_of(pool.decode_attend(to_dev(q, dev, qdtype), hq, now=7.0, decay=decay))
+    want, acc_ref = reference(q, lens, acc0)
+    for c, L in enumerate(lens):
+        if L == 0:
+            assert not out[c].any()
+            continue
+        rms = np.sqrt((want[c].astype(np.float64) ** 2).mean()) + 1e-12
+        assert np.abs(out[c] - want[c]).max() <= 1e-3 * rms, (c, np.abs(out[c] - want[c]).max(), rms)
+    np.testing.assert_allclose(np_of(pool.acc), acc_ref, rtol=1e-3, atol=1e-5)
+    ts = np_of(pool.ts)
+    for c, L in enumerate(lens):
+        rows = ref.valid_rows(c)
+        assert (ts[rows[:L]] == 7.0).all()
+    touched = np.zeros(pool.rows, bool)
+    for c, L in enumerate(lens):
+        touched[ref.valid_rows(c)[:L]] = True
+    assert (ts[~touched] == -3.0).all() and np.array_equal(np_of(pool.acc)[~touched], acc0[~touched])
+    # same result as the three public steps
+    scores, tmax, tsum = pool.scores(to_dev(q, dev, qdtype), hq)
+    pool.h2o_accumulate(scores, tmax, tsum, now=7.0, stats_only=True)
+    out3 = np_of(pool.attend_values(scores, pool.head_stats))
+    assert np.abs(out - out3).max() <= 1e-3 * (np.sqrt((out3.astype(np.float64) ** 2).mean()) + 1e-12)
+    # second call on the same workspace, without the bookkeeping, covering fewer rows than cached
+    acc_now = np_of(pool.acc).copy()
+    q2 = O.bf16_round(r.standard_normal((len(caps), hq, dh)).astype(np.float32))
+    out2 = np_of(pool.decode_attend(to_dev(q2, dev, qdtype), hq, now=8.0, accumulate=False, max_len=4300))
+    want2, _ = reference(q2, lens, acc_now)
+    for c, L in enumerate(lens):
+        if L:
+            rms = np.sqrt((want2[c].astype(np.float64) ** 2).mean()) + 1e-12
+            assert np.abs(out2[c] - want2[c]).max() <= 1e-3 * rms
+    assert np.array_equal(np_of(pool.acc), acc_now)
+    out_short = np_of(pool.decode_attend(to_dev(q2, dev, qdtype), hq, accumulate=False, max_len=200))
+    want_s, _ = reference(q2, [min(L, 200) for L in lens], acc_now)
+    for c, L in enumerate(lens):
+        if L:
+            rms = np.sqrt((want_s[c].astype(np.float64) ** 2).mean()) + 1e-12
+            assert np.abs(out_short[c] - want_s[c]).max() <= 1e-3 * rms
