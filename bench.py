@@ -31,11 +31,25 @@ sys.path.insert(0, ROOT)
 
 METRIC = "routed KV tokens/s (quant+scatter+gather+dequant), 1 MI355X; % HBM peak"
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the quantise+scatter kernel on this workload, from the
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
-# profiles/bench_all_workloads.md (counters scaled by what a plain 1 GiB
-# device copy reads on them: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
-K2_TRAFFIC_BYTES_PROFILED = 1099.2e6
+
+
+def profiled_traffic(kernel_prefix: str):
+    """HBM bytes per launch (fetched + written) of the roofline kernel as the rocprofv3 --pmc
+    runs recorded them: read from the machine-readable block at the end of profiles/prefill.md
+    (written by bench_profile.py, counters scaled by a streaming probe of known traffic in the
+    same run).  None when the summary is missing or has no such kernel."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, "profiles", "prefill.md")).read()
+        blob = json.loads(re.search(r"<!-- machine-readable: (.*) -->", text).group(1))
+    except (OSError, AttributeError, ValueError):
+        return None
+    best = None
+    for name, rec in blob.get("kernels", {}).items():
+        if name.startswith(kernel_prefix) and rec.get("fetch_bytes") is not None and rec.get("write_bytes") is not None:
+            if best is None or rec["calls"] > best["calls"]:
+                best = rec
+    return None if best is None else float(best["fetch_bytes"] + best["write_bytes"])
 
 WORKLOAD = dict(name="prefill compress-write", batch=16, seq=2048, hidden=4096, experts=8, top_k=2,
                 capacity_factor=1.25, heads=32, head_dim=128, cache_slots=8192,
@@ -335,6 +349,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only-headline", action="store_true",
                     help="skip the per-kernel figures of the decode, wide-routing and pyramid workloads")
+    ap.add_argument("--workload", default="all",
+                    choices=["all", "prefill", "decode_read", "decode_read_int8_gqa8", "wide_routing", "pyramid"],
+                    help="run one workload only (for profiling; the bench line proper is the default, all)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the streaming probes over 1 GiB (kernels of known traffic, to scale "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit")
@@ -367,6 +384,13 @@ def main():
                           "kernels": {"stream_probe_kernel<0,false>": "reads n", "stream_probe_kernel<1,false>": "writes n",
                                       "stream_probe_kernel<2,false>": "reads n and writes n"},
                           "hbm_ceiling": hbm_ceiling(torch, dev, 10)}))
+        return
+    others = {"decode_read": decode_read_workload, "decode_read_int8_gqa8": decode_read_int8_workload,
+              "wide_routing": wide_routing_workload, "pyramid": pyramid_workload}
+    if args.workload in others:
+        it = max(5, min(args.steps, 20))
+        print(json.dumps({"workload_only": args.workload, "hbm_ceiling": hbm_ceiling(torch, dev, 10),
+                          args.workload: others[args.workload](torch, ops, dev, it)}))
         return
     w = WORKLOAD
     T, E, k = w["batch"] * w["seq"], w["experts"], w["top_k"]
@@ -431,7 +455,8 @@ def main():
                    "kept_assignments": kept, "assignments": A},
         "roofline": {"bound": "hbm", "kernel": "quant_scatter_kernel<I8_SYM,bf16>",
                      "achieved": gbps(b_quant, t_quant), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": gbps(b_quant, t_quant) / HBM_PEAK_GBPS, "traffic": K2_TRAFFIC_BYTES_PROFILED,
+                     "frac": gbps(b_quant, t_quant) / HBM_PEAK_GBPS,
+                     "traffic": profiled_traffic("quant_scatter_kernel<0, 1, 2, true>"),
                      "algorithmic_bytes": b_quant, "avg_launch_ms": t_quant},
         "kernels": {
             "router": {"ms": t_router, "GBps": gbps(b_router, t_router)},
@@ -443,11 +468,10 @@ def main():
         },
     }
     out["hbm_ceiling"] = hbm_ceiling(torch, dev, 10)
-    if not args.only_headline:
+    if not args.only_headline and args.workload == "all":
         it = max(5, min(args.steps, 20))
         out["other_workloads"] = {}
-        for name, fn in (("decode_read", decode_read_workload), ("decode_read_int8_gqa8", decode_read_int8_workload),
-                         ("wide_routing", wide_routing_workload), ("pyramid", pyramid_workload)):
+        for name, fn in others.items():
             out["other_workloads"][name] = fn(torch, ops, dev, it)
             torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
