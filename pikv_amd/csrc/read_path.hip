@@ -144,45 +144,61 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
     qsum[r] = sacc;
   }
   const int64_t base_row = a.row_base[c];
-  constexpr int UN = 4;  // token steps in flight per lane
+  constexpr int UN = 4;  // token steps per batch of loads
+  const int batch = tok_per_step * UN;  // tokens of the tile covered by one batch
 
-  for (int s0 = 0; s0 < kTile; s0 += tok_per_step * UN) {
+  // Two register sets: the loads of the next batch are in flight while the current one is
+  // multiplied.  Loads are issued unconditionally from clamped rows (a token past the end of
+  // the cache or of the tile re-reads the last valid one and is masked when its score is
+  // staged): loads under conditions would make the wait before the arithmetic cover the
+  // prefetch as well.
+  struct Batch {
     uint4 v[UN];
     float sc[UN], zr[UN];
-    bool ok[UN];
+  };
+  const char* const code_base = reinterpret_cast<const char*>(a.codes) + ((base_row + n0) * lanes_per_row + part) * 16;
+  const int64_t meta_base = (base_row + n0) * groups_per_row + (part * EPL) / a.group;
+  const int last_tl = (len - n0 < kTile ? (int)(len - n0) : kTile) - 1;   // last token of the tile that exists
+  auto load_batch = [&](int s0, Batch& t) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int tl = s0 + u * tok_per_step + tok_in_step;
-      const int64_t n = n0 + tl;
-      ok[u] = tl < kTile && n < len;
-      v[u] = make_uint4(0, 0, 0, 0);
-      sc[u] = 0.f;
-      zr[u] = 0.f;
-      if (ok[u]) {
-        const int64_t row = base_row + n;
-        v[u] = ld16(reinterpret_cast<const char*>(a.codes) + (row * lanes_per_row + part) * 16);
-        const int64_t mi = row * groups_per_row + (part * EPL) / a.group;
-        sc[u] = load_meta<SCHEME>(a.scale, mi);
-        if constexpr (!Q::sym) zr[u] = load_meta<SCHEME>(a.zero, mi);
-      }
+      int tl = s0 + u * tok_per_step + tok_in_step;
+      tl = tl < last_tl ? tl : last_tl;
+      t.v[u] = ld16(code_base + (int64_t)tl * lanes_per_row * 16);
+      const int64_t mi = meta_base + (int64_t)tl * groups_per_row;
+      t.sc[u] = load_meta<SCHEME>(a.scale, mi);
+      if constexpr (!Q::sym) t.zr[u] = load_meta<SCHEME>(a.zero, mi);
+      else t.zr[u] = 0.f;
     }
+  };
+  auto mul_batch = [&](int s0, const Batch& t) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int tl = s0 + u * tok_per_step + tok_in_step;
+      const bool ok = tl < kTile && n0 + tl < len;
       float cf[EPL];
-      unpack_codes_unsigned<SCHEME>(v[u], cf);
-      const float zu = zr[u] - (float)Q::qmin;  // zero point of the unsigned stored form
+      unpack_codes_unsigned<SCHEME>(t.v[u], cf);
+      const float zu = t.zr[u] - (float)Q::qmin;  // zero point of the unsigned stored form
 #pragma unroll
       for (int r = 0; r < REP; ++r) {
         float d = 0.f;
 #pragma unroll
         for (int j = 0; j < EPL; ++j) d = fmaf(qv[r][j], cf[j], d);
-        d = (d - zu * qsum[r]) * sc[u];
+        d = (d - zu * qsum[r]) * t.sc[u];
         d = group_sum_dpp(d, lanes_per_head);
         if ((part % lanes_per_head) == 0 && tl < kTile)
-          stage[(kvl * REP + r) * kTile + tl] = ok[u] ? d * a.scale_qk : -__builtin_inff();
+          stage[(kvl * REP + r) * kTile + tl] = ok ? d * a.scale_qk : -__builtin_inff();
       }
     }
+  };
+  Batch ba, bb;
+  load_batch(0, ba);
+  for (int s0 = 0; s0 < kTile; s0 += 2 * batch) {
+    load_batch(s0 + batch, bb);
+    mul_batch(s0, ba);
+    if (s0 + batch >= kTile) break;
+    load_batch(s0 + 2 * batch, ba);
+    mul_batch(s0 + batch, bb);
   }
   __syncthreads();
 
