@@ -189,8 +189,9 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads) {
          (size_t)4 * n_kv_heads * kAttPRow * 4;
 }
 
-// HKS = log2(n_kv_heads); at most 4 query heads per kv head.
-template <int SCHEME, int HKS>
+// HKS = log2(n_kv_heads); at most 4 query heads per kv head.  EXCH: the scores come in the exchange
+// format of pikv_decode_attend (a.escores, a.tile_max) instead of a.scores.
+template <int SCHEME, int HKS, bool EXCH = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i4_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
@@ -259,7 +260,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const float s_off = normalise ? -INFINITY : 0.f;  // what a token past the end contributes: p = 0
   // exchange format: eight values exp(score - tile max) per thread and tile, and the tile's max of the head;
   // the rows of a tile lie side by side, [tile][q head][64], so a block reads one contiguous run
-  const bool exch = a.escores != nullptr;
+  constexpr bool exch = EXCH;
   const float* const ep = exch ? a.escores + ((int64_t)c * a.n_tiles * a.n_q_heads + s_hq) * kAttTile + st8 : nullptr;
   const float* const tmp = exch ? a.tile_max + (int64_t)c * a.n_tiles * a.n_q_heads + s_hq : nullptr;
   float ptm = 0.f;
@@ -809,14 +810,14 @@ static void launch_attend_mfma8(int n_kv_heads, dim3 grid, hipStream_t st, const
   }
 }
 
-template <int SCHEME>
+template <int SCHEME, bool EXCH = false>
 static void launch_attend_mfma(int n_kv_heads, dim3 grid, hipStream_t st, const AttendArgs& a) {
   const size_t lds = attend_mfma_lds_bytes(n_kv_heads, a.n_q_heads);
   switch (n_kv_heads) {
-    case 1: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 0>), grid, dim3(256), lds, st, a); break;
-    case 2: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 1>), grid, dim3(256), lds, st, a); break;
-    case 4: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 2>), grid, dim3(256), lds, st, a); break;
-    default: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 3>), grid, dim3(256), lds, st, a); break;
+    case 1: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 0, EXCH>), grid, dim3(256), lds, st, a); break;
+    case 2: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 1, EXCH>), grid, dim3(256), lds, st, a); break;
+    case 4: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 2, EXCH>), grid, dim3(256), lds, st, a); break;
+    default: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 3, EXCH>), grid, dim3(256), lds, st, a); break;
   }
 }
 
@@ -1006,8 +1007,8 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
       for (int off = 0; off < rep; off += 4) {   // four query heads of every kv group per launch
         a.head_off = off;
         if (off > 0) a.decay = 1.0f;
-        if (asym) launch_attend_mfma<PIKV_Q_I4_ASYM>(n_kv_heads, grid, st, a);
-        else launch_attend_mfma<PIKV_Q_I4_SYM>(n_kv_heads, grid, st, a);
+        if (asym) launch_attend_mfma<PIKV_Q_I4_ASYM, true>(n_kv_heads, grid, st, a);
+        else launch_attend_mfma<PIKV_Q_I4_SYM, true>(n_kv_heads, grid, st, a);
       }
       const int64_t total = (int64_t)n_caches * n_q_heads * head_dim;
       hipLaunchKernelGGL(attend_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,

@@ -95,7 +95,6 @@ struct ScoreArgs {
   int head_dim;
   float* escores;    // when set (4-bit GQA kernel only), written INSTEAD of scores: [cache][tile][q head][64] floats,
                      // exp(score - tile max) of every token - the exchange format of pikv_decode_attend
-  int score_vec;    // score rows start on 16-byte boundaries (stride % 4 == 0, aligned base)
   int max_len;      // rows of a cache beyond max_len are not read (a cache may hold more than the caller covers)
   int rep;          // scores_kernel: query heads per kv head, and the first head of every kv group that
   int head_off;     //   this launch serves (it serves REP of them; other ratios take several launches)
@@ -384,15 +383,62 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) { return (x & m) | o; }
 
 // Tile statistics and score rows from the staged scores [q head][token in tile], four
-// heads per wavefront pass: lane (rg, nl) owns the four consecutive tokens 4 nl .. 4 nl + 3 of
-// head h4 + rg, so that a score row leaves as one 16-byte store per lane (256 contiguous
-// bytes per head and instruction; a quarter of the store instructions of a token-strided
-// map); the 16 lanes of a row reduce with DPP.  Rows that are not 16-byte aligned
-// (a.score_vec == 0) are stored element by element.
+// heads per wavefront pass: lane (rg, nl) owns tokens nl, nl+16, nl+32, nl+48 of head
+// h4 + rg; the 16 lanes of a row reduce with DPP.
 // GROUPED: the staged rows are [kv head][SLOTS] (row SLOTS g + r = head g * rep + r, rows
 // r >= rep unused), so that the row of a kv head sits at a compile-time offset for the writers.
 template <bool GROUPED, int SLOTS = 4>
 __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float* stage, int c, int64_t tile,
+                                                 int64_t n0, int len, int wave, int rg, int nl, int rep = 4) {
+  const int n_pass_rows = GROUPED ? a.n_kv_heads * SLOTS : a.n_q_heads;
+  for (int h4 = wave * 4; h4 < n_pass_rows; h4 += 16) {
+    const int srow = h4 + rg;                                  // staged row = kv head * SLOTS + slot
+    const int slot = srow % SLOTS;
+    const int hq = GROUPED ? (srow / SLOTS) * rep + slot : srow;  // query head
+    const bool hok = GROUPED ? slot < rep : hq < a.n_q_heads;
+    float x[4];
+    bool okk[4];
+    float m = -__builtin_inff();
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      okk[k] = hok && (n0 + nl + 16 * k < len);
+      x[k] = okk[k] ? stage[srow * kTile + nl + 16 * k] : -__builtin_inff();
+      m = fmaxf(m, x[k]);
+    }
+    m = dpp_max<kDppXor1>(m);
+    m = dpp_max<kDppXor2>(m);
+    m = dpp_max<kDppHalfMirror>(m);
+    m = dpp_max<kDppMirror>(m);
+    float sum = 0.f;
+    float* out = a.scores + ((int64_t)c * a.n_q_heads + (hok ? hq : 0)) * a.score_stride + n0 + nl;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (okk[k]) {
+        sum += __builtin_amdgcn_exp2f((x[k] - m) * 1.4426950408889634f);
+        out[16 * k] = x[k];
+      }
+    }
+    sum = dpp_add<kDppXor1>(sum);
+    sum = dpp_add<kDppXor2>(sum);
+    sum = dpp_add<kDppHalfMirror>(sum);
+    sum = dpp_add<kDppMirror>(sum);
+    if (nl == 0 && hok) {
+      const int64_t ti = ((int64_t)c * a.n_tiles + tile) * a.n_q_heads + hq;  // heads of a tile side by side
+      a.tile_max[ti] = m;
+      a.tile_sum[ti] = sum;
+    }
+  }
+}
+
+// The same for the exchange format of pikv_decode_attend (a.escores set): lane (rg, nl) owns the
+// four consecutive tokens 4 nl .. 4 nl + 3 of head h4 + rg and stores exp(score - tile max) of
+// them as one 16-byte vector into [cache][tile][q head][64]; the heads of a tile lie side by
+// side, so a block's output is one contiguous run.  (For the public [head][token] score rows the
+// same 16-byte stores were measured and changed nothing; they keep the token-strided map.)
+// GROUPED: the staged rows are [kv head][SLOTS] (row SLOTS g + r = head g * rep + r, rows
+// r >= rep unused), so that the row of a kv head sits at a compile-time offset for the writers.
+template <bool GROUPED, int SLOTS = 4>
+__device__ __forceinline__ void tile_stats_exchange(const ScoreArgs& a, const float* stage, int c, int64_t tile,
                                                  int64_t n0, int len, int wave, int rg, int nl, int rep = 4) {
   const int n_pass_rows = GROUPED ? a.n_kv_heads * SLOTS : a.n_q_heads;
   const int left = len - (int)n0 - 4 * nl;                     // tokens of this lane's run that exist
@@ -416,24 +462,9 @@ __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float
 #pragma unroll
     for (int k = 0; k < 4; ++k)   // exp2(-inf) = 0 for the tokens that do not exist
       e[k] = (m > ninf) ? __builtin_amdgcn_exp2f((x[k] - m) * 1.4426950408889634f) : 0.f;  // (a row without tokens: -inf - -inf)
-    if (a.escores) {
-      // whole tiles, heads of a tile side by side: the block's output is one contiguous run
-      if (hok) {
-        *reinterpret_cast<float4*>(a.escores + (((int64_t)c * a.n_tiles + tile) * a.n_q_heads + hq) * kTile + 4 * nl) =
-            make_float4(e[0], e[1], e[2], e[3]);
-      }
-    } else {
-      float* out = a.scores + ((int64_t)c * a.n_q_heads + (hok ? hq : 0)) * a.score_stride + n0 + 4 * nl;
-      if (hok && left > 0) {
-        if (a.score_vec && left >= 4) {
-          *reinterpret_cast<float4*>(out) = sv;
-        } else {
-#pragma unroll
-          for (int k = 0; k < 4; ++k)
-            if (k < left) out[k] = x[k];
-        }
-      }
-    }
+    if (hok)   // whole tiles: tokens that do not exist are stored as zeros
+      *reinterpret_cast<float4*>(a.escores + (((int64_t)c * a.n_tiles + tile) * a.n_q_heads + hq) * kTile + 4 * nl) =
+          make_float4(e[0], e[1], e[2], e[3]);
     float sum = (e[0] + e[1]) + (e[2] + e[3]);
     sum = dpp_add<kDppXor1>(sum);
     sum = dpp_add<kDppXor2>(sum);
@@ -464,7 +495,7 @@ static size_t gqa_lds_bytes(int n_kv_heads, int nset) {
 // multiplied (two register sets, used alternately).
 // NSET sets of four query heads per kv head (1: up to 4 heads, 2: up to 8): the unpacked codes
 // of a kv head are multiplied with one block-diagonal A operand per set.
-template <int SCHEME, int NKV, int NSET = 1>  // NKV = n_kv_heads rounded up to 4/8/16
+template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false>  // NKV = n_kv_heads rounded up to 4/8/16; EXCH: exchange format out
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET <= 8 ? 4 : 2))) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
   constexpr int SL = 4 * NSET;  // head slots per kv head
   using Q = QScheme<SCHEME>;
@@ -635,7 +666,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     }
     __syncthreads();
 
-    tile_stats_store<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep);
+    if constexpr (EXCH) tile_stats_exchange<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep);
+    else tile_stats_store<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep);
     __syncthreads();  // stage and the metadata rows are reused by the next tile
     return true;
   };
@@ -790,7 +822,7 @@ static int launch_i8_mfma(const ScoreArgs& a, int n_caches, int64_t n_tiles, hip
   return PIKV_OK;
 }
 
-template <int SCHEME>
+template <int SCHEME, bool EXCH = false>
 static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
   const int rep = a.n_q_heads / a.n_kv_heads;
   const int nset = rep <= 4 ? 1 : 2;
@@ -799,17 +831,17 @@ static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStre
   const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
   if (nset == 1) {
     if (a.n_kv_heads <= 4)
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1, EXCH>), grid, dim3(256), lds, st, a);
     else if (a.n_kv_heads <= 8)
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1, EXCH>), grid, dim3(256), lds, st, a);
     else
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 16, 1>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 16, 1, EXCH>), grid, dim3(256), lds, st, a);
   } else {
     // 5-8 query heads per kv head; 16 kv heads x 8 would need more than 64 KB of LDS
     if (a.n_kv_heads <= 4)
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2, EXCH>), grid, dim3(256), lds, st, a);
     else
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH>), grid, dim3(256), lds, st, a);
   }
   return PIKV_OK;
 }
@@ -989,10 +1021,10 @@ int scores_exchange_launch(const void* k_codes, const void* k_scale, const void*
   if (n_q_heads / n_kv_heads > 8 || n_q_heads > kMaxQHeads || max_len < 1) return PIKV_ERR_UNSUPPORTED;
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
   ScoreArgs a{k_codes, k_scale, k_zero, q, cache_row_base, cache_fill, nullptr, tile_max, tile_sum,
-              0, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim, escores, 0,
+              0, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim, escores,
               (int)(max_len < 0x7fffffffLL ? max_len : 0x7fffffffLL), n_q_heads / n_kv_heads, 0, 1};
-  const int rc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(a, n_caches, n_tiles, st)
-                                            : launch_gqa<PIKV_Q_I4_SYM>(a, n_caches, n_tiles, st);
+  const int rc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM, true>(a, n_caches, n_tiles, st)
+                                            : launch_gqa<PIKV_Q_I4_SYM, true>(a, n_caches, n_tiles, st);
   if (rc != PIKV_OK) return rc;
   hipLaunchKernelGGL(head_stats_kernel, dim3((unsigned)((n_q_heads + 15) / 16), (unsigned)n_caches), dim3(256), 0,
                      st, tile_max, tile_sum, cache_fill, n_q_heads, n_tiles, head_stats);
@@ -1069,7 +1101,6 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   if (n_tiles > 0x7fffffffLL) return PIKV_ERR_SHAPE;
   ScoreArgs a{k_codes, k_scale, k_zero, q, cache_row_base, cache_fill, scores, tile_max, tile_sum,
               score_stride, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim, nullptr,
-              (score_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(scores) & 15) == 0) ? 1 : 0,
               (int)(max_len < 0x7fffffffLL ? max_len : 0x7fffffffLL), n_q_heads / n_kv_heads, 0, 1};
   const dim3 grid((unsigned)n_tiles, (unsigned)n_caches);
   hipStream_t st = (hipStream_t)stream;
