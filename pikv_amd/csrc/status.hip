@@ -13,4 +13,4 @@ extern "C" const char* pikv_status_string(int status) {
   return "unknown status";
 }
 
-extern "C" int pikv_abi_version(void) { return 1002; }  // 1.2: + pikv_capacity_slots_static
+extern "C" int pikv_abi_version(void) { return 1003; }  // 1.3: + pikv_quant8_minshift, pikv_decode_attend, pikv_stream_probe
