@@ -185,8 +185,9 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads) {
   // codes [64 tokens][n_kv_heads*64 + 8 bytes]; scale and zero + bias as float4 (4 groups)
   // [64 tokens][kv head] in padded token rows; A operands per wavefront [4 groups][8 rows][kAttARow];
   // probabilities [query head][kAttPRow]
+  // + one all-zero piece of an A row (32 bytes) for the lanes whose row holds no head
   return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * att_meta_bytes(n_kv_heads) + 4 * (size_t)4 * 8 * kAttARow +
-         (size_t)4 * n_kv_heads * kAttPRow * 4;
+         (size_t)4 * n_kv_heads * kAttPRow * 4 + 32;
 }
 
 // HKS = log2(n_kv_heads); at most 4 query heads per kv head.  EXCH: the scores come in the exchange
@@ -209,6 +210,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int wave = threadIdx.x >> 6;
   unsigned char* abuf = lzterm + att_meta_bytes(HK) + wave * (4 * 8 * kAttARow);
   float* lprob = reinterpret_cast<float*>(lzterm + att_meta_bytes(HK) + 4 * (4 * 8 * kAttARow));
+  unsigned char* azero = reinterpret_cast<unsigned char*>(lprob + 4 * HK * kAttPRow);
+  if (threadIdx.x < 8) reinterpret_cast<uint32_t*>(azero)[threadIdx.x] = 0u;  // visible after the loop's first barrier
 
   const int c = blockIdx.y;
   const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
@@ -286,14 +289,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int64_t urow = base_row + n0;
     if (a.row_acc && igrp == 0 && it < rem) pacc = (a.row_acc + urow)[it];
     if (exch) {
-      if (s_on) {
-        const int64_t tile = n0 / kAttTile;
-        const float4 lo4 = *reinterpret_cast<const float4*>(ep + tile * a.n_q_heads * kAttTile);
-        const float4 hi4 = *reinterpret_cast<const float4*>(ep + tile * a.n_q_heads * kAttTile + 4);
-        psc[0] = lo4.x, psc[1] = lo4.y, psc[2] = lo4.z, psc[3] = lo4.w;
-        psc[4] = hi4.x, psc[5] = hi4.y, psc[6] = hi4.z, psc[7] = hi4.w;
-        ptm = tmp[tile * a.n_q_heads];
-      }
+      // staged rows without a head read head 0 (and are multiplied by zero): no branch around the loads
+      const int64_t tile = n0 / kAttTile;
+      const float4 lo4 = *reinterpret_cast<const float4*>(ep + tile * a.n_q_heads * kAttTile);
+      const float4 hi4 = *reinterpret_cast<const float4*>(ep + tile * a.n_q_heads * kAttTile + 4);
+      psc[0] = lo4.x, psc[1] = lo4.y, psc[2] = lo4.z, psc[3] = lo4.w;
+      psc[4] = hi4.x, psc[5] = hi4.y, psc[6] = hi4.z, psc[7] = hi4.w;
+      ptm = tmp[tile * a.n_q_heads];
     } else if (s_on) {
       const float* spn = sp + n0;
       if (s_vec && st8 + 8 <= rem) {
@@ -306,22 +308,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
         for (int k = 0; k < 8; ++k) psc[k] = st8 + k < rem ? spn[k] : s_off;
       }
     }
+    // Every load is issued, from an offset clamped to the tile's last cached row: tokens past the
+    // end of a short tile see a copy of that row, and their weight is zero (p = 0, finite scale).
     const char* cb = reinterpret_cast<const char*>(a.codes) + urow * (LPR * 16);
+    const unsigned c_last = (unsigned)(rem * LPR - 1) * 16u;
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
-      pc[k] = make_uint4(0, 0, 0, 0);
-      if ((int)threadIdx.x < rem * LPR - k * 256) pc[k] = ld16(cb + k * 4096 + threadIdx.x * 16);
+      const unsigned off = k * 4096u + threadIdx.x * 16u;
+      pc[k] = ld16(cb + (off < c_last ? off : c_last));
     }
-    const uint16_t* sb = reinterpret_cast<const uint16_t*>(a.scale) + urow * LPR;
-    const uint16_t* zb = reinterpret_cast<const uint16_t*>(a.zero) + urow * LPR;
+    const char* sb = reinterpret_cast<const char*>(a.scale) + urow * (LPR * 2);
+    const char* zb = reinterpret_cast<const char*>(a.zero) + urow * (LPR * 2);
+    const unsigned m_last = (unsigned)(rem * HK - 1) * 8u;
 #pragma unroll
     for (int k = 0; k < NMC; ++k) {
-      ps[k] = make_uint2(0, 0);
+      const unsigned off = k * 2048u + threadIdx.x * 8u;
+      const unsigned mo = off < m_last ? off : m_last;
+      ps[k] = *reinterpret_cast<const uint2*>(sb + mo);
       pz[k] = make_uint2(0, 0);
-      if ((int)threadIdx.x < rem * HK - k * 256) {
-        ps[k] = *reinterpret_cast<const uint2*>(sb + k * 1024 + threadIdx.x * 4);
-        if constexpr (!Q::sym) pz[k] = *reinterpret_cast<const uint2*>(zb + k * 1024 + threadIdx.x * 4);
-      }
+      if constexpr (!Q::sym) pz[k] = *reinterpret_cast<const uint2*>(zb + mo);
     }
   };
   auto h2f = [](uint32_t w, int hi) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> (16 * hi))); };
@@ -364,6 +369,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       }
     }
   };
+
+  // A-operand piece of this lane: row i of group sg (8 rows of kAttARow bytes per group), or the zero piece
+  const unsigned char* const a_row = i < 2 * rep ? abuf + i * kAttARow + kg * 32 : azero;
+  const int a_step = i < 2 * rep ? 8 * kAttARow : 0;
+  // two nibbles -> two bf16 values 128 + code.  Both constants are kept in vector registers (the
+  // empty statement hides their values from the compiler, it emits no instruction): with a literal
+  // operand the three-operand and-or instruction cannot be encoded and every expansion falls apart
+  // into an AND and an OR.
+  uint32_t kNib = 0x000f000fu, kExp = 0x43004300u;
+  asm volatile("" : "+v"(kNib), "+v"(kExp));
 
   fetch(t0);
   for (int64_t n0 = t0; n0 < t1; n0 += kAttTile) {
@@ -452,12 +467,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       // ---- products: rows 2r / 2r+1 of A against 16 dimensions of 64 tokens ----
 #pragma unroll
       for (int sg = 0; sg < 4; ++sg) {
-        uint4 a1 = make_uint4(0, 0, 0, 0), a2 = make_uint4(0, 0, 0, 0);
-        if (i < 2 * rep) {
-          const uint4* ap = reinterpret_cast<const uint4*>(abuf + (sg * 8 + i) * kAttARow + kg * 32);
-          a1 = ap[0];
-          a2 = ap[1];
-        }
+        // a lane whose A row holds no head reads the zero piece: no branch, no cleared registers
+        const uint4* ap = reinterpret_cast<const uint4*>(a_row + sg * a_step);
+        const uint4 a1 = ap[0], a2 = ap[1];
 #pragma unroll
         for (int dbl = 0; dbl < 2; ++dbl) {
           const int db = 2 * sg + dbl;
@@ -468,9 +480,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             const uint32_t u = Q::sym ? ((uint32_t)tr[half] ^ 0x88888888u) : (uint32_t)tr[half];
-            const uint4 bb = make_uint4((u & 0x000f000fu) | 0x43004300u, ((u >> 4) & 0x000f000fu) | 0x43004300u,
-                                        ((u >> 8) & 0x000f000fu) | 0x43004300u,
-                                        ((u >> 12) & 0x000f000fu) | 0x43004300u);
+            const uint4 bb = make_uint4(and_or(u, kNib, kExp), and_or(u >> 4, kNib, kExp), and_or(u >> 8, kNib, kExp),
+                                        and_or(u >> 12, kNib, kExp));
             C[hs][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                 __builtin_bit_cast(pikv_bf16x8, half ? a2 : a1), __builtin_bit_cast(pikv_bf16x8, bb), C[hs][db], 0, 0, 0);
           }

@@ -433,4 +433,9 @@ int scores_exchange_launch(const void* k_codes, const void* k_scale, const void*
                            const int64_t* cache_row_base, const int32_t* cache_fill, int n_caches, int64_t max_len,
                            float* escores, float* tile_max, float* tile_sum, float* head_stats, hipStream_t st);
 
+// (x & m) | o.  Plain C on purpose: the value feeds a matrix-core operand, and a
+// result produced inside an inline-asm block is invisible to the compiler's
+// hazard handling between vector and matrix-core instructions.
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) { return (x & m) | o; }
+
 }  // namespace pikv

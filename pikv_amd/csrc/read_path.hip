@@ -109,6 +109,7 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
 
   const int c = blockIdx.y;
   const int64_t tile = blockIdx.x;
+  const int64_t base_row = a.row_base[c];  // asked for together with the fill: one round trip, not two
   const int len = a.fill[c] < a.max_len ? a.fill[c] : a.max_len;
   const int64_t n0 = tile * kTile;
   if (n0 >= len) return;  // uniform for the block
@@ -129,20 +130,6 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   const int kvh = kv0 + kvl;
   const int d0 = (part % lanes_per_head) * EPL;
 
-  // Query slices of the REP heads that read this kv head, and their sums (for the
-  // zero-point term: dot(q, (c - z) * s) = s * (dot(q, c) - z * sum(q))).
-  float qv[REP][EPL];
-  float qsum[REP];
-#pragma unroll
-  for (int r = 0; r < REP; ++r) {
-    const int hq = kvh * a.rep + a.head_off + r;
-    load_as_float<Q_DT, EPL>(a.q, ((int64_t)c * a.n_q_heads + hq) * a.head_dim + d0, qv[r]);
-    float sacc = 0.f;
-#pragma unroll
-    for (int j = 0; j < EPL; ++j) sacc += qv[r][j];
-    qsum[r] = sacc;
-  }
-  const int64_t base_row = a.row_base[c];
   constexpr int UN = 4;  // token steps per batch of loads
   const int batch = tok_per_step * UN;  // tokens of the tile covered by one batch
 
@@ -170,6 +157,25 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
       else t.zr[u] = 0.f;
     }
   };
+  // The first batch goes out before the queries are fetched: the block's first rows and its
+  // query slices then share one memory round trip.
+  Batch ba, bb;
+  load_batch(0, ba);
+
+  // Query slices of the REP heads that read this kv head, and their sums (for the
+  // zero-point term: dot(q, (c - z) * s) = s * (dot(q, c) - z * sum(q))).
+  float qv[REP][EPL];
+  float qsum[REP];
+#pragma unroll
+  for (int r = 0; r < REP; ++r) {
+    const int hq = kvh * a.rep + a.head_off + r;
+    load_as_float<Q_DT, EPL>(a.q, ((int64_t)c * a.n_q_heads + hq) * a.head_dim + d0, qv[r]);
+    float sacc = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) sacc += qv[r][j];
+    qsum[r] = sacc;
+  }
+
   auto mul_batch = [&](int s0, const Batch& t) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
@@ -190,13 +196,11 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
       }
     }
   };
-  Batch ba, bb;
-  load_batch(0, ba);
   for (int s0 = 0; s0 < kTile; s0 += 2 * batch) {
-    load_batch(s0 + batch, bb);
+    if (s0 + batch < kTile) load_batch(s0 + batch, bb);
     mul_batch(s0, ba);
     if (s0 + batch >= kTile) break;
-    load_batch(s0 + 2 * batch, ba);
+    if (s0 + 2 * batch < kTile) load_batch(s0 + 2 * batch, ba);
     mul_batch(s0 + batch, bb);
   }
   __syncthreads();
@@ -281,6 +285,10 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 
   const float zbias = 128.0f - (float)Q::qmin;  // 128 (asymmetric) or 136 (symmetric)
   const int64_t base_row = a.row_base[c];
+  // two nibbles -> two bf16 values 128 + code; both constants held in vector registers so that the
+  // three-operand and-or instruction can be encoded (the empty statement emits no instruction)
+  uint32_t kNib = 0x000f000fu, kExp = 0x43004300u;
+  asm volatile("" : "+v"(kNib), "+v"(kExp));
 
   for (int g = wave; g < a.n_kv_heads; g += 4) {
     // A operands of this kv head: lane (row m = nl, k-slice rg) of group gq holds
@@ -331,9 +339,8 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
         const uint32_t w = Q::sym ? (v[tg][gq] ^ 0x88888888u) : v[tg][gq];
-        const uint4 b = make_uint4((w & 0x000f000fu) | 0x43004300u, ((w >> 4) & 0x000f000fu) | 0x43004300u,
-                                   ((w >> 8) & 0x000f000fu) | 0x43004300u,
-                                   ((w >> 12) & 0x000f000fu) | 0x43004300u);
+        const uint4 b = make_uint4(and_or(w, kNib, kExp), and_or(w >> 4, kNib, kExp), and_or(w >> 8, kNib, kExp),
+                                   and_or(w >> 12, kNib, kExp));
         const pikv_f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
         const pikv_f32x4 pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
             amat[gq], __builtin_bit_cast(pikv_bf16x8, b), zero4, 0, 0, 0);
@@ -377,10 +384,6 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 // the (scale, zero) it loaded itself: no transpose, one epilogue per 16 tokens
 // instead of one per MFMA, and a 3-swap transpose-reduction over the four
 // row-groups leaves row-group r with the finished score of head r.
-// (x & m) | o.  Plain C on purpose: the value feeds a matrix-core operand, and a
-// result produced inside an inline-asm block is invisible to the compiler's
-// hazard handling between vector and matrix-core instructions.
-__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) { return (x & m) | o; }
 
 // Tile statistics and score rows from the staged scores [q head][token in tile], four
 // heads per wavefront pass: lane (rg, nl) owns tokens nl, nl+16, nl+32, nl+48 of head
@@ -718,7 +721,10 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   const int groups_per_row = (a.n_kv_heads * 128) / a.group;
   const int64_t base_row = a.row_base[c];
   const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * 128;
-  const uint32_t kNib = 0x00780078u, kExp = 0x41804180u;  // two nibbles -> two bf16 values 16 + nibble
+  // two nibbles -> two bf16 values 16 + nibble; both constants held in vector registers so that the
+  // three-operand and-or instruction can be encoded (the empty statement emits no instruction)
+  uint32_t kNib = 0x00780078u, kExp = 0x41804180u;
+  asm volatile("" : "+v"(kNib), "+v"(kExp));
 
   // A operands of this wavefront's kv heads: lane (row nl = query head, k-slice rg), k-step
   // (half, b2) covers dimensions d0 = 64*half + 16*rg + 4*b2 .. +3 in the slot order
@@ -1130,8 +1136,9 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
     PIKV_CHECK_LAUNCH();
     return PIKV_OK;
   }
-  // rows wider than one wavefront are split by kv heads over several blocks per tile
-  while (lanes_per_row / a.head_split > 64 && n_kv_heads % (a.head_split * 2) == 0) a.head_split *= 2;
+  // rows wider than 512 bytes are split by kv heads over several blocks per tile: short-lived blocks
+  // of 64 tokens x 512 bytes keep more loads in flight per compute unit than fewer, longer ones
+  while (lanes_per_row / a.head_split > 32 && n_kv_heads % (a.head_split * 2) == 0) a.head_split *= 2;
   const dim3 vgrid((unsigned)n_tiles, (unsigned)n_caches, (unsigned)a.head_split);
   int rc = PIKV_ERR_UNSUPPORTED;
   switch (scheme) {
