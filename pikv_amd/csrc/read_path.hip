@@ -98,7 +98,7 @@ struct ScoreArgs {
   int max_len;      // rows of a cache beyond max_len are not read (a cache may hold more than the caller covers)
   int rep;          // scores_kernel: query heads per kv head, and the first head of every kv group that
   int head_off;     //   this launch serves (it serves REP of them; other ratios take several launches)
-  int head_split;   // scores_kernel: blocks along z share a tile, each owns n_kv_heads/head_split heads
+  int head_split;   // scores_kernel: head_split blocks share a tile, each owns n_kv_heads/head_split heads
 };
 
 template <int SCHEME, int REP, int Q_DT>
@@ -107,8 +107,12 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   constexpr int EPL = Q::epl;
   extern __shared__ float stage[];  // [q head of this block][token in tile]
 
+  // blockIdx.x = tile * head_split + piece: the blocks that share a tile's rows are dispatched side
+  // by side, so that whole rows are in flight at any time and not the same 512-byte piece of every
+  // 4 KB row (which lands on a fraction of the memory channels)
   const int c = blockIdx.y;
-  const int64_t tile = blockIdx.x;
+  const int64_t tile = blockIdx.x / a.head_split;
+  const int piece = blockIdx.x - (int)tile * a.head_split;
   const int64_t base_row = a.row_base[c];  // asked for together with the fill: one round trip, not two
   const int len = a.fill[c] < a.max_len ? a.fill[c] : a.max_len;
   const int64_t n0 = tile * kTile;
@@ -116,7 +120,7 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   // A block owns the kv heads [kv0, kv0 + kv_blk) of its tile: wide rows are split
   // over several blocks so that while one block reduces its tile, others still load.
   const int kv_blk = a.n_kv_heads / a.head_split;
-  const int kv0 = blockIdx.z * kv_blk;
+  const int kv0 = piece * kv_blk;
   const int D = a.n_kv_heads * a.head_dim;
   const int lanes_per_row = D / EPL;                         // lanes of a whole cached row
   const int lanes_per_head = a.head_dim / EPL;               // power of two
@@ -1139,7 +1143,8 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   // rows wider than 512 bytes are split by kv heads over several blocks per tile: short-lived blocks
   // of 64 tokens x 512 bytes keep more loads in flight per compute unit than fewer, longer ones
   while (lanes_per_row / a.head_split > 32 && n_kv_heads % (a.head_split * 2) == 0) a.head_split *= 2;
-  const dim3 vgrid((unsigned)n_tiles, (unsigned)n_caches, (unsigned)a.head_split);
+  if (n_tiles * a.head_split > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+  const dim3 vgrid((unsigned)(n_tiles * a.head_split), (unsigned)n_caches);
   int rc = PIKV_ERR_UNSUPPORTED;
   switch (scheme) {
     case PIKV_Q_I8_SYM: rc = launch_scores<PIKV_Q_I8_SYM>(rep, vgrid, st, q_dtype, a); break;
