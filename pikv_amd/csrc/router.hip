@@ -26,6 +26,7 @@
 namespace pikv {
 
 constexpr int kSlotChunk = 512;  // assignments per block in the slot pass
+constexpr int64_t kSlotSelfPrefixWords = 8192;  // chunks x experts up to which a rank block sums the earlier chunks itself
 constexpr int kRowsTailMinK = 2;  // standalone tail, 33-64 experts: lanes per token instead of per expert from this k on
 
 struct TailParams {
@@ -918,16 +919,38 @@ __global__ __launch_bounds__(64) void slot_scan_kernel(int32_t* __restrict__ ws,
   if (count && lane == 63) count[e] = incl;
 }
 
+// SELF_PREFIX: ws holds the raw per-chunk histograms and every block adds up the chunks before
+// its own by itself (integer sums: the order does not matter); the last block also writes the
+// totals.  For short assignment streams this saves the scan launch, which is all latency there.
+template <bool SELF_PREFIX>
 __global__ __launch_bounds__(256) void slot_rank_kernel(const int32_t* __restrict__ idx, int64_t A,
                                                         int E, int64_t capacity,
                                                         const int32_t* __restrict__ ws,
-                                                        int32_t* __restrict__ slot) {
+                                                        int32_t* __restrict__ slot,
+                                                        int32_t* __restrict__ count) {
   __shared__ int running[64];
   __shared__ int wcnt[4][64];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  if ((int)threadIdx.x < 64)
-    running[threadIdx.x] = ((int)threadIdx.x < E) ? ws[(int64_t)blockIdx.x * E + threadIdx.x] : 0;
+  if constexpr (SELF_PREFIX) {
+    if (threadIdx.x < 64) running[threadIdx.x] = 0;
+    __syncthreads();
+    const int n = (int)blockIdx.x * E;  // words of the earlier chunks, [chunk][expert]
+    for (int p0 = threadIdx.x; p0 < n; p0 += 256 * 8) {
+      int v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = (p0 + u * 256 < n) ? ws[p0 + u * 256] : 0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (v[u]) atomicAdd(&running[(p0 + u * 256) % E], v[u]);
+    }
+    __syncthreads();
+    if (count && blockIdx.x == gridDim.x - 1 && (int)threadIdx.x < E)
+      count[threadIdx.x] = running[threadIdx.x] + ws[n + threadIdx.x];
+  } else {
+    if ((int)threadIdx.x < 64)
+      running[threadIdx.x] = ((int)threadIdx.x < E) ? ws[(int64_t)blockIdx.x * E + threadIdx.x] : 0;
+  }
   const int64_t base = (int64_t)blockIdx.x * kSlotChunk;
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
   for (int step = 0; step < kSlotChunk / 256; ++step) {
@@ -988,9 +1011,14 @@ static int launch_slots(const int32_t* idx, int64_t A, int E, int64_t capacity, 
   const int64_t nb = slot_chunks(A);
   if (nb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
   hipLaunchKernelGGL(slot_hist_kernel, dim3((unsigned)nb), dim3(256), 0, st, idx, A, E, (int32_t*)ws);
-  hipLaunchKernelGGL(slot_scan_kernel, dim3((unsigned)E), dim3(64), 0, st, (int32_t*)ws, nb, E, count);
-  hipLaunchKernelGGL(slot_rank_kernel, dim3((unsigned)nb), dim3(256), 0, st, idx, A, E, capacity,
-                     (const int32_t*)ws, slot);
+  if (nb * E <= kSlotSelfPrefixWords) {
+    hipLaunchKernelGGL((slot_rank_kernel<true>), dim3((unsigned)nb), dim3(256), 0, st, idx, A, E, capacity,
+                       (const int32_t*)ws, slot, count);
+  } else {
+    hipLaunchKernelGGL(slot_scan_kernel, dim3((unsigned)E), dim3(64), 0, st, (int32_t*)ws, nb, E, count);
+    hipLaunchKernelGGL((slot_rank_kernel<false>), dim3((unsigned)nb), dim3(256), 0, st, idx, A, E, capacity,
+                       (const int32_t*)ws, slot, count);
+  }
   PIKV_CHECK_LAUNCH();
   return PIKV_OK;
 }
