@@ -76,7 +76,12 @@ class PiKVKernels:
     # ---- eviction ------------------------------------------------------------------
     def evict_cache(self, keys, values, timestamps, usage_counts, current_time: int,
                     policy: EvictionPolicy, window_threshold: int = 1024,
-                    quest_threshold: float = 0.1):
+                    quest_threshold: float = 0.1, inplace: bool = False):
+        """Returns (keys, values, timestamps, usage_counts, new_size) of the surviving rows, in order.
+        inplace=False (the reference's behaviour, core/single/pikv_kernels.py:386-420): the inputs are
+        left as they are and the survivors are moved inside copies.  inplace=True: the survivors are
+        moved to the front of the caller's own (contiguous) tensors, no copy is made, and the returned
+        tensors are views of their first new_size rows."""
         n, hidden = keys.shape
         dev = keys.device
         if dev.type != "cuda":
@@ -89,8 +94,13 @@ class PiKVKernels:
         new_size = int(keep_index.numel())
         if new_size == 0:
             return keys[:0], values[:0], timestamps[:0], usage_counts[:0], 0
-        planes = [keys.clone().contiguous(), values.clone().contiguous(),
-                  timestamps.clone().contiguous(), usage_counts.clone().contiguous()]
+        if inplace:
+            planes = [keys, values, timestamps, usage_counts]
+            if not all(p.is_contiguous() for p in planes):
+                raise ValueError("inplace=True needs contiguous tensors")
+        else:
+            planes = [keys.clone().contiguous(), values.clone().contiguous(),
+                      timestamps.clone().contiguous(), usage_counts.clone().contiguous()]
         if any((p[0].numel() * p.element_size()) % 4 for p in planes):
             raise ValueError("rows must be a multiple of 4 bytes")
         # one cache spanning all rows: keep_index is already the ascending survivor list

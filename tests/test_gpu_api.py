@@ -352,6 +352,16 @@ def test_kernels_facade(dev):
                         EvictionPolicy.QUEST, quest_threshold=thr)
     valid = score >= thr
     assert out[4] == valid.sum() and np.array_equal(np_of(out[0]), keys[valid])
+    # inputs are left alone by default; inplace=True moves the survivors inside the caller's tensors
+    tens = [torch.from_numpy(a).to(dev) for a in (keys, vals, ts, use)]
+    out = K.evict_cache(*tens, 1000, EvictionPolicy.SLIDING, window_threshold=600)
+    assert np.array_equal(np_of(tens[0]), keys) and np.array_equal(np_of(tens[2]), ts)
+    out = K.evict_cache(*tens, 1000, EvictionPolicy.SLIDING, window_threshold=600, inplace=True)
+    valid = (1000 - ts) <= 600
+    m = int(valid.sum())
+    assert out[4] == m and out[0].data_ptr() == tens[0].data_ptr()
+    assert np.array_equal(np_of(tens[0][:m]), keys[valid]) and np.array_equal(np_of(tens[1][:m]), vals[valid])
+    assert np.array_equal(np_of(tens[2][:m]), ts[valid]) and np.array_equal(np_of(tens[3][:m]), use[valid])
     with pytest.raises(NotImplementedError):
         K.compress_kv(torch.zeros(4, 64, device=dev), torch.zeros(4, 64, device=dev), CompressionMode.LORA)
 

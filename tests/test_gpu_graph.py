@@ -124,3 +124,58 @@ def test_decode_read_replays(dev):
         valid = (torch.arange(N, device=dev).unsqueeze(0) < lens.unsqueeze(1)).reshape(-1)
         assert torch.equal(pool.ts[valid], want_ts[valid]), rep
         assert bool((pool.ts[~valid] == -1.0).all()), rep
+
+
+def test_decode_attend_replays(dev):
+    """The one-call decode read under capture: its workspace is allocated before the capture, and every
+    replay must rebuild the attention output and the H2O accumulators from scribbled memory."""
+    import torch
+    from pikv_amd import ops
+    g = torch.Generator(device=dev).manual_seed(9)
+    B, N, hkv, hq, dh = 3, 4500, 8, 32, 128
+    D = hkv * dh
+    lens = torch.tensor([4500, 2049, 64], dtype=torch.int32, device=dev)
+
+    def filled():
+        pool = ops.CachePool([N] * B, hkv, dh, 32, ops.Q_I4_ASYM, dev, with_v=True)
+        gg = torch.Generator(device=dev).manual_seed(10)
+        ks = torch.randn(B * N, D, generator=gg, device=dev).to(torch.bfloat16)
+        vs = torch.randn(B * N, D, generator=gg, device=dev).to(torch.bfloat16)
+        cid = torch.arange(B, device=dev, dtype=torch.int32).repeat_interleave(N)
+        slot = torch.arange(N, device=dev, dtype=torch.int32).repeat(B)
+        pool.quant_scatter(ks, vs, cid, slot, 1, now=0.0)
+        pool.fill.copy_(lens)
+        return pool
+
+    q = torch.randn(B, hq, dh, generator=g, device=dev).to(torch.bfloat16)
+
+    def read(pool):
+        pool.acc.zero_()
+        return pool.decode_attend(q, hq, now=2.0)
+
+    eager_pool = filled()
+    want_out = read(eager_pool).clone()
+    want_acc, want_ts = eager_pool.acc.clone(), eager_pool.ts.clone()
+
+    pool = filled()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            read(pool)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = read(pool)
+    valid = (torch.arange(N, device=dev).unsqueeze(0) < lens.unsqueeze(1)).reshape(-1)
+    for rep in range(4):
+        pool.acc.fill_(7.0)
+        pool.ts.fill_(-1.0)
+        out.fill_(123.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want_out), rep
+        assert torch.equal(pool.acc, want_acc), rep
+        assert torch.equal(pool.ts[valid], want_ts[valid]), rep
+        assert bool((pool.ts[~valid] == -1.0).all()), rep
