@@ -358,7 +358,19 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
     steps = step0 + steps_per_slice < steps ? step0 + steps_per_slice : steps;
   }
   constexpr int UN = (MT >= 8) ? 1 : (MT + NT > 4) ? 2 : 4;  // registers: 2 wavefronts per SIMD must fit
-  for (int st0 = step0 + wave; st0 < steps; st0 += WAVES * UN) {
+  // Every block starts its walk along the rows at another offset (a hash of the block index, in
+  // whole iterations, wrapping around): with all blocks walking front to back together the whole
+  // chip reads the same 1 KB window of its 8 KB rows at any time, which loads the memory channels
+  // unevenly (config[1]: router call 73.5 -> 70 us).  The pattern matters: offsets that are small
+  // multiples of the block index moved the time both ways (73 ... 90 us), a scattered assignment or
+  // one that changes every 64 blocks gained.  The order of a wavefront's additions, and so the last
+  // bits of a logit, depend on the block a token falls into.
+  const int n_it = (steps - step0 + WAVES * UN - 1) / (WAVES * UN);
+  const int rot = PARTIAL ? 0 : (int)(((blockIdx.x * 0x9E3779B1u) >> 16) % (unsigned)n_it);
+  for (int it = 0; it < n_it; ++it) {
+    int itr = it + rot;
+    if (itr >= n_it) itr -= n_it;
+    const int st0 = step0 + wave + itr * (WAVES * UN);
     uint4 av[UN][MT], bv[UN][NT];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
