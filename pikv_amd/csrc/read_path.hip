@@ -110,9 +110,23 @@ __global__ __launch_bounds__(256) void scores_kernel(ScoreArgs a) {
   // blockIdx.x = tile * head_split + piece: the blocks that share a tile's rows are dispatched side
   // by side, so that whole rows are in flight at any time and not the same 512-byte piece of every
   // 4 KB row (which lands on a fraction of the memory channels)
+  // ... and, inside a run of 8 tiles, block r serves piece r / 8 of tile r % 8: consecutive block
+  // indices go round the 8 XCDs, so the pieces of one tile meet in one L2 and the scale rows and
+  // queries they share are fetched from memory once, not once per piece.  (Any dispatch order gives
+  // the same results; a ragged last run keeps the plain order.)
   const int c = blockIdx.y;
-  const int64_t tile = blockIdx.x / a.head_split;
-  const int piece = blockIdx.x - (int)tile * a.head_split;
+  const unsigned run = 8u * (unsigned)a.head_split;
+  const unsigned run0 = blockIdx.x / run * run;
+  int64_t tile;
+  int piece;
+  if (run0 + run <= gridDim.x) {
+    const unsigned r = blockIdx.x - run0;
+    tile = (int64_t)(run0 / (unsigned)a.head_split) + (r & 7u);
+    piece = (int)(r >> 3);
+  } else {
+    tile = blockIdx.x / a.head_split;
+    piece = blockIdx.x - (int)tile * a.head_split;
+  }
   const int64_t base_row = a.row_base[c];  // asked for together with the fill: one round trip, not two
   const int len = a.fill[c] < a.max_len ? a.fill[c] : a.max_len;
   const int64_t n0 = tile * kTile;
