@@ -28,7 +28,7 @@ typedef __bf16 pikv_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float pikv_f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kAttTile = 64;          // cached tokens per step of the matrix-core form
-constexpr int kAttTokensPerBlock = 2048;
+constexpr int kAttMaxTokensPerBlock = 4096;  // cached tokens one block walks: chosen per call, see attend_tokens_per_block
 
 struct AttendArgs {
   const float* scores;      // [n_caches, n_q_heads, score_stride]
@@ -57,6 +57,7 @@ struct AttendArgs {
   const float* tile_max;
   int64_t n_tiles;
   int head_off;  // attend_mfma_i4_kernel: first query head of every kv group handled by this launch
+  int tokens_per_block;  // cached tokens per block (a multiple of 64): block x covers tokens [x * tokens_per_block, ...)
 };
 
 __device__ __forceinline__ float prob_of(float s, float mx, float rz, bool normalise) {
@@ -72,8 +73,8 @@ __global__ __launch_bounds__(256) void attend_valu_kernel(AttendArgs a) {
   __shared__ float red[256 * EPL];
   const int c = blockIdx.y;
   const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
-  const int64_t t0 = (int64_t)blockIdx.x * kAttTokensPerBlock;
-  const int64_t t1 = (t0 + kAttTokensPerBlock < len) ? t0 + kAttTokensPerBlock : len;
+  const int64_t t0 = (int64_t)blockIdx.x * a.tokens_per_block;
+  const int64_t t1 = (t0 + a.tokens_per_block < len) ? t0 + a.tokens_per_block : len;
   const int rep = a.n_q_heads / a.n_kv_heads;
   const int r0 = blockIdx.z * RP;
   const int D = a.n_kv_heads * a.head_dim;
@@ -215,8 +216,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
   const int c = blockIdx.y;
   const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
-  const int64_t t0 = (int64_t)blockIdx.x * kAttTokensPerBlock;
-  const int64_t t1 = (t0 + kAttTokensPerBlock < len) ? t0 + kAttTokensPerBlock : len;
+  const int64_t t0 = (int64_t)blockIdx.x * a.tokens_per_block;
+  const int64_t t1 = (t0 + a.tokens_per_block < len) ? t0 + a.tokens_per_block : len;
   if (t0 >= t1) {  // nothing cached in this range: the partial is zero
     for (int idx = threadIdx.x; idx < a.n_q_heads * 128; idx += 256)
       a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * 128 + idx] = 0.f;
@@ -571,8 +572,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
   const int c = blockIdx.y;
   const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
-  const int64_t t0 = (int64_t)blockIdx.x * kAttTokensPerBlock;
-  const int64_t t1 = (t0 + kAttTokensPerBlock < len) ? t0 + kAttTokensPerBlock : len;
+  const int64_t t0 = (int64_t)blockIdx.x * a.tokens_per_block;
+  const int64_t t1 = (t0 + a.tokens_per_block < len) ? t0 + a.tokens_per_block : len;
   if (t0 >= t1) {  // nothing cached in this range: the partial is zero
     for (int idx = threadIdx.x; idx < a.n_q_heads * 128; idx += 256)
       a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * 128 + idx] = 0.f;
@@ -836,12 +837,12 @@ static void launch_attend_mfma(int n_kv_heads, dim3 grid, hipStream_t st, const 
 __global__ __launch_bounds__(256) void attend_reduce_kernel(const float* __restrict__ partial,
                                                            const int32_t* __restrict__ fill, int n_caches,
                                                            int n_q_heads, int head_dim, int n_splits,
-                                                           float* __restrict__ out) {
+                                                           int tokens_per_block, float* __restrict__ out) {
   const int64_t per_cache = (int64_t)n_q_heads * head_dim;
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= per_cache * n_caches) return;
   const int c = (int)(idx / per_cache);
-  const int64_t used = ((int64_t)fill[c] + kAttTokensPerBlock - 1) / kAttTokensPerBlock;
+  const int64_t used = ((int64_t)fill[c] + tokens_per_block - 1) / tokens_per_block;
   const int lim = used < n_splits ? (int)used : n_splits;
   float s = 0.f;
   for (int sp = 0; sp < lim; ++sp) s += partial[(int64_t)sp * per_cache * n_caches + idx];
@@ -852,13 +853,34 @@ __global__ __launch_bounds__(256) void attend_reduce_kernel(const float* __restr
 
 using namespace pikv;
 
-static int64_t attend_splits(int64_t max_len) {
-  return (max_len + kAttTokensPerBlock - 1) / kAttTokensPerBlock;
+// Cached tokens per block.  Two blocks are resident per compute unit (512 on the chip): the longest
+// walk that still fills the chip wins (64 caches x 32768 tokens: 4096 tokens per block, one round of
+// 512 blocks, 342 us; 2048: 346 us; 1024: 361 us; 512: 380 us), a small batch is cut finer so that more
+// compute units take part, and a count of blocks that would leave the last round mostly idle is avoided.
+static int attend_tokens_per_block(int n_caches, int64_t max_len) {
+  constexpr int64_t kResident = 512;
+  int best = 256;
+  double best_eff = -1.0;
+  for (int tpb = kAttMaxTokensPerBlock; tpb >= 256; tpb >>= 1) {
+    const int64_t blocks = (int64_t)n_caches * ((max_len + tpb - 1) / tpb);
+    const int64_t rounds = (blocks + kResident - 1) / kResident;
+    const double eff = rounds > 0 ? (double)blocks / (double)(rounds * kResident) : 0.0;
+    if (eff >= 0.85) return tpb;
+    if (eff > best_eff) {  // nothing fills the chip: the finest cut has the most blocks
+      best_eff = eff;
+      best = tpb;
+    }
+  }
+  return best;
+}
+static int64_t attend_splits(int n_caches, int64_t max_len) {
+  const int tpb = attend_tokens_per_block(n_caches, max_len);
+  return (max_len + tpb - 1) / tpb;
 }
 
 extern "C" int64_t pikv_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim, int64_t max_len) {
   if (n_caches < 1 || n_q_heads < 1 || head_dim < 1 || max_len < 0) return 0;
-  return attend_splits(max_len) * n_caches * (int64_t)n_q_heads * head_dim * (int64_t)sizeof(float);
+  return attend_splits(n_caches, max_len) * n_caches * (int64_t)n_q_heads * head_dim * (int64_t)sizeof(float);
 }
 
 extern "C" int pikv_attend_values(const float* scores, const float* head_stats, int64_t score_stride,
@@ -885,7 +907,7 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
   if (lanes_per_row > 256 || 256 % lanes_per_row != 0) return PIKV_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   const int64_t total = (int64_t)n_caches * n_q_heads * head_dim;
-  const int64_t splits = attend_splits(max_len);
+  const int64_t splits = attend_splits(n_caches, max_len);
   if (splits > 65535) return PIKV_ERR_SHAPE;
   if (max_len > 0) {
     if (!workspace) return PIKV_ERR_NULL;
@@ -894,7 +916,7 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
   }
   AttendArgs a{scores, head_stats, v_codes, v_scale, v_zero, cache_row_base, cache_fill,
                (float*)workspace, score_stride, group, n_kv_heads, n_q_heads, head_dim, n_caches,
-               row_acc, row_ts, decay, now, max_len, nullptr, nullptr, 0, 0};
+               row_acc, row_ts, decay, now, max_len, nullptr, nullptr, 0, 0, attend_tokens_per_block(n_caches, max_len)};
   const int rep = n_q_heads / n_kv_heads;
   if (max_len > 0) {
     const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;
@@ -942,7 +964,8 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
     }
   }
   hipLaunchKernelGGL(attend_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                     (const float*)workspace, cache_fill, n_caches, n_q_heads, head_dim, (int)splits, out);
+                     (const float*)workspace, cache_fill, n_caches, n_q_heads, head_dim, (int)splits,
+                     a.tokens_per_block, out);
   PIKV_CHECK_LAUNCH();
   return PIKV_OK;
 }
@@ -1003,7 +1026,7 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
   const bool asym = scheme == PIKV_Q_I4_ASYM;
   const int rep = n_q_heads % n_kv_heads == 0 ? n_q_heads / n_kv_heads : 0;
   const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;
-  const int64_t splits = attend_splits(max_len);
+  const int64_t splits = attend_splits(n_caches, max_len);
   if ((scheme == PIKV_Q_I4_ASYM || scheme == PIKV_Q_I4_SYM) && group == 32 && head_dim == 128 && rep >= 1 &&
       rep <= 8 && hk_ok && q_dtype == PIKV_BF16 && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {
     float* esc = reinterpret_cast<float*>(ws + w.scores);
@@ -1013,7 +1036,7 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
     if (rc == PIKV_OK) {
       AttendArgs a{nullptr, stats, v_codes, v_scale, v_zero, cache_row_base, cache_fill,
                    (float*)partial, 0, group, n_kv_heads, n_q_heads, head_dim, n_caches,
-                   row_acc, row_ts, decay, now, max_len, esc, tmax, w.n_tiles, 0};
+                   row_acc, row_ts, decay, now, max_len, esc, tmax, w.n_tiles, 0, attend_tokens_per_block(n_caches, max_len)};
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       for (int off = 0; off < rep; off += 4) {   // four query heads of every kv group per launch
         a.head_off = off;
@@ -1023,7 +1046,8 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
       }
       const int64_t total = (int64_t)n_caches * n_q_heads * head_dim;
       hipLaunchKernelGGL(attend_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                         (const float*)partial, cache_fill, n_caches, n_q_heads, head_dim, (int)splits, out);
+                         (const float*)partial, cache_fill, n_caches, n_q_heads, head_dim, (int)splits,
+                         a.tokens_per_block, out);
       PIKV_CHECK_LAUNCH();
       return PIKV_OK;
     }

@@ -499,7 +499,7 @@ __device__ __forceinline__ void tile_stats_exchange(const ScoreArgs& a, const fl
   }
 }
 
-constexpr int kGqaTilesPerBlock = 4;   // consecutive 64-token tiles handled by one block
+constexpr int kGqaTilesPerBlock = 2;   // consecutive 64-token tiles handled by one block (4: 1.6 % slower in the one-call decode read; 8 and 16 as 4)
 constexpr int kGqaMaxKvHeads = 16;     // code vectors of one 16-token slice kept in registers
 
 // LDS bytes of scores_mfma_i4_gqa_kernel: score staging, query sums, compact A
