@@ -161,6 +161,59 @@ def test_decode_read_full(dev):
     assert torch.equal(pool.k_codes, k0)
 
 
+def test_decode_attend_full(dev):
+    """Attention output and the one-call decode read at the full decode shape (64 x 32768 tokens,
+    blocks of 4096 cached tokens), through properties: with every cached V row equal the output IS
+    that row whatever the probabilities are (they sum to one over all 32768 tokens); the
+    accumulators grow by one per query head and cache; the one call agrees with the three public
+    steps; two sequences are checked against dequantise + softmax + matmul in float32."""
+    import torch
+    from pikv_amd import ops
+    B, N, hkv, hq, dh = 64, 32768, 8, 32, 128
+    D = hkv * dh
+    g = torch.Generator(device=dev).manual_seed(22)
+    pool = ops.CachePool([N] * B, hkv, dh, 32, ops.Q_I4_ASYM, dev, with_v=True)
+    chunk = 8
+    slot = torch.arange(N, device=dev, dtype=torch.int32).repeat(chunk)
+    for b0 in range(0, B, chunk):
+        ks = torch.randn(chunk * N, D, generator=g, device=dev).to(torch.bfloat16)
+        vs = torch.randn(chunk * N, D, generator=g, device=dev).to(torch.bfloat16)
+        cid = torch.arange(b0, b0 + chunk, device=dev, dtype=torch.int32).repeat_interleave(N)
+        pool.quant_scatter(ks, vs, cid, slot, 1)
+        del ks, vs
+    pool.fill.fill_(N)
+    q = torch.randn(B, hq, dh, generator=g, device=dev).to(torch.bfloat16)
+    pool.acc.zero_()
+    out = pool.decode_attend(q, hq, now=3.0)
+    # H2O: every query head spreads a total of one over the cache
+    assert torch.allclose(pool.acc.view(B, N).sum(1), torch.full((B,), float(hq), device=dev), rtol=1e-3)
+    assert bool((pool.ts == 3.0).all())
+    # the three public steps give the same output
+    s1, tm, tsu = pool.scores(q, hq)
+    pool.h2o_accumulate(s1, tm, tsu, now=3.0, stats_only=True)
+    out3 = pool.attend_values(s1, pool.head_stats)
+    assert float((out - out3).abs().max()) <= 1e-4    # both sum the same summands of RMS 1, in different splits
+    # two sequences against float64 torch on the dequantised rows.  With 32768 nearly uniform
+    # probabilities the output (RMS 0.01) is what is left of summands of RMS 1 after cancellation:
+    # the error is measured against the summands (1e-4 of their RMS; observed 2e-5)
+    for b in (0, B - 1):
+        kh = pool.gather_dequant("k", row0=b * N, n=N).view(N, hkv, dh).repeat_interleave(hq // hkv, dim=1)
+        vh = pool.gather_dequant("v", row0=b * N, n=N).view(N, hkv, dh).repeat_interleave(hq // hkv, dim=1)
+        sc = torch.einsum("hd,nhd->hn", q[b].float(), kh) / math.sqrt(dh)
+        want = torch.einsum("hn,nhd->hd", torch.softmax(sc.double(), dim=1), vh.double()).float()
+        assert float((out[b] - want).abs().max()) <= 1e-4 * float(vh.pow(2).mean().sqrt())
+        del kh, vh, sc
+    # every V row the same: the output is that row, bit patterns of the probabilities do not matter
+    pool.v_codes.copy_(pool.v_codes[:1].expand_as(pool.v_codes))
+    pool.v_scale.copy_(pool.v_scale[:1].expand_as(pool.v_scale))
+    pool.v_zero.copy_(pool.v_zero[:1].expand_as(pool.v_zero))
+    row = pool.gather_dequant("v", row0=0, n=1).view(hkv, dh).repeat_interleave(hq // hkv, dim=0)
+    out_c = pool.decode_attend(q, hq, now=4.0, accumulate=False)
+    assert float((out_c - row.unsqueeze(0)).abs().max()) <= 2e-5 * float(row.abs().max())
+    del pool
+    torch.cuda.empty_cache()
+
+
 def test_wide_routing_full(dev):
     import torch
     from pikv_amd import ops
