@@ -379,9 +379,10 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
         av[u][mt] = (ok && tok_ok[mt]) ? ld16(xrow[mt] + (int64_t)st * 64) : make_uint4(0, 0, 0, 0);
+      // (columns of experts that do not exist are zero in the re-laid weights: not loaded at all)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        bv[u][t] = ok ? ld16(wlane + ((int64_t)st * EP + t * 16) * 64) : make_uint4(0, 0, 0, 0);
+        bv[u][t] = (ok && t * 16 + m < p.E) ? ld16(wlane + ((int64_t)st * EP + t * 16) * 64) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u)
