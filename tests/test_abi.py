@@ -83,8 +83,11 @@ def test_pure_host_entry_points():
                                  1, None, 1, None, None, None, None, None, 0.0, None) == -1
     assert lib.pikv_attend_values(1, None, 64, 1, 1, None, 0, 128, 3, 4, 128, 1, 1, 1, 64, 1.0, 0.0, None, None,
                                   1, 1, 1 << 20, None) == -2
+    # partial outputs, one per block of cached tokens: a small batch is cut into 256-token pieces so that
+    # more compute units take part, a batch that fills the chip walks 4096 tokens per block
     ws = lib.pikv_attend_workspace_bytes(2, 4, 128, 5000)
-    assert ws == 3 * 2 * 4 * 128 * 4
+    assert ws == 20 * 2 * 4 * 128 * 4
+    assert lib.pikv_attend_workspace_bytes(64, 32, 128, 32768) == 8 * 64 * 32 * 128 * 4
     assert lib.pikv_attend_values(1, None, 5000, 1, 1, None, 0, 128, 4, 4, 128, 1, 1, 2, 5000, 1.0, 0.0, None, None,
                                   1, 1, ws - 1, None) == -4
 
