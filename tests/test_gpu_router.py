@@ -102,7 +102,10 @@ def test_router_tail_special_values_both_forms(dev, E):
 
 
 @pytest.mark.parametrize("A,E,cap", [(1, 4, 1), (2047, 8, 100), (2049, 8, 3), (100000, 64, 1500),
-                                      (65536, 8, 10240), (5000, 3, 0)])
+                                      (65536, 8, 10240), (5000, 3, 0),
+                                      # 8192 (chunk, expert) words is where the rank blocks stop summing the
+                                      # earlier chunks themselves: both sides of it, and an odd expert count
+                                      (65536, 64, 900), (66000, 64, 1100), (40000, 5, 7000), (513, 64, 4)])
 def test_capacity_slots_exact(dev, A, E, cap):
     from pikv_amd import ops
     r = rng(A + E)
