@@ -210,3 +210,46 @@ def test_decode_attend_one_call(dev, scheme, group, heads, hq, dh, qdtype, decay
         if L:
             rms = np.sqrt((want_s[c].astype(np.float64) ** 2).mean()) + 1e-12
             assert np.abs(out_short[c] - want_s[c]).max() <= 1e-3 * rms
+
+
+@pytest.mark.parametrize("n_caches,length,scheme,heads,hq", [
+    (64, 4096, O.Q_I4_ASYM, 1, 4),     # 512 blocks of 512 cached tokens
+    (64, 7168, O.Q_I4_SYM, 1, 2),      # 448 blocks of 1024
+    (56, 16384, O.Q_I4_ASYM, 1, 1),    # 448 blocks of 2048
+    (40, 2500, O.Q_I8_SYM, 1, 2),      # 8-bit matrix-core form, 400 blocks of 256, ragged lengths
+])
+def test_attend_block_lengths(dev, n_caches, length, scheme, heads, hq):
+    """The number of cached tokens a block walks is chosen per call from the batch (256 ... 4096, so that
+    the blocks fill the chip); batches that select the longer walks, attention output and H2O
+    accumulators of three caches against float64 on the restatement's dequantised rows, for the
+    separate steps and for the one call."""
+    dh, group = 128, (32 if scheme in (O.Q_I4_ASYM, O.Q_I4_SYM) else 128)
+    r = rng(n_caches + length)
+    lens = [length - (17 * c) % 300 for c in range(n_caches)]
+    lens[0] = length
+    pool, ref = _fill_pool(dev, r, [length] * n_caches, lens, heads, dh, group, scheme)
+    q = O.bf16_round(r.standard_normal((n_caches, hq, dh)).astype(np.float32) * 2)
+    qd = to_dev(q, dev, "bf16")
+    scale_qk = 1.0 / np.sqrt(dh)
+    pool.acc.zero_()
+    out1 = np_of(pool.decode_attend(qd, hq, now=5.0))
+    acc1 = np_of(pool.acc).copy()
+    pool.acc.zero_()
+    scores, tmax, tsum = pool.scores(qd, hq)
+    pool.h2o_accumulate(scores, tmax, tsum, now=5.0, stats_only=True)
+    out3 = np_of(pool.attend_values(scores, pool.head_stats, accumulate=True, now=5.0))
+    acc3 = np_of(pool.acc)
+    for c in (0, n_caches // 2, n_caches - 1):
+        rows = ref.valid_rows(c)[:lens[c]]
+        k_hat = O.dequantize_groups(ref.k_codes[rows], ref.k_scale[rows], ref.k_zero[rows], group)
+        v_hat = O.dequantize_groups(ref.v_codes[rows], ref.v_scale[rows], ref.v_zero[rows], group)
+        s = O.attention_scores(q[c], k_hat, heads, scale_qk)
+        p, imp = O.h2o_importance(s)
+        want = O.attend_values(p, v_hat, heads)
+        rms = np.sqrt((want.astype(np.float64) ** 2).mean()) + 1e-12
+        v_rms = np.sqrt((v_hat.astype(np.float64) ** 2).mean())
+        tol = max(1e-3 * rms, 1e-4 * v_rms)       # a long, nearly uniform sum is what cancellation leaves of its terms
+        assert np.abs(out1[c] - want).max() <= tol, (c, "one call")
+        assert np.abs(out3[c] - want).max() <= tol, (c, "three steps")
+        np.testing.assert_allclose(acc1[rows], imp, rtol=1e-3, atol=1e-6)
+        np.testing.assert_allclose(acc3[rows], imp, rtol=1e-3, atol=1e-6)
