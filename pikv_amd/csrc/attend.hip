@@ -106,7 +106,8 @@ __global__ __launch_bounds__(256) void attend_valu_kernel(AttendArgs a) {
     for (int j = 0; j < EPL; ++j) acc[r][j] = 0.f;
   }
   const int64_t base_row = a.row_base[c];
-  for (int64_t n = t0 + tok_in_step; n < t1; n += tok_per_step) {
+  // (a row's lanes need not divide the block: the threads beyond the last whole row stay idle)
+  for (int64_t n = tok_in_step < tok_per_step ? t0 + tok_in_step : t1; n < t1; n += tok_per_step) {
     const int64_t row = base_row + n;
     const uint4 v = ld16(reinterpret_cast<const char*>(a.codes) + (row * lanes_per_row + part) * 16);
     const int64_t mi = row * groups_per_row + (part * EPL) / a.group;
@@ -193,6 +194,10 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads) {
 
 // HKS = log2(n_kv_heads); at most 4 query heads per kv head.  EXCH: the scores come in the exchange
 // format of pikv_decode_attend (a.escores, a.tile_max) instead of a.scores.
+// Heads narrower than 128 (a.head_dim 64 or 32): the kernel's kv heads are 128-dimension slabs of
+// the cached row, each the stored bytes of hps = 128 / head_dim neighbouring kv heads, and the query
+// heads of a slab are the heads of those kv heads in order.  A query head is multiplied with the
+// whole slab and only the dimensions of its own kv head are written out.
 template <int SCHEME, int HKS, bool EXCH = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i4_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
@@ -219,8 +224,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int64_t t0 = (int64_t)blockIdx.x * a.tokens_per_block;
   const int64_t t1 = (t0 + a.tokens_per_block < len) ? t0 + a.tokens_per_block : len;
   if (t0 >= t1) {  // nothing cached in this range: the partial is zero
-    for (int idx = threadIdx.x; idx < a.n_q_heads * 128; idx += 256)
-      a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * 128 + idx] = 0.f;
+    for (int idx = threadIdx.x; idx < a.n_q_heads * a.head_dim; idx += 256)
+      a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * a.head_dim + idx] = 0.f;
     return;
   }
   // A launch covers up to 4 query heads of every kv group: heads head_off .. head_off+nr-1.
@@ -500,6 +505,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   // spread over the 16 lanes that prepared head r.
   __syncthreads();
   float* zl = reinterpret_cast<float*>(att_lds);  // [wave][head slot][r][sg]
+  const int hps = 128 / a.head_dim;   // kv heads per slab
+  const int rep1 = rep_all / hps;     // query heads per kv head
 #pragma unroll
   for (int hs = 0; hs < NH; ++hs)
 #pragma unroll
@@ -516,10 +523,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     for (int rr = 0; rr < 2; ++rr) {
       const int ro = 2 * kg + rr;  // head (inside the kv group) held by this lane
       if (ro >= rep) continue;
-      float* o = a.partial + (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + ro) * 128;
+      // kv head hh of the slab owns the 16-dimension blocks db with db * hps / 8 == hh
+      const int hh = (a.head_off + ro) / rep1;
+      float* o = a.partial +
+                 (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + ro) * a.head_dim -
+                 hh * a.head_dim;
 #pragma unroll
       for (int db = 0; db < 8; ++db)
-        o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NH + hs) * 4 + ro) * 4 + (db >> 1)];
+        if ((db * hps) >> 3 == hh)
+          o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NH + hs) * 4 + ro) * 4 + (db >> 1)];
     }
   }
 }
@@ -904,7 +916,7 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
   if (D % group != 0) return PIKV_ERR_SHAPE;
   if (!is_pow2(head_dim) || head_dim < epl || group % epl != 0) return PIKV_ERR_UNSUPPORTED;
   const int lanes_per_row = D / epl;
-  if (lanes_per_row > 256 || 256 % lanes_per_row != 0) return PIKV_ERR_UNSUPPORTED;
+  if (lanes_per_row > 256) return PIKV_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   const int64_t total = (int64_t)n_caches * n_q_heads * head_dim;
   const int64_t splits = attend_splits(n_caches, max_len);
@@ -919,16 +931,20 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
                row_acc, row_ts, decay, now, max_len, nullptr, nullptr, 0, 0, attend_tokens_per_block(n_caches, max_len)};
   const int rep = n_q_heads / n_kv_heads;
   if (max_len > 0) {
+    // the matrix-core kernels see 128-dimension slabs of the row: one kv head, or 2 / 4 narrow ones
+    const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
+    const int slabs = hps > 0 ? n_kv_heads / hps : 0;
     const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;
-    if (!eight && group == 32 && head_dim == 128 && rep <= 8 && hk_ok) {
+    const bool slabs_ok = slabs == 1 || slabs == 2 || slabs == 4 || slabs == 8;
+    if (!eight && group == 32 && slabs_ok && rep * hps <= 8) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       // four query heads of every kv group per launch; a second launch (same codes, next four
       // heads) adds its share to the accumulators that the first one has already decayed
-      for (int off = 0; off < rep; off += 4) {
+      for (int off = 0; off < rep * hps; off += 4) {
         a.head_off = off;
         if (off > 0) a.decay = 1.0f;
-        if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(n_kv_heads, grid, st, a);
-        else launch_attend_mfma<PIKV_Q_I4_SYM>(n_kv_heads, grid, st, a);
+        if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(slabs, grid, st, a);
+        else launch_attend_mfma<PIKV_Q_I4_SYM>(slabs, grid, st, a);
       }
     } else if (eight && group % 128 == 0 && head_dim == 128 && rep >= 2 && rep <= 8 && hk_ok) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
@@ -1025,10 +1041,12 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
   // fast form: the 4-bit matrix-core kernels meet in the exchange format
   const bool asym = scheme == PIKV_Q_I4_ASYM;
   const int rep = n_q_heads % n_kv_heads == 0 ? n_q_heads / n_kv_heads : 0;
-  const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;
+  const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);   // 128-dimension slabs: one kv head, or 2 / 4 narrow ones
+  const int slabs = hps > 0 ? n_kv_heads / hps : 0;
+  const bool hk_ok = slabs == 1 || slabs == 2 || slabs == 4 || slabs == 8;
   const int64_t splits = attend_splits(n_caches, max_len);
-  if ((scheme == PIKV_Q_I4_ASYM || scheme == PIKV_Q_I4_SYM) && group == 32 && head_dim == 128 && rep >= 1 &&
-      rep <= 8 && hk_ok && q_dtype == PIKV_BF16 && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {
+  if ((scheme == PIKV_Q_I4_ASYM || scheme == PIKV_Q_I4_SYM) && group == 32 && rep >= 1 &&
+      rep * hps <= 8 && hk_ok && q_dtype == PIKV_BF16 && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {
     float* esc = reinterpret_cast<float*>(ws + w.scores);
     const int rc = scores_exchange_launch(k_codes, k_scale, k_zero, scheme, group, n_kv_heads, n_q_heads, head_dim, q,
                                           q_dtype, scale_qk, cache_row_base, cache_fill, n_caches, max_len, esc, tmax,
@@ -1038,11 +1056,11 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
                    (float*)partial, 0, group, n_kv_heads, n_q_heads, head_dim, n_caches,
                    row_acc, row_ts, decay, now, max_len, esc, tmax, w.n_tiles, 0, attend_tokens_per_block(n_caches, max_len)};
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
-      for (int off = 0; off < rep; off += 4) {   // four query heads of every kv group per launch
+      for (int off = 0; off < rep * hps; off += 4) {   // four query heads of every slab per launch
         a.head_off = off;
         if (off > 0) a.decay = 1.0f;
-        if (asym) launch_attend_mfma<PIKV_Q_I4_ASYM, true>(n_kv_heads, grid, st, a);
-        else launch_attend_mfma<PIKV_Q_I4_SYM, true>(n_kv_heads, grid, st, a);
+        if (asym) launch_attend_mfma<PIKV_Q_I4_ASYM, true>(slabs, grid, st, a);
+        else launch_attend_mfma<PIKV_Q_I4_SYM, true>(slabs, grid, st, a);
       }
       const int64_t total = (int64_t)n_caches * n_q_heads * head_dim;
       hipLaunchKernelGGL(attend_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,

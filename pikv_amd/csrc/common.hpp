@@ -424,6 +424,15 @@ __device__ __forceinline__ float load_meta(const void* plane, int64_t idx) {
 
 __host__ __device__ inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 
+// The matrix-core read kernels work on 128-dimension slabs of a cached row: one kv head of 128
+// dimensions, or the stored bytes of 2 / 4 neighbouring kv heads of 64 / 32.  Heads per slab, or 0
+// when the head width is another one or the heads of a row do not fill whole slabs.
+inline int mfma_heads_per_slab(int head_dim, int n_kv_heads) {
+  if (head_dim != 128 && head_dim != 64 && head_dim != 32) return 0;
+  const int hps = 128 / head_dim;
+  return n_kv_heads % hps == 0 ? hps : 0;
+}
+
 // read_path.hip, for pikv_decode_attend in attend.hip: the 4-bit matrix-core score kernel writing the
 // exchange format (escores [cache][tile][q head][64] floats = exp(score - tile max); tile_max, tile_sum
 // [cache][tile][q head]) followed by the merge of the tile statistics into head_stats [cache][q head][2].

@@ -537,12 +537,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   const int64_t tok0 = tile0 * kTile;
   if (tok0 >= len) return;  // uniform for the block
   const int rep = a.n_q_heads / a.n_kv_heads;  // <= 4 NSET
+  // Heads narrower than 128: a.n_kv_heads counts 128-dimension slabs of the cached row, each the
+  // stored bytes of hps = 128 / head_dim neighbouring kv heads, and the rep query heads of a slab
+  // are the heads of those kv heads, rep1 each, in order.  Query head r of a slab belongs to kv
+  // head r / rep1 of it and its A rows are zero outside that head's gph groups - the products
+  // with the neighbours' codes vanish exactly.
+  const int hps = 128 / a.head_dim;
+  const int rep1 = rep / hps;
+  const int gph = 4 / hps;
   const int lanes_per_row = a.n_kv_heads * 4;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nl = lane & 15;
   const int rg = lane >> 4;
-  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * 128;
+  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * a.head_dim;
   const int64_t base_row = a.row_base[c];
 
   // Code vectors of this wavefront's slice of tile tt (one 16-byte load per kv
@@ -587,14 +595,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
 
   // Prologue: group sums of q, and the non-zero part of the block-diagonal A
   // operands: entry (g, b, gq, r) = q[g*rep + r][32*gq + 8*b + {0,4,1,5,2,6,3,7}].
-  // (set s holds heads g*rep + 4 s + r of kv head g)
+  // (set s holds heads g*rep + 4 s + r of kv head g; with narrow heads gq counts the groups of
+  // the slab and the head's own dimensions start at group (r / rep1) * gph)
   for (int i = threadIdx.x; i < NSET * a.n_kv_heads * 16; i += 256) {
     const int set = i / (a.n_kv_heads * 16), ig = i - set * a.n_kv_heads * 16;
     const int g = ig >> 4, gq = (ig >> 2) & 3, r = (ig & 3) + 4 * set;
     float sacc = 0.f;
-    if (r < rep) {
+    if (r < rep && gq / gph == r / rep1) {
       float h32[32];
-      load_as_float<PIKV_BF16, 32>(qbase, (int64_t)(g * rep + r) * 128 + gq * 32, h32);
+      load_as_float<PIKV_BF16, 32>(qbase, (int64_t)(g * rep + r) * a.head_dim + (gq % gph) * 32, h32);
 #pragma unroll
       for (int k = 0; k < 32; ++k) sacc += h32[k];
     }
@@ -604,7 +613,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     const int set = i / (a.n_kv_heads * 64), ig = i - set * a.n_kv_heads * 64;
     const int g = ig >> 6, b2 = (ig >> 4) & 3, gq = (ig >> 2) & 3, r = (ig & 3) + 4 * set;
     uint4 d = make_uint4(0, 0, 0, 0);
-    if (r < rep) d = ld16(qbase + (int64_t)(g * rep + r) * 128 + gq * 32 + b2 * 8);
+    if (r < rep && gq / gph == r / rep1)
+      d = ld16(qbase + (int64_t)(g * rep + r) * a.head_dim + (gq % gph) * 32 + b2 * 8);
     alds[i] = make_uint4((d.x & 0xffffu) | (d.z << 16), (d.x >> 16) | (d.z & 0xffff0000u),
                          (d.y & 0xffffu) | (d.w << 16), (d.y >> 16) | (d.w & 0xffff0000u));
     if (set == 0) azero[ig] = make_uint4(0, 0, 0, 0);
@@ -1041,12 +1051,15 @@ int scores_exchange_launch(const void* k_codes, const void* k_scale, const void*
                            const int64_t* cache_row_base, const int32_t* cache_fill, int n_caches, int64_t max_len,
                            float* escores, float* tile_max, float* tile_sum, float* head_stats, hipStream_t st) {
   if (scheme != PIKV_Q_I4_ASYM && scheme != PIKV_Q_I4_SYM) return PIKV_ERR_UNSUPPORTED;
-  if (group != 32 || head_dim != 128 || q_dtype != PIKV_BF16 || n_q_heads % n_kv_heads != 0) return PIKV_ERR_UNSUPPORTED;
-  if (n_q_heads / n_kv_heads > 8 || n_q_heads > kMaxQHeads || max_len < 1) return PIKV_ERR_UNSUPPORTED;
+  if (group != 32 || q_dtype != PIKV_BF16 || n_q_heads % n_kv_heads != 0) return PIKV_ERR_UNSUPPORTED;
+  const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
+  if (hps == 0) return PIKV_ERR_UNSUPPORTED;
+  const int slabs = n_kv_heads / hps;   // the kernel's kv heads are 128-dimension slabs of the row
+  if (n_q_heads / slabs > 8 || n_q_heads > kMaxQHeads || max_len < 1) return PIKV_ERR_UNSUPPORTED;
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
   ScoreArgs a{k_codes, k_scale, k_zero, q, cache_row_base, cache_fill, nullptr, tile_max, tile_sum,
-              0, n_tiles, scale_qk, group, n_kv_heads, n_q_heads, head_dim, escores,
-              (int)(max_len < 0x7fffffffLL ? max_len : 0x7fffffffLL), n_q_heads / n_kv_heads, 0, 1};
+              0, n_tiles, scale_qk, group, slabs, n_q_heads, head_dim, escores,
+              (int)(max_len < 0x7fffffffLL ? max_len : 0x7fffffffLL), n_q_heads / slabs, 0, 1};
   const int rc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM, true>(a, n_caches, n_tiles, st)
                                             : launch_gqa<PIKV_Q_I4_SYM, true>(a, n_caches, n_tiles, st);
   if (rc != PIKV_OK) return rc;
@@ -1118,7 +1131,6 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   if (D % group != 0) return PIKV_ERR_SHAPE;
   if (!is_pow2(head_dim) || head_dim < epl || group % epl != 0) return PIKV_ERR_UNSUPPORTED;
   const int lanes_per_row = D / epl;
-  if (lanes_per_row > 256 || 256 % lanes_per_row != 0) return PIKV_ERR_UNSUPPORTED;
   if (n_q_heads > kMaxQHeads) return PIKV_ERR_UNSUPPORTED;
   if (max_len == 0) return PIKV_OK;
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
@@ -1129,22 +1141,31 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   const dim3 grid((unsigned)n_tiles, (unsigned)n_caches);
   hipStream_t st = (hipStream_t)stream;
   const int rep = n_q_heads / n_kv_heads;
-  // grouped 4-bit caches read with bf16 queries go to the matrix-core kernel
-  if (!eight && group == 32 && head_dim == 128 && q_dtype == PIKV_BF16 && rep <= 16) {
+  // grouped 4-bit caches read with bf16 queries go to the matrix-core kernels; heads of 64 or 32
+  // dimensions are served as 128-dimension slabs of two or four neighbouring kv heads
+  const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
+  if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_BF16 && rep * hps <= (hps == 1 ? 16 : 8)) {
     int grc = PIKV_ERR_UNSUPPORTED;
     const size_t mlds = (size_t)n_q_heads * (kTile + 4) * sizeof(float);
-    if (rep <= 8)
-      grc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(a, n_caches, n_tiles, st)
-                                       : launch_gqa<PIKV_Q_I4_SYM>(a, n_caches, n_tiles, st);
-    if (grc == PIKV_OK) {
-      // launched above
-    } else if (scheme == PIKV_Q_I4_ASYM) {
-      hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_ASYM>), grid, dim3(256), mlds, st, a);
-    } else {
-      hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_SYM>), grid, dim3(256), mlds, st, a);
+    if (rep * hps <= 8) {
+      ScoreArgs as = a;
+      as.n_kv_heads = n_kv_heads / hps;
+      grc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(as, n_caches, n_tiles, st)
+                                       : launch_gqa<PIKV_Q_I4_SYM>(as, n_caches, n_tiles, st);
     }
-    PIKV_CHECK_LAUNCH();
-    return PIKV_OK;
+    if (grc == PIKV_OK) {
+      PIKV_CHECK_LAUNCH();
+      return PIKV_OK;
+    }
+    if (hps == 1) {
+      if (scheme == PIKV_Q_I4_ASYM)
+        hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_ASYM>), grid, dim3(256), mlds, st, a);
+      else
+        hipLaunchKernelGGL((scores_mfma_i4_kernel<PIKV_Q_I4_SYM>), grid, dim3(256), mlds, st, a);
+      PIKV_CHECK_LAUNCH();
+      return PIKV_OK;
+    }
+    // narrow heads that do not fit the slab kernel: the vector form below
   }
   // 8-bit caches with per-head (or coarser) scales, several bf16 query heads per kv head
   if (eight && head_dim == 128 && group % 128 == 0 && q_dtype == PIKV_BF16 && rep >= 2 && rep <= 16 &&
@@ -1154,9 +1175,13 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
     PIKV_CHECK_LAUNCH();
     return PIKV_OK;
   }
-  // rows wider than 512 bytes are split by kv heads over several blocks per tile: short-lived blocks
-  // of 64 tokens x 512 bytes keep more loads in flight per compute unit than fewer, longer ones
+  // The blocks of a tile own a power-of-two number of kv heads each (a block's lanes per token must
+  // divide 256): 12 kv heads are three blocks of four.  Rows wider than 512 bytes are split further:
+  // short-lived blocks of 64 tokens x 512 bytes keep more loads in flight per compute unit than
+  // fewer, longer ones.
+  a.head_split = n_kv_heads / (n_kv_heads & -n_kv_heads);
   while (lanes_per_row / a.head_split > 32 && n_kv_heads % (a.head_split * 2) == 0) a.head_split *= 2;
+  if (lanes_per_row / a.head_split > 256) return PIKV_ERR_UNSUPPORTED;
   if (n_tiles * a.head_split > 0x7fffffffLL) return PIKV_ERR_SHAPE;
   const dim3 vgrid((unsigned)(n_tiles * a.head_split), (unsigned)n_caches);
   int rc = PIKV_ERR_UNSUPPORTED;

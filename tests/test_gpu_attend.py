@@ -31,6 +31,14 @@ pytestmark = pytest.mark.gpu
     (O.Q_I8_SYM, 256, 4, 8, 128),      # ... one scale per two heads
     (O.Q_I8_ASYM, 128, 1, 6, 128),     # ... one kv head, 6 q heads
     (O.Q_I4_SYM, 64, 4, 4, 64),
+    (O.Q_I4_ASYM, 32, 4, 8, 64),       # heads of 64: two kv heads share a 128-dimension slab of the matrix-core form
+    (O.Q_I4_SYM, 32, 2, 8, 64),        # ... 4 q heads per kv head: two launches over the one slab
+    (O.Q_I4_ASYM, 32, 16, 16, 64),     # ... eight slabs
+    (O.Q_I4_SYM, 32, 4, 12, 64),       # ... 3 q heads per kv head: the second launch half empty
+    (O.Q_I4_ASYM, 32, 8, 16, 32),      # heads of 32: four kv heads per slab
+    (O.Q_I4_ASYM, 32, 12, 12, 64),     # six slabs: vector form
+    (O.Q_I8_SYM, 64, 12, 12, 64),      # 12 kv heads, vector form: five whole rows per pass of a block
+    (O.Q_I4_SYM, 32, 3, 6, 128),       # 3 kv heads
 ])
 @pytest.mark.parametrize("form", ["stats", "probs"])
 def test_attend_values(dev, scheme, group, heads, hq, dh, form):
@@ -71,6 +79,9 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
     (O.Q_I8_SYM, 128, 4, 8, 128),      # 8-bit matrix-core form
     (O.Q_I8_ASYM, 128, 8, 64, 128),    # ... 64 query heads
     (O.Q_I8_SYM, 64, 4, 8, 64),        # vector form: importance in a kernel of its own
+    (O.Q_I4_ASYM, 32, 4, 8, 64),       # heads of 64 on the matrix-core form
+    (O.Q_I4_SYM, 32, 2, 8, 64),        # ... two launches
+    (O.Q_I4_ASYM, 32, 8, 8, 32),       # heads of 32
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.95])
 def test_attend_accumulates_importance(dev, scheme, group, heads, hq, dh, decay):
@@ -136,6 +147,14 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I8_SYM, 128, 8, 32, 128, "bf16"),   # 8-bit matrix-core kernels
     (O.Q_I8_ASYM, 64, 2, 16, 64, "f32"),     # vector forms
     (O.Q_I4_SYM, 64, 4, 12, 64, "bf16"),
+    (O.Q_I4_ASYM, 32, 4, 8, 64, "bf16"),     # heads of 64: exchange format, two kv heads per 128-dimension slab
+    (O.Q_I4_SYM, 32, 2, 8, 64, "bf16"),      # ... 4 q heads per kv head
+    (O.Q_I4_ASYM, 32, 16, 16, 64, "bf16"),   # ... eight slabs
+    (O.Q_I4_ASYM, 32, 8, 16, 32, "bf16"),    # heads of 32
+    (O.Q_I4_SYM, 32, 12, 12, 64, "bf16"),    # six slabs: the three public steps inside the call
+    (O.Q_I4_ASYM, 32, 2, 6, 64, "f32"),
+    (O.Q_I8_SYM, 64, 12, 12, 64, "f32"),     # 12 kv heads of 64, 8-bit
+    (O.Q_I4_ASYM, 32, 3, 6, 128, "bf16"),    # 3 kv heads
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.9])
 def test_decode_attend_one_call(dev, scheme, group, heads, hq, dh, qdtype, decay):

@@ -59,6 +59,16 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I8_SYM, 256, 4, 64, 128),     # ... 16 q heads per kv head, one scale per two heads
     (O.Q_I8_ASYM, 128, 16, 32, 128),   # ... 16 kv heads (four per wavefront)
     (O.Q_I8_SYM, 1024, 8, 16, 128),    # ... one scale per token
+    (O.Q_I4_ASYM, 32, 4, 8, 64),       # heads of 64: two kv heads share a 128-dimension slab of the matrix-core kernel
+    (O.Q_I4_SYM, 32, 12, 12, 64),      # ... 12 x 64, one q head each (six slabs)
+    (O.Q_I4_ASYM, 32, 2, 8, 64),       # ... 4 q heads per kv head: two sets of A rows
+    (O.Q_I4_SYM, 32, 4, 12, 64),       # ... 3 per kv head
+    (O.Q_I4_ASYM, 32, 8, 16, 32),      # heads of 32: four kv heads per slab
+    (O.Q_I4_ASYM, 32, 3, 3, 64),       # an odd number of narrow heads fills no slab: vector form
+    (O.Q_I4_ASYM, 32, 2, 10, 64),      # 5 q heads per narrow kv head: vector form
+    (O.Q_I8_SYM, 64, 12, 12, 64),      # 12 kv heads: three blocks of four heads per tile
+    (O.Q_I4_ASYM, 32, 3, 6, 128),      # 3 kv heads
+    (O.Q_I8_ASYM, 128, 5, 10, 128),    # 5 kv heads: one block per head
 ])
 @pytest.mark.parametrize("qdtype", ["f32", "bf16"])
 def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
