@@ -11,7 +11,7 @@
 //  * attend_valu_kernel - any scheme / group / head size: one lane owns 16 code
 //    bytes of a token (as in the score kernel), w = p * scale multiplies the codes
 //    into float accumulators, the zero-point term is carried as one extra sum.
-//  * attend_mfma_i4_kernel - 4-bit codes, groups of 32, head_dim 128, bf16-exact:
+//  * attend_mfma_i4_kernel - 4-bit codes, groups of 32, head_dim 128 (64 and 32 as slabs of two / four heads), bf16-exact:
 //    the contraction runs over TOKENS, so the matrix-core B operand needs, per lane,
 //    the codes of 8 tokens for ONE dimension - the transpose of how rows are stored.
 //    The codes of a 64-token tile are staged in LDS as they are and read back with
@@ -537,7 +537,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 }
 
 // ---- matrix-core form, 8-bit codes ------------------------------------------------------
-// Per-head (or coarser) scales, head_dim 128, 2..8 query heads per kv head.  Same plan as
+// Per-head (or coarser) scales, head_dim 128 (64 and 32 as slabs of two / four heads), 2..8 query heads per
+// slab.  Same plan as
 // the 4-bit kernel - contraction over tokens, codes staged in LDS as stored and read back
 // transposed - with two differences.  An 8-bit code is not exact as one bf16, so a stored
 // byte u is fed as its nibbles, u = 16*hi + lo, each exact as 128 + nibble, against two
@@ -555,15 +556,20 @@ constexpr int kAtt8Tile = 32;    // cached tokens per step
 constexpr int kAtt8ARow = 80;    // bytes per staged A row: 32 tokens x bf16 + 16 (bank spread)
 constexpr int kAtt8PRow = 36;    // floats per query head of staged probabilities: 32 tokens + 4
 
-static size_t attend_mfma8_lds_bytes(int n_kv_heads, int n_q_heads) {
-  // codes [32 tokens][n_kv_heads*128 + 8]; scale and zero term [32][n_kv_heads] float; A rows per
+static size_t attend_mfma8_lds_bytes(int n_slabs, int n_q_heads, int hps) {
+  // codes [32 tokens][n_slabs*128 + 8]; scale and zero term [32][n_slabs*hps] float; A rows per
   // wavefront [2 copies][16 rows][kAtt8ARow]; probabilities [query head][kAtt8PRow]
-  return (size_t)kAtt8Tile * (n_kv_heads * 128 + 8) + 2 * (size_t)kAtt8Tile * n_kv_heads * 4 +
+  return (size_t)kAtt8Tile * (n_slabs * 128 + 8) + 2 * (size_t)kAtt8Tile * n_slabs * hps * 4 +
          4 * (size_t)2 * 16 * kAtt8ARow + (size_t)n_q_heads * kAtt8PRow * 4;
 }
 
 // HKS = log2(n_kv_heads) <= 3; 2..8 query heads per kv head, at most 64 query heads.
-template <int SCHEME, int HKS>
+// Heads narrower than 128 (HPS = 128 / head_dim = 2 or 4): the kernel's kv heads are 128-dimension
+// slabs of the cached row, each the stored bytes of HPS neighbouring kv heads with a scale (and
+// zero point) each; the query heads of a slab are the heads of those kv heads in order.  A query
+// head is weighted with its own kv head's scale, multiplied with the whole slab, and only the
+// dimensions of its own kv head are written out.
+template <int SCHEME, int HKS, int HPS = 1>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i8_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 8, "8-bit schemes only");
@@ -572,14 +578,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   constexpr int RS = HK * 128 + 8;   // bytes per token row of staged codes
   constexpr int LPR = HK * 8;        // 16-byte chunks per cached row
   constexpr int NCH = kAtt8Tile * LPR / 256;  // code chunks per thread (= HK)
+  constexpr int HR = HK * HPS;                // stored kv heads = (scale, zero) pairs per token
+  constexpr int NMT = (kAtt8Tile * HR + 255) / 256;  // metadata pairs per thread
   extern __shared__ __align__(16) unsigned char att8_lds[];
   unsigned char* lcodes = att8_lds;
   float* lscale = reinterpret_cast<float*>(att8_lds + kAtt8Tile * RS);
-  float* lzterm = lscale + kAtt8Tile * HK;
+  float* lzterm = lscale + kAtt8Tile * HR;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  unsigned char* abuf = reinterpret_cast<unsigned char*>(lzterm + kAtt8Tile * HK) + wave * (2 * 16 * kAtt8ARow);
-  float* lprob = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(lzterm + kAtt8Tile * HK) +
+  unsigned char* abuf = reinterpret_cast<unsigned char*>(lzterm + kAtt8Tile * HR) + wave * (2 * 16 * kAtt8ARow);
+  float* lprob = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(lzterm + kAtt8Tile * HR) +
                                           4 * (2 * 16 * kAtt8ARow));
 
   const int c = blockIdx.y;
@@ -587,11 +595,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int64_t t0 = (int64_t)blockIdx.x * a.tokens_per_block;
   const int64_t t1 = (t0 + a.tokens_per_block < len) ? t0 + a.tokens_per_block : len;
   if (t0 >= t1) {  // nothing cached in this range: the partial is zero
-    for (int idx = threadIdx.x; idx < a.n_q_heads * 128; idx += 256)
-      a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * 128 + idx] = 0.f;
+    for (int idx = threadIdx.x; idx < a.n_q_heads * a.head_dim; idx += 256)
+      a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * a.head_dim + idx] = 0.f;
     return;
   }
   const int rep = a.n_q_heads / HK;  // 2..8
+  const int rep1 = rep / HPS;        // query heads per stored kv head
   const int groups_per_row = (HK * 128) / a.group;
   // matrix-core roles: A row / B,C column i, token group kg (tokens 8*kg .. 8*kg+7 of the tile)
   const int i = lane & 15;
@@ -600,6 +609,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int r = lane >> 3;
   const int t4 = (lane & 7) * 4;
   const bool row_on = r < rep;
+  const int hh_w = (HPS > 1 && row_on) ? r / rep1 : 0;   // stored kv head, inside its slab, of the head this lane weights
   const bool normalise = a.head_stats != nullptr;
   const int64_t base_row = a.row_base[c];
 
@@ -626,7 +636,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
   // registers that carry the next tile from HBM to LDS
   uint4 pc[NCH];
-  float ps = 0.f, pz = 0.f, pacc = 0.f;
+  float ps[NMT], pz[NMT], pacc = 0.f;
   float psc[8];
   auto fetch = [&](int64_t n0) {
     if (a.row_acc && igrp == 0 && n0 + it < t1) pacc = (a.row_acc + (base_row + n0))[it];  // uniform base + lane
@@ -650,14 +660,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       if (n0 + tok < t1)
         pc[k] = ld16(reinterpret_cast<const char*>(a.codes) + ((base_row + n0 + tok) * LPR + off) * 16);
     }
-    {  // one (token, kv head) metadata pair per thread
-      const int tok = threadIdx.x >> HKS, hd = threadIdx.x & (HK - 1);
-      ps = 0.f;
-      pz = 0.f;
+#pragma unroll
+    for (int k = 0; k < NMT; ++k) {  // (token, stored kv head) metadata pairs
+      const int ch = k * 256 + threadIdx.x;
+      const int tok = ch / HR, hd = ch % HR;
+      ps[k] = 0.f;
+      pz[k] = 0.f;
       if (tok < kAtt8Tile && n0 + tok < t1) {
-        const int64_t mi = (base_row + n0 + tok) * groups_per_row + (hd * 128) / a.group;
-        ps = reinterpret_cast<const float*>(a.scale)[mi];
-        if constexpr (!Q::sym) pz = reinterpret_cast<const float*>(a.zero)[mi];
+        const int64_t mi = (base_row + n0 + tok) * groups_per_row + (hd * (128 / HPS)) / a.group;
+        ps[k] = reinterpret_cast<const float*>(a.scale)[mi];
+        if constexpr (!Q::sym) pz[k] = reinterpret_cast<const float*>(a.zero)[mi];
       }
     }
   };
@@ -679,11 +691,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       dst[0] = make_uint2(pc[k].x, pc[k].y);
       dst[1] = make_uint2(pc[k].z, pc[k].w);
     }
-    {
-      const int tok = threadIdx.x >> HKS, hd = threadIdx.x & (HK - 1);
-      if (tok < kAtt8Tile) {
-        lscale[tok * HK + hd] = ps;
-        lzterm[tok * HK + hd] = -(272.0f + (Q::sym ? 128.0f : pz));
+#pragma unroll
+    for (int k = 0; k < NMT; ++k) {
+      const int ch = k * 256 + threadIdx.x;   // = tok * HR + stored kv head
+      if (ch < kAtt8Tile * HR) {
+        lscale[ch] = ps[k];
+        lzterm[ch] = -(272.0f + (Q::sym ? 128.0f : pz[k]));
       }
     }
   };
@@ -732,7 +745,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       uint32_t hi[4], lo[4], hi16[4], lo16[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float w = p4[j] * lscale[(t4 + j) * HK + g];
+        const float w = p4[j] * lscale[(t4 + j) * HR + g * HPS + hh_w];
         const float wh = __uint_as_float(bf16_hi(w));
         const float wl = __uint_as_float(bf16_hi(w - wh));
         hi[j] = __float_as_uint(wh) >> 16;
@@ -759,21 +772,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       }
       // the offset column of tokens 8*kg .. 8*kg+7 (the same for every dimension), as a bf16
       // high part and - asymmetric schemes, whose zero points are arbitrary floats - a remainder
+      // (narrow heads: the column of the stored kv head that owns the dimensions, rebuilt where the
+      // 16-dimension blocks pass from one kv head to the next)
       uint4 bz = make_uint4(0, 0, 0, 0), bzl = make_uint4(0, 0, 0, 0);
-      {
-        uint32_t zh[8], zlw[8];
-#pragma unroll
-        for (int q8 = 0; q8 < 8; ++q8) {
-          const float zt = lzterm[(kg * 8 + q8) * HK + g];
-          const float zhf = __uint_as_float(bf16_hi(zt));
-          zh[q8] = __float_as_uint(zhf) >> 16;
-          zlw[q8] = bf16_hi(zt - zhf) >> 16;
-        }
-        bz = make_uint4(zh[0] | (zh[1] << 16), zh[2] | (zh[3] << 16), zh[4] | (zh[5] << 16), zh[6] | (zh[7] << 16));
-        bzl = make_uint4(zlw[0] | (zlw[1] << 16), zlw[2] | (zlw[3] << 16), zlw[4] | (zlw[5] << 16), zlw[6] | (zlw[7] << 16));
-      }
 #pragma unroll
       for (int db = 0; db < 8; ++db) {
+        if (db % (8 / HPS) == 0) {
+          uint32_t zh[8], zlw[8];
+#pragma unroll
+          for (int q8 = 0; q8 < 8; ++q8) {
+            const float zt = lzterm[(kg * 8 + q8) * HR + g * HPS + db / (8 / HPS)];
+            const float zhf = __uint_as_float(bf16_hi(zt));
+            zh[q8] = __float_as_uint(zhf) >> 16;
+            zlw[q8] = bf16_hi(zt - zhf) >> 16;
+          }
+          bz = make_uint4(zh[0] | (zh[1] << 16), zh[2] | (zh[3] << 16), zh[4] | (zh[5] << 16), zh[6] | (zh[7] << 16));
+          bzl = make_uint4(zlw[0] | (zlw[1] << 16), zlw[2] | (zlw[3] << 16), zlw[4] | (zlw[5] << 16), zlw[6] | (zlw[7] << 16));
+        }
         // source lane i points at token 8*kg + i/2, dims 16*db + 8*(i%2) .. +7; result lane i
         // holds dimension 16*db + i of tokens 8*kg .. 8*kg+7
         const pikv_i32x2 tr = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
@@ -816,22 +831,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     for (int rr = 0; rr < 2; ++rr) {
       const int ro = 2 * kg + rr;  // head (inside the kv group) held by this lane
       if (ro >= rep) continue;
-      float* o = a.partial + (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep + ro) * 128;
+      const int hh = HPS > 1 ? ro / rep1 : 0;   // stored kv head of the slab that owns this head: blocks db with db * HPS / 8 == hh
+      float* o = a.partial + (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep + ro) * (128 / HPS) -
+                 hh * (128 / HPS);
 #pragma unroll
-      for (int db = 0; db < 8; ++db) o[db * 16 + i] = C[hs][db][2 * rr] + C[hs][db][2 * rr + 1];
+      for (int db = 0; db < 8; ++db)
+        if (HPS == 1 || db / (8 / HPS) == hh) o[db * 16 + i] = C[hs][db][2 * rr] + C[hs][db][2 * rr + 1];
     }
   }
 }
 
-template <int SCHEME>
-static void launch_attend_mfma8(int n_kv_heads, dim3 grid, hipStream_t st, const AttendArgs& a) {
-  const size_t lds = attend_mfma8_lds_bytes(n_kv_heads, a.n_q_heads);
-  switch (n_kv_heads) {
-    case 1: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 0>), grid, dim3(256), lds, st, a); break;
-    case 2: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 1>), grid, dim3(256), lds, st, a); break;
-    case 4: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 2>), grid, dim3(256), lds, st, a); break;
-    default: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 3>), grid, dim3(256), lds, st, a); break;
+template <int SCHEME, int HPS>
+static void launch_attend_mfma8_slabs(int n_slabs, dim3 grid, hipStream_t st, const AttendArgs& a) {
+  const size_t lds = attend_mfma8_lds_bytes(n_slabs, a.n_q_heads, HPS);
+  switch (n_slabs) {
+    case 1: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 0, HPS>), grid, dim3(256), lds, st, a); break;
+    case 2: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 1, HPS>), grid, dim3(256), lds, st, a); break;
+    case 4: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 2, HPS>), grid, dim3(256), lds, st, a); break;
+    default: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 3, HPS>), grid, dim3(256), lds, st, a); break;
   }
+}
+template <int SCHEME>
+static void launch_attend_mfma8(int n_slabs, int hps, dim3 grid, hipStream_t st, const AttendArgs& a) {
+  if (hps == 1) launch_attend_mfma8_slabs<SCHEME, 1>(n_slabs, grid, st, a);
+  else if (hps == 2) launch_attend_mfma8_slabs<SCHEME, 2>(n_slabs, grid, st, a);
+  else launch_attend_mfma8_slabs<SCHEME, 4>(n_slabs, grid, st, a);
 }
 
 template <int SCHEME, bool EXCH = false>
@@ -934,7 +958,6 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
     // the matrix-core kernels see 128-dimension slabs of the row: one kv head, or 2 / 4 narrow ones
     const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
     const int slabs = hps > 0 ? n_kv_heads / hps : 0;
-    const bool hk_ok = n_kv_heads == 1 || n_kv_heads == 2 || n_kv_heads == 4 || n_kv_heads == 8;
     const bool slabs_ok = slabs == 1 || slabs == 2 || slabs == 4 || slabs == 8;
     if (!eight && group == 32 && slabs_ok && rep * hps <= 8) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
@@ -946,10 +969,10 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
         if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(slabs, grid, st, a);
         else launch_attend_mfma<PIKV_Q_I4_SYM>(slabs, grid, st, a);
       }
-    } else if (eight && group % 128 == 0 && head_dim == 128 && rep >= 2 && rep <= 8 && hk_ok) {
+    } else if (eight && slabs_ok && group % head_dim == 0 && rep * hps >= 2 && rep * hps <= 8) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
-      if (scheme == PIKV_Q_I8_SYM) launch_attend_mfma8<PIKV_Q_I8_SYM>(n_kv_heads, grid, st, a);
-      else launch_attend_mfma8<PIKV_Q_I8_ASYM>(n_kv_heads, grid, st, a);
+      if (scheme == PIKV_Q_I8_SYM) launch_attend_mfma8<PIKV_Q_I8_SYM>(slabs, hps, grid, st, a);
+      else launch_attend_mfma8<PIKV_Q_I8_ASYM>(slabs, hps, grid, st, a);
     } else {
       if (row_acc || row_ts)
         hipLaunchKernelGGL(attend_importance_kernel, dim3((unsigned)((max_len + 255) / 256), (unsigned)n_caches),

@@ -710,7 +710,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
 }
 
 // ---- 8-bit scores on the matrix cores ------------------------------------------------
-// Per-head (or coarser) scales, head_dim 128, bf16 queries, up to 16 query heads per kv
+// Per-head (or coarser) scales, head_dim 128 (64 and 32 as slabs of two / four heads), bf16 queries, up to 16 query heads per kv
 // head.  The vector form above is instruction-bound as soon as several query heads share
 // a kv head (measured at 64 x 32768 cached tokens, 8 kv heads: 793 us for 4 heads per kv
 // head, 2143 us for 8, where HBM allows about 440 us).  An 8-bit code does not fit one
@@ -729,7 +729,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
 // halves of its token's head row, so one load instruction fetches whole 128-byte lines.
 constexpr int kI8TilesPerBlock = 4;
 
-template <int SCHEME, int NHW>  // NHW = kv heads per wavefront: ceil(n_kv_heads / 4), 1, 2 or 4
+// Heads narrower than 128 (HPS = 128 / head_dim = 2 or 4): a.n_kv_heads counts 128-dimension slabs of
+// the cached row, each the stored bytes of HPS neighbouring kv heads; the rep query heads of a slab
+// are the heads of those kv heads, rep / HPS each, in order.  A query head's A rows are zero outside
+// its own kv head's dimensions, and its scores take that kv head's scale and zero point.
+template <int SCHEME, int NHW, int HPS = 1>  // NHW = kv heads per wavefront: ceil(n_kv_heads / 4), 1, 2 or 4
 __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 8, "8-bit schemes only");
@@ -748,7 +752,12 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   const int64_t row_bytes = (int64_t)a.n_kv_heads * 128;
   const int groups_per_row = (a.n_kv_heads * 128) / a.group;
   const int64_t base_row = a.row_base[c];
-  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * 128;
+  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * a.head_dim;
+  const int rep1 = rep / HPS;        // query heads per kv head
+  const int hh_a = nl / rep1;        // kv head (inside the slab) of the query head in A row nl
+  int hh_c[4];                       // ... of the query heads in this lane's four C rows
+#pragma unroll
+  for (int qq = 0; qq < 4; ++qq) hh_c[qq] = (4 * rg + qq) / rep1 < HPS ? (4 * rg + qq) / rep1 : HPS - 1;
   // two nibbles -> two bf16 values 16 + nibble; both constants held in vector registers so that the
   // three-operand and-or instruction can be encoded (the empty statement emits no instruction)
   uint32_t kNib = 0x00780078u, kExp = 0x41804180u;
@@ -766,7 +775,9 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       uint2 qd = make_uint2(0, 0);
-      if (on) qd = *reinterpret_cast<const uint2*>(qbase + (int64_t)(g * rep + nl) * 128 + 64 * (ks >> 2) + 16 * rg + 4 * (ks & 3));
+      const int ds = 64 * (ks >> 2) + 16 * rg + 4 * (ks & 3);   // dimension inside the slab
+      if (on && (HPS == 1 || ds / a.head_dim == hh_a))
+        qd = *reinterpret_cast<const uint2*>(qbase + (int64_t)(g * rep + nl) * a.head_dim + (ds - hh_a * a.head_dim));
       // bf16 x 16: through float, exact (zero stays zero)
       auto x16 = [](uint32_t h) { return __float_as_uint(__uint_as_float(h << 16) * 16.0f) >> 16; };
       const uint32_t q0 = qd.x & 0xffffu, q1 = qd.x >> 16, q2 = qd.y & 0xffffu, q3 = qd.y >> 16;
@@ -793,22 +804,25 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
       if (g >= a.n_kv_heads) continue;  // uniform
       // the four 16-token slices of the tile: two 16-byte halves and the metadata of each
       uint4 cv[4][2];
-      float sc[4], zr[4];
+      float sc[4][HPS], zr[4][HPS];
       bool ok[4];
 #pragma unroll
       for (int sl = 0; sl < 4; ++sl) {
         const int64_t n = n0 + 16 * sl + nl;
         ok[sl] = n < len;
         cv[sl][0] = cv[sl][1] = make_uint4(0, 0, 0, 0);
-        sc[sl] = 0.f;
-        zr[sl] = 0.f;
+#pragma unroll
+        for (int k = 0; k < HPS; ++k) sc[sl][k] = zr[sl][k] = 0.f;
         if (ok[sl]) {
           const char* rowp = reinterpret_cast<const char*>(a.codes) + (base_row + n) * row_bytes + g * 128 + 16 * rg;
           cv[sl][0] = ld16(rowp);
           cv[sl][1] = ld16(rowp + 64);
-          const int64_t mi = (base_row + n) * groups_per_row + (g * 128) / a.group;
-          sc[sl] = reinterpret_cast<const float*>(a.scale)[mi];
-          if constexpr (!Q::sym) zr[sl] = reinterpret_cast<const float*>(a.zero)[mi];
+#pragma unroll
+          for (int k = 0; k < HPS; ++k) {   // one (scale, zero) per kv head of the slab
+            const int64_t mi = (base_row + n) * groups_per_row + (g * 128 + k * (128 / HPS)) / a.group;
+            sc[sl][k] = reinterpret_cast<const float*>(a.scale)[mi];
+            if constexpr (!Q::sym) zr[sl][k] = reinterpret_cast<const float*>(a.zero)[mi];
+          }
         }
       }
 #pragma unroll
@@ -826,12 +840,18 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
                                                          __builtin_bit_cast(pikv_bf16x8, bb), pc, 0, 0, 0);
           }
         }
-        const float zz = 272.0f + (Q::sym ? 128.0f : zr[sl]);
 #pragma unroll
         for (int qq = 0; qq < 4; ++qq) {
           const int r = 4 * rg + qq;
           if (r < rep) {
-            const float score = sc[sl] * fmaf(-zz, qs[hs][qq], pc[qq]) * a.scale_qk;
+            float scl = sc[sl][0], zrl = zr[sl][0];
+#pragma unroll
+            for (int k = 1; k < HPS; ++k) {
+              scl = hh_c[qq] == k ? sc[sl][k] : scl;
+              zrl = hh_c[qq] == k ? zr[sl][k] : zrl;
+            }
+            const float zz = 272.0f + (Q::sym ? 128.0f : zrl);
+            const float score = scl * fmaf(-zz, qs[hs][qq], pc[qq]) * a.scale_qk;
             stage[(g * rep + r) * kTile + 16 * sl + nl] = ok[sl] ? score : -__builtin_inff();
           }
         }
@@ -843,16 +863,16 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   }
 }
 
-template <int SCHEME>
+template <int SCHEME, int HPS = 1>
 static int launch_i8_mfma(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
   const size_t lds = (size_t)a.n_q_heads * kTile * sizeof(float);
   const dim3 grid((unsigned)((n_tiles + kI8TilesPerBlock - 1) / kI8TilesPerBlock), (unsigned)n_caches);
   if (a.n_kv_heads <= 4)
-    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 1>), grid, dim3(256), lds, st, a);
+    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 1, HPS>), grid, dim3(256), lds, st, a);
   else if (a.n_kv_heads <= 8)
-    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 2>), grid, dim3(256), lds, st, a);
+    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 2, HPS>), grid, dim3(256), lds, st, a);
   else
-    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 4>), grid, dim3(256), lds, st, a);
+    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 4, HPS>), grid, dim3(256), lds, st, a);
   return PIKV_OK;
 }
 
@@ -1168,10 +1188,15 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
     // narrow heads that do not fit the slab kernel: the vector form below
   }
   // 8-bit caches with per-head (or coarser) scales, several bf16 query heads per kv head
-  if (eight && head_dim == 128 && group % 128 == 0 && q_dtype == PIKV_BF16 && rep >= 2 && rep <= 16 &&
-      n_kv_heads <= 16) {
-    if (scheme == PIKV_Q_I8_SYM) launch_i8_mfma<PIKV_Q_I8_SYM>(a, n_caches, n_tiles, st);
-    else launch_i8_mfma<PIKV_Q_I8_ASYM>(a, n_caches, n_tiles, st);
+  // (heads of 64 or 32 dimensions as 128-dimension slabs of two or four neighbouring kv heads)
+  if (eight && hps > 0 && group % head_dim == 0 && q_dtype == PIKV_BF16 && rep >= 2 && rep * hps <= 16 &&
+      n_kv_heads / hps <= 16) {
+    ScoreArgs as = a;
+    as.n_kv_heads = n_kv_heads / hps;
+    const bool sym = scheme == PIKV_Q_I8_SYM;
+    if (hps == 1) sym ? launch_i8_mfma<PIKV_Q_I8_SYM>(as, n_caches, n_tiles, st) : launch_i8_mfma<PIKV_Q_I8_ASYM>(as, n_caches, n_tiles, st);
+    else if (hps == 2) sym ? launch_i8_mfma<PIKV_Q_I8_SYM, 2>(as, n_caches, n_tiles, st) : launch_i8_mfma<PIKV_Q_I8_ASYM, 2>(as, n_caches, n_tiles, st);
+    else sym ? launch_i8_mfma<PIKV_Q_I8_SYM, 4>(as, n_caches, n_tiles, st) : launch_i8_mfma<PIKV_Q_I8_ASYM, 4>(as, n_caches, n_tiles, st);
     PIKV_CHECK_LAUNCH();
     return PIKV_OK;
   }

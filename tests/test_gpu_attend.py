@@ -37,6 +37,11 @@ pytestmark = pytest.mark.gpu
     (O.Q_I4_SYM, 32, 4, 12, 64),       # ... 3 q heads per kv head: the second launch half empty
     (O.Q_I4_ASYM, 32, 8, 16, 32),      # heads of 32: four kv heads per slab
     (O.Q_I4_ASYM, 32, 12, 12, 64),     # six slabs: vector form
+    (O.Q_I8_SYM, 64, 8, 16, 64),       # 8-bit heads of 64 on the matrix-core form: a scale per kv head, two per slab
+    (O.Q_I8_ASYM, 64, 4, 16, 64),      # ... 4 q heads per kv head: all 16 operand rows, zero points per kv head
+    (O.Q_I8_SYM, 128, 4, 8, 64),       # ... one scale per slab
+    (O.Q_I8_ASYM, 32, 8, 16, 32),      # ... heads of 32
+    (O.Q_I8_ASYM, 64, 16, 32, 64),     # ... eight slabs
     (O.Q_I8_SYM, 64, 12, 12, 64),      # 12 kv heads, vector form: five whole rows per pass of a block
     (O.Q_I4_SYM, 32, 3, 6, 128),       # 3 kv heads
 ])
@@ -82,6 +87,7 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
     (O.Q_I4_ASYM, 32, 4, 8, 64),       # heads of 64 on the matrix-core form
     (O.Q_I4_SYM, 32, 2, 8, 64),        # ... two launches
     (O.Q_I4_ASYM, 32, 8, 8, 32),       # heads of 32
+    (O.Q_I8_ASYM, 64, 8, 16, 64),      # 8-bit heads of 64 on the matrix-core form
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.95])
 def test_attend_accumulates_importance(dev, scheme, group, heads, hq, dh, decay):
@@ -153,6 +159,7 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I4_ASYM, 32, 8, 16, 32, "bf16"),    # heads of 32
     (O.Q_I4_SYM, 32, 12, 12, 64, "bf16"),    # six slabs: the three public steps inside the call
     (O.Q_I4_ASYM, 32, 2, 6, 64, "f32"),
+    (O.Q_I8_ASYM, 64, 8, 16, 64, "bf16"),    # 8-bit heads of 64 on the matrix-core kernels
     (O.Q_I8_SYM, 64, 12, 12, 64, "f32"),     # 12 kv heads of 64, 8-bit
     (O.Q_I4_ASYM, 32, 3, 6, 128, "bf16"),    # 3 kv heads
 ])

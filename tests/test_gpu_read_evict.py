@@ -66,6 +66,11 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I4_ASYM, 32, 8, 16, 32),      # heads of 32: four kv heads per slab
     (O.Q_I4_ASYM, 32, 3, 3, 64),       # an odd number of narrow heads fills no slab: vector form
     (O.Q_I4_ASYM, 32, 2, 10, 64),      # 5 q heads per narrow kv head: vector form
+    (O.Q_I8_SYM, 64, 8, 16, 64),       # 8-bit heads of 64 on the matrix-core kernel: a scale per kv head, two per slab
+    (O.Q_I8_ASYM, 64, 4, 16, 64),      # ... 4 q heads per kv head, zero points
+    (O.Q_I8_SYM, 128, 4, 8, 64),       # ... one scale per slab
+    (O.Q_I8_ASYM, 32, 8, 16, 32),      # ... heads of 32
+    (O.Q_I8_SYM, 64, 32, 64, 64),      # ... 16 slabs (four per wavefront)
     (O.Q_I8_SYM, 64, 12, 12, 64),      # 12 kv heads: three blocks of four heads per tile
     (O.Q_I4_ASYM, 32, 3, 6, 128),      # 3 kv heads
     (O.Q_I8_ASYM, 128, 5, 10, 128),    # 5 kv heads: one block per head
