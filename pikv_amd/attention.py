@@ -245,10 +245,9 @@ class PiKVAttention(nn.Module):
         """q [B, heads, head_dim] against the whole compressed cache of each sequence."""
         pool = self.pool
         qq = q.to(torch.bfloat16) if q.dtype == torch.bfloat16 else q.float()
-        scores, tmax, tsum = pool.scores(qq.contiguous(), self.num_heads, 1.0 / math.sqrt(self.head_dim))
-        pool.h2o_accumulate(scores, tmax, tsum, now=float(self.clock), stats_only=True)
-        # probabilities x V rows and the H2O importance of the same probabilities in one pass
-        return pool.attend_values(scores, pool.head_stats, accumulate=True, now=float(self.clock))
+        # scores, softmax, probabilities x V rows and the H2O importance of the same probabilities: one call
+        return pool.decode_attend(qq.contiguous(), self.num_heads, now=float(self.clock),
+                                  scale_qk=1.0 / math.sqrt(self.head_dim))
 
     def _dense_attention(self, q, k, v, attention_mask, causal_mask, past=None):
         """core/single/pikv_attention.py:104-191 over [cached rows ; rows of this call]

@@ -19,7 +19,9 @@ def _f64(t):
     return t.detach().double().cpu().numpy()
 
 
-@pytest.mark.parametrize("quant,group,heads,kv_heads,dh", [("int4", 32, 8, 2, 128), ("int8", 64, 4, 4, 64)])
+@pytest.mark.parametrize("quant,group,heads,kv_heads,dh", [("int4", 32, 8, 2, 128), ("int8", 64, 4, 4, 64),
+                                                         ("int4", 32, 12, 12, 64),    # the head geometry of GPT-2 small
+                                                         ("int8", 64, 12, 12, 64)])
 def test_decode_step_over_quantised_cache(dev, quant, group, heads, kv_heads, dh):
     import torch
     from pikv_amd.attention import PiKVAttention
