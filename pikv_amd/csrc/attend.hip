@@ -192,17 +192,18 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads) {
          (size_t)4 * n_kv_heads * kAttPRow * 4 + 32;
 }
 
-// HKS = log2(n_kv_heads); at most 4 query heads per kv head.  EXCH: the scores come in the exchange
+// HK = n_kv_heads (1..8); at most 4 query heads per kv head.  EXCH: the scores come in the exchange
 // format of pikv_decode_attend (a.escores, a.tile_max) instead of a.scores.
 // Heads narrower than 128 (a.head_dim 64 or 32): the kernel's kv heads are 128-dimension slabs of
 // the cached row, each the stored bytes of hps = 128 / head_dim neighbouring kv heads, and the query
 // heads of a slab are the heads of those kv heads in order.  A query head is multiplied with the
 // whole slab and only the dimensions of its own kv head are written out.
-template <int SCHEME, int HKS, bool EXCH = false>
+// NARROW selects that form at compile time: the kernel for heads of 128 carries none of it.
+template <int SCHEME, int HK, bool EXCH = false, bool NARROW = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i4_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
-  constexpr int HK = 1 << HKS;
+  static_assert(HK >= 1 && HK <= 8, "1 to 8 kv heads");
   constexpr int NH = (HK + 3) / 4;        // kv heads per wavefront
   constexpr int RS = HK * 64 + 8;         // bytes per token row of staged codes
   constexpr int LPR = HK * 4;             // 16-byte chunks per cached row
@@ -224,8 +225,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int64_t t0 = (int64_t)blockIdx.x * a.tokens_per_block;
   const int64_t t1 = (t0 + a.tokens_per_block < len) ? t0 + a.tokens_per_block : len;
   if (t0 >= t1) {  // nothing cached in this range: the partial is zero
-    for (int idx = threadIdx.x; idx < a.n_q_heads * a.head_dim; idx += 256)
-      a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * a.head_dim + idx] = 0.f;
+    const int hd = NARROW ? a.head_dim : 128;
+    for (int idx = threadIdx.x; idx < a.n_q_heads * hd; idx += 256)
+      a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * hd + idx] = 0.f;
     return;
   }
   // A launch covers up to 4 query heads of every kv group: heads head_off .. head_off+nr-1.
@@ -355,7 +357,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
       const int ch = k * 256 + threadIdx.x;
-      const int tok = ch >> (HKS + 2), off = ch & (LPR - 1);
+      const int tok = ch / LPR, off = ch % LPR;
       if (tok < kAttTile) {
         uint2* dst = reinterpret_cast<uint2*>(lcodes + tok * RS + off * 16);  // rows are 8-byte aligned only
         dst[0] = make_uint2(pc[k].x, pc[k].y);
@@ -365,7 +367,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 #pragma unroll
     for (int k = 0; k < NMC; ++k) {
       const int ch = k * 256 + threadIdx.x;
-      const int tok = ch >> HKS, hd = ch & (HK - 1);
+      const int tok = ch / HK, hd = ch % HK;
       if (tok < kAttTile) {
         const int mo = att_meta_off(tok, hd, HK);
         *reinterpret_cast<float4*>(lscale + mo) =
@@ -505,8 +507,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   // spread over the 16 lanes that prepared head r.
   __syncthreads();
   float* zl = reinterpret_cast<float*>(att_lds);  // [wave][head slot][r][sg]
-  const int hps = 128 / a.head_dim;   // kv heads per slab
-  const int rep1 = rep_all / hps;     // query heads per kv head
+  const int hps = NARROW ? 128 / a.head_dim : 1;   // kv heads per slab
+  const int rep1 = rep_all / hps;                  // query heads per kv head
 #pragma unroll
   for (int hs = 0; hs < NH; ++hs)
 #pragma unroll
@@ -523,15 +525,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     for (int rr = 0; rr < 2; ++rr) {
       const int ro = 2 * kg + rr;  // head (inside the kv group) held by this lane
       if (ro >= rep) continue;
-      // kv head hh of the slab owns the 16-dimension blocks db with db * hps / 8 == hh
-      const int hh = (a.head_off + ro) / rep1;
-      float* o = a.partial +
-                 (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + ro) * a.head_dim -
-                 hh * a.head_dim;
+      const int64_t ohead = ((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + ro;
+      if constexpr (!NARROW) {
+        float* o = a.partial + ohead * 128;
 #pragma unroll
-      for (int db = 0; db < 8; ++db)
-        if ((db * hps) >> 3 == hh)
+        for (int db = 0; db < 8; ++db)
           o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NH + hs) * 4 + ro) * 4 + (db >> 1)];
+      } else {
+        // kv head hh of the slab owns the 16-dimension blocks db with db * hps / 8 == hh
+        const int hh = (a.head_off + ro) / rep1;
+        float* o = a.partial + ohead * a.head_dim - hh * a.head_dim;
+#pragma unroll
+        for (int db = 0; db < 8; ++db)
+          if ((db * hps) >> 3 == hh)
+            o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NH + hs) * 4 + ro) * 4 + (db >> 1)];
+      }
     }
   }
 }
@@ -563,17 +571,17 @@ static size_t attend_mfma8_lds_bytes(int n_slabs, int n_q_heads, int hps) {
          4 * (size_t)2 * 16 * kAtt8ARow + (size_t)n_q_heads * kAtt8PRow * 4;
 }
 
-// HKS = log2(n_kv_heads) <= 3; 2..8 query heads per kv head, at most 64 query heads.
+// HK = n_kv_heads (1..8); 2..8 query heads per kv head, at most 64 query heads.
 // Heads narrower than 128 (HPS = 128 / head_dim = 2 or 4): the kernel's kv heads are 128-dimension
 // slabs of the cached row, each the stored bytes of HPS neighbouring kv heads with a scale (and
 // zero point) each; the query heads of a slab are the heads of those kv heads in order.  A query
 // head is weighted with its own kv head's scale, multiplied with the whole slab, and only the
 // dimensions of its own kv head are written out.
-template <int SCHEME, int HKS, int HPS = 1>
+template <int SCHEME, int HK, int HPS = 1>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i8_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 8, "8-bit schemes only");
-  constexpr int HK = 1 << HKS;
+  static_assert(HK >= 1 && HK <= 8, "1 to 8 kv heads");
   constexpr int NH = (HK + 3) / 4;   // kv heads per wavefront
   constexpr int RS = HK * 128 + 8;   // bytes per token row of staged codes
   constexpr int LPR = HK * 8;        // 16-byte chunks per cached row
@@ -655,7 +663,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
       const int ch = k * 256 + threadIdx.x;
-      const int tok = ch >> (HKS + 3), off = ch & (LPR - 1);
+      const int tok = ch / LPR, off = ch % LPR;
       pc[k] = make_uint4(0, 0, 0, 0);
       if (n0 + tok < t1)
         pc[k] = ld16(reinterpret_cast<const char*>(a.codes) + ((base_row + n0 + tok) * LPR + off) * 16);
@@ -686,7 +694,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
       const int ch = k * 256 + threadIdx.x;
-      const int tok = ch >> (HKS + 3), off = ch & (LPR - 1);
+      const int tok = ch / LPR, off = ch % LPR;
       uint2* dst = reinterpret_cast<uint2*>(lcodes + tok * RS + off * 16);  // rows are 8-byte aligned only
       dst[0] = make_uint2(pc[k].x, pc[k].y);
       dst[1] = make_uint2(pc[k].z, pc[k].w);
@@ -845,10 +853,14 @@ template <int SCHEME, int HPS>
 static void launch_attend_mfma8_slabs(int n_slabs, dim3 grid, hipStream_t st, const AttendArgs& a) {
   const size_t lds = attend_mfma8_lds_bytes(n_slabs, a.n_q_heads, HPS);
   switch (n_slabs) {
-    case 1: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 0, HPS>), grid, dim3(256), lds, st, a); break;
-    case 2: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 1, HPS>), grid, dim3(256), lds, st, a); break;
-    case 4: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 2, HPS>), grid, dim3(256), lds, st, a); break;
-    default: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 3, HPS>), grid, dim3(256), lds, st, a); break;
+    case 1: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 1, HPS>), grid, dim3(256), lds, st, a); break;
+    case 2: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 2, HPS>), grid, dim3(256), lds, st, a); break;
+    case 3: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 3, HPS>), grid, dim3(256), lds, st, a); break;
+    case 4: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 4, HPS>), grid, dim3(256), lds, st, a); break;
+    case 5: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 5, HPS>), grid, dim3(256), lds, st, a); break;
+    case 6: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 6, HPS>), grid, dim3(256), lds, st, a); break;
+    case 7: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 7, HPS>), grid, dim3(256), lds, st, a); break;
+    default: hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 8, HPS>), grid, dim3(256), lds, st, a); break;
   }
 }
 template <int SCHEME>
@@ -858,15 +870,24 @@ static void launch_attend_mfma8(int n_slabs, int hps, dim3 grid, hipStream_t st,
   else launch_attend_mfma8_slabs<SCHEME, 4>(n_slabs, grid, st, a);
 }
 
-template <int SCHEME, bool EXCH = false>
-static void launch_attend_mfma(int n_kv_heads, dim3 grid, hipStream_t st, const AttendArgs& a) {
-  const size_t lds = attend_mfma_lds_bytes(n_kv_heads, a.n_q_heads);
-  switch (n_kv_heads) {
-    case 1: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 0, EXCH>), grid, dim3(256), lds, st, a); break;
-    case 2: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 1, EXCH>), grid, dim3(256), lds, st, a); break;
-    case 4: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 2, EXCH>), grid, dim3(256), lds, st, a); break;
-    default: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 3, EXCH>), grid, dim3(256), lds, st, a); break;
+template <int SCHEME, bool EXCH, bool NARROW>
+static void launch_attend_mfma_slabs(int n_slabs, dim3 grid, hipStream_t st, const AttendArgs& a) {
+  const size_t lds = attend_mfma_lds_bytes(n_slabs, a.n_q_heads);
+  switch (n_slabs) {
+    case 1: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
+    case 2: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 2, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
+    case 3: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 3, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
+    case 4: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 4, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
+    case 5: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 5, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
+    case 6: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 6, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
+    case 7: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 7, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
+    default: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 8, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
   }
+}
+template <int SCHEME, bool EXCH = false>
+static void launch_attend_mfma(int n_slabs, dim3 grid, hipStream_t st, const AttendArgs& a) {
+  if (a.head_dim == 128) launch_attend_mfma_slabs<SCHEME, EXCH, false>(n_slabs, grid, st, a);
+  else launch_attend_mfma_slabs<SCHEME, EXCH, true>(n_slabs, grid, st, a);
 }
 
 // out[c,h,d] = sum over the splits that hold tokens of cache c, in split order
@@ -958,7 +979,7 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
     // the matrix-core kernels see 128-dimension slabs of the row: one kv head, or 2 / 4 narrow ones
     const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
     const int slabs = hps > 0 ? n_kv_heads / hps : 0;
-    const bool slabs_ok = slabs == 1 || slabs == 2 || slabs == 4 || slabs == 8;
+    const bool slabs_ok = slabs >= 1 && slabs <= 8;
     if (!eight && group == 32 && slabs_ok && rep * hps <= 8) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       // four query heads of every kv group per launch; a second launch (same codes, next four
@@ -1066,7 +1087,7 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
   const int rep = n_q_heads % n_kv_heads == 0 ? n_q_heads / n_kv_heads : 0;
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);   // 128-dimension slabs: one kv head, or 2 / 4 narrow ones
   const int slabs = hps > 0 ? n_kv_heads / hps : 0;
-  const bool hk_ok = slabs == 1 || slabs == 2 || slabs == 4 || slabs == 8;
+  const bool hk_ok = slabs >= 1 && slabs <= 8;
   const int64_t splits = attend_splits(n_caches, max_len);
   if ((scheme == PIKV_Q_I4_ASYM || scheme == PIKV_Q_I4_SYM) && group == 32 && rep >= 1 &&
       rep * hps <= 8 && hk_ok && q_dtype == PIKV_BF16 && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {

@@ -516,7 +516,8 @@ static size_t gqa_lds_bytes(int n_kv_heads, int nset) {
 // multiplied (two register sets, used alternately).
 // NSET sets of four query heads per kv head (1: up to 4 heads, 2: up to 8): the unpacked codes
 // of a kv head are multiplied with one block-diagonal A operand per set.
-template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false>  // NKV = n_kv_heads rounded up to 4/8/16; EXCH: exchange format out
+// NARROW: heads of 64 or 32 dimensions (below); the kernel for heads of 128 carries none of it.
+template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false, bool NARROW = false>  // NKV = n_kv_heads rounded up to 4/8/16; EXCH: exchange format out
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET <= 8 ? 4 : 2))) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
   constexpr int SL = 4 * NSET;  // head slots per kv head
   using Q = QScheme<SCHEME>;
@@ -540,17 +541,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   // Heads narrower than 128: a.n_kv_heads counts 128-dimension slabs of the cached row, each the
   // stored bytes of hps = 128 / head_dim neighbouring kv heads, and the rep query heads of a slab
   // are the heads of those kv heads, rep1 each, in order.  Query head r of a slab belongs to kv
-  // head r / rep1 of it and its A rows are zero outside that head's gph groups - the products
+  // head r / rep1 of it and its A rows are zero outside that head's groups - the products
   // with the neighbours' codes vanish exactly.
-  const int hps = 128 / a.head_dim;
-  const int rep1 = rep / hps;
-  const int gph = 4 / hps;
+  // (hps is 1, 2 or 4: shifts and comparisons, no integer division in a prologue that every block of
+  // two tiles runs)
+  const int head_dim = NARROW ? a.head_dim : 128;
+  const int gshift = head_dim == 64 ? 1 : 0;          // log2 of a narrow head's groups of 32
+  const int rep1 = head_dim == 64 ? rep >> 1 : rep >> 2;
+  auto owns = [&](int r, int gq) {                    // group gq of the slab belongs to query head r's kv head
+    return !NARROW || (gq >> gshift) == (r >= rep1) + (r >= 2 * rep1) + (r >= 3 * rep1);
+  };
+  auto group_in_head = [&](int gq) { return NARROW ? gq & ((1 << gshift) - 1) : gq; };
   const int lanes_per_row = a.n_kv_heads * 4;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nl = lane & 15;
   const int rg = lane >> 4;
-  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * a.head_dim;
+  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * head_dim;
   const int64_t base_row = a.row_base[c];
 
   // Code vectors of this wavefront's slice of tile tt (one 16-byte load per kv
@@ -601,9 +608,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     const int set = i / (a.n_kv_heads * 16), ig = i - set * a.n_kv_heads * 16;
     const int g = ig >> 4, gq = (ig >> 2) & 3, r = (ig & 3) + 4 * set;
     float sacc = 0.f;
-    if (r < rep && gq / gph == r / rep1) {
+    if (r < rep && owns(r, gq)) {
       float h32[32];
-      load_as_float<PIKV_BF16, 32>(qbase, (int64_t)(g * rep + r) * a.head_dim + (gq % gph) * 32, h32);
+      load_as_float<PIKV_BF16, 32>(qbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32, h32);
 #pragma unroll
       for (int k = 0; k < 32; ++k) sacc += h32[k];
     }
@@ -613,8 +620,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     const int set = i / (a.n_kv_heads * 64), ig = i - set * a.n_kv_heads * 64;
     const int g = ig >> 6, b2 = (ig >> 4) & 3, gq = (ig >> 2) & 3, r = (ig & 3) + 4 * set;
     uint4 d = make_uint4(0, 0, 0, 0);
-    if (r < rep && gq / gph == r / rep1)
-      d = ld16(qbase + (int64_t)(g * rep + r) * a.head_dim + (gq % gph) * 32 + b2 * 8);
+    if (r < rep && owns(r, gq))
+      d = ld16(qbase + (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32 + b2 * 8);
     alds[i] = make_uint4((d.x & 0xffffu) | (d.z << 16), (d.x >> 16) | (d.z & 0xffff0000u),
                          (d.y & 0xffffu) | (d.w << 16), (d.y >> 16) | (d.w & 0xffff0000u));
     if (set == 0) azero[ig] = make_uint4(0, 0, 0, 0);
@@ -752,12 +759,14 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   const int64_t row_bytes = (int64_t)a.n_kv_heads * 128;
   const int groups_per_row = (a.n_kv_heads * 128) / a.group;
   const int64_t base_row = a.row_base[c];
-  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * a.head_dim;
-  const int rep1 = rep / HPS;        // query heads per kv head
-  const int hh_a = nl / rep1;        // kv head (inside the slab) of the query head in A row nl
-  int hh_c[4];                       // ... of the query heads in this lane's four C rows
+  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * (128 / HPS);
+  const int rep1 = HPS == 1 ? rep : HPS == 2 ? rep >> 1 : rep >> 2;   // query heads per kv head
+  // kv head (inside the slab) of query head r: comparisons, no integer division
+  auto head_in_slab = [&](int r) { return HPS == 1 ? 0 : (r >= rep1) + (r >= 2 * rep1) + (r >= 3 * rep1); };
+  const int hh_a = head_in_slab(nl);  // ... of the query head in A row nl (rows >= rep hold no head)
+  int hh_c[4];                        // ... of the query heads in this lane's four C rows
 #pragma unroll
-  for (int qq = 0; qq < 4; ++qq) hh_c[qq] = (4 * rg + qq) / rep1 < HPS ? (4 * rg + qq) / rep1 : HPS - 1;
+  for (int qq = 0; qq < 4; ++qq) hh_c[qq] = head_in_slab(4 * rg + qq) < HPS ? head_in_slab(4 * rg + qq) : HPS - 1;
   // two nibbles -> two bf16 values 16 + nibble; both constants held in vector registers so that the
   // three-operand and-or instruction can be encoded (the empty statement emits no instruction)
   uint32_t kNib = 0x00780078u, kExp = 0x41804180u;
@@ -776,8 +785,8 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
     for (int ks = 0; ks < 8; ++ks) {
       uint2 qd = make_uint2(0, 0);
       const int ds = 64 * (ks >> 2) + 16 * rg + 4 * (ks & 3);   // dimension inside the slab
-      if (on && (HPS == 1 || ds / a.head_dim == hh_a))
-        qd = *reinterpret_cast<const uint2*>(qbase + (int64_t)(g * rep + nl) * a.head_dim + (ds - hh_a * a.head_dim));
+      if (on && (HPS == 1 || ds / (128 / HPS) == hh_a))
+        qd = *reinterpret_cast<const uint2*>(qbase + (int64_t)(g * rep + nl) * (128 / HPS) + (ds - hh_a * (128 / HPS)));
       // bf16 x 16: through float, exact (zero stays zero)
       auto x16 = [](uint32_t h) { return __float_as_uint(__uint_as_float(h << 16) * 16.0f) >> 16; };
       const uint32_t q0 = qd.x & 0xffffu, q1 = qd.x >> 16, q2 = qd.y & 0xffffu, q3 = qd.y >> 16;
@@ -876,8 +885,8 @@ static int launch_i8_mfma(const ScoreArgs& a, int n_caches, int64_t n_tiles, hip
   return PIKV_OK;
 }
 
-template <int SCHEME, bool EXCH = false>
-static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
+template <int SCHEME, bool EXCH, bool NARROW>
+static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
   const int rep = a.n_q_heads / a.n_kv_heads;
   const int nset = rep <= 4 ? 1 : 2;
   const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset);
@@ -885,19 +894,25 @@ static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStre
   const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
   if (nset == 1) {
     if (a.n_kv_heads <= 4)
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1, EXCH>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a);
     else if (a.n_kv_heads <= 8)
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1, EXCH>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a);
     else
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 16, 1, EXCH>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 16, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a);
   } else {
     // 5-8 query heads per kv head; 16 kv heads x 8 would need more than 64 KB of LDS
     if (a.n_kv_heads <= 4)
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2, EXCH>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2, EXCH, NARROW>), grid, dim3(256), lds, st, a);
     else
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH, NARROW>), grid, dim3(256), lds, st, a);
   }
   return PIKV_OK;
+}
+// a.n_kv_heads counts 128-dimension slabs, a.head_dim is the width of a stored kv head
+template <int SCHEME, bool EXCH = false>
+static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
+  return a.head_dim == 128 ? launch_gqa_slabs<SCHEME, EXCH, false>(a, n_caches, n_tiles, st)
+                           : launch_gqa_slabs<SCHEME, EXCH, true>(a, n_caches, n_tiles, st);
 }
 
 // Final max and sum per (cache, q head) from the tile statistics [cache][tile][head].

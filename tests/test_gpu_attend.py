@@ -36,14 +36,23 @@ pytestmark = pytest.mark.gpu
     (O.Q_I4_ASYM, 32, 16, 16, 64),     # ... eight slabs
     (O.Q_I4_SYM, 32, 4, 12, 64),       # ... 3 q heads per kv head: the second launch half empty
     (O.Q_I4_ASYM, 32, 8, 16, 32),      # heads of 32: four kv heads per slab
-    (O.Q_I4_ASYM, 32, 12, 12, 64),     # six slabs: vector form
+    (O.Q_I4_ASYM, 32, 12, 12, 64),     # ... six slabs
+    (O.Q_I4_ASYM, 32, 20, 20, 64),     # ten slabs: vector form
     (O.Q_I8_SYM, 64, 8, 16, 64),       # 8-bit heads of 64 on the matrix-core form: a scale per kv head, two per slab
     (O.Q_I8_ASYM, 64, 4, 16, 64),      # ... 4 q heads per kv head: all 16 operand rows, zero points per kv head
     (O.Q_I8_SYM, 128, 4, 8, 64),       # ... one scale per slab
     (O.Q_I8_ASYM, 32, 8, 16, 32),      # ... heads of 32
     (O.Q_I8_ASYM, 64, 16, 32, 64),     # ... eight slabs
     (O.Q_I8_SYM, 64, 12, 12, 64),      # 12 kv heads, vector form: five whole rows per pass of a block
-    (O.Q_I4_SYM, 32, 3, 6, 128),       # 3 kv heads
+    (O.Q_I4_SYM, 32, 3, 6, 128),       # 3 kv heads: matrix-core form with a kv head count that is no power of two
+    (O.Q_I4_ASYM, 32, 6, 12, 128),     # ... 6
+    (O.Q_I4_ASYM, 32, 5, 5, 128),      # ... 5, one q head each
+    (O.Q_I4_SYM, 32, 7, 42, 128),      # ... 7 x 6: two launches
+    (O.Q_I8_SYM, 128, 3, 6, 128),      # 8-bit matrix-core form, 3 kv heads
+    (O.Q_I8_ASYM, 128, 6, 12, 128),    # ... 6
+    (O.Q_I8_SYM, 128, 5, 40, 128),     # ... 5 x 8
+    (O.Q_I8_ASYM, 128, 7, 14, 128),    # ... 7
+    (O.Q_I8_SYM, 64, 12, 24, 64),      # ... 12 heads of 64: six slabs
 ])
 @pytest.mark.parametrize("form", ["stats", "probs"])
 def test_attend_values(dev, scheme, group, heads, hq, dh, form):
@@ -88,6 +97,8 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
     (O.Q_I4_SYM, 32, 2, 8, 64),        # ... two launches
     (O.Q_I4_ASYM, 32, 8, 8, 32),       # heads of 32
     (O.Q_I8_ASYM, 64, 8, 16, 64),      # 8-bit heads of 64 on the matrix-core form
+    (O.Q_I4_ASYM, 32, 6, 36, 128),     # 6 kv heads x 6: two launches
+    (O.Q_I8_SYM, 128, 3, 12, 128),     # 8-bit, 3 kv heads
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.95])
 def test_attend_accumulates_importance(dev, scheme, group, heads, hq, dh, decay):
@@ -157,7 +168,11 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I4_SYM, 32, 2, 8, 64, "bf16"),      # ... 4 q heads per kv head
     (O.Q_I4_ASYM, 32, 16, 16, 64, "bf16"),   # ... eight slabs
     (O.Q_I4_ASYM, 32, 8, 16, 32, "bf16"),    # heads of 32
-    (O.Q_I4_SYM, 32, 12, 12, 64, "bf16"),    # six slabs: the three public steps inside the call
+    (O.Q_I4_SYM, 32, 12, 12, 64, "bf16"),    # ... six slabs
+    (O.Q_I4_ASYM, 32, 6, 24, 128, "bf16"),   # kv head counts that are no power of two: 6
+    (O.Q_I4_SYM, 32, 5, 10, 128, "bf16"),    # ... 5
+    (O.Q_I4_ASYM, 32, 7, 7, 128, "bf16"),    # ... 7
+    (O.Q_I4_ASYM, 32, 20, 20, 64, "bf16"),   # ten slabs: the three public steps inside the call
     (O.Q_I4_ASYM, 32, 2, 6, 64, "f32"),
     (O.Q_I8_ASYM, 64, 8, 16, 64, "bf16"),    # 8-bit heads of 64 on the matrix-core kernels
     (O.Q_I8_SYM, 64, 12, 12, 64, "f32"),     # 12 kv heads of 64, 8-bit
