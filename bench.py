@@ -107,13 +107,19 @@ def cpu_baseline(torch, w, hidden, gate_w, k_src, v_src, q, reps=5):
                       f"(OpenMP, {CO.threads()} threads), {best:.2f} s per step"}
 
 
-def _median_ms(torch, fn, iters, warm=3):
+def _median_ms(torch, fn, iters, warm=3, setup=None):
+    """Median time of fn over `iters` calls; `setup` (state restoring, not part of the measured
+    work) runs before every call, ahead of the opening event."""
     for _ in range(warm):
+        if setup:
+            setup()
         fn()
     torch.cuda.synchronize()
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
            for _ in range(iters)]
     for a, b in evs:
+        if setup:
+            setup()
         a.record()
         fn()
         b.record()
@@ -188,11 +194,11 @@ def decode_read_workload(torch, ops, dev, iters):
     one = torch.ones(B, device=dev, dtype=torch.int32)
 
     def decode_step():
-        pool.fill.fill_(N - 1)
         pool.quant_scatter(new_k, new_v, seq_id, zero_slot, 1, now=2.0)
         pool.advance(one)
         return pool.decode_attend(q, hq, now=2.0)     # scores + softmax + attention output + H2O accumulate
-    t_step = _median_ms(torch, decode_step, iters)
+    # every step starts from caches of N - 1 rows: the reset is the bench's, not the step's
+    t_step = _median_ms(torch, decode_step, iters, setup=lambda: pool.fill.fill_(N - 1))
     t_fused = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=2.0), iters)
     t_att_acc = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats, accumulate=True, now=1.0), iters)
     pool.fill.fill_(N)
