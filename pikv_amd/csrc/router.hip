@@ -320,10 +320,15 @@ __global__ __launch_bounds__(256) void gate_weight_relayout_kernel(const uint16_
 // PARTIAL (short token streams): blockIdx.y picks a slice of the k-steps, and the block
 // writes its partial logits to part[slice][T][E] instead of running the tail - with a few
 // dozen tokens a single block would walk all of H alone, one load latency per k-step.
-template <int NT, int MT, int WAVES, bool PARTIAL = false>
+// DIRECT (up to 16 experts): wb is the caller's [E, H] weight matrix itself, lane (expert m, kg)
+// reads its 16 bytes of a k-step from row m.  Every block starts its walk at another k-step (below),
+// so the rows - a multiple of 2 KB apart - no longer meet in one L2 channel at the same time, and the
+// launch that re-lays the weights is saved (config[1], router call: 65.2 -> 63.0 us).
+template <int NT, int MT, int WAVES, bool PARTIAL = false, bool DIRECT = false>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2))) void router_gate_mfma_kernel(
     const void* __restrict__ x, const void* __restrict__ wb, int H, TailParams p, float* __restrict__ part = nullptr,
     int steps_per_slice = 0) {
+  static_assert(!DIRECT || (NT == 1 && !PARTIAL), "direct weights: one expert tile, whole rows per block");
   constexpr int EP = 16 * NT;
   constexpr int TB = 16 * MT;  // tokens per block
   // Partial sums of the wavefronts: one slab each, or - when those would not leave room
@@ -344,7 +349,8 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
     xrow[mt] = reinterpret_cast<const char*>(x) +
                ((tok_ok[mt] ? tok0 + mt * 16 + m : 0) * (int64_t)H + kg * 8) * 2;
   }
-  const char* wlane = reinterpret_cast<const char*>(wb) + (m * 32 + kg * 8) * 2;
+  const char* wlane = DIRECT ? reinterpret_cast<const char*>(wb) + ((int64_t)(m < p.E ? m : 0) * H + kg * 8) * 2
+                             : reinterpret_cast<const char*>(wb) + (m * 32 + kg * 8) * 2;
   pikv_f32x4 acc[MT][NT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -382,7 +388,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
       // (columns of experts that do not exist are zero in the re-laid weights: not loaded at all)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        bv[u][t] = (ok && t * 16 + m < p.E) ? ld16(wlane + ((int64_t)st * EP + t * 16) * 64) : make_uint4(0, 0, 0, 0);
+        bv[u][t] = (ok && t * 16 + m < p.E)
+                       ? ld16(DIRECT ? wlane + (int64_t)st * 64 : wlane + ((int64_t)st * EP + t * 16) * 64)
+                       : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u)
@@ -1177,8 +1185,6 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
     if (mfma) {
       const int ep = gate_epad(E);
       const int64_t chunks = (int64_t)(H / 32) * ep * 4;
-      hipLaunchKernelGGL(gate_weight_relayout_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256),
-                         0, st, (const uint16_t*)w, H, E, ep, (uint4*)wb);
       // 64 tokens per block.  Few experts: 8 wavefronts share the k-steps; many
       // experts: 4 (the accumulators of 4 x 4 tiles and the partial sums in LDS
       // leave room for two such blocks per compute unit)
@@ -1197,6 +1203,11 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
       const bool t128 = tiled && ep != 16 && H % 128 == 0 && (T > 32768 || H % 256 != 0);
       const bool t64 = tiled && !t128 && H % 256 == 0;
       const dim3 g64((unsigned)((T + 63) / 64)), g128((unsigned)((T + 127) / 128));
+      // up to 16 experts on the untiled kernel: the weights are read where they lie
+      const bool direct = slices <= 1 && !t64 && !t128 && ep == 16;
+      if (!direct)
+        hipLaunchKernelGGL(gate_weight_relayout_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256),
+                           0, st, (const uint16_t*)w, H, E, ep, (uint4*)wb);
       if (slices > 1) {
         // short token streams: partial logits per slice of H, then the tail on their sum
         float* part = reinterpret_cast<float*>(wb + align256(gate_weight_bytes(H, E)));
@@ -1230,7 +1241,7 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
         hipLaunchKernelGGL((router_gate_mfma_kernel<4, 8, 4>), dim3((unsigned)((T + 127) / 128)), dim3(256), 0, st,
                            x, wb, H, p);
       else if (ep == 16)
-        hipLaunchKernelGGL((router_gate_mfma_kernel<1, 4, 8>), grid, dim3(512), 0, st, x, wb, H, p);
+        hipLaunchKernelGGL((router_gate_mfma_kernel<1, 4, 8, false, true>), grid, dim3(512), 0, st, x, w, H, p);
       else if (ep == 32)
         hipLaunchKernelGGL((router_gate_mfma_kernel<2, 4, 4>), grid, dim3(256), 0, st, x, wb, H, p);
       else
