@@ -183,13 +183,13 @@ __device__ __forceinline__ int att_meta_off(int tok, int g, int hk) {
 
 constexpr int kAttPRow = 68;  // floats per query head of staged probabilities: 64 tokens + 4 (bank spread)
 
-static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads) {
+static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads, int nsets = 1) {
   // codes [64 tokens][n_kv_heads*64 + 8 bytes]; scale and zero + bias as float4 (4 groups)
   // [64 tokens][kv head] in padded token rows; A operands per wavefront [4 groups][8 rows][kAttARow];
   // probabilities [query head][kAttPRow]
   // + one all-zero piece of an A row (32 bytes) for the lanes whose row holds no head
   return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * att_meta_bytes(n_kv_heads) + 4 * (size_t)4 * 8 * kAttARow +
-         (size_t)4 * n_kv_heads * kAttPRow * 4 + 32;
+         (size_t)4 * n_kv_heads * nsets * kAttPRow * 4 + 32;
 }
 
 // HK = n_kv_heads (1..8); at most 4 query heads per kv head.  EXCH: the scores come in the exchange
@@ -199,12 +199,17 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads) {
 // heads of a slab are the heads of those kv heads in order.  A query head is multiplied with the
 // whole slab and only the dimensions of its own kv head are written out.
 // NARROW selects that form at compile time: the kernel for heads of 128 carries none of it.
-template <int SCHEME, int HK, bool EXCH = false, bool NARROW = false>
+// NSETS = 2 (up to 4 kv heads): a launch covers up to 8 query heads of every kv head as two sets of
+// four that are multiplied, one after the other, with the same staged tile - the V codes of a cache
+// with 5 to 8 query heads per kv head are read from memory once instead of once per launch.
+template <int SCHEME, int HK, bool EXCH = false, bool NARROW = false, int NSETS = 1>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i4_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
   static_assert(HK >= 1 && HK <= 8, "1 to 8 kv heads");
   constexpr int NH = (HK + 3) / 4;        // kv heads per wavefront
+  constexpr int NI = NH * NSETS;          // (kv head, set of four query heads) pairs per wavefront
+  static_assert(NSETS == 1 || (NSETS == 2 && HK <= 4), "two sets: the staged rows of 8 x 4 heads, accumulators of one kv head");
   constexpr int RS = HK * 64 + 8;         // bytes per token row of staged codes
   constexpr int LPR = HK * 4;             // 16-byte chunks per cached row
   constexpr int NCH = kAttTile * LPR / 256 > 0 ? kAttTile * LPR / 256 : 1;  // code chunks per thread
@@ -217,7 +222,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int wave = threadIdx.x >> 6;
   unsigned char* abuf = lzterm + att_meta_bytes(HK) + wave * (4 * 8 * kAttARow);
   float* lprob = reinterpret_cast<float*>(lzterm + att_meta_bytes(HK) + 4 * (4 * 8 * kAttARow));
-  unsigned char* azero = reinterpret_cast<unsigned char*>(lprob + 4 * HK * kAttPRow);
+  unsigned char* azero = reinterpret_cast<unsigned char*>(lprob + 4 * HK * NSETS * kAttPRow);
   if (threadIdx.x < 8) reinterpret_cast<uint32_t*>(azero)[threadIdx.x] = 0u;  // visible after the loop's first barrier
 
   const int c = blockIdx.y;
@@ -233,7 +238,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   // A launch covers up to 4 query heads of every kv group: heads head_off .. head_off+nr-1.
   // More than 4 heads per kv head are served by a second launch over the same codes.
   const int rep_all = a.n_q_heads / HK;
-  const int rep = rep_all - a.head_off < 4 ? rep_all - a.head_off : 4;  // heads of a group in this launch
+  const int rep = rep_all - a.head_off < 4 ? rep_all - a.head_off : 4;  // heads of a group in this launch (first set)
+  const int rep_b = NSETS == 1 ? 0 : rep_all - a.head_off - 4 < 0 ? 0 : rep_all - a.head_off - 4 < 4 ? rep_all - a.head_off - 4 : 4;  // second set
   // matrix-core roles: A row / B,C column i, token group kg
   const int i = lane & 15;
   const int kg = lane >> 4;
@@ -241,26 +247,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int r = lane >> 4;
   const int wkg = (lane >> 2) & 3;
   const int tk = wkg * 16 + (lane & 3);
-  const bool row_on = r < rep;
   const bool normalise = a.head_stats != nullptr;
   const float zbias = 128.0f - (float)Q::qmin;
   const int64_t base_row = a.row_base[c];
 
-  pikv_f32x4 C[NH][8];
-  float zacc[NH][4];
+  pikv_f32x4 C[NI][8];
+  float zacc[NI][4];
 #pragma unroll
-  for (int hs = 0; hs < NH; ++hs) {
+  for (int hs = 0; hs < NI; ++hs) {
 #pragma unroll
     for (int d = 0; d < 8; ++d) C[hs][d] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int sg = 0; sg < 4; ++sg) zacc[hs][sg] = 0.f;
   }
-  // score-staging role: staged row sh = 4 * kv head + head of this launch, tokens st8..st8+7 of
-  // the tile (32 rows x 8 runs); rows without a head stage zeros
+  // score-staging role: staged row sh = 4 * (set * HK + kv head) + head of the set, tokens
+  // st8..st8+7 of the tile (32 rows x 8 runs); rows without a head stage zeros
   const int sh = threadIdx.x >> 3;
   const int st8 = (threadIdx.x & 7) * 8;
-  const bool s_on = (sh >> 2) < HK && (sh & 3) < rep;
-  const int s_hq = s_on ? (sh >> 2) * rep_all + a.head_off + (sh & 3) : 0;
+  const int s_set = NSETS == 1 ? 0 : sh / (4 * HK);
+  const int s_g = NSETS == 1 ? sh >> 2 : (sh >> 2) % HK;
+  const bool s_on = s_set < NSETS && s_g < HK && (sh & 3) < (s_set ? rep_b : rep);
+  const int s_hq = s_on ? s_g * rep_all + a.head_off + 4 * s_set + (sh & 3) : 0;
   const float* srow = a.scores + ((int64_t)c * a.n_q_heads + s_hq) * a.score_stride;
   float smx = 0.f, srz = 1.f;
   if (normalise) {
@@ -379,8 +386,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   };
 
   // A-operand piece of this lane: row i of group sg (8 rows of kAttARow bytes per group), or the zero piece
-  const unsigned char* const a_row = i < 2 * rep ? abuf + i * kAttARow + kg * 32 : azero;
-  const int a_step = i < 2 * rep ? 8 * kAttARow : 0;
+  const unsigned char* a_row[NSETS];
+  int a_step[NSETS];
+#pragma unroll
+  for (int set = 0; set < NSETS; ++set) {
+    const bool on = i < 2 * (set ? rep_b : rep);
+    a_row[set] = on ? abuf + i * kAttARow + kg * 32 : azero;
+    a_step[set] = on ? 8 * kAttARow : 0;
+  }
   // two nibbles -> two bf16 values 128 + code.  Both constants are kept in vector registers (the
   // empty statement hides their values from the compiler, it emits no instruction): with a literal
   // operand the three-operand and-or instruction cannot be encoded and every expansion falls apart
@@ -407,7 +420,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       float* const ts_rows = a.row_ts ? a.row_ts + (base_row + n0) : nullptr;
       const float* lp = lprob + (t & ~15) + (t & 3) * 4 + ((t >> 2) & 3);
       float imp = 0.f;
-      for (int hq = grp; hq < 4 * HK; hq += 4) imp = imp + lp[hq * kAttPRow];
+      for (int hq = grp; hq < 4 * HK * NSETS; hq += 4) imp = imp + lp[hq * kAttPRow];
       imp = imp + __shfl_xor(imp, 16, 64);
       imp = imp + __shfl_xor(imp, 32, 64);
       if (mine) {
@@ -428,12 +441,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     if (n0 + kAttTile < t1) fetch(n0 + kAttTile);  // in flight while this tile is multiplied
 
 #pragma unroll
-    for (int hs = 0; hs < NH; ++hs) {
-      const int g = wave + 4 * hs;
+    for (int hs = 0; hs < NI; ++hs) {   // hs = kv head slot * NSETS + set
+      const int set = hs % NSETS;
+      const int g = wave + 4 * (hs / NSETS);
       if (g >= HK) continue;  // uniform
+      const bool row_on = r < (set ? rep_b : rep);
       // ---- weights: this lane prepares head r for four tokens, all four groups ----
       float4 s4[4], z4[4];
-      const float4 pv = *reinterpret_cast<const float4*>(lprob + (row_on ? g * 4 + r : 0) * kAttPRow + wkg * 16 +
+      const float4 pv = *reinterpret_cast<const float4*>(lprob + (row_on ? (set * HK + g) * 4 + r : 0) * kAttPRow + wkg * 16 +
                                                          (lane & 3) * 4);
       const float p4[4] = {row_on ? pv.x : 0.f, row_on ? pv.y : 0.f, row_on ? pv.z : 0.f, row_on ? pv.w : 0.f};
 #pragma unroll
@@ -476,7 +491,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 #pragma unroll
       for (int sg = 0; sg < 4; ++sg) {
         // a lane whose A row holds no head reads the zero piece: no branch, no cleared registers
-        const uint4* ap = reinterpret_cast<const uint4*>(a_row + sg * a_step);
+        const uint4* ap = reinterpret_cast<const uint4*>(a_row[set] + sg * a_step[set]);
         const uint4 a1 = ap[0], a2 = ap[1];
 #pragma unroll
         for (int dbl = 0; dbl < 2; ++dbl) {
@@ -506,39 +521,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   // head r, so head 2*kg is q = 0,1 and head 2*kg+1 is q = 2,3.  The zero-point sums sit
   // spread over the 16 lanes that prepared head r.
   __syncthreads();
-  float* zl = reinterpret_cast<float*>(att_lds);  // [wave][head slot][r][sg]
+  float* zl = reinterpret_cast<float*>(att_lds);  // [wave][kv head slot, set][r][sg]
   const int hps = NARROW ? 128 / a.head_dim : 1;   // kv heads per slab
   const int rep1 = rep_all / hps;                  // query heads per kv head
 #pragma unroll
-  for (int hs = 0; hs < NH; ++hs)
+  for (int hs = 0; hs < NI; ++hs)
 #pragma unroll
     for (int sg = 0; sg < 4; ++sg) {
       const float z = group_sum_dpp(zacc[hs][sg], 16);
-      if ((lane & 15) == 0) zl[((wave * NH + hs) * 4 + r) * 4 + sg] = z;
+      if ((lane & 15) == 0) zl[((wave * NI + hs) * 4 + r) * 4 + sg] = z;
     }
   __syncthreads();
 #pragma unroll
-  for (int hs = 0; hs < NH; ++hs) {
-    const int g = wave + 4 * hs;
+  for (int hs = 0; hs < NI; ++hs) {
+    const int set = hs % NSETS;
+    const int g = wave + 4 * (hs / NSETS);
     if (g >= HK) continue;
 #pragma unroll
     for (int rr = 0; rr < 2; ++rr) {
-      const int ro = 2 * kg + rr;  // head (inside the kv group) held by this lane
-      if (ro >= rep) continue;
-      const int64_t ohead = ((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + ro;
+      const int ro = 2 * kg + rr;  // head (inside the set) held by this lane
+      if (ro >= (set ? rep_b : rep)) continue;
+      const int hro = a.head_off + 4 * set + ro;   // head inside the kv group
+      const int64_t ohead = ((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep_all + hro;
       if constexpr (!NARROW) {
         float* o = a.partial + ohead * 128;
 #pragma unroll
         for (int db = 0; db < 8; ++db)
-          o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NH + hs) * 4 + ro) * 4 + (db >> 1)];
+          o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NI + hs) * 4 + ro) * 4 + (db >> 1)];
       } else {
         // kv head hh of the slab owns the 16-dimension blocks db with db * hps / 8 == hh
-        const int hh = (a.head_off + ro) / rep1;
+        const int hh = hro / rep1;
         float* o = a.partial + ohead * a.head_dim - hh * a.head_dim;
 #pragma unroll
         for (int db = 0; db < 8; ++db)
           if ((db * hps) >> 3 == hh)
-            o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NH + hs) * 4 + ro) * 4 + (db >> 1)];
+            o[db * 16 + i] = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NI + hs) * 4 + ro) * 4 + (db >> 1)];
       }
     }
   }
@@ -871,8 +888,17 @@ static void launch_attend_mfma8(int n_slabs, int hps, dim3 grid, hipStream_t st,
 }
 
 template <int SCHEME, bool EXCH, bool NARROW>
-static void launch_attend_mfma_slabs(int n_slabs, dim3 grid, hipStream_t st, const AttendArgs& a) {
-  const size_t lds = attend_mfma_lds_bytes(n_slabs, a.n_q_heads);
+static void launch_attend_mfma_slabs(int n_slabs, int nsets, dim3 grid, hipStream_t st, const AttendArgs& a) {
+  const size_t lds = attend_mfma_lds_bytes(n_slabs, a.n_q_heads, nsets);
+  if (nsets == 2) {
+    switch (n_slabs) {
+      case 1: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 1, EXCH, NARROW, 2>), grid, dim3(256), lds, st, a); break;
+      case 2: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 2, EXCH, NARROW, 2>), grid, dim3(256), lds, st, a); break;
+      case 3: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 3, EXCH, NARROW, 2>), grid, dim3(256), lds, st, a); break;
+      default: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 4, EXCH, NARROW, 2>), grid, dim3(256), lds, st, a); break;
+    }
+    return;
+  }
   switch (n_slabs) {
     case 1: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
     case 2: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 2, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
@@ -884,10 +910,17 @@ static void launch_attend_mfma_slabs(int n_slabs, dim3 grid, hipStream_t st, con
     default: hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 8, EXCH, NARROW>), grid, dim3(256), lds, st, a); break;
   }
 }
+// All query heads of every slab: four per launch, or - up to 4 slabs - eight per launch in two sets.  A
+// later launch (same codes, next heads) adds its share to the accumulators that the first one has decayed.
 template <int SCHEME, bool EXCH = false>
-static void launch_attend_mfma(int n_slabs, dim3 grid, hipStream_t st, const AttendArgs& a) {
-  if (a.head_dim == 128) launch_attend_mfma_slabs<SCHEME, EXCH, false>(n_slabs, grid, st, a);
-  else launch_attend_mfma_slabs<SCHEME, EXCH, true>(n_slabs, grid, st, a);
+static void launch_attend_mfma(int n_slabs, int heads_per_slab, dim3 grid, hipStream_t st, AttendArgs a) {
+  const int nsets = (n_slabs <= 4 && heads_per_slab > 4) ? 2 : 1;
+  for (int off = 0; off < heads_per_slab; off += 4 * nsets) {
+    a.head_off = off;
+    if (off > 0) a.decay = 1.0f;
+    if (a.head_dim == 128) launch_attend_mfma_slabs<SCHEME, EXCH, false>(n_slabs, nsets, grid, st, a);
+    else launch_attend_mfma_slabs<SCHEME, EXCH, true>(n_slabs, nsets, grid, st, a);
+  }
 }
 
 // out[c,h,d] = sum over the splits that hold tokens of cache c, in split order
@@ -982,14 +1015,8 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
     const bool slabs_ok = slabs >= 1 && slabs <= 8;
     if (!eight && group == 32 && slabs_ok && rep * hps <= 8) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
-      // four query heads of every kv group per launch; a second launch (same codes, next four
-      // heads) adds its share to the accumulators that the first one has already decayed
-      for (int off = 0; off < rep * hps; off += 4) {
-        a.head_off = off;
-        if (off > 0) a.decay = 1.0f;
-        if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(slabs, grid, st, a);
-        else launch_attend_mfma<PIKV_Q_I4_SYM>(slabs, grid, st, a);
-      }
+      if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(slabs, rep * hps, grid, st, a);
+      else launch_attend_mfma<PIKV_Q_I4_SYM>(slabs, rep * hps, grid, st, a);
     } else if (eight && slabs_ok && group % head_dim == 0 && rep * hps >= 2 && rep * hps <= 8) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       if (scheme == PIKV_Q_I8_SYM) launch_attend_mfma8<PIKV_Q_I8_SYM>(slabs, hps, grid, st, a);
@@ -1100,12 +1127,8 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
                    (float*)partial, 0, group, n_kv_heads, n_q_heads, head_dim, n_caches,
                    row_acc, row_ts, decay, now, max_len, esc, tmax, w.n_tiles, 0, attend_tokens_per_block(n_caches, max_len)};
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
-      for (int off = 0; off < rep * hps; off += 4) {   // four query heads of every slab per launch
-        a.head_off = off;
-        if (off > 0) a.decay = 1.0f;
-        if (asym) launch_attend_mfma<PIKV_Q_I4_ASYM, true>(slabs, grid, st, a);
-        else launch_attend_mfma<PIKV_Q_I4_SYM, true>(slabs, grid, st, a);
-      }
+      if (asym) launch_attend_mfma<PIKV_Q_I4_ASYM, true>(slabs, rep * hps, grid, st, a);
+      else launch_attend_mfma<PIKV_Q_I4_SYM, true>(slabs, rep * hps, grid, st, a);
       const int64_t total = (int64_t)n_caches * n_q_heads * head_dim;
       hipLaunchKernelGGL(attend_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
                          (const float*)partial, cache_fill, n_caches, n_q_heads, head_dim, (int)splits,
