@@ -188,7 +188,7 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads, int nsets = 1
   // [64 tokens][kv head] in padded token rows; A operands per wavefront [4 groups][8 rows][kAttARow];
   // probabilities [query head][kAttPRow]
   // + one all-zero piece of an A row (32 bytes) for the lanes whose row holds no head
-  return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * att_meta_bytes(n_kv_heads) + 4 * (size_t)4 * 8 * kAttARow +
+  return (size_t)kAttTile * (n_kv_heads * 64 + 8) + 2 * att_meta_bytes(n_kv_heads) + 4 * (size_t)nsets * 4 * 8 * kAttARow +
          (size_t)4 * n_kv_heads * nsets * kAttPRow * 4 + 32;
 }
 
@@ -200,8 +200,8 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads, int nsets = 1
 // whole slab and only the dimensions of its own kv head are written out.
 // NARROW selects that form at compile time: the kernel for heads of 128 carries none of it.
 // NSETS = 2 (up to 4 kv heads): a launch covers up to 8 query heads of every kv head as two sets of
-// four that are multiplied, one after the other, with the same staged tile - the V codes of a cache
-// with 5 to 8 query heads per kv head are read from memory once instead of once per launch.
+// four that are multiplied with the same staged tile and the same expanded codes - the V codes of a
+// cache with 5 to 8 query heads per kv head are read from memory once instead of once per launch.
 template <int SCHEME, int HK, bool EXCH = false, bool NARROW = false, int NSETS = 1>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i4_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
@@ -220,8 +220,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   unsigned char* lzterm = lscale + att_meta_bytes(HK);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  unsigned char* abuf = lzterm + att_meta_bytes(HK) + wave * (4 * 8 * kAttARow);
-  float* lprob = reinterpret_cast<float*>(lzterm + att_meta_bytes(HK) + 4 * (4 * 8 * kAttARow));
+  unsigned char* abuf = lzterm + att_meta_bytes(HK) + wave * (NSETS * 4 * 8 * kAttARow);   // [set][4 groups][8 rows]
+  float* lprob = reinterpret_cast<float*>(lzterm + att_meta_bytes(HK) + 4 * (NSETS * 4 * 8 * kAttARow));
   unsigned char* azero = reinterpret_cast<unsigned char*>(lprob + 4 * HK * NSETS * kAttPRow);
   if (threadIdx.x < 8) reinterpret_cast<uint32_t*>(azero)[threadIdx.x] = 0u;  // visible after the loop's first barrier
 
@@ -391,7 +391,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 #pragma unroll
   for (int set = 0; set < NSETS; ++set) {
     const bool on = i < 2 * (set ? rep_b : rep);
-    a_row[set] = on ? abuf + i * kAttARow + kg * 32 : azero;
+    a_row[set] = on ? abuf + set * (4 * 8 * kAttARow) + i * kAttARow + kg * 32 : azero;
     a_step[set] = on ? 8 * kAttARow : 0;
   }
   // two nibbles -> two bf16 values 128 + code.  Both constants are kept in vector registers (the
@@ -441,58 +441,68 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     if (n0 + kAttTile < t1) fetch(n0 + kAttTile);  // in flight while this tile is multiplied
 
 #pragma unroll
-    for (int hs = 0; hs < NI; ++hs) {   // hs = kv head slot * NSETS + set
-      const int set = hs % NSETS;
-      const int g = wave + 4 * (hs / NSETS);
+    for (int hk = 0; hk < NH; ++hk) {   // kv head slot of this wavefront
+      const int g = wave + 4 * hk;
       if (g >= HK) continue;  // uniform
-      const bool row_on = r < (set ? rep_b : rep);
-      // ---- weights: this lane prepares head r for four tokens, all four groups ----
+      // ---- weights: this lane prepares head r of every set for four tokens, all four groups ----
       float4 s4[4], z4[4];
-      const float4 pv = *reinterpret_cast<const float4*>(lprob + (row_on ? (set * HK + g) * 4 + r : 0) * kAttPRow + wkg * 16 +
-                                                         (lane & 3) * 4);
-      const float p4[4] = {row_on ? pv.x : 0.f, row_on ? pv.y : 0.f, row_on ? pv.z : 0.f, row_on ? pv.w : 0.f};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         s4[j] = *reinterpret_cast<const float4*>(lscale + att_meta_off(tk + 4 * j, g, HK));
         z4[j] = *reinterpret_cast<const float4*>(lzterm + att_meta_off(tk + 4 * j, g, HK));
       }
 #pragma unroll
-      for (int sg = 0; sg < 4; ++sg) {
-        // w = p * scale cut into a bf16 high part and a bf16 remainder.  The zero-point
-        // sum uses the SAME two-part value, so that what the matrix core multiplies with
-        // 128 + u is taken off again exactly.
-        float hi[4], lo[4];
-        float zsum = 0.f;
+      for (int set = 0; set < NSETS; ++set) {
+        const int hs = hk * NSETS + set;
+        const bool row_on = r < (set ? rep_b : rep);
+        unsigned char* const aset = abuf + set * (4 * 8 * kAttARow);
+        const float4 pv = *reinterpret_cast<const float4*>(lprob + (row_on ? (set * HK + g) * 4 + r : 0) * kAttPRow +
+                                                           wkg * 16 + (lane & 3) * 4);
+        const float p4[4] = {row_on ? pv.x : 0.f, row_on ? pv.y : 0.f, row_on ? pv.z : 0.f, row_on ? pv.w : 0.f};
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float sc = sg == 0 ? s4[j].x : sg == 1 ? s4[j].y : sg == 2 ? s4[j].z : s4[j].w;
-          const float zt = sg == 0 ? z4[j].x : sg == 1 ? z4[j].y : sg == 2 ? z4[j].z : z4[j].w;
-          const float w = p4[j] * sc;
-          hi[j] = __uint_as_float(__float_as_uint(w) & 0xffff0000u);
-          lo[j] = __uint_as_float(__float_as_uint(w - hi[j]) & 0xffff0000u);
-          zsum = fmaf(hi[j] + lo[j], zt, zsum);
-        }
-        zacc[hs][sg] += zsum;
-        // operand order inside 8 tokens is {0,4,1,5,2,6,3,7}: tokens (k, k+4) share a dword
-        if (row_on) {
-          uint32_t* rowh = reinterpret_cast<uint32_t*>(abuf + (sg * 8 + 2 * r) * kAttARow + wkg * 32) + (lane & 3);
-          uint32_t* rowl = reinterpret_cast<uint32_t*>(abuf + (sg * 8 + 2 * r + 1) * kAttARow + wkg * 32) + (lane & 3);
-          rowh[0] = (__float_as_uint(hi[0]) >> 16) | __float_as_uint(hi[1]);
-          rowh[4] = (__float_as_uint(hi[2]) >> 16) | __float_as_uint(hi[3]);
-          rowl[0] = (__float_as_uint(lo[0]) >> 16) | __float_as_uint(lo[1]);
-          rowl[4] = (__float_as_uint(lo[2]) >> 16) | __float_as_uint(lo[3]);
+        for (int sg = 0; sg < 4; ++sg) {
+          // w = p * scale cut into a bf16 high part and a bf16 remainder.  The zero-point
+          // sum uses the SAME two-part value, so that what the matrix core multiplies with
+          // 128 + u is taken off again exactly.
+          float hi[4], lo[4];
+          float zsum = 0.f;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float sc = sg == 0 ? s4[j].x : sg == 1 ? s4[j].y : sg == 2 ? s4[j].z : s4[j].w;
+            const float zt = sg == 0 ? z4[j].x : sg == 1 ? z4[j].y : sg == 2 ? z4[j].z : z4[j].w;
+            const float w = p4[j] * sc;
+            hi[j] = __uint_as_float(__float_as_uint(w) & 0xffff0000u);
+            lo[j] = __uint_as_float(__float_as_uint(w - hi[j]) & 0xffff0000u);
+            zsum = fmaf(hi[j] + lo[j], zt, zsum);
+          }
+          zacc[hs][sg] += zsum;
+          // operand order inside 8 tokens is {0,4,1,5,2,6,3,7}: tokens (k, k+4) share a dword
+          if (row_on) {
+            uint32_t* rowh = reinterpret_cast<uint32_t*>(aset + (sg * 8 + 2 * r) * kAttARow + wkg * 32) + (lane & 3);
+            uint32_t* rowl = reinterpret_cast<uint32_t*>(aset + (sg * 8 + 2 * r + 1) * kAttARow + wkg * 32) + (lane & 3);
+            rowh[0] = (__float_as_uint(hi[0]) >> 16) | __float_as_uint(hi[1]);
+            rowh[4] = (__float_as_uint(hi[2]) >> 16) | __float_as_uint(hi[3]);
+            rowl[0] = (__float_as_uint(lo[0]) >> 16) | __float_as_uint(lo[1]);
+            rowl[4] = (__float_as_uint(lo[2]) >> 16) | __float_as_uint(lo[3]);
+          }
         }
       }
       // the rows were written by other lanes of this wavefront
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      // ---- products: rows 2r / 2r+1 of A against 16 dimensions of 64 tokens ----
+      // ---- products: rows 2r / 2r+1 of A against 16 dimensions of 64 tokens; the expanded
+      // codes of a 16-dimension block serve every set ----
 #pragma unroll
       for (int sg = 0; sg < 4; ++sg) {
         // a lane whose A row holds no head reads the zero piece: no branch, no cleared registers
-        const uint4* ap = reinterpret_cast<const uint4*>(a_row[set] + sg * a_step[set]);
-        const uint4 a1 = ap[0], a2 = ap[1];
+        uint4 a1[NSETS], a2[NSETS];
+#pragma unroll
+        for (int set = 0; set < NSETS; ++set) {
+          const uint4* ap = reinterpret_cast<const uint4*>(a_row[set] + sg * a_step[set]);
+          a1[set] = ap[0];
+          a2[set] = ap[1];
+        }
 #pragma unroll
         for (int dbl = 0; dbl < 2; ++dbl) {
           const int db = 2 * sg + dbl;
@@ -505,8 +515,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
             const uint32_t u = Q::sym ? ((uint32_t)tr[half] ^ 0x88888888u) : (uint32_t)tr[half];
             const uint4 bb = make_uint4(and_or(u, kNib, kExp), and_or(u >> 4, kNib, kExp), and_or(u >> 8, kNib, kExp),
                                         and_or(u >> 12, kNib, kExp));
-            C[hs][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                __builtin_bit_cast(pikv_bf16x8, half ? a2 : a1), __builtin_bit_cast(pikv_bf16x8, bb), C[hs][db], 0, 0, 0);
+#pragma unroll
+            for (int set = 0; set < NSETS; ++set)
+              C[hk * NSETS + set][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  __builtin_bit_cast(pikv_bf16x8, half ? a2[set] : a1[set]), __builtin_bit_cast(pikv_bf16x8, bb),
+                  C[hk * NSETS + set][db], 0, 0, 0);
           }
         }
       }
