@@ -517,12 +517,17 @@ static size_t gqa_lds_bytes(int n_kv_heads, int nset) {
 // NSET sets of four query heads per kv head (1: up to 4 heads, 2: up to 8): the unpacked codes
 // of a kv head are multiplied with one block-diagonal A operand per set.
 // NARROW: heads of 64 or 32 dimensions (below); the kernel for heads of 128 carries none of it.
-template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false, bool NARROW = false>  // NKV = n_kv_heads rounded up to 4/8/16; EXCH: exchange format out
+// QF32 (two sets, up to 4 query heads per kv head): float32 queries.  A query element goes in as two
+// bf16 limbs, q = hi + lo + (at most 2^-17 |q|), hi = the float cut to its upper 16 bits, lo = the rest
+// rounded to bf16: set 0 holds the hi limbs of the heads, set 1 the lo limbs, and the two scores of a
+// head are added before they are staged.
+template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false, bool NARROW = false, bool QF32 = false>  // NKV = n_kv_heads rounded up to 4/8/16; EXCH: exchange format out
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET <= 8 ? 4 : 2))) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
   constexpr int SL = 4 * NSET;  // head slots per kv head
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
   static_assert(kGqaTilesPerBlock % 2 == 0, "tiles are processed in pairs");
+  static_assert(!QF32 || NSET == 2, "float32 queries: one set per limb");
   extern __shared__ float gqa_lds[];
   float* stage = gqa_lds;                            // [kv head][SL head slots][token in tile]
   float4* qs4 = reinterpret_cast<float4*>(stage + a.n_kv_heads * SL * kTile);  // [set][kv head][group]: q sums of the set's 4 heads
@@ -558,6 +563,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   const int nl = lane & 15;
   const int rg = lane >> 4;
   const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * head_dim;
+  const float* qfbase = reinterpret_cast<const float*>(a.q) + (int64_t)c * a.n_q_heads * head_dim;
+  // bf16 bits of limb `set` of a float32 query element
+  auto limb_bits = [](float v, int set) -> uint32_t {
+    const uint32_t hb = __float_as_uint(v) & 0xffff0000u;
+    return set == 0 ? hb >> 16 : float_to_bf16_bits(v - __uint_as_float(hb));
+  };
   const int64_t base_row = a.row_base[c];
 
   // Code vectors of this wavefront's slice of tile tt (one 16-byte load per kv
@@ -606,11 +617,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   // the slab and the head's own dimensions start at group (r / rep1) * gph)
   for (int i = threadIdx.x; i < NSET * a.n_kv_heads * 16; i += 256) {
     const int set = i / (a.n_kv_heads * 16), ig = i - set * a.n_kv_heads * 16;
-    const int g = ig >> 4, gq = (ig >> 2) & 3, r = (ig & 3) + 4 * set;
+    const int g = ig >> 4, gq = (ig >> 2) & 3, r = (ig & 3) + (QF32 ? 0 : 4 * set);
     float sacc = 0.f;
     if (r < rep && owns(r, gq)) {
       float h32[32];
-      load_as_float<PIKV_BF16, 32>(qbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32, h32);
+      if constexpr (QF32) {
+        load_as_float<PIKV_F32, 32>(qfbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32, h32);
+#pragma unroll
+        for (int k = 0; k < 32; ++k) h32[k] = bf16_bits_to_float(limb_bits(h32[k], set));
+      } else {
+        load_as_float<PIKV_BF16, 32>(qbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32, h32);
+      }
 #pragma unroll
       for (int k = 0; k < 32; ++k) sacc += h32[k];
     }
@@ -618,10 +635,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   }
   for (int i = threadIdx.x; i < NSET * a.n_kv_heads * 64; i += 256) {
     const int set = i / (a.n_kv_heads * 64), ig = i - set * a.n_kv_heads * 64;
-    const int g = ig >> 6, b2 = (ig >> 4) & 3, gq = (ig >> 2) & 3, r = (ig & 3) + 4 * set;
+    const int g = ig >> 6, b2 = (ig >> 4) & 3, gq = (ig >> 2) & 3, r = (ig & 3) + (QF32 ? 0 : 4 * set);
     uint4 d = make_uint4(0, 0, 0, 0);
-    if (r < rep && owns(r, gq))
-      d = ld16(qbase + (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32 + b2 * 8);
+    if (r < rep && owns(r, gq)) {
+      if constexpr (QF32) {
+        float f8[8];
+        load_as_float<PIKV_F32, 8>(qfbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32 + b2 * 8, f8);
+        d = make_uint4(limb_bits(f8[0], set) | (limb_bits(f8[1], set) << 16), limb_bits(f8[2], set) | (limb_bits(f8[3], set) << 16),
+                       limb_bits(f8[4], set) | (limb_bits(f8[5], set) << 16), limb_bits(f8[6], set) | (limb_bits(f8[7], set) << 16));
+      } else {
+        d = ld16(qbase + (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32 + b2 * 8);
+      }
+    }
     alds[i] = make_uint4((d.x & 0xffffu) | (d.z << 16), (d.x >> 16) | (d.z & 0xffff0000u),
                          (d.y & 0xffffu) | (d.w << 16), (d.y >> 16) | (d.w & 0xffff0000u));
     if (set == 0) azero[ig] = make_uint4(0, 0, 0, 0);
@@ -686,6 +711,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
         const int mo = tl * meta_stride + g * 4 + rg;
         const float sc = (float)__builtin_bit_cast(_Float16, smeta[mo]);
         const float zq = (Q::sym ? 0.f : (float)__builtin_bit_cast(_Float16, zmeta[mo])) + zbias;
+        float limb_sum = 0.f;
 #pragma unroll
         for (int set = 0; set < NSET; ++set) {
           const float4 qv = qs4[(set * a.n_kv_heads + g) * 4 + rg];
@@ -698,7 +724,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
           const float u23 = __uint_as_float(s23[0]) + __uint_as_float(s23[1]);
           auto sf = __builtin_amdgcn_permlane32_swap(__float_as_uint(u01), __float_as_uint(u23), false, false);
           const float score = (__uint_as_float(sf[0]) + __uint_as_float(sf[1])) * a.scale_qk;
-          if (4 * set + rg < rep) stage[(g * SL + 4 * set + rg) * kTile + tl] = okt ? score : -__builtin_inff();
+          if constexpr (QF32) {
+            limb_sum += score;
+            if (set == NSET - 1 && rg < rep) stage[(g * SL + rg) * kTile + tl] = okt ? limb_sum : -__builtin_inff();
+          } else {
+            if (4 * set + rg < rep) stage[(g * SL + 4 * set + rg) * kTile + tl] = okt ? score : -__builtin_inff();
+          }
         }
       }
     }
@@ -886,13 +917,18 @@ static int launch_i8_mfma(const ScoreArgs& a, int n_caches, int64_t n_tiles, hip
 }
 
 template <int SCHEME, bool EXCH, bool NARROW>
-static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
+static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st, bool qf32) {
   const int rep = a.n_q_heads / a.n_kv_heads;
-  const int nset = rep <= 4 ? 1 : 2;
+  const int nset = (rep <= 4 && !qf32) ? 1 : 2;   // float32 queries: the second set holds their low limbs
   const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset);
-  if (rep > 8 || lds > 64 * 1024 || a.n_kv_heads > kGqaMaxKvHeads) return PIKV_ERR_UNSUPPORTED;
+  if (rep > (qf32 ? 4 : 8) || lds > 64 * 1024 || a.n_kv_heads > (qf32 ? 8 : kGqaMaxKvHeads)) return PIKV_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
-  if (nset == 1) {
+  if (qf32) {
+    if (a.n_kv_heads <= 4)
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
+    else
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
+  } else if (nset == 1) {
     if (a.n_kv_heads <= 4)
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a);
     else if (a.n_kv_heads <= 8)
@@ -910,9 +946,9 @@ static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, h
 }
 // a.n_kv_heads counts 128-dimension slabs, a.head_dim is the width of a stored kv head
 template <int SCHEME, bool EXCH = false>
-static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
-  return a.head_dim == 128 ? launch_gqa_slabs<SCHEME, EXCH, false>(a, n_caches, n_tiles, st)
-                           : launch_gqa_slabs<SCHEME, EXCH, true>(a, n_caches, n_tiles, st);
+static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st, bool qf32 = false) {
+  return a.head_dim == 128 ? launch_gqa_slabs<SCHEME, EXCH, false>(a, n_caches, n_tiles, st, qf32)
+                           : launch_gqa_slabs<SCHEME, EXCH, true>(a, n_caches, n_tiles, st, qf32);
 }
 
 // Final max and sum per (cache, q head) from the tile statistics [cache][tile][head].
@@ -1112,7 +1148,7 @@ int scores_exchange_launch(const void* k_codes, const void* k_scale, const void*
                            const int64_t* cache_row_base, const int32_t* cache_fill, int n_caches, int64_t max_len,
                            float* escores, float* tile_max, float* tile_sum, float* head_stats, hipStream_t st) {
   if (scheme != PIKV_Q_I4_ASYM && scheme != PIKV_Q_I4_SYM) return PIKV_ERR_UNSUPPORTED;
-  if (group != 32 || q_dtype != PIKV_BF16 || n_q_heads % n_kv_heads != 0) return PIKV_ERR_UNSUPPORTED;
+  if (group != 32 || (q_dtype != PIKV_BF16 && q_dtype != PIKV_F32) || n_q_heads % n_kv_heads != 0) return PIKV_ERR_UNSUPPORTED;
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
   if (hps == 0) return PIKV_ERR_UNSUPPORTED;
   const int slabs = n_kv_heads / hps;   // the kernel's kv heads are 128-dimension slabs of the row
@@ -1121,8 +1157,9 @@ int scores_exchange_launch(const void* k_codes, const void* k_scale, const void*
   ScoreArgs a{k_codes, k_scale, k_zero, q, cache_row_base, cache_fill, nullptr, tile_max, tile_sum,
               0, n_tiles, scale_qk, group, slabs, n_q_heads, head_dim, escores,
               (int)(max_len < 0x7fffffffLL ? max_len : 0x7fffffffLL), n_q_heads / slabs, 0, 1};
-  const int rc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM, true>(a, n_caches, n_tiles, st)
-                                            : launch_gqa<PIKV_Q_I4_SYM, true>(a, n_caches, n_tiles, st);
+  const bool qf32 = q_dtype == PIKV_F32;
+  const int rc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM, true>(a, n_caches, n_tiles, st, qf32)
+                                            : launch_gqa<PIKV_Q_I4_SYM, true>(a, n_caches, n_tiles, st, qf32);
   if (rc != PIKV_OK) return rc;
   launch_head_stats(tile_max, tile_sum, cache_fill, n_q_heads, n_tiles, n_caches, head_stats, st);
   return PIKV_OK;
@@ -1204,6 +1241,17 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   // grouped 4-bit caches read with bf16 queries go to the matrix-core kernels; heads of 64 or 32
   // dimensions are served as 128-dimension slabs of two or four neighbouring kv heads
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
+  // (float32 queries, up to 4 heads per slab: as two bf16 limbs on the same kernel)
+  if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_F32 && rep * hps <= 4) {
+    ScoreArgs as = a;
+    as.n_kv_heads = n_kv_heads / hps;
+    const int grc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(as, n_caches, n_tiles, st, true)
+                                               : launch_gqa<PIKV_Q_I4_SYM>(as, n_caches, n_tiles, st, true);
+    if (grc == PIKV_OK) {
+      PIKV_CHECK_LAUNCH();
+      return PIKV_OK;
+    }
+  }
   if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_BF16 && rep * hps <= (hps == 1 ? 16 : 8)) {
     int grc = PIKV_ERR_UNSUPPORTED;
     const size_t mlds = (size_t)n_q_heads * (kTile + 4) * sizeof(float);

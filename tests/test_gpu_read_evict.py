@@ -115,6 +115,43 @@ def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
     assert np.array_equal(np_of(pool.ts), ts_ref)
 
 
+@pytest.mark.parametrize("scheme,heads,hq,dh", [
+    (O.Q_I4_ASYM, 8, 32, 128),     # decode shape
+    (O.Q_I4_SYM, 2, 2, 128),
+    (O.Q_I4_ASYM, 4, 8, 64),       # two heads of 64 per slab, 2 query heads each
+    (O.Q_I4_ASYM, 3, 12, 128),     # 3 kv heads x 4
+])
+def test_scores_float32_queries_as_two_limbs(dev, scheme, heads, hq, dh):
+    """float32 queries on the 4-bit matrix-core kernel: every query element goes in as two bf16 limbs,
+    q = hi + lo + (at most 2^-17 |q|).  The scores against float64 on the dequantised rows: the error
+    bound of the limbs (2^-17 of sum |q k|) plus float32 accumulation, far inside the 1e-3 of the
+    row RMS that the float path is held to - and queries that ARE bf16 numbers give the scores of
+    the bf16 call bit for bit (their low limbs are zero)."""
+    group = 32
+    r = rng(90 + heads)
+    caps, lens = [200, 70], [193, 64]
+    pool, ref = _fill_pool(dev, r, caps, lens, heads, dh, group, scheme)
+    q = (r.standard_normal((2, hq, dh)) * (1.0 + 1e-3 * r.standard_normal((2, hq, dh)))).astype(np.float32)
+    assert not np.array_equal(q, O.bf16_round(q))
+    scale_qk = 1.0 / np.sqrt(dh)
+    sc = np_of(pool.scores(to_dev(q, dev, "f32"), hq)[0])
+    rep = hq // heads
+    for c, L in enumerate(lens):
+        rows = ref.valid_rows(c)
+        k_hat = O.dequantize_groups(ref.k_codes[rows], ref.k_scale[rows], ref.k_zero[rows], group).astype(np.float64)
+        k_hat = k_hat.reshape(L, heads, dh)
+        for h in range(hq):
+            want = k_hat[:, h // rep, :] @ q[c, h].astype(np.float64) * scale_qk
+            bound = (np.abs(k_hat[:, h // rep, :]) @ np.abs(q[c, h]).astype(np.float64)) * scale_qk
+            err = np.abs(sc[c, h, :L] - want)
+            assert (err <= 2.0 ** -15 * bound + 1e-7).all(), (c, h, (err / bound).max())
+    qb = O.bf16_round(q)
+    s_f = np_of(pool.scores(to_dev(qb, dev, "f32"), hq)[0])
+    s_b = np_of(pool.scores(to_dev(qb, dev, "bf16"), hq)[0])
+    for c, L in enumerate(lens):
+        assert np.array_equal(s_f[c, :, :L], s_b[c, :, :L])
+
+
 @pytest.mark.parametrize("scheme,group,heads,hq,dh,qdtype", [
     (O.Q_I4_ASYM, 32, 8, 32, 128, "bf16"),    # matrix-core 4-bit kernels
     (O.Q_I4_ASYM, 32, 8, 64, 128, "bf16"),    # ... two sets of query heads
