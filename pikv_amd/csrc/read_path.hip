@@ -504,9 +504,10 @@ constexpr int kGqaMaxKvHeads = 16;     // code vectors of one 16-token slice kep
 
 // LDS bytes of scores_mfma_i4_gqa_kernel: score staging, query sums, compact A
 // operands plus an all-zero twin, and the (scale, zero) rows of one tile.
-static size_t gqa_lds_bytes(int n_kv_heads, int nset) {
+// (na = copies of the A operands: one per set, or the two limbs of float32 queries)
+static size_t gqa_lds_bytes(int n_kv_heads, int nset, int na) {
   return (size_t)nset * n_kv_heads * 4 * kTile * sizeof(float) + (size_t)nset * n_kv_heads * 16 * sizeof(float) +
-         (size_t)(nset + 1) * n_kv_heads * 4 * 16 * 16 + 2 * (size_t)kTile * (n_kv_heads * 4 + 2) * sizeof(uint16_t);
+         (size_t)(na + 1) * n_kv_heads * 4 * 16 * 16 + 2 * (size_t)kTile * (n_kv_heads * 4 + 2) * sizeof(uint16_t);
 }
 
 // A wavefront owns one 16-token slice of the tile and walks over ALL kv heads, so
@@ -517,22 +518,23 @@ static size_t gqa_lds_bytes(int n_kv_heads, int nset) {
 // NSET sets of four query heads per kv head (1: up to 4 heads, 2: up to 8): the unpacked codes
 // of a kv head are multiplied with one block-diagonal A operand per set.
 // NARROW: heads of 64 or 32 dimensions (below); the kernel for heads of 128 carries none of it.
-// QF32 (two sets, up to 4 query heads per kv head): float32 queries.  A query element goes in as two
+// QF32 (one set, up to 4 query heads per kv head): float32 queries.  A query element goes in as two
 // bf16 limbs, q = hi + lo + (at most 2^-17 |q|), hi = the float cut to its upper 16 bits, lo = the rest
-// rounded to bf16: set 0 holds the hi limbs of the heads, set 1 the lo limbs, and the two scores of a
-// head are added before they are staged.
+// rounded to bf16: two copies of the A operands, one per limb, are multiplied with the same unpacked
+// codes into the same accumulators, and the group sums of q are those of hi + lo.
 template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false, bool NARROW = false, bool QF32 = false>  // NKV = n_kv_heads rounded up to 4/8/16; EXCH: exchange format out
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET <= 8 ? 4 : 2))) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
   constexpr int SL = 4 * NSET;  // head slots per kv head
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
   static_assert(kGqaTilesPerBlock % 2 == 0, "tiles are processed in pairs");
-  static_assert(!QF32 || NSET == 2, "float32 queries: one set per limb");
+  static_assert(!QF32 || NSET == 1, "float32 queries: one set, two limbs");
+  constexpr int NA = QF32 ? 2 : NSET;  // copies of the A operands
   extern __shared__ float gqa_lds[];
   float* stage = gqa_lds;                            // [kv head][SL head slots][token in tile]
   float4* qs4 = reinterpret_cast<float4*>(stage + a.n_kv_heads * SL * kTile);  // [set][kv head][group]: q sums of the set's 4 heads
   uint4* alds = reinterpret_cast<uint4*>(qs4 + NSET * a.n_kv_heads * 4);  // [set][kv head][b][gq*4 + r]
-  uint4* azero = alds + NSET * a.n_kv_heads * 64;                         // [kv head][b][gq*4 + r], all zero
+  uint4* azero = alds + NA * a.n_kv_heads * 64;                           // [kv head][b][gq*4 + r], all zero
   const int meta_stride = a.n_kv_heads * 4 + 2;      // halves; +2 spreads the tokens over banks
   uint16_t* smeta = reinterpret_cast<uint16_t*>(azero + a.n_kv_heads * 64);
   uint16_t* zmeta = smeta + kTile * meta_stride;
@@ -617,14 +619,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   // the slab and the head's own dimensions start at group (r / rep1) * gph)
   for (int i = threadIdx.x; i < NSET * a.n_kv_heads * 16; i += 256) {
     const int set = i / (a.n_kv_heads * 16), ig = i - set * a.n_kv_heads * 16;
-    const int g = ig >> 4, gq = (ig >> 2) & 3, r = (ig & 3) + (QF32 ? 0 : 4 * set);
+    const int g = ig >> 4, gq = (ig >> 2) & 3, r = (ig & 3) + 4 * set;
     float sacc = 0.f;
     if (r < rep && owns(r, gq)) {
       float h32[32];
       if constexpr (QF32) {
         load_as_float<PIKV_F32, 32>(qfbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32, h32);
 #pragma unroll
-        for (int k = 0; k < 32; ++k) h32[k] = bf16_bits_to_float(limb_bits(h32[k], set));
+        for (int k = 0; k < 32; ++k) h32[k] = bf16_bits_to_float(limb_bits(h32[k], 0)) + bf16_bits_to_float(limb_bits(h32[k], 1));
       } else {
         load_as_float<PIKV_BF16, 32>(qbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32, h32);
       }
@@ -633,7 +635,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     }
     reinterpret_cast<float*>(qs4)[i] = sacc;
   }
-  for (int i = threadIdx.x; i < NSET * a.n_kv_heads * 64; i += 256) {
+  for (int i = threadIdx.x; i < NA * a.n_kv_heads * 64; i += 256) {   // set = copy: a set of heads, or a limb
     const int set = i / (a.n_kv_heads * 64), ig = i - set * a.n_kv_heads * 64;
     const int g = ig >> 6, b2 = (ig >> 4) & 3, gq = (ig >> 2) & 3, r = (ig & 3) + (QF32 ? 0 : 4 * set);
     uint4 d = make_uint4(0, 0, 0, 0);
@@ -655,9 +657,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   const float zbias = 128.0f - (float)Q::qmin;  // 128 (asymmetric) or 136 (symmetric)
   // a lane whose k-slice does not meet its row's group reads zeros
   const bool a_on = (nl >> 2) == rg;
-  const uint4* a_lane[NSET];
+  const uint4* a_lane[NA];
 #pragma unroll
-  for (int set = 0; set < NSET; ++set) a_lane[set] = (a_on ? alds + set * a.n_kv_heads * 64 : azero) + nl;
+  for (int set = 0; set < NA; ++set) a_lane[set] = (a_on ? alds + set * a.n_kv_heads * 64 : azero) + nl;
   // two nibbles -> two bf16 values 128 + code.  Both constants are kept in vector registers
   // (the empty statement hides their values from the compiler, it emits no instruction): with
   // a literal or scalar operand the three-operand and-or instruction cannot be encoded and
@@ -702,16 +704,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
           const uint4 bb = make_uint4(and_or(w, kNib, kExp), and_or(w >> 4, kNib, kExp),
                                       and_or(w >> 8, kNib, kExp), and_or(w >> 12, kNib, kExp));
 #pragma unroll
-          for (int set = 0; set < NSET; ++set) {
+          for (int set = 0; set < NA; ++set) {   // the limbs of float32 queries meet in one accumulator
             const uint4 av = a_lane[set][(g * 4 + b2) * 16];
-            pc[set] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, av),
-                                                              __builtin_bit_cast(pikv_bf16x8, bb), pc[set], 0, 0, 0);
+            pc[QF32 ? 0 : set] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                __builtin_bit_cast(pikv_bf16x8, av), __builtin_bit_cast(pikv_bf16x8, bb), pc[QF32 ? 0 : set], 0, 0, 0);
           }
         }
         const int mo = tl * meta_stride + g * 4 + rg;
         const float sc = (float)__builtin_bit_cast(_Float16, smeta[mo]);
         const float zq = (Q::sym ? 0.f : (float)__builtin_bit_cast(_Float16, zmeta[mo])) + zbias;
-        float limb_sum = 0.f;
 #pragma unroll
         for (int set = 0; set < NSET; ++set) {
           const float4 qv = qs4[(set * a.n_kv_heads + g) * 4 + rg];
@@ -724,12 +725,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
           const float u23 = __uint_as_float(s23[0]) + __uint_as_float(s23[1]);
           auto sf = __builtin_amdgcn_permlane32_swap(__float_as_uint(u01), __float_as_uint(u23), false, false);
           const float score = (__uint_as_float(sf[0]) + __uint_as_float(sf[1])) * a.scale_qk;
-          if constexpr (QF32) {
-            limb_sum += score;
-            if (set == NSET - 1 && rg < rep) stage[(g * SL + rg) * kTile + tl] = okt ? limb_sum : -__builtin_inff();
-          } else {
-            if (4 * set + rg < rep) stage[(g * SL + 4 * set + rg) * kTile + tl] = okt ? score : -__builtin_inff();
-          }
+          if (4 * set + rg < rep) stage[(g * SL + 4 * set + rg) * kTile + tl] = okt ? score : -__builtin_inff();
         }
       }
     }
@@ -919,15 +915,15 @@ static int launch_i8_mfma(const ScoreArgs& a, int n_caches, int64_t n_tiles, hip
 template <int SCHEME, bool EXCH, bool NARROW>
 static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st, bool qf32) {
   const int rep = a.n_q_heads / a.n_kv_heads;
-  const int nset = (rep <= 4 && !qf32) ? 1 : 2;   // float32 queries: the second set holds their low limbs
-  const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset);
+  const int nset = rep <= 4 ? 1 : 2;
+  const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset, qf32 ? 2 : nset);   // float32 queries: a copy of the A operands per limb
   if (rep > (qf32 ? 4 : 8) || lds > 64 * 1024 || a.n_kv_heads > (qf32 ? 8 : kGqaMaxKvHeads)) return PIKV_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
   if (qf32) {
     if (a.n_kv_heads <= 4)
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
     else
-      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
   } else if (nset == 1) {
     if (a.n_kv_heads <= 4)
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a);

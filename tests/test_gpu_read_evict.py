@@ -123,10 +123,11 @@ def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
 ])
 def test_scores_float32_queries_as_two_limbs(dev, scheme, heads, hq, dh):
     """float32 queries on the 4-bit matrix-core kernel: every query element goes in as two bf16 limbs,
-    q = hi + lo + (at most 2^-17 |q|).  The scores against float64 on the dequantised rows: the error
-    bound of the limbs (2^-17 of sum |q k|) plus float32 accumulation, far inside the 1e-3 of the
-    row RMS that the float path is held to - and queries that ARE bf16 numbers give the scores of
-    the bf16 call bit for bit (their low limbs are zero)."""
+    q = hi + lo + (at most 2^-17 |q|).  The scores against float64 on the dequantised rows: within
+    2^-14 of sum |q k| - the limbs' 2^-17 plus the float32 rounding of accumulators that carry the
+    codes with an offset of 128 (the same for bf16 queries) - far inside the 1e-3 of the row RMS
+    that the float path is held to; and queries that ARE bf16 numbers give the scores of the bf16
+    call bit for bit (their low limbs are zero)."""
     group = 32
     r = rng(90 + heads)
     caps, lens = [200, 70], [193, 64]
@@ -144,7 +145,7 @@ def test_scores_float32_queries_as_two_limbs(dev, scheme, heads, hq, dh):
             want = k_hat[:, h // rep, :] @ q[c, h].astype(np.float64) * scale_qk
             bound = (np.abs(k_hat[:, h // rep, :]) @ np.abs(q[c, h]).astype(np.float64)) * scale_qk
             err = np.abs(sc[c, h, :L] - want)
-            assert (err <= 2.0 ** -15 * bound + 1e-7).all(), (c, h, (err / bound).max())
+            assert (err <= 2.0 ** -14 * bound + 1e-7).all(), (c, h, (err / bound).max())
     qb = O.bf16_round(q)
     s_f = np_of(pool.scores(to_dev(qb, dev, "f32"), hq)[0])
     s_b = np_of(pool.scores(to_dev(qb, dev, "bf16"), hq)[0])
