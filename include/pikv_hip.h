@@ -311,7 +311,7 @@ int pikv_gather_dequant(const void* codes, const void* scale, const void* zero,
  *   the number of rows per cache the caller wants covered.
  *   D = n_kv_heads*head_dim; head_dim a power of two >= 16 (8-bit) / 32 (4-bit);
  *   any number of kv heads, any n_q_heads that is a multiple of n_kv_heads, for
- *   either q_dtype.  float32 queries against 4-bit group-32 caches with up to 4
+ *   either q_dtype.  float32 queries against 4-bit group-32 caches with up to 8
  *   query heads per 128 dimensions of kv heads are multiplied on the matrix cores as
  *   two bf16 limbs (q = hi + lo to 2^-17 |q|; float32 accumulation). */
 #define PIKV_SCORE_TILE 64
@@ -389,8 +389,8 @@ int64_t pikv_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim,
  * Same results as pikv_gather_dequant_scores + pikv_h2o_accumulate + pikv_attend_values
  * (to the float tolerance of those), but the score matrix never leaves the library: for
  * 4-bit caches with group 32, rows that are 1 to 8 slabs of 128 dimensions (a slab is one kv
- * head of 128 dimensions, two of 64 or four of 32) and up to 8 query heads per slab (bf16
- * queries; float32 queries: up to 4) the two matrix-core kernels exchange exp(score - tile max)
+ * head of 128 dimensions, two of 64 or four of 32) and up to 8 query heads per slab (5 to 8
+ * heads with float32 queries: up to 7 slabs) the two matrix-core kernels exchange exp(score - tile max)
  * with a tile's heads side by side, so that both sides stream contiguous 8 KB runs instead
  * of the 256-byte pieces of a [head][token] score matrix; every other format runs the three
  * steps with float scores in the workspace.

@@ -1130,7 +1130,7 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
   const bool hk_ok = slabs >= 1 && slabs <= 8;
   const int64_t splits = attend_splits(n_caches, max_len);
   if ((scheme == PIKV_Q_I4_ASYM || scheme == PIKV_Q_I4_SYM) && group == 32 && rep >= 1 &&
-      rep * hps <= 8 && hk_ok && (q_dtype == PIKV_BF16 || (q_dtype == PIKV_F32 && rep * hps <= 4)) && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {
+      rep * hps <= 8 && hk_ok && (q_dtype == PIKV_BF16 || q_dtype == PIKV_F32) && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {
     float* esc = reinterpret_cast<float*>(ws + w.scores);
     const int rc = scores_exchange_launch(k_codes, k_scale, k_zero, scheme, group, n_kv_heads, n_q_heads, head_dim, q,
                                           q_dtype, scale_qk, cache_row_base, cache_fill, n_caches, max_len, esc, tmax,

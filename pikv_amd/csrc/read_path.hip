@@ -518,18 +518,18 @@ static size_t gqa_lds_bytes(int n_kv_heads, int nset, int na) {
 // NSET sets of four query heads per kv head (1: up to 4 heads, 2: up to 8): the unpacked codes
 // of a kv head are multiplied with one block-diagonal A operand per set.
 // NARROW: heads of 64 or 32 dimensions (below); the kernel for heads of 128 carries none of it.
-// QF32 (one set, up to 4 query heads per kv head): float32 queries.  A query element goes in as two
-// bf16 limbs, q = hi + lo + (at most 2^-17 |q|), hi = the float cut to its upper 16 bits, lo = the rest
-// rounded to bf16: two copies of the A operands, one per limb, are multiplied with the same unpacked
-// codes into the same accumulators, and the group sums of q are those of hi + lo.
+// QF32: float32 queries.  A query element goes in as two bf16 limbs, q = hi + lo + (at most
+// 2^-17 |q|), hi = the float cut to its upper 16 bits, lo = the rest rounded to bf16: two copies of a
+// set's A operands, one per limb, are multiplied with the same unpacked codes into the same
+// accumulators, and the group sums of q are those of hi + lo.
 template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false, bool NARROW = false, bool QF32 = false>  // NKV = n_kv_heads rounded up to 4/8/16; EXCH: exchange format out
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET <= 8 ? 4 : 2))) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
   constexpr int SL = 4 * NSET;  // head slots per kv head
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
   static_assert(kGqaTilesPerBlock % 2 == 0, "tiles are processed in pairs");
-  static_assert(!QF32 || NSET == 1, "float32 queries: one set, two limbs");
-  constexpr int NA = QF32 ? 2 : NSET;  // copies of the A operands
+  constexpr int NL = QF32 ? 2 : 1;     // limbs of a query element
+  constexpr int NA = NL * NSET;        // copies of the A operands: copy = set * NL + limb
   extern __shared__ float gqa_lds[];
   float* stage = gqa_lds;                            // [kv head][SL head slots][token in tile]
   float4* qs4 = reinterpret_cast<float4*>(stage + a.n_kv_heads * SL * kTile);  // [set][kv head][group]: q sums of the set's 4 heads
@@ -635,23 +635,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     }
     reinterpret_cast<float*>(qs4)[i] = sacc;
   }
-  for (int i = threadIdx.x; i < NA * a.n_kv_heads * 64; i += 256) {   // set = copy: a set of heads, or a limb
-    const int set = i / (a.n_kv_heads * 64), ig = i - set * a.n_kv_heads * 64;
-    const int g = ig >> 6, b2 = (ig >> 4) & 3, gq = (ig >> 2) & 3, r = (ig & 3) + (QF32 ? 0 : 4 * set);
+  for (int i = threadIdx.x; i < NA * a.n_kv_heads * 64; i += 256) {
+    const int copy = i / (a.n_kv_heads * 64), ig = i - copy * a.n_kv_heads * 64;
+    const int set = copy / NL, limb = copy % NL;
+    const int g = ig >> 6, b2 = (ig >> 4) & 3, gq = (ig >> 2) & 3, r = (ig & 3) + 4 * set;
     uint4 d = make_uint4(0, 0, 0, 0);
     if (r < rep && owns(r, gq)) {
       if constexpr (QF32) {
         float f8[8];
         load_as_float<PIKV_F32, 8>(qfbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32 + b2 * 8, f8);
-        d = make_uint4(limb_bits(f8[0], set) | (limb_bits(f8[1], set) << 16), limb_bits(f8[2], set) | (limb_bits(f8[3], set) << 16),
-                       limb_bits(f8[4], set) | (limb_bits(f8[5], set) << 16), limb_bits(f8[6], set) | (limb_bits(f8[7], set) << 16));
+        d = make_uint4(limb_bits(f8[0], limb) | (limb_bits(f8[1], limb) << 16), limb_bits(f8[2], limb) | (limb_bits(f8[3], limb) << 16),
+                       limb_bits(f8[4], limb) | (limb_bits(f8[5], limb) << 16), limb_bits(f8[6], limb) | (limb_bits(f8[7], limb) << 16));
       } else {
         d = ld16(qbase + (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32 + b2 * 8);
       }
     }
     alds[i] = make_uint4((d.x & 0xffffu) | (d.z << 16), (d.x >> 16) | (d.z & 0xffff0000u),
                          (d.y & 0xffffu) | (d.w << 16), (d.y >> 16) | (d.w & 0xffff0000u));
-    if (set == 0) azero[ig] = make_uint4(0, 0, 0, 0);
+    if (copy == 0) azero[ig] = make_uint4(0, 0, 0, 0);
   }
 
   const float zbias = 128.0f - (float)Q::qmin;  // 128 (asymmetric) or 136 (symmetric)
@@ -704,10 +705,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
           const uint4 bb = make_uint4(and_or(w, kNib, kExp), and_or(w >> 4, kNib, kExp),
                                       and_or(w >> 8, kNib, kExp), and_or(w >> 12, kNib, kExp));
 #pragma unroll
-          for (int set = 0; set < NA; ++set) {   // the limbs of float32 queries meet in one accumulator
-            const uint4 av = a_lane[set][(g * 4 + b2) * 16];
-            pc[QF32 ? 0 : set] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                __builtin_bit_cast(pikv_bf16x8, av), __builtin_bit_cast(pikv_bf16x8, bb), pc[QF32 ? 0 : set], 0, 0, 0);
+          for (int copy = 0; copy < NA; ++copy) {   // the limbs of float32 queries meet in one accumulator
+            const uint4 av = a_lane[copy][(g * 4 + b2) * 16];
+            pc[copy / NL] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                __builtin_bit_cast(pikv_bf16x8, av), __builtin_bit_cast(pikv_bf16x8, bb), pc[copy / NL], 0, 0, 0);
           }
         }
         const int mo = tl * meta_stride + g * 4 + rg;
@@ -916,14 +917,19 @@ template <int SCHEME, bool EXCH, bool NARROW>
 static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st, bool qf32) {
   const int rep = a.n_q_heads / a.n_kv_heads;
   const int nset = rep <= 4 ? 1 : 2;
-  const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset, qf32 ? 2 : nset);   // float32 queries: a copy of the A operands per limb
-  if (rep > (qf32 ? 4 : 8) || lds > 64 * 1024 || a.n_kv_heads > (qf32 ? 8 : kGqaMaxKvHeads)) return PIKV_ERR_UNSUPPORTED;
+  const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset, qf32 ? 2 * nset : nset);   // float32 queries: a copy of the A operands per limb
+  if (rep > 8 || lds > 64 * 1024 || a.n_kv_heads > (qf32 ? 8 : kGqaMaxKvHeads)) return PIKV_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
-  if (qf32) {
+  if (qf32 && nset == 1) {
     if (a.n_kv_heads <= 4)
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
     else
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
+  } else if (qf32) {
+    if (a.n_kv_heads <= 4)
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
+    else
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
   } else if (nset == 1) {
     if (a.n_kv_heads <= 4)
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a);
@@ -1237,8 +1243,8 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   // grouped 4-bit caches read with bf16 queries go to the matrix-core kernels; heads of 64 or 32
   // dimensions are served as 128-dimension slabs of two or four neighbouring kv heads
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
-  // (float32 queries, up to 4 heads per slab: as two bf16 limbs on the same kernel)
-  if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_F32 && rep * hps <= 4) {
+  // (float32 queries: as two bf16 limbs on the same kernel, where its operands fit)
+  if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_F32 && rep * hps <= 8) {
     ScoreArgs as = a;
     as.n_kv_heads = n_kv_heads / hps;
     const int grc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(as, n_caches, n_tiles, st, true)

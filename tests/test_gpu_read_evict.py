@@ -120,6 +120,8 @@ def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
     (O.Q_I4_SYM, 2, 2, 128),
     (O.Q_I4_ASYM, 4, 8, 64),       # two heads of 64 per slab, 2 query heads each
     (O.Q_I4_ASYM, 3, 12, 128),     # 3 kv heads x 4
+    (O.Q_I4_ASYM, 4, 28, 128),     # 7 query heads per kv head: two sets of heads, two limbs each
+    (O.Q_I4_SYM, 1, 8, 128),
 ])
 def test_scores_float32_queries_as_two_limbs(dev, scheme, heads, hq, dh):
     """float32 queries on the 4-bit matrix-core kernel: every query element goes in as two bf16 limbs,
