@@ -311,9 +311,10 @@ int pikv_gather_dequant(const void* codes, const void* scale, const void* zero,
  *   the number of rows per cache the caller wants covered.
  *   D = n_kv_heads*head_dim; head_dim a power of two >= 16 (8-bit) / 32 (4-bit);
  *   any number of kv heads, any n_q_heads that is a multiple of n_kv_heads, for
- *   either q_dtype.  float32 queries against 4-bit group-32 caches with up to 8
- *   query heads per 128 dimensions of kv heads are multiplied on the matrix cores as
- *   two bf16 limbs (q = hi + lo to 2^-17 |q|; float32 accumulation). */
+ *   either q_dtype.  float32 queries against 4-bit group-32 caches, or 8-bit caches
+ *   with a scale per kv head or coarser, with up to 8 query heads per 128 dimensions
+ *   of kv heads are multiplied on the matrix cores as two bf16 limbs (q = hi + lo to
+ *   2^-17 |q|; float32 accumulation). */
 #define PIKV_SCORE_TILE 64
 int pikv_gather_dequant_scores(const void* k_codes, const void* k_scale,
                                const void* k_zero, int scheme, int group,

@@ -768,7 +768,10 @@ constexpr int kI8TilesPerBlock = 4;
 // the cached row, each the stored bytes of HPS neighbouring kv heads; the rep query heads of a slab
 // are the heads of those kv heads, rep / HPS each, in order.  A query head's A rows are zero outside
 // its own kv head's dimensions, and its scores take that kv head's scale and zero point.
-template <int SCHEME, int NHW, int HPS = 1>  // NHW = kv heads per wavefront: ceil(n_kv_heads / 4), 1, 2 or 4
+// QF32 (up to 8 query heads per slab): float32 queries as two bf16 limbs, q = hi + lo + (at most
+// 2^-17 |q|): A rows 2r and 2r+1 hold the limbs of head r, and the two rows' scores - they sit in
+// the same lane - are added before they are staged.
+template <int SCHEME, int NHW, int HPS = 1, bool QF32 = false>  // NHW = kv heads per wavefront: ceil(n_kv_heads / 4), 1, 2 or 4
 __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 8, "8-bit schemes only");
@@ -791,10 +794,13 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   const int rep1 = HPS == 1 ? rep : HPS == 2 ? rep >> 1 : rep >> 2;   // query heads per kv head
   // kv head (inside the slab) of query head r: comparisons, no integer division
   auto head_in_slab = [&](int r) { return HPS == 1 ? 0 : (r >= rep1) + (r >= 2 * rep1) + (r >= 3 * rep1); };
-  const int hh_a = head_in_slab(nl);  // ... of the query head in A row nl (rows >= rep hold no head)
-  int hh_c[4];                        // ... of the query heads in this lane's four C rows
+  constexpr int RSH = QF32 ? 1 : 0;   // A / C row -> query head of the kv group: row >> RSH (two limb rows per head)
+  const int hh_a = head_in_slab(nl >> RSH);  // ... of the query head in A row nl (rows past the heads hold none)
+  int hh_c[4];                               // ... of the query heads in this lane's four C rows
 #pragma unroll
-  for (int qq = 0; qq < 4; ++qq) hh_c[qq] = head_in_slab(4 * rg + qq) < HPS ? head_in_slab(4 * rg + qq) : HPS - 1;
+  for (int qq = 0; qq < 4; ++qq)
+    hh_c[qq] = head_in_slab((4 * rg + qq) >> RSH) < HPS ? head_in_slab((4 * rg + qq) >> RSH) : HPS - 1;
+  const float* qfbase = reinterpret_cast<const float*>(a.q) + (int64_t)c * a.n_q_heads * (128 / HPS);
   // two nibbles -> two bf16 values 16 + nibble; both constants held in vector registers so that the
   // three-operand and-or instruction can be encoded (the empty statement emits no instruction)
   uint32_t kNib = 0x00780078u, kExp = 0x41804180u;
@@ -808,13 +814,27 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
 #pragma unroll
   for (int hs = 0; hs < NHW; ++hs) {
     const int g = wave + 4 * hs;
-    const bool on = g < a.n_kv_heads && nl < rep;
+    const bool on = g < a.n_kv_heads && (nl >> RSH) < rep;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       uint2 qd = make_uint2(0, 0);
       const int ds = 64 * (ks >> 2) + 16 * rg + 4 * (ks & 3);   // dimension inside the slab
-      if (on && (HPS == 1 || ds / (128 / HPS) == hh_a))
-        qd = *reinterpret_cast<const uint2*>(qbase + (int64_t)(g * rep + nl) * (128 / HPS) + (ds - hh_a * (128 / HPS)));
+      if (on && (HPS == 1 || ds / (128 / HPS) == hh_a)) {
+        const int64_t qo = (int64_t)(g * rep + (nl >> RSH)) * (128 / HPS) + (ds - hh_a * (128 / HPS));
+        if constexpr (QF32) {
+          float f4[4];
+          load_as_float<PIKV_F32, 4>(qfbase, qo, f4);
+          uint32_t lb[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {   // limb nl & 1: the float cut to its upper 16 bits, or the rest rounded to bf16
+            const uint32_t hb = __float_as_uint(f4[k]) & 0xffff0000u;
+            lb[k] = (nl & 1) ? float_to_bf16_bits(f4[k] - __uint_as_float(hb)) : hb >> 16;
+          }
+          qd = make_uint2(lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16));
+        } else {
+          qd = *reinterpret_cast<const uint2*>(qbase + qo);
+        }
+      }
       // bf16 x 16: through float, exact (zero stays zero)
       auto x16 = [](uint32_t h) { return __float_as_uint(__uint_as_float(h << 16) * 16.0f) >> 16; };
       const uint32_t q0 = qd.x & 0xffffu, q1 = qd.x >> 16, q2 = qd.y & 0xffffu, q3 = qd.y >> 16;
@@ -877,19 +897,31 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
                                                          __builtin_bit_cast(pikv_bf16x8, bb), pc, 0, 0, 0);
           }
         }
+        float row_score[4];
 #pragma unroll
         for (int qq = 0; qq < 4; ++qq) {
-          const int r = 4 * rg + qq;
-          if (r < rep) {
-            float scl = sc[sl][0], zrl = zr[sl][0];
+          float scl = sc[sl][0], zrl = zr[sl][0];
 #pragma unroll
-            for (int k = 1; k < HPS; ++k) {
-              scl = hh_c[qq] == k ? sc[sl][k] : scl;
-              zrl = hh_c[qq] == k ? zr[sl][k] : zrl;
-            }
-            const float zz = 272.0f + (Q::sym ? 128.0f : zrl);
-            const float score = scl * fmaf(-zz, qs[hs][qq], pc[qq]) * a.scale_qk;
-            stage[(g * rep + r) * kTile + 16 * sl + nl] = ok[sl] ? score : -__builtin_inff();
+          for (int k = 1; k < HPS; ++k) {
+            scl = hh_c[qq] == k ? sc[sl][k] : scl;
+            zrl = hh_c[qq] == k ? zr[sl][k] : zrl;
+          }
+          const float zz = 272.0f + (Q::sym ? 128.0f : zrl);
+          row_score[qq] = scl * fmaf(-zz, qs[hs][qq], pc[qq]) * a.scale_qk;
+        }
+        if constexpr (QF32) {
+#pragma unroll
+          for (int hq2 = 0; hq2 < 2; ++hq2) {   // rows (2 hq2, 2 hq2 + 1) of this lane: the limbs of one head
+            const int r = 2 * rg + hq2;
+            if (r < rep)
+              stage[(g * rep + r) * kTile + 16 * sl + nl] =
+                  ok[sl] ? row_score[2 * hq2] + row_score[2 * hq2 + 1] : -__builtin_inff();
+          }
+        } else {
+#pragma unroll
+          for (int qq = 0; qq < 4; ++qq) {
+            const int r = 4 * rg + qq;
+            if (r < rep) stage[(g * rep + r) * kTile + 16 * sl + nl] = ok[sl] ? row_score[qq] : -__builtin_inff();
           }
         }
       }
@@ -900,16 +932,21 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   }
 }
 
-template <int SCHEME, int HPS = 1>
-static int launch_i8_mfma(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
+template <int SCHEME, int HPS, bool QF32>
+static void launch_i8_mfma_q(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
   const size_t lds = (size_t)a.n_q_heads * kTile * sizeof(float);
   const dim3 grid((unsigned)((n_tiles + kI8TilesPerBlock - 1) / kI8TilesPerBlock), (unsigned)n_caches);
   if (a.n_kv_heads <= 4)
-    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 1, HPS>), grid, dim3(256), lds, st, a);
+    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 1, HPS, QF32>), grid, dim3(256), lds, st, a);
   else if (a.n_kv_heads <= 8)
-    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 2, HPS>), grid, dim3(256), lds, st, a);
+    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 2, HPS, QF32>), grid, dim3(256), lds, st, a);
   else
-    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 4, HPS>), grid, dim3(256), lds, st, a);
+    hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 4, HPS, QF32>), grid, dim3(256), lds, st, a);
+}
+template <int SCHEME, int HPS = 1>
+static int launch_i8_mfma(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st, bool qf32) {
+  if (qf32) launch_i8_mfma_q<SCHEME, HPS, true>(a, n_caches, n_tiles, st);
+  else launch_i8_mfma_q<SCHEME, HPS, false>(a, n_caches, n_tiles, st);
   return PIKV_OK;
 }
 
@@ -1279,14 +1316,15 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   }
   // 8-bit caches with per-head (or coarser) scales, several bf16 query heads per kv head
   // (heads of 64 or 32 dimensions as 128-dimension slabs of two or four neighbouring kv heads)
-  if (eight && hps > 0 && group % head_dim == 0 && q_dtype == PIKV_BF16 && rep >= 2 && rep * hps <= 16 &&
-      n_kv_heads / hps <= 16) {
+  // (float32 queries as two bf16 limbs, two operand rows per head: up to 8 heads per slab)
+  const bool qf32 = q_dtype == PIKV_F32;
+  if (eight && hps > 0 && group % head_dim == 0 && rep >= 2 && rep * hps <= (qf32 ? 8 : 16) && n_kv_heads / hps <= 16) {
     ScoreArgs as = a;
     as.n_kv_heads = n_kv_heads / hps;
     const bool sym = scheme == PIKV_Q_I8_SYM;
-    if (hps == 1) sym ? launch_i8_mfma<PIKV_Q_I8_SYM>(as, n_caches, n_tiles, st) : launch_i8_mfma<PIKV_Q_I8_ASYM>(as, n_caches, n_tiles, st);
-    else if (hps == 2) sym ? launch_i8_mfma<PIKV_Q_I8_SYM, 2>(as, n_caches, n_tiles, st) : launch_i8_mfma<PIKV_Q_I8_ASYM, 2>(as, n_caches, n_tiles, st);
-    else sym ? launch_i8_mfma<PIKV_Q_I8_SYM, 4>(as, n_caches, n_tiles, st) : launch_i8_mfma<PIKV_Q_I8_ASYM, 4>(as, n_caches, n_tiles, st);
+    if (hps == 1) sym ? launch_i8_mfma<PIKV_Q_I8_SYM>(as, n_caches, n_tiles, st, qf32) : launch_i8_mfma<PIKV_Q_I8_ASYM>(as, n_caches, n_tiles, st, qf32);
+    else if (hps == 2) sym ? launch_i8_mfma<PIKV_Q_I8_SYM, 2>(as, n_caches, n_tiles, st, qf32) : launch_i8_mfma<PIKV_Q_I8_ASYM, 2>(as, n_caches, n_tiles, st, qf32);
+    else sym ? launch_i8_mfma<PIKV_Q_I8_SYM, 4>(as, n_caches, n_tiles, st, qf32) : launch_i8_mfma<PIKV_Q_I8_ASYM, 4>(as, n_caches, n_tiles, st, qf32);
     PIKV_CHECK_LAUNCH();
     return PIKV_OK;
   }

@@ -115,22 +115,24 @@ def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
     assert np.array_equal(np_of(pool.ts), ts_ref)
 
 
-@pytest.mark.parametrize("scheme,heads,hq,dh", [
-    (O.Q_I4_ASYM, 8, 32, 128),     # decode shape
-    (O.Q_I4_SYM, 2, 2, 128),
-    (O.Q_I4_ASYM, 4, 8, 64),       # two heads of 64 per slab, 2 query heads each
-    (O.Q_I4_ASYM, 3, 12, 128),     # 3 kv heads x 4
-    (O.Q_I4_ASYM, 4, 28, 128),     # 7 query heads per kv head: two sets of heads, two limbs each
-    (O.Q_I4_SYM, 1, 8, 128),
+@pytest.mark.parametrize("scheme,group,heads,hq,dh", [
+    (O.Q_I4_ASYM, 32, 8, 32, 128),     # decode shape
+    (O.Q_I4_SYM, 32, 2, 2, 128),
+    (O.Q_I4_ASYM, 32, 4, 8, 64),       # two heads of 64 per slab, 2 query heads each
+    (O.Q_I4_ASYM, 32, 3, 12, 128),     # 3 kv heads x 4
+    (O.Q_I4_ASYM, 32, 4, 28, 128),     # 7 query heads per kv head: two sets of heads, two limbs each
+    (O.Q_I4_SYM, 32, 1, 8, 128),
+    (O.Q_I8_SYM, 128, 8, 32, 128),     # 8-bit kernel: two operand rows per head
+    (O.Q_I8_ASYM, 128, 2, 16, 128),    # ... all 16 rows in use
+    (O.Q_I8_ASYM, 64, 4, 16, 64),      # ... heads of 64
 ])
-def test_scores_float32_queries_as_two_limbs(dev, scheme, heads, hq, dh):
-    """float32 queries on the 4-bit matrix-core kernel: every query element goes in as two bf16 limbs,
+def test_scores_float32_queries_as_two_limbs(dev, scheme, group, heads, hq, dh):
+    """float32 queries on the matrix-core score kernels: every query element goes in as two bf16 limbs,
     q = hi + lo + (at most 2^-17 |q|).  The scores against float64 on the dequantised rows: within
     2^-14 of sum |q k| - the limbs' 2^-17 plus the float32 rounding of accumulators that carry the
     codes with an offset of 128 (the same for bf16 queries) - far inside the 1e-3 of the row RMS
     that the float path is held to; and queries that ARE bf16 numbers give the scores of the bf16
     call bit for bit (their low limbs are zero)."""
-    group = 32
     r = rng(90 + heads)
     caps, lens = [200, 70], [193, 64]
     pool, ref = _fill_pool(dev, r, caps, lens, heads, dh, group, scheme)
