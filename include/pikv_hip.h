@@ -389,7 +389,8 @@ int64_t pikv_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim,
  *   H2OScheduler.update_attention_scores (core/single/cache_scheduling.py:69-73).
  * Same results as pikv_gather_dequant_scores + pikv_h2o_accumulate + pikv_attend_values
  * (to the float tolerance of those), but the score matrix never leaves the library: for
- * 4-bit caches with group 32, rows that are 1 to 8 slabs of 128 dimensions (a slab is one kv
+ * 4-bit caches with group 32, rows that are 1 to 8 slabs of 128 dimensions, or whole groups
+ * of 8 kv heads of 128 dimensions (a slab is one kv
  * head of 128 dimensions, two of 64 or four of 32) and up to 8 query heads per slab (5 to 8
  * heads with float32 queries: up to 7 slabs) the two matrix-core kernels exchange exp(score - tile max)
  * with a tile's heads side by side, so that both sides stream contiguous 8 KB runs instead

@@ -58,6 +58,7 @@ struct AttendArgs {
   int64_t n_tiles;
   int head_off;  // attend_mfma_i4_kernel: first query head of every kv group handled by this launch
   int tokens_per_block;  // cached tokens per block (a multiple of 64): block x covers tokens [x * tokens_per_block, ...)
+  int row_slabs;         // attend_mfma_i4_kernel<SPLIT>: 128-dimension slabs of a whole cached row (the block takes 8 of them)
 };
 
 __device__ __forceinline__ float prob_of(float s, float mx, float rz, bool normalise) {
@@ -168,6 +169,40 @@ __global__ __launch_bounds__(256) void attend_importance_kernel(AttendArgs a) {
   if (a.row_ts) a.row_ts[row] = a.now;
 }
 
+// H2O bookkeeping from the exchange format of pikv_decode_attend, for the attention kernels that
+// cannot do it themselves (split rows: a block sees only some heads of a token):
+//   p[h][n] = e[c][tile][h][n % 64] * exp(tile max[h] - head max[h]) / head sum[h],  imp[n] = sum_h p[h][n]
+// One block per 64-token tile; four lanes per token add every fourth head, then the four partial sums.
+__global__ __launch_bounds__(256) void exch_importance_kernel(AttendArgs a) {
+  __shared__ float part[4][kAttTile];
+  const int c = blockIdx.y;
+  const int64_t tile = blockIdx.x;
+  const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
+  const int64_t n0 = tile * kAttTile;
+  if (n0 >= len) return;  // uniform
+  const int t = threadIdx.x & 63, hl = threadIdx.x >> 6;
+  const int64_t trow = ((int64_t)c * a.n_tiles + tile) * a.n_q_heads;
+  float imp = 0.f;
+  for (int h = hl; h < a.n_q_heads; h += 4) {
+    const int64_t hi = (int64_t)c * a.n_q_heads + h;
+    const float coef = __builtin_amdgcn_exp2f((a.tile_max[trow + h] - a.head_stats[hi * 2]) * 1.4426950408889634f) *
+                       (1.0f / a.head_stats[hi * 2 + 1]);
+    imp = imp + a.escores[(trow + h) * kAttTile + t] * coef;
+  }
+  part[hl][t] = imp;
+  __syncthreads();
+  if (hl == 0 && n0 + t < len) {
+    imp = (part[0][t] + part[1][t]) + (part[2][t] + part[3][t]);
+    const int64_t row = a.row_base[c] + n0 + t;
+    if (a.row_acc) {
+      float acc = a.row_acc[row];
+      if (a.decay != 1.0f) acc = acc * a.decay;
+      a.row_acc[row] = acc + imp;
+    }
+    if (a.row_ts) a.row_ts[row] = a.now;
+  }
+}
+
 // ---- matrix-core form -----------------------------------------------------------------
 typedef int pikv_i32x2 __attribute__((ext_vector_type(2)));
 
@@ -202,7 +237,11 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads, int nsets = 1
 // NSETS = 2 (up to 4 kv heads): a launch covers up to 8 query heads of every kv head as two sets of
 // four that are multiplied with the same staged tile and the same expanded codes - the V codes of a
 // cache with 5 to 8 query heads per kv head are read from memory once instead of once per launch.
-template <int SCHEME, int HK, bool EXCH = false, bool NARROW = false, int NSETS = 1>
+// SPLIT (rows of more than 8 slabs, e.g. 32 kv heads of 128; HK = 8): neighbouring blocks take the
+// groups of 8 slabs of one token range, block index = range * groups + group; a group is a 512-byte
+// piece of every cached row.  The H2O bookkeeping needs all heads of a token and is left to a kernel
+// of its own (row_acc and row_ts are not touched here).
+template <int SCHEME, int HK, bool EXCH = false, bool NARROW = false, int NSETS = 1, bool SPLIT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i4_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
@@ -227,17 +266,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
   const int c = blockIdx.y;
   const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
-  const int64_t t0 = (int64_t)blockIdx.x * a.tokens_per_block;
+  static_assert(!SPLIT || (HK == 8 && !NARROW && NSETS == 1), "split rows: groups of 8 slabs of 128 dimensions");
+  const int n_groups = SPLIT ? a.row_slabs / HK : 1;
+  const int xb = SPLIT ? blockIdx.x / n_groups : blockIdx.x;            // token range of this block
+  const int kv_off = SPLIT ? (blockIdx.x % n_groups) * HK : 0;          // its first slab
+  const int row_slabs = SPLIT ? a.row_slabs : HK;
+  const int64_t t0 = (int64_t)xb * a.tokens_per_block;
   const int64_t t1 = (t0 + a.tokens_per_block < len) ? t0 + a.tokens_per_block : len;
-  if (t0 >= t1) {  // nothing cached in this range: the partial is zero
+  if (t0 >= t1) {  // nothing cached in this range: the partial (of this block's heads) is zero
     const int hd = NARROW ? a.head_dim : 128;
-    for (int idx = threadIdx.x; idx < a.n_q_heads * hd; idx += 256)
-      a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * hd + idx] = 0.f;
+    const int nh = a.n_q_heads / n_groups;   // query heads of the block's slabs, a contiguous run
+    for (int idx = threadIdx.x; idx < nh * hd; idx += 256)
+      a.partial[(((int64_t)xb * a.n_caches + c) * a.n_q_heads + (SPLIT ? (blockIdx.x % n_groups) * nh : 0)) * hd + idx] = 0.f;
     return;
   }
   // A launch covers up to 4 query heads of every kv group: heads head_off .. head_off+nr-1.
   // More than 4 heads per kv head are served by a second launch over the same codes.
-  const int rep_all = a.n_q_heads / HK;
+  const int rep_all = a.n_q_heads / row_slabs;   // query heads per slab
   const int rep = rep_all - a.head_off < 4 ? rep_all - a.head_off : 4;  // heads of a group in this launch (first set)
   const int rep_b = NSETS == 1 ? 0 : rep_all - a.head_off - 4 < 0 ? 0 : rep_all - a.head_off - 4 < 4 ? rep_all - a.head_off - 4 : 4;  // second set
   // matrix-core roles: A row / B,C column i, token group kg
@@ -267,7 +312,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int s_set = NSETS == 1 ? 0 : sh / (4 * HK);
   const int s_g = NSETS == 1 ? sh >> 2 : (sh >> 2) % HK;
   const bool s_on = s_set < NSETS && s_g < HK && (sh & 3) < (s_set ? rep_b : rep);
-  const int s_hq = s_on ? s_g * rep_all + a.head_off + 4 * s_set + (sh & 3) : 0;
+  const int s_hq = s_on ? (kv_off + s_g) * rep_all + a.head_off + 4 * s_set + (sh & 3) : 0;
   const float* srow = a.scores + ((int64_t)c * a.n_q_heads + s_hq) * a.score_stride;
   float smx = 0.f, srz = 1.f;
   if (normalise) {
@@ -325,6 +370,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     }
     // Every load is issued, from an offset clamped to the tile's last cached row: tokens past the
     // end of a short tile see a copy of that row, and their weight is zero (p = 0, finite scale).
+    if constexpr (SPLIT) {
+      // the block's slabs are a piece of every row: (token, piece) from the chunk index, the token clamped
+      const char* cb = reinterpret_cast<const char*>(a.codes) + (urow * row_slabs + kv_off) * 64;
+#pragma unroll
+      for (int k = 0; k < NCH; ++k) {
+        const int ch = k * 256 + threadIdx.x;
+        const int tok = ch / LPR < rem ? ch / LPR : rem - 1;
+        pc[k] = ld16(cb + (int64_t)tok * row_slabs * 64 + (ch % LPR) * 16);
+      }
+      const char* sb = reinterpret_cast<const char*>(a.scale) + (urow * row_slabs + kv_off) * 8;
+      const char* zb = reinterpret_cast<const char*>(a.zero) + (urow * row_slabs + kv_off) * 8;
+#pragma unroll
+      for (int k = 0; k < NMC; ++k) {
+        const int ch = k * 256 + threadIdx.x;
+        const int tok = ch / HK < rem ? ch / HK : rem - 1;
+        const int64_t mo = (int64_t)tok * row_slabs * 8 + (ch % HK) * 8;
+        ps[k] = *reinterpret_cast<const uint2*>(sb + mo);
+        pz[k] = make_uint2(0, 0);
+        if constexpr (!Q::sym) pz[k] = *reinterpret_cast<const uint2*>(zb + mo);
+      }
+    } else {
     const char* cb = reinterpret_cast<const char*>(a.codes) + urow * (LPR * 16);
     const unsigned c_last = (unsigned)(rem * LPR - 1) * 16u;
 #pragma unroll
@@ -342,6 +408,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       ps[k] = *reinterpret_cast<const uint2*>(sb + mo);
       pz[k] = make_uint2(0, 0);
       if constexpr (!Q::sym) pz[k] = *reinterpret_cast<const uint2*>(zb + mo);
+    }
     }
   };
   auto h2f = [](uint32_t w, int hi) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> (16 * hi))); };
@@ -555,7 +622,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       const int ro = 2 * kg + rr;  // head (inside the set) held by this lane
       if (ro >= (set ? rep_b : rep)) continue;
       const int hro = a.head_off + 4 * set + ro;   // head inside the kv group
-      const int64_t ohead = ((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep_all + hro;
+      const int64_t ohead = ((int64_t)xb * a.n_caches + c) * a.n_q_heads + (kv_off + g) * rep_all + hro;
       if constexpr (!NARROW) {
         float* o = a.partial + ohead * 128;
 #pragma unroll
@@ -927,6 +994,25 @@ static void launch_attend_mfma_slabs(int n_slabs, int nsets, dim3 grid, hipStrea
 // later launch (same codes, next heads) adds its share to the accumulators that the first one has decayed.
 template <int SCHEME, bool EXCH = false>
 static void launch_attend_mfma(int n_slabs, int heads_per_slab, dim3 grid, hipStream_t st, AttendArgs a) {
+  if (n_slabs > 8) {
+    // split rows (heads of 128, whole groups of 8 slabs - checked by the caller): the groups of a token
+    // range are neighbouring blocks; the H2O bookkeeping runs first, as a kernel of its own
+    if (a.row_acc || a.row_ts) {
+      const dim3 ig((unsigned)((a.max_len + kAttTile - 1) / kAttTile), (unsigned)a.n_caches);
+      if (EXCH) hipLaunchKernelGGL(exch_importance_kernel, ig, dim3(256), 0, st, a);
+      else hipLaunchKernelGGL(attend_importance_kernel, dim3((unsigned)((a.max_len + 255) / 256), (unsigned)a.n_caches), dim3(256), 0, st, a);
+    }
+    a.row_acc = nullptr;
+    a.row_ts = nullptr;
+    a.row_slabs = n_slabs;
+    const dim3 sgrid(grid.x * (unsigned)(n_slabs / 8), grid.y);
+    const size_t lds = attend_mfma_lds_bytes(8, a.n_q_heads, 1);
+    for (int off = 0; off < heads_per_slab; off += 4) {
+      a.head_off = off;
+      hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 8, EXCH, false, 1, true>), sgrid, dim3(256), lds, st, a);
+    }
+    return;
+  }
   const int nsets = (n_slabs <= 4 && heads_per_slab > 4) ? 2 : 1;
   for (int off = 0; off < heads_per_slab; off += 4 * nsets) {
     a.head_off = off;
@@ -1025,12 +1111,12 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
     // the matrix-core kernels see 128-dimension slabs of the row: one kv head, or 2 / 4 narrow ones
     const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
     const int slabs = hps > 0 ? n_kv_heads / hps : 0;
-    const bool slabs_ok = slabs >= 1 && slabs <= 8;
+    const bool slabs_ok = (slabs >= 1 && slabs <= 8) || (hps == 1 && slabs > 8 && slabs % 8 == 0 && splits * (slabs / 8) <= 0x7fffffffLL);
     if (!eight && group == 32 && slabs_ok && rep * hps <= 8) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(slabs, rep * hps, grid, st, a);
       else launch_attend_mfma<PIKV_Q_I4_SYM>(slabs, rep * hps, grid, st, a);
-    } else if (eight && slabs_ok && group % head_dim == 0 && rep * hps >= 2 && rep * hps <= 8) {
+    } else if (eight && slabs >= 1 && slabs <= 8 && group % head_dim == 0 && rep * hps >= 2 && rep * hps <= 8) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       if (scheme == PIKV_Q_I8_SYM) launch_attend_mfma8<PIKV_Q_I8_SYM>(slabs, hps, grid, st, a);
       else launch_attend_mfma8<PIKV_Q_I8_ASYM>(slabs, hps, grid, st, a);
@@ -1127,7 +1213,7 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
   const int rep = n_q_heads % n_kv_heads == 0 ? n_q_heads / n_kv_heads : 0;
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);   // 128-dimension slabs: one kv head, or 2 / 4 narrow ones
   const int slabs = hps > 0 ? n_kv_heads / hps : 0;
-  const bool hk_ok = slabs >= 1 && slabs <= 8;
+  const bool hk_ok = (slabs >= 1 && slabs <= 8) || (hps == 1 && slabs > 8 && slabs % 8 == 0);
   const int64_t splits = attend_splits(n_caches, max_len);
   if ((scheme == PIKV_Q_I4_ASYM || scheme == PIKV_Q_I4_SYM) && group == 32 && rep >= 1 &&
       rep * hps <= 8 && hk_ok && (q_dtype == PIKV_BF16 || q_dtype == PIKV_F32) && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {

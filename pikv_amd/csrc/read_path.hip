@@ -99,6 +99,7 @@ struct ScoreArgs {
   int rep;          // scores_kernel: query heads per kv head, and the first head of every kv group that
   int head_off;     //   this launch serves (it serves REP of them; other ratios take several launches)
   int head_split;   // scores_kernel: head_split blocks share a tile, each owns n_kv_heads/head_split heads
+  int row_slabs;    // scores_mfma_i4_gqa_kernel<SPLIT>: 128-dimension slabs of a whole cached row (n_kv_heads of them per block)
 };
 
 template <int SCHEME, int REP, int Q_DT>
@@ -410,12 +411,13 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 // r >= rep unused), so that the row of a kv head sits at a compile-time offset for the writers.
 template <bool GROUPED, int SLOTS = 4>
 __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float* stage, int c, int64_t tile,
-                                                 int64_t n0, int len, int wave, int rg, int nl, int rep = 4) {
+                                                 int64_t n0, int len, int wave, int rg, int nl, int rep = 4,
+                                                 int hq0 = 0) {  // hq0: first query head of the block's kv heads
   const int n_pass_rows = GROUPED ? a.n_kv_heads * SLOTS : a.n_q_heads;
   for (int h4 = wave * 4; h4 < n_pass_rows; h4 += 16) {
     const int srow = h4 + rg;                                  // staged row = kv head * SLOTS + slot
     const int slot = srow % SLOTS;
-    const int hq = GROUPED ? (srow / SLOTS) * rep + slot : srow;  // query head
+    const int hq = hq0 + (GROUPED ? (srow / SLOTS) * rep + slot : srow);  // query head
     const bool hok = GROUPED ? slot < rep : hq < a.n_q_heads;
     float x[4];
     bool okk[4];
@@ -460,13 +462,14 @@ __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float
 // r >= rep unused), so that the row of a kv head sits at a compile-time offset for the writers.
 template <bool GROUPED, int SLOTS = 4>
 __device__ __forceinline__ void tile_stats_exchange(const ScoreArgs& a, const float* stage, int c, int64_t tile,
-                                                 int64_t n0, int len, int wave, int rg, int nl, int rep = 4) {
+                                                 int64_t n0, int len, int wave, int rg, int nl, int rep = 4,
+                                                 int hq0 = 0) {  // hq0: first query head of the block's kv heads
   const int n_pass_rows = GROUPED ? a.n_kv_heads * SLOTS : a.n_q_heads;
   const int left = len - (int)n0 - 4 * nl;                     // tokens of this lane's run that exist
   for (int h4 = wave * 4; h4 < n_pass_rows; h4 += 16) {
     const int srow = h4 + rg;                                  // staged row = kv head * SLOTS + slot
     const int slot = srow % SLOTS;
-    const int hq = GROUPED ? (srow / SLOTS) * rep + slot : srow;  // query head
+    const int hq = hq0 + (GROUPED ? (srow / SLOTS) * rep + slot : srow);  // query head
     const bool hok = GROUPED ? slot < rep : hq < a.n_q_heads;
     const float4 sv = hok ? *reinterpret_cast<const float4*>(stage + srow * kTile + 4 * nl)
                           : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -522,7 +525,10 @@ static size_t gqa_lds_bytes(int n_kv_heads, int nset, int na) {
 // 2^-17 |q|), hi = the float cut to its upper 16 bits, lo = the rest rounded to bf16: two copies of a
 // set's A operands, one per limb, are multiplied with the same unpacked codes into the same
 // accumulators, and the group sums of q are those of hi + lo.
-template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false, bool NARROW = false, bool QF32 = false>  // NKV = n_kv_heads rounded up to 4/8/16; EXCH: exchange format out
+// SPLIT (rows of more than 16 slabs, e.g. 32 kv heads of 128): a block takes a group of a.n_kv_heads slabs
+// out of the a.row_slabs of a cached row; the groups of a tile are independent blocks with neighbouring
+// block indices, so that whole rows are in flight at any time and not one 512-byte window of every row.
+template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false, bool NARROW = false, bool QF32 = false, bool SPLIT = false>  // NKV = n_kv_heads rounded up to 4/8/16; EXCH: exchange format out
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET <= 8 ? 4 : 2))) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
   constexpr int SL = 4 * NSET;  // head slots per kv head
   using Q = QScheme<SCHEME>;
@@ -541,10 +547,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
 
   const int c = blockIdx.y;
   const int len = a.fill[c] < a.max_len ? a.fill[c] : a.max_len;
-  const int64_t tile0 = (int64_t)blockIdx.x * kGqaTilesPerBlock;
+  const int n_groups = SPLIT ? a.row_slabs / a.n_kv_heads : 1;
+  const int64_t tile0 = (int64_t)(SPLIT ? blockIdx.x / n_groups : blockIdx.x) * kGqaTilesPerBlock;
   const int64_t tok0 = tile0 * kTile;
   if (tok0 >= len) return;  // uniform for the block
-  const int rep = a.n_q_heads / a.n_kv_heads;  // <= 4 NSET
+  const int rep = a.n_q_heads / (SPLIT ? a.row_slabs : a.n_kv_heads);  // query heads per slab, <= 4 NSET
   // Heads narrower than 128: a.n_kv_heads counts 128-dimension slabs of the cached row, each the
   // stored bytes of hps = 128 / head_dim neighbouring kv heads, and the rep query heads of a slab
   // are the heads of those kv heads, rep1 each, in order.  Query head r of a slab belongs to kv
@@ -559,13 +566,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     return !NARROW || (gq >> gshift) == (r >= rep1) + (r >= 2 * rep1) + (r >= 3 * rep1);
   };
   auto group_in_head = [&](int gq) { return NARROW ? gq & ((1 << gshift) - 1) : gq; };
-  const int lanes_per_row = a.n_kv_heads * 4;
+  const int lanes_per_row = SPLIT ? a.row_slabs * 4 : a.n_kv_heads * 4;   // 16-byte pieces of a whole cached row
+  const int kv_off = SPLIT ? (blockIdx.x % n_groups) * a.n_kv_heads : 0;  // first slab of this block
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nl = lane & 15;
   const int rg = lane >> 4;
-  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)c * a.n_q_heads * head_dim;
-  const float* qfbase = reinterpret_cast<const float*>(a.q) + (int64_t)c * a.n_q_heads * head_dim;
+  // (the queries of this block's slabs: heads kv_off * rep ...)
+  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)c * a.n_q_heads + kv_off * rep) * head_dim;
+  const float* qfbase = reinterpret_cast<const float*>(a.q) + ((int64_t)c * a.n_q_heads + kv_off * rep) * head_dim;
   // bf16 bits of limb `set` of a float32 query element
   auto limb_bits = [](float v, int set) -> uint32_t {
     const uint32_t hb = __float_as_uint(v) & 0xffff0000u;
@@ -586,7 +595,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   // rows is the (token, kv head) pair, 4*ch halves into the rows (lanes_per_row = 4 kv heads).
   // (64-bit lane addresses per chunk had cost the registers whose spill reloads waited,
   // inside the loop, for the code loads just issued.)
-  const int code_lane_off = ((wave * 16 + nl) * lanes_per_row + rg) * 16;
+  const int code_lane_off = ((wave * 16 + nl) * lanes_per_row + kv_off * 4 + rg) * 16;
   auto issue = [&](int tt, TileRegs& t) {
     const int64_t t0 = tok0 + tt * kTile;
     const int64_t left = len - t0;
@@ -605,8 +614,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
       t.sv[j] = make_uint2(0, 0);
       t.zv[j] = make_uint2(0, 0);
       if ((int)threadIdx.x < rem * a.n_kv_heads - j * 256) {
-        t.sv[j] = *reinterpret_cast<const uint2*>(sb + j * 1024 + threadIdx.x * 4);
-        if constexpr (!Q::sym) t.zv[j] = *reinterpret_cast<const uint2*>(zb + j * 1024 + threadIdx.x * 4);
+        int mo = j * 1024 + threadIdx.x * 4;   // halves into the tile's metadata rows
+        if constexpr (SPLIT) {                 // the block's slabs are a piece of every row
+          const int ch = j * 256 + threadIdx.x, tok = ch / a.n_kv_heads;
+          mo = (tok * a.row_slabs + kv_off + (ch - tok * a.n_kv_heads)) * 4;
+        }
+        t.sv[j] = *reinterpret_cast<const uint2*>(sb + mo);
+        if constexpr (!Q::sym) t.zv[j] = *reinterpret_cast<const uint2*>(zb + mo);
       }
     }
   };
@@ -732,8 +746,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     }
     __syncthreads();
 
-    if constexpr (EXCH) tile_stats_exchange<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep);
-    else tile_stats_store<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep);
+    if constexpr (EXCH) tile_stats_exchange<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep, kv_off * rep);
+    else tile_stats_store<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep, kv_off * rep);
     __syncthreads();  // stage and the metadata rows are reused by the next tile
     return true;
   };
@@ -983,9 +997,34 @@ static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, h
   }
   return PIKV_OK;
 }
+// Rows of more than 16 slabs (heads of 128 dimensions): groups of 8 slabs as independent blocks, grid z.
+template <int SCHEME, bool EXCH>
+static int launch_gqa_split(const ScoreArgs& a0, int n_caches, int64_t n_tiles, hipStream_t st, bool qf32) {
+  if (a0.head_dim != 128 || a0.n_kv_heads % 8 != 0) return PIKV_ERR_UNSUPPORTED;
+  ScoreArgs a = a0;
+  a.row_slabs = a0.n_kv_heads;
+  a.n_kv_heads = 8;
+  const int rep = a.n_q_heads / a.row_slabs;
+  const int nset = rep <= 4 ? 1 : 2;
+  const size_t lds = gqa_lds_bytes(8, nset, qf32 ? 2 * nset : nset);
+  if (rep > 8 || lds > 64 * 1024) return PIKV_ERR_UNSUPPORTED;
+  const int64_t gx = (n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock * (a.row_slabs / 8);
+  if (gx > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+  const dim3 grid((unsigned)gx, (unsigned)n_caches);
+  if (qf32 && nset == 1)
+    hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1, EXCH, false, true, true>), grid, dim3(256), lds, st, a);
+  else if (qf32)
+    hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH, false, true, true>), grid, dim3(256), lds, st, a);
+  else if (nset == 1)
+    hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1, EXCH, false, false, true>), grid, dim3(256), lds, st, a);
+  else
+    hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH, false, false, true>), grid, dim3(256), lds, st, a);
+  return PIKV_OK;
+}
 // a.n_kv_heads counts 128-dimension slabs, a.head_dim is the width of a stored kv head
 template <int SCHEME, bool EXCH = false>
 static int launch_gqa(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st, bool qf32 = false) {
+  if (a.n_kv_heads > 16) return launch_gqa_split<SCHEME, EXCH>(a, n_caches, n_tiles, st, qf32);
   return a.head_dim == 128 ? launch_gqa_slabs<SCHEME, EXCH, false>(a, n_caches, n_tiles, st, qf32)
                            : launch_gqa_slabs<SCHEME, EXCH, true>(a, n_caches, n_tiles, st, qf32);
 }

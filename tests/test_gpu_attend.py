@@ -18,7 +18,10 @@ pytestmark = pytest.mark.gpu
     (O.Q_I4_SYM, 32, 2, 4, 128),       # matrix-core form, symmetric codes
     (O.Q_I4_ASYM, 32, 1, 8, 128),      # matrix-core form, all 16 operand rows in use
     (O.Q_I4_ASYM, 32, 4, 4, 128),      # matrix-core form, one row pair per kv head
-    (O.Q_I4_ASYM, 32, 16, 16, 128),    # more kv heads than the matrix-core form takes: vector form
+    (O.Q_I4_ASYM, 32, 16, 16, 128),    # 16 kv heads: two groups of 8 as neighbouring blocks of the matrix-core form
+    (O.Q_I4_ASYM, 32, 32, 32, 128),    # ... 32 kv heads, four groups
+    (O.Q_I4_SYM, 32, 24, 120, 128),    # ... three groups, 5 q heads per kv head: two launches
+    (O.Q_I4_ASYM, 32, 12, 12, 128),    # 12 kv heads are no whole groups of 8: vector form
     (O.Q_I4_ASYM, 32, 8, 24, 128),     # 3 q heads per kv head: a row pair of every kv head stays empty
     (O.Q_I4_ASYM, 32, 8, 64, 128),     # 8 q heads per kv head: two launches of four heads each
     (O.Q_I4_SYM, 32, 2, 12, 128),      # 6 q heads per kv head: the second launch half empty
@@ -99,6 +102,8 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
     (O.Q_I8_ASYM, 64, 8, 16, 64),      # 8-bit heads of 64 on the matrix-core form
     (O.Q_I4_ASYM, 32, 6, 36, 128),     # 6 kv heads x 6: two launches
     (O.Q_I8_SYM, 128, 3, 12, 128),     # 8-bit, 3 kv heads
+    (O.Q_I4_ASYM, 32, 16, 32, 128),    # 16 kv heads in two groups: the importance comes from a kernel of its own
+    (O.Q_I4_SYM, 32, 24, 24, 128),
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.95])
 def test_attend_accumulates_importance(dev, scheme, group, heads, hq, dh, decay):
@@ -159,7 +164,10 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I4_ASYM, 32, 1, 8, 128, "bf16"),    # ... 8 q heads per kv head: two sets, two attention launches
     (O.Q_I4_ASYM, 32, 8, 24, 128, "bf16"),   # ... 3 q heads per kv head
     (O.Q_I4_SYM, 32, 4, 28, 128, "bf16"),    # ... 7 q heads per kv head
-    (O.Q_I4_ASYM, 32, 16, 16, 128, "bf16"),  # 16 kv heads: the three public steps inside the call
+    (O.Q_I4_ASYM, 32, 16, 16, 128, "bf16"),  # 16 kv heads: exchange format, the attention kernel in two groups of 8
+    (O.Q_I4_SYM, 32, 32, 32, 128, "bf16"),   # ... 32 kv heads: both kernels in four groups
+    (O.Q_I4_ASYM, 32, 24, 48, 128, "f32"),   # ... three groups, float32 queries
+    (O.Q_I4_ASYM, 32, 12, 12, 128, "bf16"),  # 12 kv heads: no whole groups, the three public steps inside the call
     (O.Q_I4_ASYM, 32, 8, 32, 128, "f32"),    # float32 queries: same
     (O.Q_I8_SYM, 128, 8, 32, 128, "bf16"),   # 8-bit matrix-core kernels
     (O.Q_I8_ASYM, 64, 2, 16, 64, "f32"),     # vector forms

@@ -71,6 +71,9 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I8_SYM, 128, 4, 8, 64),       # ... one scale per slab
     (O.Q_I8_ASYM, 32, 8, 16, 32),      # ... heads of 32
     (O.Q_I8_SYM, 64, 32, 64, 64),      # ... 16 slabs (four per wavefront)
+    (O.Q_I4_ASYM, 32, 32, 32, 128),    # 32 kv heads of 128: four groups of 8 slabs as independent blocks of the matrix-core kernel
+    (O.Q_I4_SYM, 32, 24, 48, 128),     # ... three groups, 2 q heads per kv head
+    (O.Q_I4_ASYM, 32, 24, 120, 128),   # ... 5 q heads per kv head: two sets
     (O.Q_I8_SYM, 64, 12, 12, 64),      # 12 kv heads: three blocks of four heads per tile
     (O.Q_I4_ASYM, 32, 3, 6, 128),      # 3 kv heads
     (O.Q_I8_ASYM, 128, 5, 10, 128),    # 5 kv heads: one block per head
