@@ -108,20 +108,37 @@ __global__ __launch_bounds__(256) void attend_valu_kernel(AttendArgs a) {
   }
   const int64_t base_row = a.row_base[c];
   // (a row's lanes need not divide the block: the threads beyond the last whole row stay idle)
-  for (int64_t n = tok_in_step < tok_per_step ? t0 + tok_in_step : t1; n < t1; n += tok_per_step) {
-    const int64_t row = base_row + n;
-    const uint4 v = ld16(reinterpret_cast<const char*>(a.codes) + (row * lanes_per_row + part) * 16);
-    const int64_t mi = row * groups_per_row + (part * EPL) / a.group;
-    const float sc = load_meta<SCHEME>(a.scale, mi);
-    const float zu = (Q::sym ? 0.f : load_meta<SCHEME>(a.zero, mi)) - (float)Q::qmin;
-    float cf[EPL];
-    unpack_codes_unsigned<SCHEME>(v, cf);
+  // UN tokens per thread and trip: their codes, metadata and scores are asked for together, one
+  // memory round trip instead of UN (a step past the end re-reads the trip's first token, weight 0)
+  constexpr int UN = RP >= 8 ? 2 : 4;
+  for (int64_t n = tok_in_step < tok_per_step ? t0 + tok_in_step : t1; n < t1; n += (int64_t)tok_per_step * UN) {
+    uint4 v[UN];
+    float sc[UN], zu[UN], sv[UN][RP];
+    bool ok[UN];
 #pragma unroll
-    for (int r = 0; r < RP; ++r) {
-      const float w = prob_of(srow[r][n], mx[r], rz[r], normalise) * sc;
-      zacc[r] = fmaf(w, zu, zacc[r]);
+    for (int u = 0; u < UN; ++u) {
+      const int64_t nn = n + (int64_t)u * tok_per_step;
+      ok[u] = nn < t1;
+      const int64_t nc = ok[u] ? nn : n;
+      const int64_t row = base_row + nc;
+      v[u] = ld16(reinterpret_cast<const char*>(a.codes) + (row * lanes_per_row + part) * 16);
+      const int64_t mi = row * groups_per_row + (part * EPL) / a.group;
+      sc[u] = load_meta<SCHEME>(a.scale, mi);
+      zu[u] = (Q::sym ? 0.f : load_meta<SCHEME>(a.zero, mi)) - (float)Q::qmin;
 #pragma unroll
-      for (int j = 0; j < EPL; ++j) acc[r][j] = fmaf(w, cf[j], acc[r][j]);
+      for (int r = 0; r < RP; ++r) sv[u][r] = srow[r][nc];
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      float cf[EPL];
+      unpack_codes_unsigned<SCHEME>(v[u], cf);
+#pragma unroll
+      for (int r = 0; r < RP; ++r) {
+        const float w = ok[u] ? prob_of(sv[u][r], mx[r], rz[r], normalise) * sc[u] : 0.f;
+        zacc[r] = fmaf(w, zu[u], zacc[r]);
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) acc[r][j] = fmaf(w, cf[j], acc[r][j]);
+      }
     }
   }
   // add the token slots of the block (threads that share `part`), one head at a time
