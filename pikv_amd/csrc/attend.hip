@@ -171,11 +171,18 @@ __global__ __launch_bounds__(256) void attend_importance_kernel(AttendArgs a) {
   if (n >= a.fill[c] || n >= a.max_len) return;
   const bool normalise = a.head_stats != nullptr;
   float imp = 0.f;
-  for (int hq = 0; hq < a.n_q_heads; ++hq) {
-    const int64_t hi = (int64_t)c * a.n_q_heads + hq;
-    const float mx = normalise ? a.head_stats[hi * 2] : 0.f;
-    const float rz = normalise ? 1.0f / a.head_stats[hi * 2 + 1] : 1.f;
-    imp = imp + prob_of(a.scores[hi * a.score_stride + n], mx, rz, normalise);
+  for (int h0 = 0; h0 < a.n_q_heads; h0 += 8) {   // eight heads in flight per thread
+    float sv[8], mx[8], hz[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t hi = (int64_t)c * a.n_q_heads + (h0 + u < a.n_q_heads ? h0 + u : 0);
+      sv[u] = a.scores[hi * a.score_stride + n];
+      mx[u] = normalise ? a.head_stats[hi * 2] : 0.f;
+      hz[u] = normalise ? a.head_stats[hi * 2 + 1] : 1.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (h0 + u < a.n_q_heads) imp = imp + prob_of(sv[u], mx[u], 1.0f / hz[u], normalise);
   }
   const int64_t row = a.row_base[c] + n;
   if (a.row_acc) {
@@ -200,11 +207,21 @@ __global__ __launch_bounds__(256) void exch_importance_kernel(AttendArgs a) {
   const int t = threadIdx.x & 63, hl = threadIdx.x >> 6;
   const int64_t trow = ((int64_t)c * a.n_tiles + tile) * a.n_q_heads;
   float imp = 0.f;
-  for (int h = hl; h < a.n_q_heads; h += 4) {
-    const int64_t hi = (int64_t)c * a.n_q_heads + h;
-    const float coef = __builtin_amdgcn_exp2f((a.tile_max[trow + h] - a.head_stats[hi * 2]) * 1.4426950408889634f) *
-                       (1.0f / a.head_stats[hi * 2 + 1]);
-    imp = imp + a.escores[(trow + h) * kAttTile + t] * coef;
+  for (int h0 = hl; h0 < a.n_q_heads; h0 += 4 * 8) {   // eight heads in flight per thread
+    float e[8], tm[8], hm[8], hz[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int h = h0 + 4 * u < a.n_q_heads ? h0 + 4 * u : hl;
+      const int64_t hi = (int64_t)c * a.n_q_heads + h;
+      e[u] = a.escores[(trow + h) * kAttTile + t];
+      tm[u] = a.tile_max[trow + h];
+      hm[u] = a.head_stats[hi * 2];
+      hz[u] = a.head_stats[hi * 2 + 1];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (h0 + 4 * u < a.n_q_heads)
+        imp = imp + e[u] * (__builtin_amdgcn_exp2f((tm[u] - hm[u]) * 1.4426950408889634f) * (1.0f / hz[u]));
   }
   part[hl][t] = imp;
   __syncthreads();
