@@ -303,16 +303,17 @@ typedef float pikv_f32x4 __attribute__((ext_vector_type(4)));
 // so that the B operands of one k-step are EP*64 contiguous bytes.  Rows of the
 // original [E,H] layout are a multiple of 2 KB apart for the usual hidden sizes and
 // would all fall into the same L2 channel.
-__global__ __launch_bounds__(256) void gate_weight_relayout_kernel(const uint16_t* __restrict__ w, int H,
+// (row_bytes = bytes of a row of w: a k-step is 64 bytes of it, 32 bf16 or 16 float32 values)
+__global__ __launch_bounds__(256) void gate_weight_relayout_kernel(const void* __restrict__ w, int64_t row_bytes,
                                                                   int E, int EP, uint4* __restrict__ wb) {
   const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;  // 16-byte chunk of wb
-  const int64_t total = (int64_t)(H / 32) * EP * 4;
+  const int64_t total = (row_bytes / 64) * EP * 4;
   if (chunk >= total) return;
   const int kg = (int)(chunk & 3);
   const int e = (int)((chunk >> 2) % EP);
   const int64_t st = (chunk >> 2) / EP;
   uint4 v = make_uint4(0, 0, 0, 0);
-  if (e < E) v = ld16(w + (int64_t)e * H + st * 32 + kg * 8);
+  if (e < E) v = ld16(reinterpret_cast<const char*>(w) + (int64_t)e * row_bytes + st * 64 + kg * 16);
   wb[chunk] = v;
 }
 
@@ -324,11 +325,16 @@ __global__ __launch_bounds__(256) void gate_weight_relayout_kernel(const uint16_
 // reads its 16 bytes of a k-step from row m.  Every block starts its walk at another k-step (below),
 // so the rows - a multiple of 2 KB apart - no longer meet in one L2 channel at the same time, and the
 // launch that re-lays the weights is saved (config[1], router call: 65.2 -> 63.0 us).
-template <int NT, int MT, int WAVES, bool PARTIAL = false, bool DIRECT = false>
+// F32IN: float32 activations and weights, multiplied exactly by v_mfma_f32_16x16x4_f32.  A k-step is
+// 16 values - the same 64 bytes of a row as 32 bf16 - and a lane's four floats feed four instructions:
+// lane (m, kg) holds k = k0 + 4 kg + j for instruction j on both operands, so the four cover all 16.
+template <int NT, int MT, int WAVES, bool PARTIAL = false, bool DIRECT = false, bool F32IN = false>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2))) void router_gate_mfma_kernel(
     const void* __restrict__ x, const void* __restrict__ wb, int H, TailParams p, float* __restrict__ part = nullptr,
     int steps_per_slice = 0) {
-  static_assert(!DIRECT || (NT == 1 && !PARTIAL), "direct weights: one expert tile, whole rows per block");
+  static_assert(!DIRECT || !PARTIAL, "direct weights: whole rows per block");
+  constexpr int ES = F32IN ? 4 : 2;        // bytes per element
+  constexpr int KL = 16 / ES;              // elements of a lane's 16 bytes
   constexpr int EP = 16 * NT;
   constexpr int TB = 16 * MT;  // tokens per block
   // Partial sums of the wavefronts: one slab each, or - when those would not leave room
@@ -347,9 +353,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
   for (int mt = 0; mt < MT; ++mt) {
     tok_ok[mt] = tok0 + mt * 16 + m < p.T;
     xrow[mt] = reinterpret_cast<const char*>(x) +
-               ((tok_ok[mt] ? tok0 + mt * 16 + m : 0) * (int64_t)H + kg * 8) * 2;
+               ((tok_ok[mt] ? tok0 + mt * 16 + m : 0) * (int64_t)H + kg * KL) * ES;
   }
-  const char* wlane = DIRECT ? reinterpret_cast<const char*>(wb) + ((int64_t)(m < p.E ? m : 0) * H + kg * 8) * 2
+  const char* wlane = DIRECT ? reinterpret_cast<const char*>(wb) + ((int64_t)(m < p.E ? m : 0) * H + kg * KL) * ES
                              : reinterpret_cast<const char*>(wb) + (m * 32 + kg * 8) * 2;
   pikv_f32x4 acc[MT][NT];
 #pragma unroll
@@ -358,7 +364,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
     for (int t = 0; t < NT; ++t) acc[mt][t] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
 
   // the k-steps are dealt round-robin to the wavefronts; each keeps UN steps in flight
-  int steps = H / 32, step0 = 0;
+  int steps = H / (4 * KL), step0 = 0;
   if constexpr (PARTIAL) {
     step0 = blockIdx.y * steps_per_slice;
     steps = step0 + steps_per_slice < steps ? step0 + steps_per_slice : steps;
@@ -373,34 +379,67 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
   // bits of a logit, depend on the block a token falls into.
   const int n_it = (steps - step0 + WAVES * UN - 1) / (WAVES * UN);
   const int rot = PARTIAL ? 0 : (int)(((blockIdx.x * 0x9E3779B1u) >> 16) % (unsigned)n_it);
-  for (int it = 0; it < n_it; ++it) {
+  struct Ops {
+    uint4 av[UN][MT], bv[UN][NT];
+  };
+  auto load_ops = [&](int it, Ops& o) {
     int itr = it + rot;
     if (itr >= n_it) itr -= n_it;
     const int st0 = step0 + wave + itr * (WAVES * UN);
-    uint4 av[UN][MT], bv[UN][NT];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int st = st0 + u * WAVES;
       const bool ok = st < steps;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
-        av[u][mt] = (ok && tok_ok[mt]) ? ld16(xrow[mt] + (int64_t)st * 64) : make_uint4(0, 0, 0, 0);
+        o.av[u][mt] = (ok && tok_ok[mt]) ? ld16(xrow[mt] + (int64_t)st * 64) : make_uint4(0, 0, 0, 0);
       // (columns of experts that do not exist are zero in the re-laid weights: not loaded at all)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        bv[u][t] = (ok && t * 16 + m < p.E)
-                       ? ld16(DIRECT ? wlane + (int64_t)st * 64 : wlane + ((int64_t)st * EP + t * 16) * 64)
-                       : make_uint4(0, 0, 0, 0);
+        o.bv[u][t] = (ok && t * 16 + m < p.E)
+                         ? ld16(DIRECT ? wlane + (int64_t)st * 64 + (int64_t)t * 16 * H * ES
+                                       : wlane + ((int64_t)st * EP + t * 16) * 64)
+                         : make_uint4(0, 0, 0, 0);
     }
+  };
+  if constexpr (F32IN) {
+    // The float32 form is bound by the matrix instruction (32 cycles each): the operands of the next
+    // trip are asked for before this trip's instructions, or the two wavefronts of a SIMD spend half
+    // their time waiting for loads (64 experts: 923 us without).  The four instructions of a lane's
+    // 16 bytes are outermost: neighbours in the issue order write different accumulators.
+    Ops cur, nxt;
+    load_ops(0, cur);
+    for (int it = 0; it < n_it; ++it) {
+      if (it + 1 < n_it) load_ops(it + 1, nxt);
 #pragma unroll
-    for (int u = 0; u < UN; ++u)
+      for (int u = 0; u < UN; ++u)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              __builtin_bit_cast(pikv_bf16x8, av[u][mt]), __builtin_bit_cast(pikv_bf16x8, bv[u][t]),
-              acc[mt][t], 0, 0, 0);
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+              const uint4 a4 = cur.av[u][mt], b4 = cur.bv[u][t];
+              const uint32_t af = j == 0 ? a4.x : j == 1 ? a4.y : j == 2 ? a4.z : a4.w;
+              const uint32_t bf = j == 0 ? b4.x : j == 1 ? b4.y : j == 2 ? b4.z : b4.w;
+              acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(af), __uint_as_float(bf), acc[mt][t], 0, 0, 0);
+            }
+      if (it + 1 < n_it) cur = nxt;
+    }
+  } else {
+    for (int it = 0; it < n_it; ++it) {
+      Ops o;
+      load_ops(it, o);
+#pragma unroll
+      for (int u = 0; u < UN; ++u)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                __builtin_bit_cast(pikv_bf16x8, o.av[u][mt]), __builtin_bit_cast(pikv_bf16x8, o.bv[u][t]),
+                acc[mt][t], 0, 0, 0);
+    }
   }
   // C layout: lane holds rows 4*(lane/16)+i, column lane%16 of each tile.
   if constexpr (SEQ) {
@@ -1067,7 +1106,7 @@ extern "C" int64_t pikv_router_workspace_bytes(int64_t T, int E, int k) {
 }
 
 static int gate_epad(int E) { return E <= 16 ? 16 : E <= 32 ? 32 : 64; }
-static int64_t gate_weight_bytes(int H, int E) { return (int64_t)H * gate_epad(E) * 2; }
+static int64_t gate_weight_bytes(int H, int E) { return (int64_t)H * gate_epad(E) * 4; }  // re-laid weights, float32 at most
 static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
 // Short token streams split the gate projection over the hidden dimension: slices of at
@@ -1165,6 +1204,8 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
   if (H < 8) return PIKV_ERR_SHAPE;
   if (H % 8 != 0) return PIKV_ERR_UNSUPPORTED;
   const bool mfma = x_dtype == PIKV_BF16 && H % 32 == 0;
+  // float32 inputs on the matrix cores (exact products, float32 accumulation): 256 tokens and more
+  const bool mfma32 = x_dtype == PIKV_F32 && H % 16 == 0 && T >= 256;
   const int64_t slot_ws = align256(slot_workspace_bytes(T * k, E));
   if ((slot || mfma) && T > 0) {
     if (!workspace) return PIKV_ERR_NULL;
@@ -1207,7 +1248,7 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
       const bool direct = slices <= 1 && !t64 && !t128 && ep == 16;
       if (!direct)
         hipLaunchKernelGGL(gate_weight_relayout_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256),
-                           0, st, (const uint16_t*)w, H, E, ep, (uint4*)wb);
+                           0, st, w, (int64_t)H * 2, E, ep, (uint4*)wb);
       if (slices > 1) {
         // short token streams: partial logits per slice of H, then the tail on their sum
         float* part = reinterpret_cast<float*>(wb + align256(gate_weight_bytes(H, E)));
@@ -1248,6 +1289,31 @@ extern "C" int pikv_router_fused(const void* x, const void* w, int x_dtype, cons
         hipLaunchKernelGGL((router_gate_mfma_kernel<4, 4, 4>), grid, dim3(256), 0, st, x, wb, H, p);
     } else if (x_dtype == PIKV_BF16) {
       launch_gate<PIKV_BF16>(epad, (unsigned)blocks, st, x, w, H, p);
+    } else if (mfma32) {
+      const int ep = gate_epad(E);
+      const int64_t mb = (T + 63) / 64;
+      if (mb > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+      // more than 16 experts: the weights re-laid per k-step like the bf16 ones, when the caller's
+      // workspace has room for them; read in place otherwise
+      const bool relaid = ep > 16 && workspace &&
+                          workspace_bytes >= (slot ? slot_ws : 0) + align256(gate_weight_bytes(H, E));
+      if (relaid) {
+        const int64_t chunks = (int64_t)(H / 16) * ep * 4;
+        hipLaunchKernelGGL(gate_weight_relayout_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256),
+                           0, st, w, (int64_t)H * 4, E, ep, (uint4*)wb);
+      }
+      if (ep == 16)
+        hipLaunchKernelGGL((router_gate_mfma_kernel<1, 4, 8, false, true, true>), dim3((unsigned)mb), dim3(512), 0, st, x, w, H, p);
+      else if (ep == 32 && relaid)
+        hipLaunchKernelGGL((router_gate_mfma_kernel<2, 4, 4, false, false, true>), dim3((unsigned)mb), dim3(256), 0, st, x, wb, H, p);
+      else if (ep == 32)
+        hipLaunchKernelGGL((router_gate_mfma_kernel<2, 4, 4, false, true, true>), dim3((unsigned)mb), dim3(256), 0, st, x, w, H, p);
+      else if (relaid && T >= 32768)   // 128 tokens per block: every weight operand serves eight token tiles
+        hipLaunchKernelGGL((router_gate_mfma_kernel<4, 8, 4, false, false, true>), dim3((unsigned)((T + 127) / 128)), dim3(256), 0, st, x, wb, H, p);
+      else if (relaid)
+        hipLaunchKernelGGL((router_gate_mfma_kernel<4, 4, 4, false, false, true>), dim3((unsigned)mb), dim3(256), 0, st, x, wb, H, p);
+      else
+        hipLaunchKernelGGL((router_gate_mfma_kernel<4, 4, 4, false, true, true>), dim3((unsigned)mb), dim3(256), 0, st, x, w, H, p);
     } else {
       launch_gate<PIKV_F32>(epad, (unsigned)blocks, st, x, w, H, p);
     }

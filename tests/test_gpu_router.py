@@ -120,7 +120,10 @@ def test_capacity_slots_exact(dev, A, E, cap):
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("T,H,E,k", [(128, 256, 4, 2), (1000, 512, 8, 2), (257, 1024, 16, 4),
-                                      (130, 7168, 64, 8), (64, 264, 5, 2)])
+                                      (130, 7168, 64, 8), (64, 264, 5, 2),
+                                      (300, 272, 24, 4),       # float32: matrix cores, 17 k-steps of 16, two expert tiles
+                                      (1000, 512, 64, 8),      # ... four expert tiles, weights re-laid
+                                      (32768 + 37, 256, 64, 8)])  # ... 128-token blocks, ragged last one
 def test_router_fused(dev, dtype, T, H, E, k):
     from pikv_amd import ops
     r = rng(T + H + E)
@@ -162,6 +165,31 @@ def test_router_fused(dev, dtype, T, H, E, k):
     slot, count = O.capacity_slots(got, E, cap)
     assert np.array_equal(np_of(out.slot), slot)
     assert np.array_equal(np_of(out.count), count)
+
+
+def test_router_float32_without_workspace(dev):
+    """float32 inputs, no slots requested, no workspace passed: the call is valid (only bf16 inputs
+    need one), more than 16 experts are then read from the weight matrix where it lies - same results
+    as with a workspace, where the weights are re-laid first."""
+    import torch
+    from pikv_amd import _native as N
+    from pikv_amd import ops
+    r = rng(77)
+    T, H, E, k = 700, 320, 40, 3
+    x = to_dev(r.standard_normal((T, H)).astype(np.float32), dev)
+    w = to_dev((0.05 * r.standard_normal((E, H))).astype(np.float32), dev)
+    ref = ops.router_fused(x, w, top_k=k, return_logits=True)
+    probs = torch.empty(T, E, device=dev)
+    logits = torch.empty(T, E, device=dev)
+    idx = torch.empty(T, k, dtype=torch.int32, device=dev)
+    wts = torch.empty(T, k, device=dev)
+    N.call("pikv_router_fused", x.data_ptr(), w.data_ptr(), N.F32, None, None, None, 1.0, 0.0, 0, T, H, E, k, 0,
+           probs.data_ptr(), logits.data_ptr(), idx.data_ptr(), wts.data_ptr(), None, None, None, 0,
+           torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(idx, ref.topk_idx)
+    assert torch.equal(logits, ref.logits)      # the same products in the same order, whichever way the weights come
+    assert torch.equal(wts, ref.topk_w)
 
 
 @pytest.mark.parametrize("T,H,E,k", [(32768 + 37, 256, 64, 8), (32768, 128, 40, 3), (32768 + 5, 416, 64, 8),
