@@ -29,21 +29,54 @@ __device__ __forceinline__ uint32_t minshift_code(float x, float mn, float s) {
   return (uint32_t)y;
 }
 
+// four consecutive source elements as floats (16 bytes of float32, 8 of bf16)
+template <int DT>
+__device__ __forceinline__ void load4_as_float(const void* base, int64_t elem_off, float (&out)[4]) {
+  if constexpr (DT == PIKV_BF16) {
+    const uint2 v = *reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(base) + elem_off * 2);
+    out[0] = __uint_as_float(v.x << 16);
+    out[1] = __uint_as_float(v.x & 0xffff0000u);
+    out[2] = __uint_as_float(v.y << 16);
+    out[3] = __uint_as_float(v.y & 0xffff0000u);
+  } else {
+    const uint4 v = ld16(reinterpret_cast<const char*>(base) + elem_off * 4);
+    out[0] = __uint_as_float(v.x);
+    out[1] = __uint_as_float(v.y);
+    out[2] = __uint_as_float(v.z);
+    out[3] = __uint_as_float(v.w);
+  }
+}
+
 template <int DT, bool VEC>
 __global__ __launch_bounds__(256) void minshift_rows_kernel(const void* __restrict__ src, int64_t n_rows, int D,
                                                             uint8_t* __restrict__ codes, float* __restrict__ dq,
                                                             float* __restrict__ scale, float* __restrict__ row_min) {
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int wave = threadIdx.x >> 6;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
   if (row >= n_rows) return;  // uniform for the wavefront
   const int64_t e0 = row * D;
   float mn = __builtin_inff(), mx = -__builtin_inff();
+  // VEC: a wavefront walks its row in pieces of 1024 elements.  Float32 values (the source, the
+  // dequantised output) move as four accesses of 16 bytes per lane, each of them one contiguous
+  // kilobyte of the row: lane l, access j holds elements 256 j + 4 l .. + 3 of the piece.  (Sixteen
+  // consecutive elements per lane make every access 16 bytes at a stride of 64, which stores at
+  // a fraction of the rate: 341 us for 32768 x 4096 float32 against 293 us.)  The four code words of a lane cross LDS
+  // so that the codes, too, leave as 16 bytes per lane.
+  __shared__ uint32_t cx[4][256];
+  constexpr int PIECE = 1024;
   if constexpr (VEC) {
-    for (int ch = lane; ch < D / 16; ch += 64) {
-      float x[16];
-      load_as_float<DT, 16>(src, e0 + 16 * ch, x);
+    for (int p0 = 0; p0 < D; p0 += PIECE) {
 #pragma unroll
-      for (int j = 0; j < 16; ++j) { mn = fminf(mn, x[j]); mx = fmaxf(mx, x[j]); }
+      for (int j = 0; j < 4; ++j) {
+        const int e = p0 + 256 * j + 4 * lane;
+        if (e < D) {
+          float x[4];
+          load4_as_float<DT>(src, e0 + e, x);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) { mn = fminf(mn, x[q]); mx = fmaxf(mx, x[q]); }
+        }
+      }
     }
   } else {
     for (int i = lane; i < D; i += 64) {
@@ -59,28 +92,39 @@ __global__ __launch_bounds__(256) void minshift_rows_kernel(const void* __restri
     row_min[row] = mn;
   }
   if constexpr (VEC) {
-    for (int ch = lane; ch < D / 16; ch += 64) {
-      float x[16];
-      load_as_float<DT, 16>(src, e0 + 16 * ch, x);
-      uint32_t w[4];
+    for (int p0 = 0; p0 < D; p0 += PIECE) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        uint32_t c[4];
+      for (int j = 0; j < 4; ++j) {
+        const int e = p0 + 256 * j + 4 * lane;
+        uint32_t w = 0;
+        if (e < D) {
+          float x[4];
+          load4_as_float<DT>(src, e0 + e, x);
+          uint32_t c[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) c[j] = minshift_code(x[4 * i + j], mn, s);
-        w[i] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
-        if (dq) {
-          float o[4];
+          for (int q = 0; q < 4; ++q) c[q] = minshift_code(x[q], mn, s);
+          w = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+          if (dq) {
+            float o[4];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float t = (float)c[j] * s;
-            o[j] = t + mn;
+            for (int q = 0; q < 4; ++q) {
+              const float t = (float)c[q] * s;
+              o[q] = t + mn;
+            }
+            st16(dq + e0 + e,
+                 make_uint4(__float_as_uint(o[0]), __float_as_uint(o[1]), __float_as_uint(o[2]), __float_as_uint(o[3])));
           }
-          st16(dq + e0 + 16 * ch + 4 * i,
-               make_uint4(__float_as_uint(o[0]), __float_as_uint(o[1]), __float_as_uint(o[2]), __float_as_uint(o[3])));
         }
+        cx[wave][64 * j + lane] = w;   // code word of elements 256 j + 4 lane ..: word 64 j + lane of the piece
       }
-      st16(codes + e0 + 16 * ch, make_uint4(w[0], w[1], w[2], w[3]));
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      if (p0 + 16 * lane < D)   // D is a multiple of 16: whole 16-byte runs
+        st16(codes + e0 + p0 + 16 * lane, *reinterpret_cast<const uint4*>(&cx[wave][4 * lane]));
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
   } else {
     for (int i = lane; i < D; i += 64) {
