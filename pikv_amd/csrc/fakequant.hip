@@ -40,10 +40,32 @@ __global__ __launch_bounds__(256) void fq_minmax_kernel(const float* __restrict_
   const int64_t r0 = chunk * kFqRows;
   const int64_t rows = (N - r0) < kFqRows ? (N - r0) : kFqRows;
   float mn = __builtin_inff(), mx = -__builtin_inff();
-  for (int64_t e = threadIdx.x; e < rows * gw; e += 256) {
-    const float v = x[(r0 + e / gw) * H + c0 + (int)(e % gw)];
-    mn = fminf(mn, v);
-    mx = fmaxf(mx, v);
+  // 16-byte accesses, four of them in flight per thread, where the block's columns and the rows allow
+  // it (32768 x 4096 float32, fake-quantisation as a whole: 507 -> 341 us); else one element at a time
+  const bool vec = (gw % 4 == 0) && (H % 4 == 0) && (c0 % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+  if (vec) {
+    const int q4 = gw / 4;
+    const int64_t n4 = rows * q4;
+    for (int64_t e0 = threadIdx.x; e0 < n4; e0 += 256 * 4) {
+      uint4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t e = e0 + 256 * u < n4 ? e0 + 256 * u : e0;
+        v[u] = ld16(reinterpret_cast<const char*>(x + (r0 + e / q4) * H + c0 + 4 * (int)(e % q4)));
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float f[4] = {__uint_as_float(v[u].x), __uint_as_float(v[u].y), __uint_as_float(v[u].z), __uint_as_float(v[u].w)};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) { mn = fminf(mn, f[q]); mx = fmaxf(mx, f[q]); }
+      }
+    }
+  } else {
+    for (int64_t e = threadIdx.x; e < rows * gw; e += 256) {
+      const float v = x[(r0 + e / gw) * H + c0 + (int)(e % gw)];
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    }
   }
   mn = block_reduce_minmax(mn, false, sh);
   mx = block_reduce_minmax(mx, true, sh);
@@ -105,17 +127,45 @@ __global__ __launch_bounds__(256) void fq_apply_kernel(const float* __restrict__
   const float qmin = symmetric ? -(float)(1 << (bits - 1)) : 0.f;
   const float qmax = symmetric ? (float)((1 << (bits - 1)) - 1) : (float)((1 << bits) - 1);
   double err = 0.0;
-  for (int64_t e = threadIdx.x; e < rows * gw; e += 256) {
-    const int64_t i = (r0 + e / gw) * H + c0 + (int)(e % gw);
-    const float v = x[i];
+  auto fq = [&](float v) {
     float y = v / scale;
     y = y + zero;
     y = rintf(y);
     y = fminf(fmaxf(y, qmin), qmax);
     const float dq = (y - zero) * scale;
-    out[i] = dq;
     const double d = (double)v - (double)dq;
     err += d * d;
+    return dq;
+  };
+  const bool vec = (gw % 4 == 0) && (H % 4 == 0) && (c0 % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
+                   ((reinterpret_cast<uintptr_t>(out) & 15) == 0);
+  if (vec) {   // 16-byte accesses, four of them in flight per thread
+    const int q4 = gw / 4;
+    const int64_t n4 = rows * q4;
+    for (int64_t e0 = threadIdx.x; e0 < n4; e0 += 256 * 4) {
+      uint4 v[4];
+      int64_t idx[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t e = e0 + 256 * u < n4 ? e0 + 256 * u : e0;
+        idx[u] = (r0 + e / q4) * H + c0 + 4 * (int)(e % q4);
+        v[u] = ld16(reinterpret_cast<const char*>(x + idx[u]));
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (e0 + 256 * u < n4) {
+          const float o0 = fq(__uint_as_float(v[u].x)), o1 = fq(__uint_as_float(v[u].y));
+          const float o2 = fq(__uint_as_float(v[u].z)), o3 = fq(__uint_as_float(v[u].w));
+          st16(reinterpret_cast<char*>(out + idx[u]),
+               make_uint4(__float_as_uint(o0), __float_as_uint(o1), __float_as_uint(o2), __float_as_uint(o3)));
+        }
+      }
+    }
+  } else {
+    for (int64_t e = threadIdx.x; e < rows * gw; e += 256) {
+      const int64_t i = (r0 + e / gw) * H + c0 + (int)(e % gw);
+      out[i] = fq(x[i]);
+    }
   }
   shd[threadIdx.x] = err;
   __syncthreads();
