@@ -271,10 +271,12 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads, int nsets = 1
 // NSETS = 2 (up to 4 kv heads): a launch covers up to 8 query heads of every kv head as two sets of
 // four that are multiplied with the same staged tile and the same expanded codes - the V codes of a
 // cache with 5 to 8 query heads per kv head are read from memory once instead of once per launch.
-// SPLIT (rows of more than 8 slabs, e.g. 32 kv heads of 128; HK = 8): neighbouring blocks take the
-// groups of 8 slabs of one token range, block index = range * groups + group; a group is a 512-byte
-// piece of every cached row.  The H2O bookkeeping needs all heads of a token and is left to a kernel
-// of its own (row_acc and row_ts are not touched here).
+// SPLIT (rows of a.row_slabs = groups x HK slabs): neighbouring blocks take the groups of HK slabs of
+// one token range, block index = range * groups + group; a group is a piece of HK x 64 bytes of every
+// cached row.  Rows of more than 8 slabs (e.g. 32 kv heads of 128) go as groups of 8; rows of 6, 8 or
+// more slabs with 5 to 8 query heads per kv head go as groups of 3 or 4 with two sets each, so that
+// also their V codes are read once.  The H2O bookkeeping needs all heads of a token and is left to a
+// kernel of its own (row_acc and row_ts are not touched here).
 template <int SCHEME, int HK, bool EXCH = false, bool NARROW = false, int NSETS = 1, bool SPLIT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i4_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
@@ -300,7 +302,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
   const int c = blockIdx.y;
   const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
-  static_assert(!SPLIT || (HK == 8 && !NARROW && NSETS == 1), "split rows: groups of 8 slabs of 128 dimensions");
+  static_assert(!SPLIT || !NARROW, "split rows: groups of HK slabs, heads of 128 dimensions");
   const int n_groups = SPLIT ? a.row_slabs / HK : 1;
   const int xb = SPLIT ? blockIdx.x / n_groups : blockIdx.x;            // token range of this block
   const int kv_off = SPLIT ? (blockIdx.x % n_groups) * HK : 0;          // its first slab
@@ -1028,9 +1030,11 @@ static void launch_attend_mfma_slabs(int n_slabs, int nsets, dim3 grid, hipStrea
 // later launch (same codes, next heads) adds its share to the accumulators that the first one has decayed.
 template <int SCHEME, bool EXCH = false>
 static void launch_attend_mfma(int n_slabs, int heads_per_slab, dim3 grid, hipStream_t st, AttendArgs a) {
-  if (n_slabs > 8) {
-    // split rows (heads of 128, whole groups of 8 slabs - checked by the caller): the groups of a token
-    // range are neighbouring blocks; the H2O bookkeeping runs first, as a kernel of its own
+  // split rows (heads of 128; whole groups of 8 slabs for more than 8 are checked by the caller): slabs per group
+  const bool wide = heads_per_slab > 4 && a.head_dim == 128;
+  const int gs = wide && n_slabs >= 8 && n_slabs % 4 == 0 ? 4 : wide && n_slabs == 6 ? 3 : n_slabs > 8 ? 8 : 0;
+  if (gs) {
+    // the groups of a token range are neighbouring blocks; the H2O bookkeeping runs first, as a kernel of its own
     if (a.row_acc || a.row_ts) {
       const dim3 ig((unsigned)((a.max_len + kAttTile - 1) / kAttTile), (unsigned)a.n_caches);
       if (EXCH) hipLaunchKernelGGL(exch_importance_kernel, ig, dim3(256), 0, st, a);
@@ -1039,11 +1043,14 @@ static void launch_attend_mfma(int n_slabs, int heads_per_slab, dim3 grid, hipSt
     a.row_acc = nullptr;
     a.row_ts = nullptr;
     a.row_slabs = n_slabs;
-    const dim3 sgrid(grid.x * (unsigned)(n_slabs / 8), grid.y);
-    const size_t lds = attend_mfma_lds_bytes(8, a.n_q_heads, 1);
-    for (int off = 0; off < heads_per_slab; off += 4) {
+    const dim3 sgrid(grid.x * (unsigned)(n_slabs / gs), grid.y);
+    const int nsets = gs == 8 ? 1 : 2;
+    const size_t lds = attend_mfma_lds_bytes(gs, a.n_q_heads, nsets);
+    for (int off = 0; off < heads_per_slab; off += 4 * nsets) {
       a.head_off = off;
-      hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 8, EXCH, false, 1, true>), sgrid, dim3(256), lds, st, a);
+      if (gs == 8) hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 8, EXCH, false, 1, true>), sgrid, dim3(256), lds, st, a);
+      else if (gs == 4) hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 4, EXCH, false, 2, true>), sgrid, dim3(256), lds, st, a);
+      else hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, 3, EXCH, false, 2, true>), sgrid, dim3(256), lds, st, a);
     }
     return;
   }

@@ -20,10 +20,10 @@ pytestmark = pytest.mark.gpu
     (O.Q_I4_ASYM, 32, 4, 4, 128),      # matrix-core form, one row pair per kv head
     (O.Q_I4_ASYM, 32, 16, 16, 128),    # 16 kv heads: two groups of 8 as neighbouring blocks of the matrix-core form
     (O.Q_I4_ASYM, 32, 32, 32, 128),    # ... 32 kv heads, four groups
-    (O.Q_I4_SYM, 32, 24, 120, 128),    # ... three groups, 5 q heads per kv head: two launches
+    (O.Q_I4_SYM, 32, 24, 120, 128),    # ... 5 q heads per kv head: six groups of 4, two sets
     (O.Q_I4_ASYM, 32, 12, 12, 128),    # 12 kv heads are no whole groups of 8: vector form
     (O.Q_I4_ASYM, 32, 8, 24, 128),     # 3 q heads per kv head: a row pair of every kv head stays empty
-    (O.Q_I4_ASYM, 32, 8, 64, 128),     # 8 q heads per kv head: two launches of four heads each
+    (O.Q_I4_ASYM, 32, 8, 64, 128),     # 8 q heads per kv head: two groups of 4 kv heads side by side, two sets of four heads each
     (O.Q_I4_SYM, 32, 2, 12, 128),      # 6 q heads per kv head: the second launch half empty
     (O.Q_I8_SYM, 128, 4, 4, 128),      # int8 per token per head
     (O.Q_I8_SYM, 256, 4, 8, 64),       # one scale per token
@@ -92,7 +92,7 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
     (O.Q_I4_ASYM, 32, 2, 4, 128),
     (O.Q_I4_ASYM, 32, 4, 32, 128),     # two launches: the second adds to what the first decayed
     (O.Q_I4_ASYM, 32, 8, 24, 128),     # 3 q heads per kv head
-    (O.Q_I4_SYM, 32, 8, 40, 128),      # 5 per kv head: second launch with a single head
+    (O.Q_I4_SYM, 32, 8, 40, 128),      # 5 per kv head: two groups of 4 kv heads, the second set with a single head
     (O.Q_I8_SYM, 128, 4, 8, 128),      # 8-bit matrix-core form
     (O.Q_I8_ASYM, 128, 8, 64, 128),    # ... 64 query heads
     (O.Q_I8_SYM, 64, 4, 8, 64),        # vector form: importance in a kernel of its own
@@ -100,7 +100,7 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
     (O.Q_I4_SYM, 32, 2, 8, 64),        # ... two launches
     (O.Q_I4_ASYM, 32, 8, 8, 32),       # heads of 32
     (O.Q_I8_ASYM, 64, 8, 16, 64),      # 8-bit heads of 64 on the matrix-core form
-    (O.Q_I4_ASYM, 32, 6, 36, 128),     # 6 kv heads x 6: two launches
+    (O.Q_I4_ASYM, 32, 6, 36, 128),     # 6 kv heads x 6: two groups of 3
     (O.Q_I8_SYM, 128, 3, 12, 128),     # 8-bit, 3 kv heads
     (O.Q_I4_ASYM, 32, 16, 32, 128),    # 16 kv heads in two groups: the importance comes from a kernel of its own
     (O.Q_I4_SYM, 32, 24, 24, 128),
@@ -185,6 +185,10 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I8_ASYM, 64, 8, 16, 64, "bf16"),    # 8-bit heads of 64 on the matrix-core kernels
     (O.Q_I8_SYM, 64, 12, 12, 64, "f32"),     # 12 kv heads of 64, 8-bit
     (O.Q_I4_ASYM, 32, 3, 6, 128, "bf16"),    # 3 kv heads
+    (O.Q_I4_ASYM, 32, 8, 64, 128, "bf16"),   # 8 q heads per kv head of 8: two groups of 4 kv heads, two sets each
+    (O.Q_I4_SYM, 32, 6, 36, 128, "f32"),     # ... 6 x 6: two groups of 3
+    (O.Q_I4_ASYM, 32, 16, 80, 128, "bf16"),  # ... 16 x 5: four groups of 4, the second set with one head
+    (O.Q_I4_SYM, 32, 7, 35, 128, "bf16"),    # 7 kv heads cannot be halved: two launches over all of them
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.9])
 def test_decode_attend_one_call(dev, scheme, group, heads, hq, dh, qdtype, decay):
