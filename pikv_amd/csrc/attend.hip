@@ -277,7 +277,12 @@ static size_t attend_mfma_lds_bytes(int n_kv_heads, int n_q_heads, int nsets = 1
 // more slabs with 5 to 8 query heads per kv head go as groups of 3 or 4 with two sets each, so that
 // also their V codes are read once.  The H2O bookkeeping needs all heads of a token and is left to a
 // kernel of its own (row_acc and row_ts are not touched here).
-template <int SCHEME, int HK, bool EXCH = false, bool NARROW = false, int NSETS = 1, bool SPLIT = false>
+// TI > 1 (rows of few slabs: 1 to 4 kv heads of 128): TI neighbouring cached rows - they lie side by side in
+// memory - are taken as ONE row of HK = TI x (real slabs) slabs, slab g' = (row parity) * slabs + g.  A tile
+// is then 64 x TI tokens: TI times fewer trips of the tile loop (each pays a memory round trip and two block
+// barriers, which is what bounds small rows) and every wavefront has a slab to multiply.  Slab g' sees the
+// probabilities of its own tokens only; the TI partial outputs of a head are added at the end, in order.
+template <int SCHEME, int HK, bool EXCH = false, bool NARROW = false, int NSETS = 1, bool SPLIT = false, int TI = 1>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i4_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 4, "4-bit schemes only");
@@ -285,6 +290,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   constexpr int NH = (HK + 3) / 4;        // kv heads per wavefront
   constexpr int NI = NH * NSETS;          // (kv head, set of four query heads) pairs per wavefront
   static_assert(NSETS == 1 || (NSETS == 2 && HK <= 4), "two sets: the staged rows of 8 x 4 heads, accumulators of one kv head");
+  static_assert(TI == 1 || (!NARROW && !SPLIT && HK % TI == 0), "interleaved rows: whole rows of 128-wide heads");
+  constexpr int HR = HK / TI;             // slabs of a cached row
+  constexpr int TT = kAttTile * TI;       // cached tokens per tile
   constexpr int RS = HK * 64 + 8;         // bytes per token row of staged codes
   constexpr int LPR = HK * 4;             // 16-byte chunks per cached row
   constexpr int NCH = kAttTile * LPR / 256 > 0 ? kAttTile * LPR / 256 : 1;  // code chunks per thread
@@ -306,7 +314,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int n_groups = SPLIT ? a.row_slabs / HK : 1;
   const int xb = SPLIT ? blockIdx.x / n_groups : blockIdx.x;            // token range of this block
   const int kv_off = SPLIT ? (blockIdx.x % n_groups) * HK : 0;          // its first slab
-  const int row_slabs = SPLIT ? a.row_slabs : HK;
+  const int row_slabs = SPLIT ? a.row_slabs : HR;
   const int64_t t0 = (int64_t)xb * a.tokens_per_block;
   const int64_t t1 = (t0 + a.tokens_per_block < len) ? t0 + a.tokens_per_block : len;
   if (t0 >= t1) {  // nothing cached in this range: the partial (of this block's heads) is zero
@@ -342,12 +350,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     for (int sg = 0; sg < 4; ++sg) zacc[hs][sg] = 0.f;
   }
   // score-staging role: staged row sh = 4 * (set * HK + kv head) + head of the set, tokens
-  // st8..st8+7 of the tile (32 rows x 8 runs); rows without a head stage zeros
-  const int sh = threadIdx.x >> 3;
-  const int st8 = (threadIdx.x & 7) * 8;
-  const int s_set = NSETS == 1 ? 0 : sh / (4 * HK);
-  const int s_g = NSETS == 1 ? sh >> 2 : (sh >> 2) % HK;
-  const bool s_on = s_set < NSETS && s_g < HK && (sh & 3) < (s_set ? rep_b : rep);
+  // st8..st8+7 of the tile (32 rows x 8 runs); rows without a head stage zeros.
+  // Interleaved rows: sh = 4 * (set * HR + kv head) + head counts the heads of the REAL rows (32 / TI of
+  // them, 8 TI runs each); a thread reads eight consecutive tokens of its head and deals them to the
+  // staged rows of the TI slabs of that kv head.
+  const int sh = TI == 1 ? threadIdx.x >> 3 : threadIdx.x / (8 * TI);
+  const int st8 = TI == 1 ? (threadIdx.x & 7) * 8 : (threadIdx.x % (8 * TI)) * 8;
+  const int s_set = NSETS == 1 && TI == 1 ? 0 : sh / (4 * HR);
+  const int s_g = NSETS == 1 && TI == 1 ? sh >> 2 : (sh >> 2) % HR;
+  const bool s_on = s_set < NSETS && s_g < HR && (sh & 3) < (s_set ? rep_b : rep);
   const int s_hq = s_on ? (kv_off + s_g) * rep_all + a.head_off + 4 * s_set + (sh & 3) : 0;
   const float* srow = a.scores + ((int64_t)c * a.n_q_heads + s_hq) * a.score_stride;
   float smx = 0.f, srz = 1.f;
@@ -360,7 +371,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   // exchange format: eight values exp(score - tile max) per thread and tile, and the tile's max of the head;
   // the rows of a tile lie side by side, [tile][q head][64], so a block reads one contiguous run
   constexpr bool exch = EXCH;
-  const float* const ep = exch ? a.escores + ((int64_t)c * a.n_tiles * a.n_q_heads + s_hq) * kAttTile + st8 : nullptr;
+  const float* const ep = exch ? a.escores + ((int64_t)c * a.n_tiles * a.n_q_heads + s_hq) * kAttTile + st8 % kAttTile : nullptr;
   const float* const tmp = exch ? a.tile_max + (int64_t)c * a.n_tiles * a.n_q_heads + s_hq : nullptr;
   float ptm = 0.f;
 
@@ -371,7 +382,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   // importance role: wavefront w owns tokens 16w..16w+15 of a tile, lanes 0..15 hold their accumulators
   const int it = wave * 16 + (lane & 15);
   const int igrp = lane >> 4;
-  float pacc = 0.f;
+  float pacc[TI];
+#pragma unroll
+  for (int k = 0; k < TI; ++k) pacc[k] = 0.f;
   // Every address below is a wave-uniform base plus a multiple of the thread index: chunk
   // ch = k * 256 + thread of the tile's code rows IS the (token, 16-byte piece) pair
   // (tok * LPR + off), and 4 * ch halves the (token, kv head) pair of the metadata rows; the
@@ -381,17 +394,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const float* const sp = srow + st8;
   auto fetch = [&](int64_t n0) {
     const int64_t left = t1 - n0;
-    const int rem = left < kAttTile ? (int)left : kAttTile;  // tokens of this tile
+    const int rem = left < TT ? (int)left : TT;  // tokens of this tile
     const int64_t urow = base_row + n0;
-    if (a.row_acc && igrp == 0 && it < rem) pacc = (a.row_acc + urow)[it];
+#pragma unroll
+    for (int k = 0; k < TI; ++k)
+      if (a.row_acc && igrp == 0 && k * kAttTile + it < rem) pacc[k] = (a.row_acc + urow)[k * kAttTile + it];
     if (exch) {
       // staged rows without a head read head 0 (and are multiplied by zero): no branch around the loads
-      const int64_t tile = n0 / kAttTile;
-      const float4 lo4 = *reinterpret_cast<const float4*>(ep + tile * a.n_q_heads * kAttTile);
-      const float4 hi4 = *reinterpret_cast<const float4*>(ep + tile * a.n_q_heads * kAttTile + 4);
+      // the 64-token tile of the exchange rows that holds this thread's tokens; with interleaved rows the
+      // last tile of the loop may reach past the range, into exchange rows that were never written
+      const int64_t tile = n0 / kAttTile + (TI == 1 ? 0 : st8 / kAttTile);
+      const bool live = TI == 1 || tile * kAttTile < t1;
+      float4 lo4 = make_float4(0.f, 0.f, 0.f, 0.f), hi4 = lo4;
+      ptm = smx;
+      if (live) {
+        lo4 = *reinterpret_cast<const float4*>(ep + tile * a.n_q_heads * kAttTile);
+        hi4 = *reinterpret_cast<const float4*>(ep + tile * a.n_q_heads * kAttTile + 4);
+        ptm = tmp[tile * a.n_q_heads];
+      }
       psc[0] = lo4.x, psc[1] = lo4.y, psc[2] = lo4.z, psc[3] = lo4.w;
       psc[4] = hi4.x, psc[5] = hi4.y, psc[6] = hi4.z, psc[7] = hi4.w;
-      ptm = tmp[tile * a.n_q_heads];
     } else if (s_on) {
       const float* spn = sp + n0;
       if (s_vec && st8 + 8 <= rem) {
@@ -427,16 +449,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
         if constexpr (!Q::sym) pz[k] = *reinterpret_cast<const uint2*>(zb + mo);
       }
     } else {
-    const char* cb = reinterpret_cast<const char*>(a.codes) + urow * (LPR * 16);
-    const unsigned c_last = (unsigned)(rem * LPR - 1) * 16u;
+    const char* cb = reinterpret_cast<const char*>(a.codes) + urow * (HR * 64);
+    const unsigned c_last = (unsigned)(rem * (HR * 4) - 1) * 16u;
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
       const unsigned off = k * 4096u + threadIdx.x * 16u;
       pc[k] = ld16(cb + (off < c_last ? off : c_last));
     }
-    const char* sb = reinterpret_cast<const char*>(a.scale) + urow * (LPR * 2);
-    const char* zb = reinterpret_cast<const char*>(a.zero) + urow * (LPR * 2);
-    const unsigned m_last = (unsigned)(rem * HK - 1) * 8u;
+    const char* sb = reinterpret_cast<const char*>(a.scale) + urow * (HR * 8);
+    const char* zb = reinterpret_cast<const char*>(a.zero) + urow * (HR * 8);
+    const unsigned m_last = (unsigned)(rem * HR - 1) * 8u;
 #pragma unroll
     for (int k = 0; k < NMC; ++k) {
       const unsigned off = k * 2048u + threadIdx.x * 8u;
@@ -459,9 +481,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       }
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
-        const int t = st8 + k;
-        lprob[sh * kAttPRow + (t & ~15) + (t & 3) * 4 + ((t >> 2) & 3)] =
-            exch ? psc[k] : (s_on ? prob_of(psc[k], smx, srz, normalise) : 0.f);
+        // token j of the tile is row j % TI of tile row t = j / TI: it belongs to slab (j % TI) * HR + kv head
+        const int t = (st8 + k) / TI;
+        const int row = TI == 1 ? sh : ((s_set * HK + ((st8 + k) % TI) * HR + s_g) * 4 + (sh & 3));
+        if (TI == 1 || s_set < NSETS)
+          lprob[row * kAttPRow + (t & ~15) + (t & 3) * 4 + ((t >> 2) & 3)] =
+              exch ? psc[k] : (s_on ? prob_of(psc[k], smx, srz, normalise) : 0.f);
       }
     }
 #pragma unroll
@@ -505,12 +530,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   asm volatile("" : "+v"(kNib), "+v"(kExp));
 
   fetch(t0);
-  for (int64_t n0 = t0; n0 < t1; n0 += kAttTile) {
+  for (int64_t n0 = t0; n0 < t1; n0 += TT) {
     __syncthreads();  // the previous tile has been consumed
     stage();
     __syncthreads();
-    float acc = pacc;
-    if (a.row_acc || a.row_ts) {  // uniform
+    if constexpr (TI > 1) {
+      if (a.row_acc || a.row_ts) {  // uniform
+        // token j = 64 k + it of the tile is row j % TI of tile row j / TI: its probabilities are the staged
+        // rows of the slabs of that parity
+        float* const acc_rows = a.row_acc ? a.row_acc + (base_row + n0) : nullptr;
+        float* const ts_rows = a.row_ts ? a.row_ts + (base_row + n0) : nullptr;
+#pragma unroll
+        for (int k = 0; k < TI; ++k) {
+          const int j = k * kAttTile + it;
+          const int vt = j / TI, par = j % TI;
+          const float* lp = lprob + igrp * kAttPRow + (vt & ~15) + (vt & 3) * 4 + ((vt >> 2) & 3);
+          float imp = 0.f;
+#pragma unroll
+          for (int hs = 0; hs < NSETS * HR; ++hs)
+            imp = imp + lp[((hs / HR) * HK + par * HR + hs % HR) * 4 * kAttPRow];
+          imp = imp + __shfl_xor(imp, 16, 64);
+          imp = imp + __shfl_xor(imp, 32, 64);
+          if (igrp == 0 && n0 + j < t1) {
+            if (acc_rows) {
+              float acc = pacc[k];
+              if (a.decay != 1.0f) acc = acc * a.decay;
+              acc_rows[j] = acc + imp;
+            }
+            if (ts_rows) {
+              float now = a.now;
+              asm volatile("" : "+v"(now));
+              ts_rows[j] = now;
+            }
+          }
+        }
+      }
+    }
+    float acc = pacc[0];
+    if (TI == 1 && (a.row_acc || a.row_ts)) {  // uniform
       // importance of the tile's tokens: four lanes per token add every fourth head, and two
       // exchanges add the four partial sums
       const int t = it;
@@ -541,7 +598,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     // The next tile's loads go out AFTER the bookkeeping stores: the wait at the top of the
     // loop covers everything outstanding, and stores issued behind the loads had been
     // adding their latency to it (366 vs 347 us).
-    if (n0 + kAttTile < t1) fetch(n0 + kAttTile);  // in flight while this tile is multiplied
+    if (n0 + TT < t1) fetch(n0 + TT);  // in flight while this tile is multiplied
 
 #pragma unroll
     for (int hk = 0; hk < NH; ++hk) {   // kv head slot of this wavefront
@@ -648,6 +705,37 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       if ((lane & 15) == 0) zl[((wave * NI + hs) * 4 + r) * 4 + sg] = z;
     }
   __syncthreads();
+  if constexpr (TI > 1) {
+    // the TI slabs of a kv head hold partial outputs over different tokens: added in LDS, parity by parity
+    float* ol = zl + 4 * NI * 4 * 4;   // [kv head][head of the launch: 4 * set + ro][128]
+    for (int par = 0; par < TI; ++par) {
+#pragma unroll
+      for (int hs = 0; hs < NI; ++hs) {
+        const int set = hs % NSETS;
+        const int g = wave + 4 * (hs / NSETS);
+        if (g >= HK || g / HR != par) continue;  // uniform
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+          const int ro = 2 * kg + rr;
+          if (ro >= (set ? rep_b : rep)) continue;
+          float* o = ol + ((g % HR) * (4 * NSETS) + 4 * set + ro) * 128;
+#pragma unroll
+          for (int db = 0; db < 8; ++db) {
+            const float v = (C[hs][db][2 * rr] + C[hs][db][2 * rr + 1]) - zl[((wave * NI + hs) * 4 + ro) * 4 + (db >> 1)];
+            o[db * 16 + i] = par == 0 ? v : o[db * 16 + i] + v;
+          }
+        }
+      }
+      __syncthreads();
+    }
+    const int heads = rep + rep_b;   // heads of a kv head in this launch
+    for (int idx = threadIdx.x; idx < HR * 4 * NSETS * 128; idx += 256) {
+      const int row = idx >> 7, g = row / (4 * NSETS), hl = row % (4 * NSETS);
+      if (hl < heads)
+        a.partial[(((int64_t)xb * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + hl) * 128 + (idx & 127)] = ol[idx];
+    }
+    return;
+  }
 #pragma unroll
   for (int hs = 0; hs < NI; ++hs) {
     const int set = hs % NSETS;
@@ -1055,10 +1143,33 @@ static void launch_attend_mfma(int n_slabs, int heads_per_slab, dim3 grid, hipSt
     return;
   }
   const int nsets = (n_slabs <= 4 && heads_per_slab > 4) ? 2 : 1;
+  // rows of few slabs: 8, 4 or 2 neighbouring rows as one (a block's token range must hold whole tiles of them)
+  int ti = 1;
+  if (a.head_dim == 128 && n_slabs <= 4) {
+    const int room = (nsets == 2 ? 4 : 8) / n_slabs;
+    ti = room >= 8 ? 8 : room >= 4 ? 4 : room >= 2 ? 2 : 1;
+    while (ti > 1 && a.tokens_per_block % (kAttTile * ti) != 0) ti >>= 1;
+    // 4 slabs already fill the wavefronts; pairs of rows gain 5 % on the exchange rows and lose 4 % on float scores
+    if (n_slabs == 4 && !EXCH) ti = 1;
+  }
   for (int off = 0; off < heads_per_slab; off += 4 * nsets) {
     a.head_off = off;
     if (off > 0) a.decay = 1.0f;
-    if (a.head_dim == 128) launch_attend_mfma_slabs<SCHEME, EXCH, false>(n_slabs, nsets, grid, st, a);
+    if (ti > 1) {
+      const int hk = n_slabs * ti;
+      const size_t lds = attend_mfma_lds_bytes(hk, a.n_q_heads, nsets);
+#define PIKV_ATT_ROWS(HKV, TIV, NS)                                                                              \
+  if (hk == HKV && ti == TIV && nsets == NS)                                                                     \
+    hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, HKV, EXCH, false, NS, false, TIV>), grid, dim3(256), lds, st, a);
+      PIKV_ATT_ROWS(8, 8, 1)   // 1 kv head
+      PIKV_ATT_ROWS(4, 4, 1)   // ... token ranges of 256
+      PIKV_ATT_ROWS(8, 4, 1)   // 2
+      PIKV_ATT_ROWS(6, 2, 1)   // 3
+      PIKV_ATT_ROWS(8, 2, 1)   // 4
+      PIKV_ATT_ROWS(4, 4, 2)   // 1 kv head, 5-8 query heads
+      PIKV_ATT_ROWS(4, 2, 2)   // 2 kv heads, 5-8 query heads each
+#undef PIKV_ATT_ROWS
+    } else if (a.head_dim == 128) launch_attend_mfma_slabs<SCHEME, EXCH, false>(n_slabs, nsets, grid, st, a);
     else launch_attend_mfma_slabs<SCHEME, EXCH, true>(n_slabs, nsets, grid, st, a);
   }
 }

@@ -104,6 +104,10 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
     (O.Q_I8_SYM, 128, 3, 12, 128),     # 8-bit, 3 kv heads
     (O.Q_I4_ASYM, 32, 16, 32, 128),    # 16 kv heads in two groups: the importance comes from a kernel of its own
     (O.Q_I4_SYM, 32, 24, 24, 128),
+    (O.Q_I4_ASYM, 32, 1, 4, 128),      # one kv head: four neighbouring rows as one row of four slabs
+    (O.Q_I4_SYM, 32, 1, 8, 128),       # ... 8 q heads: two sets
+    (O.Q_I4_ASYM, 32, 2, 12, 128),     # two kv heads x 6: pairs of rows, two sets
+    (O.Q_I4_ASYM, 32, 3, 9, 128),      # three kv heads: pairs of rows, six slabs
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.95])
 def test_attend_accumulates_importance(dev, scheme, group, heads, hq, dh, decay):
@@ -189,6 +193,9 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I4_SYM, 32, 6, 36, 128, "f32"),     # ... 6 x 6: two groups of 3
     (O.Q_I4_ASYM, 32, 16, 80, 128, "bf16"),  # ... 16 x 5: four groups of 4, the second set with one head
     (O.Q_I4_SYM, 32, 7, 35, 128, "bf16"),    # 7 kv heads cannot be halved: two launches over all of them
+    (O.Q_I4_ASYM, 32, 4, 16, 128, "bf16"),   # 4 kv heads: pairs of neighbouring rows as one row of eight slabs
+    (O.Q_I4_SYM, 32, 2, 8, 128, "f32"),      # 2 kv heads: four rows as one
+    (O.Q_I4_ASYM, 32, 1, 3, 128, "bf16"),    # 1 kv head, 3 q heads
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.9])
 def test_decode_attend_one_call(dev, scheme, group, heads, hq, dh, qdtype, decay):
@@ -266,7 +273,7 @@ def test_decode_attend_one_call(dev, scheme, group, heads, hq, dh, qdtype, decay
 
 
 @pytest.mark.parametrize("n_caches,length,scheme,heads,hq", [
-    (64, 4096, O.Q_I4_ASYM, 1, 4),     # 512 blocks of 512 cached tokens
+    (64, 4096, O.Q_I4_ASYM, 1, 4),     # 512 blocks of 512 cached tokens: eight neighbouring rows of the one kv head as one row
     (64, 7168, O.Q_I4_SYM, 1, 2),      # 448 blocks of 1024
     (56, 16384, O.Q_I4_ASYM, 1, 1),    # 448 blocks of 2048
     (40, 2500, O.Q_I8_SYM, 1, 2),      # 8-bit matrix-core form, 400 blocks of 256, ragged lengths
