@@ -558,7 +558,7 @@ static size_t gqa_lds_bytes(int n_kv_heads, int nset, int na) {
 // SPLIT (rows of more than 16 slabs, e.g. 32 kv heads of 128): a block takes a group of a.n_kv_heads slabs
 // out of the a.row_slabs of a cached row; the groups of a tile are independent blocks with neighbouring
 // block indices, so that whole rows are in flight at any time and not one 512-byte window of every row.
-template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false, bool NARROW = false, bool QF32 = false, bool SPLIT = false>  // NKV = n_kv_heads rounded up to 4/8/16; EXCH: exchange format out
+template <int SCHEME, int NKV, int NSET = 1, bool EXCH = false, bool NARROW = false, bool QF32 = false, bool SPLIT = false>  // NKV = n_kv_heads rounded up to 2/4/8/16; EXCH: exchange format out
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET <= 8 ? 4 : 2))) void scores_mfma_i4_gqa_kernel(ScoreArgs a) {
   constexpr int SL = 4 * NSET;  // head slots per kv head
   using Q = QScheme<SCHEME>;
@@ -615,7 +615,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   // Code vectors of this wavefront's slice of tile tt (one 16-byte load per kv
   // head) and this thread's share of the tile's (scale, zero) rows: chunk
   // j*256 + thread = (token, kv head), 8 bytes each.
-  constexpr int NM = NKV / 4;
+  constexpr int NM = (NKV + 3) / 4;   // 256 (token, kv head) chunks per pass
   struct TileRegs {
     uint4 cv[NKV];
     uint2 sv[NM], zv[NM];
@@ -1001,18 +1001,27 @@ static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, h
   const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset, qf32 ? 2 * nset : nset);   // float32 queries: a copy of the A operands per limb
   if (rep > 8 || lds > 64 * 1024 || a.n_kv_heads > (qf32 ? 8 : kGqaMaxKvHeads)) return PIKV_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
+  // (rows of 1 or 2 slabs have a kernel of their own: fewer registers, 8 instead of 6 blocks per compute unit,
+  // and with 5 KB tiles the bytes in flight are what bounds them - 1 kv head x 4 q heads 61.3 -> 52.1 us,
+  // 2 x 8: 83.6 -> 76.8 us at 64 caches x 32768 tokens)
   if (qf32 && nset == 1) {
-    if (a.n_kv_heads <= 4)
+    if (a.n_kv_heads <= 2)
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 2, 1, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
+    else if (a.n_kv_heads <= 4)
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
     else
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
   } else if (qf32) {
-    if (a.n_kv_heads <= 4)
+    if (a.n_kv_heads <= 2)
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 2, 2, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
+    else if (a.n_kv_heads <= 4)
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
     else
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH, NARROW, true>), grid, dim3(256), lds, st, a);
   } else if (nset == 1) {
-    if (a.n_kv_heads <= 4)
+    if (a.n_kv_heads <= 2)
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 2, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a);
+    else if (a.n_kv_heads <= 4)
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a);
     else if (a.n_kv_heads <= 8)
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a);
@@ -1020,7 +1029,9 @@ static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, h
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 16, 1, EXCH, NARROW>), grid, dim3(256), lds, st, a);
   } else {
     // 5-8 query heads per kv head; 16 kv heads x 8 would need more than 64 KB of LDS
-    if (a.n_kv_heads <= 4)
+    if (a.n_kv_heads <= 2)
+      hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 2, 2, EXCH, NARROW>), grid, dim3(256), lds, st, a);
+    else if (a.n_kv_heads <= 4)
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2, EXCH, NARROW>), grid, dim3(256), lds, st, a);
     else
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH, NARROW>), grid, dim3(256), lds, st, a);
