@@ -853,11 +853,15 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   // A operands of this wavefront's kv heads: lane (row nl = query head, k-slice rg), k-step
   // (half, b2) covers dimensions d0 = 64*half + 16*rg + 4*b2 .. +3 in the slot order
   // {d0, d0+2, 16x d0, 16x d0+2, d0+1, d0+3, 16x d0+1, 16x d0+3} that the nibble unpack produces.
+  // Rows of 1 or 2 slabs (spread): the wavefronts take (kv head, tile) pairs - item = wave + 4 * round is kv
+  // head item % n_kv_heads of tile item / n_kv_heads - so that all four load and multiply and 4 / n_kv_heads
+  // tiles of the block are in flight at a time; a wavefront's kv head is the same in every round.
+  const int spread = (NHW == 1 && a.n_kv_heads <= 2) ? a.n_kv_heads : 0;
   uint4 areg[NHW][8];
   float qs[NHW][4];
 #pragma unroll
   for (int hs = 0; hs < NHW; ++hs) {
-    const int g = wave + 4 * hs;
+    const int g = spread ? wave % spread : wave + 4 * hs;
     const bool on = g < a.n_kv_heads && (nl >> RSH) < rep;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
@@ -895,14 +899,9 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
     for (int qq = 0; qq < 4; ++qq) qs[hs][qq] = sumq[qq];
   }
 
-  for (int tt = 0; tt < kI8TilesPerBlock; ++tt) {
-    const int64_t tile = tile0 + tt;
-    const int64_t n0 = tile * kTile;
-    if (n0 >= len) break;  // uniform
-#pragma unroll
-    for (int hs = 0; hs < NHW; ++hs) {
-      const int g = wave + 4 * hs;
-      if (g >= a.n_kv_heads) continue;  // uniform
+  // kv head g (A operands of slot hs) against the tile that starts at token n0, scores into st
+  auto head_tile = [&](int hs, int g, int64_t n0, float* st) {
+    {
       // the four 16-token slices of the tile: two 16-byte halves and the metadata of each
       uint4 cv[4][2];
       float sc[4][HPS], zr[4][HPS];
@@ -958,17 +957,44 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
           for (int hq2 = 0; hq2 < 2; ++hq2) {   // rows (2 hq2, 2 hq2 + 1) of this lane: the limbs of one head
             const int r = 2 * rg + hq2;
             if (r < rep)
-              stage[(g * rep + r) * kTile + 16 * sl + nl] =
+              st[(g * rep + r) * kTile + 16 * sl + nl] =
                   ok[sl] ? row_score[2 * hq2] + row_score[2 * hq2 + 1] : -__builtin_inff();
           }
         } else {
 #pragma unroll
           for (int qq = 0; qq < 4; ++qq) {
             const int r = 4 * rg + qq;
-            if (r < rep) stage[(g * rep + r) * kTile + 16 * sl + nl] = ok[sl] ? row_score[qq] : -__builtin_inff();
+            if (r < rep) st[(g * rep + r) * kTile + 16 * sl + nl] = ok[sl] ? row_score[qq] : -__builtin_inff();
           }
         }
       }
+    }
+  };
+  if (spread) {
+    const int tpr = kI8TilesPerBlock / spread;   // tiles per round, each with a staging area of its own
+    for (int round = 0; round < spread; ++round) {
+      const int item = wave + 4 * round;
+      const int tt = item / spread;
+      if ((tile0 + tt) * kTile < len) head_tile(0, item % spread, (tile0 + tt) * kTile, stage + (tt % tpr) * a.n_q_heads * kTile);
+      __syncthreads();
+      for (int k = 0; k < tpr; ++k) {
+        const int64_t tile = tile0 + round * tpr + k;
+        if (tile * kTile < len)  // uniform
+          tile_stats_store<false>(a, stage + k * a.n_q_heads * kTile, c, tile, tile * kTile, len, wave, rg, nl);
+      }
+      __syncthreads();  // the staging areas are reused by the next round
+    }
+    return;
+  }
+  for (int tt = 0; tt < kI8TilesPerBlock; ++tt) {
+    const int64_t tile = tile0 + tt;
+    const int64_t n0 = tile * kTile;
+    if (n0 >= len) break;  // uniform
+#pragma unroll
+    for (int hs = 0; hs < NHW; ++hs) {
+      const int g = wave + 4 * hs;
+      if (g >= a.n_kv_heads) continue;  // uniform
+      head_tile(hs, g, n0, stage);
     }
     __syncthreads();
     tile_stats_store<false>(a, stage, c, tile, n0, len, wave, rg, nl);
@@ -978,7 +1004,8 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
 
 template <int SCHEME, int HPS, bool QF32>
 static void launch_i8_mfma_q(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
-  const size_t lds = (size_t)a.n_q_heads * kTile * sizeof(float);
+  // rows of 1 or 2 slabs stage 4 or 2 tiles at a time
+  const size_t lds = (size_t)a.n_q_heads * kTile * sizeof(float) * (a.n_kv_heads <= 2 ? kI8TilesPerBlock / a.n_kv_heads : 1);
   const dim3 grid((unsigned)((n_tiles + kI8TilesPerBlock - 1) / kI8TilesPerBlock), (unsigned)n_caches);
   if (a.n_kv_heads <= 4)
     hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 1, HPS, QF32>), grid, dim3(256), lds, st, a);
