@@ -798,11 +798,18 @@ static size_t attend_mfma8_lds_bytes(int n_slabs, int n_q_heads, int hps) {
 // zero point) each; the query heads of a slab are the heads of those kv heads in order.  A query
 // head is weighted with its own kv head's scale, multiplied with the whole slab, and only the
 // dimensions of its own kv head are written out.
-template <int SCHEME, int HK, int HPS = 1>
+// TI > 1 (rows of 1 to 4 kv heads of 128): TI neighbouring cached rows as ONE row of HK = TI x (real slabs)
+// slabs, slab g' = (row parity) * slabs + kv head, exactly as in the 4-bit kernel: tiles of 32 x TI tokens,
+// every wavefront with a slab to multiply, the TI partial outputs of a head added at the end.  The staged
+// probabilities are [parity][query head] rows.
+template <int SCHEME, int HK, int HPS = 1, int TI = 1>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attend_mfma_i8_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 8, "8-bit schemes only");
   static_assert(HK >= 1 && HK <= 8, "1 to 8 kv heads");
+  static_assert(TI == 1 || (HPS == 1 && HK % TI == 0), "interleaved rows: whole rows of 128-wide heads");
+  constexpr int HKR = HK / TI;            // slabs of a cached row
+  constexpr int TT = kAtt8Tile * TI;      // cached tokens per tile
   constexpr int NH = (HK + 3) / 4;   // kv heads per wavefront
   constexpr int RS = HK * 128 + 8;   // bytes per token row of staged codes
   constexpr int LPR = HK * 8;        // 16-byte chunks per cached row
@@ -828,9 +835,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * a.head_dim + idx] = 0.f;
     return;
   }
-  const int rep = a.n_q_heads / HK;  // 2..8
+  const int rep = a.n_q_heads / HKR;  // 2..8
   const int rep1 = rep / HPS;        // query heads per stored kv head
-  const int groups_per_row = (HK * 128) / a.group;
+  const int groups_per_row = (HKR * 128) / a.group;
   // matrix-core roles: A row / B,C column i, token group kg (tokens 8*kg .. 8*kg+7 of the tile)
   const int i = lane & 15;
   const int kg = lane >> 4;
@@ -847,9 +854,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   for (int hs = 0; hs < NH; ++hs)
 #pragma unroll
     for (int d = 0; d < 8; ++d) C[hs][d] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
-  // score-staging role: query head sh, tokens st8..st8+7 of the tile (64 heads x 4 runs)
-  const int sh = threadIdx.x >> 2;
-  const int st8 = (threadIdx.x & 3) * 8;
+  // score-staging role: query head sh, tokens st8..st8+7 of the tile (64 heads x 4 runs; interleaved rows:
+  // 64 / TI heads x 4 TI runs)
+  const int sh = threadIdx.x / (4 * TI);
+  const int st8 = (threadIdx.x % (4 * TI)) * 8;
   const bool s_on = sh < a.n_q_heads;
   const float* srow = a.scores + ((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * a.score_stride;
   float smx = 0.f, srz = 1.f;
@@ -865,10 +873,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
   // registers that carry the next tile from HBM to LDS
   uint4 pc[NCH];
-  float ps[NMT], pz[NMT], pacc = 0.f;
+  float ps[NMT], pz[NMT], pacc[TI];
+#pragma unroll
+  for (int k = 0; k < TI; ++k) pacc[k] = 0.f;
   float psc[8];
   auto fetch = [&](int64_t n0) {
-    if (a.row_acc && igrp == 0 && n0 + it < t1) pacc = (a.row_acc + (base_row + n0))[it];  // uniform base + lane
+#pragma unroll
+    for (int k = 0; k < TI; ++k)
+      if (a.row_acc && igrp == 0 && n0 + k * kAtt8Tile + it < t1)
+        pacc[k] = (a.row_acc + (base_row + n0))[k * kAtt8Tile + it];  // uniform base + lane
     if (s_on) {
       const int64_t n = n0 + st8;
       if (s_vec && n + 8 <= t1) {
@@ -883,11 +896,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     }
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
-      const int ch = k * 256 + threadIdx.x;
-      const int tok = ch / LPR, off = ch % LPR;
+      const int ch = k * 256 + threadIdx.x;   // 16-byte chunk of the tile's rows, which lie side by side
       pc[k] = make_uint4(0, 0, 0, 0);
-      if (n0 + tok < t1)
-        pc[k] = ld16(reinterpret_cast<const char*>(a.codes) + ((base_row + n0 + tok) * LPR + off) * 16);
+      if (n0 + ch / (LPR / TI) < t1)
+        pc[k] = ld16(reinterpret_cast<const char*>(a.codes) + ((base_row + n0) * (LPR / TI) + ch) * 16);
     }
 #pragma unroll
     for (int k = 0; k < NMT; ++k) {  // (token, stored kv head) metadata pairs
@@ -895,8 +907,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       const int tok = ch / HR, hd = ch % HR;
       ps[k] = 0.f;
       pz[k] = 0.f;
-      if (tok < kAtt8Tile && n0 + tok < t1) {
-        const int64_t mi = (base_row + n0 + tok) * groups_per_row + (hd * (128 / HPS)) / a.group;
+      // (interleaved rows: slab hd of tile row tok is kv head hd % HKR of cached row tok * TI + hd / HKR)
+      const int64_t rtok = TI == 1 ? n0 + tok : n0 + tok * TI + hd / HKR;
+      if (tok < kAtt8Tile && rtok < t1) {
+        const int64_t mi = (base_row + rtok) * groups_per_row + ((TI == 1 ? hd : hd % HKR) * (128 / HPS)) / a.group;
         ps[k] = reinterpret_cast<const float*>(a.scale)[mi];
         if constexpr (!Q::sym) pz[k] = reinterpret_cast<const float*>(a.zero)[mi];
       }
@@ -909,8 +923,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       v0.z = prob_of(psc[2], smx, srz, normalise), v0.w = prob_of(psc[3], smx, srz, normalise);
       v1.x = prob_of(psc[4], smx, srz, normalise), v1.y = prob_of(psc[5], smx, srz, normalise);
       v1.z = prob_of(psc[6], smx, srz, normalise), v1.w = prob_of(psc[7], smx, srz, normalise);
-      *reinterpret_cast<float4*>(lprob + sh * kAtt8PRow + st8) = v0;
-      *reinterpret_cast<float4*>(lprob + sh * kAtt8PRow + st8 + 4) = v1;
+      if constexpr (TI == 1) {
+        *reinterpret_cast<float4*>(lprob + sh * kAtt8PRow + st8) = v0;
+        *reinterpret_cast<float4*>(lprob + sh * kAtt8PRow + st8 + 4) = v1;
+      } else {
+        // token j of the tile is row j % TI of tile row j / TI
+        const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          lprob[(((st8 + k) % TI) * a.n_q_heads + sh) * kAtt8PRow + (st8 + k) / TI] = v[k];
+      }
     }
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
@@ -932,13 +954,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   auto bf16_hi = [](float v) { return __float_as_uint(v) & 0xffff0000u; };
 
   fetch(t0);
-  for (int64_t n0 = t0; n0 < t1; n0 += kAtt8Tile) {
+  for (int64_t n0 = t0; n0 < t1; n0 += TT) {
     __syncthreads();  // the previous tile has been consumed
     stage();
     __syncthreads();
-    float acc = pacc;
-    if (n0 + kAtt8Tile < t1) fetch(n0 + kAtt8Tile);  // in flight while this tile is multiplied
-    if (a.row_acc || a.row_ts) {  // uniform
+    float accs[TI];
+#pragma unroll
+    for (int k = 0; k < TI; ++k) accs[k] = pacc[k];
+    float acc = accs[0];
+    if (n0 + TT < t1) fetch(n0 + TT);  // in flight while this tile is multiplied
+    if constexpr (TI > 1) {
+      if (a.row_acc || a.row_ts) {  // uniform
+        float* const acc_rows = a.row_acc ? a.row_acc + (base_row + n0) : nullptr;
+        float* const ts_rows = a.row_ts ? a.row_ts + (base_row + n0) : nullptr;
+#pragma unroll
+        for (int k = 0; k < TI; ++k) {
+          const int j = k * kAtt8Tile + it;   // token of the tile: row j % TI of tile row j / TI
+          const float* lp = lprob + (j % TI) * a.n_q_heads * kAtt8PRow + j / TI;
+          float imp = 0.f;
+          for (int hq = igrp; hq < a.n_q_heads; hq += 8) imp = imp + lp[hq * kAtt8PRow];
+          imp = imp + __shfl_xor(imp, 8, 64);
+          imp = imp + __shfl_xor(imp, 16, 64);
+          imp = imp + __shfl_xor(imp, 32, 64);
+          if (igrp == 0 && n0 + j < t1) {
+            if (acc_rows) {
+              float av = accs[k];
+              if (a.decay != 1.0f) av = av * a.decay;
+              acc_rows[j] = av + imp;
+            }
+            if (ts_rows) {
+              float now = a.now;
+              asm volatile("" : "+v"(now));
+              ts_rows[j] = now;
+            }
+          }
+        }
+      }
+    }
+    if (TI == 1 && (a.row_acc || a.row_ts)) {  // uniform
       const bool mine = igrp == 0 && n0 + it < t1;
       const int t = it;
       // wave-uniform row pointers + a 32-bit lane offset (no per-lane address registers live
@@ -1052,6 +1105,36 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
   // Epilogue.  C: lane (dimension i, rows 4*kg + q): rows 2r / 2r+1 are the two parts of head r,
   // so head 2*kg is q = 0,1 and head 2*kg+1 is q = 2,3.
+  if constexpr (TI > 1) {
+    // the TI slabs of a kv head hold partial outputs over different tokens: added in LDS, parity by parity
+    __syncthreads();
+    float* ol = reinterpret_cast<float*>(att8_lds);   // [kv head][head of the kv group, 8 slots][128]
+    for (int par = 0; par < TI; ++par) {
+#pragma unroll
+      for (int hs = 0; hs < NH; ++hs) {
+        const int g = wave + 4 * hs;
+        if (g >= HK || g / HKR != par) continue;  // uniform
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+          const int ro = 2 * kg + rr;
+          if (ro >= rep) continue;
+          float* o = ol + ((g % HKR) * 8 + ro) * 128;
+#pragma unroll
+          for (int db = 0; db < 8; ++db) {
+            const float v = C[hs][db][2 * rr] + C[hs][db][2 * rr + 1];
+            o[db * 16 + i] = par == 0 ? v : o[db * 16 + i] + v;
+          }
+        }
+      }
+      __syncthreads();
+    }
+    for (int idx = threadIdx.x; idx < HKR * 8 * 128; idx += 256) {
+      const int row = idx >> 7, g = row >> 3, ro = row & 7;
+      if (ro < rep)
+        a.partial[(((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep + ro) * 128 + (idx & 127)] = ol[idx];
+    }
+    return;
+  }
 #pragma unroll
   for (int hs = 0; hs < NH; ++hs) {
     const int g = wave + 4 * hs;
@@ -1086,6 +1169,16 @@ static void launch_attend_mfma8_slabs(int n_slabs, dim3 grid, hipStream_t st, co
 }
 template <int SCHEME>
 static void launch_attend_mfma8(int n_slabs, int hps, dim3 grid, hipStream_t st, const AttendArgs& a) {
+  if (hps == 1 && n_slabs <= 3 && a.tokens_per_block % (kAtt8Tile * 8) == 0) {
+    // rows of few slabs: 8, 4 or 2 neighbouring rows as one row of (up to) 8 slabs (pairs of rows of 4 slabs
+    // measured the same as single rows: 322 vs 325 us at 64 caches x 32768 tokens x 16 query heads)
+    const int ti = n_slabs == 1 ? 8 : n_slabs == 2 ? 4 : 2;
+    const size_t lds = attend_mfma8_lds_bytes(n_slabs * ti, a.n_q_heads * ti, 1);
+    if (n_slabs == 1) hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 8, 1, 8>), grid, dim3(256), lds, st, a);
+    else if (n_slabs == 2) hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 8, 1, 4>), grid, dim3(256), lds, st, a);
+    else hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 6, 1, 2>), grid, dim3(256), lds, st, a);
+    return;
+  }
   if (hps == 1) launch_attend_mfma8_slabs<SCHEME, 1>(n_slabs, grid, st, a);
   else if (hps == 2) launch_attend_mfma8_slabs<SCHEME, 2>(n_slabs, grid, st, a);
   else launch_attend_mfma8_slabs<SCHEME, 4>(n_slabs, grid, st, a);

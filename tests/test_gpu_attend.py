@@ -108,6 +108,8 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
     (O.Q_I4_SYM, 32, 1, 8, 128),       # ... 8 q heads: two sets
     (O.Q_I4_ASYM, 32, 2, 12, 128),     # two kv heads x 6: pairs of rows, two sets
     (O.Q_I4_ASYM, 32, 3, 9, 128),      # three kv heads: pairs of rows, six slabs
+    (O.Q_I8_ASYM, 128, 1, 8, 128),     # 8-bit, one kv head: eight neighbouring rows as one row
+    (O.Q_I8_SYM, 128, 2, 4, 128),      # ... two kv heads: four rows
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.95])
 def test_attend_accumulates_importance(dev, scheme, group, heads, hq, dh, decay):
@@ -196,6 +198,14 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I4_ASYM, 32, 4, 16, 128, "bf16"),   # 4 kv heads: pairs of neighbouring rows as one row of eight slabs
     (O.Q_I4_SYM, 32, 2, 8, 128, "f32"),      # 2 kv heads: four rows as one
     (O.Q_I4_ASYM, 32, 1, 3, 128, "bf16"),    # 1 kv head, 3 q heads
+    (O.Q_I8_ASYM, 128, 2, 8, 128, "bf16"),   # 8-bit, 2 kv heads: four neighbouring rows as one row of eight slabs
+    (O.Q_I8_SYM, 128, 1, 4, 128, "f32"),     # ... 1 kv head: eight rows as one
+    (O.Q_I8_SYM, 128, 3, 12, 128, "bf16"),   # ... 3 kv heads x 4: pairs of rows, 24 staged probability rows
+    # 3 kv heads x 8: this draw has scores up to 36, and the 8-bit matrix-core scores carry an absolute error
+    # of about 1e-4 there (their nibble offsets make the accumulators ~250 times the score): the output misses
+    # the 1e-3 bar by the score side alone (1.4e-3 of its root-mean-square; the output side is 2.6e-4)
+    pytest.param(O.Q_I8_SYM, 128, 3, 24, 128, "bf16",
+                 marks=pytest.mark.xfail(reason="8-bit matrix-core scores: 1e-4 absolute at |score| 36", strict=False)),
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.9])
 def test_decode_attend_one_call(dev, scheme, group, heads, hq, dh, qdtype, decay):
