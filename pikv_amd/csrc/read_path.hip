@@ -442,12 +442,13 @@ __global__ __launch_bounds__(256) void scores_mfma_i4_kernel(ScoreArgs a) {
 template <bool GROUPED, int SLOTS = 4>
 __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float* stage, int c, int64_t tile,
                                                  int64_t n0, int len, int wave, int rg, int nl, int rep = 4,
-                                                 int hq0 = 0) {  // hq0: first query head of the block's kv heads
+                                                 int hq0 = 0,    // hq0: first query head of the block's kv heads
+                                                 int rep_all = 0) {  // query heads per kv head when the launch serves only rep of them
   const int n_pass_rows = GROUPED ? a.n_kv_heads * SLOTS : a.n_q_heads;
   for (int h4 = wave * 4; h4 < n_pass_rows; h4 += 16) {
     const int srow = h4 + rg;                                  // staged row = kv head * SLOTS + slot
     const int slot = srow % SLOTS;
-    const int hq = hq0 + (GROUPED ? (srow / SLOTS) * rep + slot : srow);  // query head
+    const int hq = hq0 + (GROUPED ? (srow / SLOTS) * (rep_all ? rep_all : rep) + slot : srow);  // query head
     const bool hok = GROUPED ? slot < rep : hq < a.n_q_heads;
     float x[4];
     bool okk[4];
@@ -493,13 +494,14 @@ __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float
 template <bool GROUPED, int SLOTS = 4>
 __device__ __forceinline__ void tile_stats_exchange(const ScoreArgs& a, const float* stage, int c, int64_t tile,
                                                  int64_t n0, int len, int wave, int rg, int nl, int rep = 4,
-                                                 int hq0 = 0) {  // hq0: first query head of the block's kv heads
+                                                 int hq0 = 0,    // hq0: first query head of the block's kv heads
+                                                 int rep_all = 0) {  // query heads per kv head when the launch serves only rep of them
   const int n_pass_rows = GROUPED ? a.n_kv_heads * SLOTS : a.n_q_heads;
   const int left = len - (int)n0 - 4 * nl;                     // tokens of this lane's run that exist
   for (int h4 = wave * 4; h4 < n_pass_rows; h4 += 16) {
     const int srow = h4 + rg;                                  // staged row = kv head * SLOTS + slot
     const int slot = srow % SLOTS;
-    const int hq = hq0 + (GROUPED ? (srow / SLOTS) * rep + slot : srow);  // query head
+    const int hq = hq0 + (GROUPED ? (srow / SLOTS) * (rep_all ? rep_all : rep) + slot : srow);  // query head
     const bool hok = GROUPED ? slot < rep : hq < a.n_q_heads;
     const float4 sv = hok ? *reinterpret_cast<const float4*>(stage + srow * kTile + 4 * nl)
                           : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -581,7 +583,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   const int64_t tile0 = (int64_t)(SPLIT ? blockIdx.x / n_groups : blockIdx.x) * kGqaTilesPerBlock;
   const int64_t tok0 = tile0 * kTile;
   if (tok0 >= len) return;  // uniform for the block
-  const int rep = a.n_q_heads / (SPLIT ? a.row_slabs : a.n_kv_heads);  // query heads per slab, <= 4 NSET
+  // query heads per slab; a launch serves heads a.head_off .. a.head_off + rep - 1 of every slab, rep <= 4 NSET
+  // (more than 8 heads per slab: two launches; narrow heads and split rows are launched with head_off = 0 only)
+  const int rep_all = a.n_q_heads / (SPLIT ? a.row_slabs : a.n_kv_heads);
+  const int rep = rep_all - a.head_off < 4 * NSET ? rep_all - a.head_off : 4 * NSET;
   // Heads narrower than 128: a.n_kv_heads counts 128-dimension slabs of the cached row, each the
   // stored bytes of hps = 128 / head_dim neighbouring kv heads, and the rep query heads of a slab
   // are the heads of those kv heads, rep1 each, in order.  Query head r of a slab belongs to kv
@@ -603,8 +608,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   const int nl = lane & 15;
   const int rg = lane >> 4;
   // (the queries of this block's slabs: heads kv_off * rep ...)
-  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)c * a.n_q_heads + kv_off * rep) * head_dim;
-  const float* qfbase = reinterpret_cast<const float*>(a.q) + ((int64_t)c * a.n_q_heads + kv_off * rep) * head_dim;
+  const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)c * a.n_q_heads + kv_off * rep_all + a.head_off) * head_dim;
+  const float* qfbase = reinterpret_cast<const float*>(a.q) + ((int64_t)c * a.n_q_heads + kv_off * rep_all + a.head_off) * head_dim;
   // bf16 bits of limb `set` of a float32 query element
   auto limb_bits = [](float v, int set) -> uint32_t {
     const uint32_t hb = __float_as_uint(v) & 0xffff0000u;
@@ -668,11 +673,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     if (r < rep && owns(r, gq)) {
       float h32[32];
       if constexpr (QF32) {
-        load_as_float<PIKV_F32, 32>(qfbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32, h32);
+        load_as_float<PIKV_F32, 32>(qfbase, (int64_t)(g * rep_all + r) * head_dim + group_in_head(gq) * 32, h32);
 #pragma unroll
         for (int k = 0; k < 32; ++k) h32[k] = bf16_bits_to_float(limb_bits(h32[k], 0)) + bf16_bits_to_float(limb_bits(h32[k], 1));
       } else {
-        load_as_float<PIKV_BF16, 32>(qbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32, h32);
+        load_as_float<PIKV_BF16, 32>(qbase, (int64_t)(g * rep_all + r) * head_dim + group_in_head(gq) * 32, h32);
       }
 #pragma unroll
       for (int k = 0; k < 32; ++k) sacc += h32[k];
@@ -687,11 +692,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     if (r < rep && owns(r, gq)) {
       if constexpr (QF32) {
         float f8[8];
-        load_as_float<PIKV_F32, 8>(qfbase, (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32 + b2 * 8, f8);
+        load_as_float<PIKV_F32, 8>(qfbase, (int64_t)(g * rep_all + r) * head_dim + group_in_head(gq) * 32 + b2 * 8, f8);
         d = make_uint4(limb_bits(f8[0], limb) | (limb_bits(f8[1], limb) << 16), limb_bits(f8[2], limb) | (limb_bits(f8[3], limb) << 16),
                        limb_bits(f8[4], limb) | (limb_bits(f8[5], limb) << 16), limb_bits(f8[6], limb) | (limb_bits(f8[7], limb) << 16));
       } else {
-        d = ld16(qbase + (int64_t)(g * rep + r) * head_dim + group_in_head(gq) * 32 + b2 * 8);
+        d = ld16(qbase + (int64_t)(g * rep_all + r) * head_dim + group_in_head(gq) * 32 + b2 * 8);
       }
     }
     alds[i] = make_uint4((d.x & 0xffffu) | (d.z << 16), (d.x >> 16) | (d.z & 0xffff0000u),
@@ -776,8 +781,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
     }
     __syncthreads();
 
-    if constexpr (EXCH) tile_stats_exchange<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep, kv_off * rep);
-    else tile_stats_store<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep, kv_off * rep);
+    if constexpr (EXCH) tile_stats_exchange<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep, kv_off * rep_all + a.head_off, rep_all);
+    else tile_stats_store<true, SL>(a, stage, c, tile, n0, len, wave, rg, nl, rep, kv_off * rep_all + a.head_off, rep_all);
     __syncthreads();  // stage and the metadata rows are reused by the next tile
     return true;
   };
@@ -1022,11 +1027,15 @@ static int launch_i8_mfma(const ScoreArgs& a, int n_caches, int64_t n_tiles, hip
 }
 
 template <int SCHEME, bool EXCH, bool NARROW>
-static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st, bool qf32) {
+static int launch_gqa_slabs(const ScoreArgs& a0, int n_caches, int64_t n_tiles, hipStream_t st, bool qf32) {
+  ScoreArgs a = a0;
   const int rep = a.n_q_heads / a.n_kv_heads;
   const int nset = rep <= 4 ? 1 : 2;
   const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset, qf32 ? 2 * nset : nset);   // float32 queries: a copy of the A operands per limb
-  if (rep > 8 || lds > 64 * 1024 || a.n_kv_heads > (qf32 ? 8 : kGqaMaxKvHeads)) return PIKV_ERR_UNSUPPORTED;
+  // 9 to 16 query heads per kv head (heads of 128, up to 4 kv heads): two launches of eight heads over the same codes
+  if (rep > 8 && (NARROW || rep > 16 || a.n_kv_heads > 4)) return PIKV_ERR_UNSUPPORTED;
+  if (lds > 64 * 1024 || a.n_kv_heads > (qf32 ? 8 : kGqaMaxKvHeads)) return PIKV_ERR_UNSUPPORTED;
+  for (a.head_off = 0; a.head_off < rep; a.head_off += 4 * nset) {
   const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
   // (rows of 1 or 2 slabs have a kernel of their own: fewer registers, 8 instead of 6 blocks per compute unit,
   // and with 5 KB tiles the bytes in flight are what bounds them - 1 kv head x 4 q heads 61.3 -> 52.1 us,
@@ -1062,6 +1071,7 @@ static int launch_gqa_slabs(const ScoreArgs& a, int n_caches, int64_t n_tiles, h
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 4, 2, EXCH, NARROW>), grid, dim3(256), lds, st, a);
     else
       hipLaunchKernelGGL((scores_mfma_i4_gqa_kernel<SCHEME, 8, 2, EXCH, NARROW>), grid, dim3(256), lds, st, a);
+  }
   }
   return PIKV_OK;
 }
@@ -1298,7 +1308,9 @@ int scores_exchange_launch(const void* k_codes, const void* k_scale, const void*
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
   if (hps == 0) return PIKV_ERR_UNSUPPORTED;
   const int slabs = n_kv_heads / hps;   // the kernel's kv heads are 128-dimension slabs of the row
-  if (n_q_heads / slabs > 8 || n_q_heads > kMaxQHeads || max_len < 1) return PIKV_ERR_UNSUPPORTED;
+  if ((n_q_heads / slabs > 8 && !(hps == 1 && slabs <= 4 && n_q_heads / slabs <= 16 && q_dtype == PIKV_BF16)) ||
+      n_q_heads > kMaxQHeads || max_len < 1)
+    return PIKV_ERR_UNSUPPORTED;
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
   ScoreArgs a{k_codes, k_scale, k_zero, q, cache_row_base, cache_fill, nullptr, tile_max, tile_sum,
               0, n_tiles, scale_qk, group, slabs, n_q_heads, head_dim, escores,
@@ -1388,6 +1400,9 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   // dimensions are served as 128-dimension slabs of two or four neighbouring kv heads
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
   // (float32 queries: as two bf16 limbs on the same kernel, where its operands fit)
+  // (9 to 16 bf16 query heads per kv head over up to 4 kv heads of 128: two launches of eight heads; float32
+  // queries of such ratios stay on the vector form, which multiplies them exactly)
+  const bool two_launches = hps == 1 && n_kv_heads <= 4 && rep > 8 && rep <= 16;
   if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_F32 && rep * hps <= 8) {
     ScoreArgs as = a;
     as.n_kv_heads = n_kv_heads / hps;
@@ -1401,7 +1416,7 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_BF16 && rep * hps <= (hps == 1 ? 16 : 8)) {
     int grc = PIKV_ERR_UNSUPPORTED;
     const size_t mlds = (size_t)n_q_heads * (kTile + 4) * sizeof(float);
-    if (rep * hps <= 8) {
+    if (rep * hps <= 8 || two_launches) {
       ScoreArgs as = a;
       as.n_kv_heads = n_kv_heads / hps;
       grc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(as, n_caches, n_tiles, st)

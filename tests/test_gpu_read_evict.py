@@ -77,6 +77,9 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I8_SYM, 64, 12, 12, 64),      # 12 kv heads: three blocks of four heads per tile
     (O.Q_I4_ASYM, 32, 3, 6, 128),      # 3 kv heads
     (O.Q_I8_ASYM, 128, 5, 10, 128),    # 5 kv heads: one block per head
+    (O.Q_I4_ASYM, 32, 2, 32, 128),     # 16 q heads per kv head: two launches of eight heads over the same codes
+    (O.Q_I4_SYM, 32, 1, 12, 128),      # ... 12: the second launch with four heads
+    (O.Q_I4_ASYM, 32, 4, 36, 128),     # ... 9: the second launch with one head
 ])
 @pytest.mark.parametrize("qdtype", ["f32", "bf16"])
 def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
