@@ -835,7 +835,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       a.partial[((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads * a.head_dim + idx] = 0.f;
     return;
   }
-  const int rep = a.n_q_heads / HKR;  // 2..8
+  // a launch serves heads a.head_off .. a.head_off + rep - 1 of every kv head (more than 8 per kv head: two
+  // launches; narrow heads are launched with head_off = 0 only); the staged rows count these heads alone
+  const int rep_all = a.n_q_heads / HKR;
+  const int rep = rep_all - a.head_off < 8 ? rep_all - a.head_off : 8;  // 1..8
+  const int nql = HKR * rep;         // staged heads: row (kv head) * rep + head of the launch
   const int rep1 = rep / HPS;        // query heads per stored kv head
   const int groups_per_row = (HKR * 128) / a.group;
   // matrix-core roles: A row / B,C column i, token group kg (tokens 8*kg .. 8*kg+7 of the tile)
@@ -858,12 +862,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   // 64 / TI heads x 4 TI runs)
   const int sh = threadIdx.x / (4 * TI);
   const int st8 = (threadIdx.x % (4 * TI)) * 8;
-  const bool s_on = sh < a.n_q_heads;
-  const float* srow = a.scores + ((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * a.score_stride;
+  const bool s_on = sh < nql;
+  const int s_hq = s_on ? (sh / rep) * rep_all + a.head_off + sh % rep : 0;   // the query head itself
+  const float* srow = a.scores + ((int64_t)c * a.n_q_heads + s_hq) * a.score_stride;
   float smx = 0.f, srz = 1.f;
   if (normalise) {
-    smx = a.head_stats[((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * 2];
-    srz = 1.0f / a.head_stats[((int64_t)c * a.n_q_heads + (s_on ? sh : 0)) * 2 + 1];
+    smx = a.head_stats[((int64_t)c * a.n_q_heads + s_hq) * 2];
+    srz = 1.0f / a.head_stats[((int64_t)c * a.n_q_heads + s_hq) * 2 + 1];
   }
   const bool s_vec = (a.score_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(a.scores) & 15) == 0;
   const float s_off = normalise ? -INFINITY : 0.f;  // what a token past the end contributes: p = 0
@@ -931,7 +936,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
         const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
         for (int k = 0; k < 8; ++k)
-          lprob[(((st8 + k) % TI) * a.n_q_heads + sh) * kAtt8PRow + (st8 + k) / TI] = v[k];
+          lprob[(((st8 + k) % TI) * nql + sh) * kAtt8PRow + (st8 + k) / TI] = v[k];
       }
     }
 #pragma unroll
@@ -970,9 +975,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 #pragma unroll
         for (int k = 0; k < TI; ++k) {
           const int j = k * kAtt8Tile + it;   // token of the tile: row j % TI of tile row j / TI
-          const float* lp = lprob + (j % TI) * a.n_q_heads * kAtt8PRow + j / TI;
+          const float* lp = lprob + (j % TI) * nql * kAtt8PRow + j / TI;
           float imp = 0.f;
-          for (int hq = igrp; hq < a.n_q_heads; hq += 8) imp = imp + lp[hq * kAtt8PRow];
+          for (int hq = igrp; hq < nql; hq += 8) imp = imp + lp[hq * kAtt8PRow];
           imp = imp + __shfl_xor(imp, 8, 64);
           imp = imp + __shfl_xor(imp, 16, 64);
           imp = imp + __shfl_xor(imp, 32, 64);
@@ -999,7 +1004,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       float* const acc_rows = a.row_acc ? a.row_acc + (base_row + n0) : nullptr;
       float* const ts_rows = a.row_ts ? a.row_ts + (base_row + n0) : nullptr;
       float imp = 0.f;
-      for (int hq = igrp; hq < a.n_q_heads; hq += 8) imp = imp + lprob[hq * kAtt8PRow + it];
+      for (int hq = igrp; hq < nql; hq += 8) imp = imp + lprob[hq * kAtt8PRow + it];
       imp = imp + __shfl_xor(imp, 8, 64);
       imp = imp + __shfl_xor(imp, 16, 64);
       imp = imp + __shfl_xor(imp, 32, 64);
@@ -1131,7 +1136,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     for (int idx = threadIdx.x; idx < HKR * 8 * 128; idx += 256) {
       const int row = idx >> 7, g = row >> 3, ro = row & 7;
       if (ro < rep)
-        a.partial[(((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep + ro) * 128 + (idx & 127)] = ol[idx];
+        a.partial[(((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + ro) * 128 + (idx & 127)] = ol[idx];
     }
     return;
   }
@@ -1144,7 +1149,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       const int ro = 2 * kg + rr;  // head (inside the kv group) held by this lane
       if (ro >= rep) continue;
       const int hh = HPS > 1 ? ro / rep1 : 0;   // stored kv head of the slab that owns this head: blocks db with db * HPS / 8 == hh
-      float* o = a.partial + (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep + ro) * (128 / HPS) -
+      float* o = a.partial + (((int64_t)blockIdx.x * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + ro) * (128 / HPS) -
                  hh * (128 / HPS);
 #pragma unroll
       for (int db = 0; db < 8; ++db)
@@ -1168,12 +1173,26 @@ static void launch_attend_mfma8_slabs(int n_slabs, dim3 grid, hipStream_t st, co
   }
 }
 template <int SCHEME>
-static void launch_attend_mfma8(int n_slabs, int hps, dim3 grid, hipStream_t st, const AttendArgs& a) {
+static void launch_attend_mfma8_heads(int n_slabs, int hps, dim3 grid, hipStream_t st, const AttendArgs& a);
+// All query heads of every kv head: up to eight per launch; a later launch (same codes, next heads) adds its
+// share of the importance to the accumulators that the first one has decayed.
+template <int SCHEME>
+static void launch_attend_mfma8(int n_slabs, int hps, dim3 grid, hipStream_t st, AttendArgs a) {
+  const int rep = a.n_q_heads / n_slabs;
+  for (int off = 0; off < rep; off += 8) {
+    a.head_off = off;
+    if (off > 0) a.decay = 1.0f;
+    launch_attend_mfma8_heads<SCHEME>(n_slabs, hps, grid, st, a);
+  }
+}
+template <int SCHEME>
+static void launch_attend_mfma8_heads(int n_slabs, int hps, dim3 grid, hipStream_t st, const AttendArgs& a) {
   if (hps == 1 && n_slabs <= 3 && a.tokens_per_block % (kAtt8Tile * 8) == 0) {
     // rows of few slabs: 8, 4 or 2 neighbouring rows as one row of (up to) 8 slabs (pairs of rows of 4 slabs
     // measured the same as single rows: 322 vs 325 us at 64 caches x 32768 tokens x 16 query heads)
     const int ti = n_slabs == 1 ? 8 : n_slabs == 2 ? 4 : 2;
-    const size_t lds = attend_mfma8_lds_bytes(n_slabs * ti, a.n_q_heads * ti, 1);
+    const int staged = a.n_q_heads < n_slabs * 8 ? a.n_q_heads : n_slabs * 8;   // heads of one launch
+    const size_t lds = attend_mfma8_lds_bytes(n_slabs * ti, staged * ti, 1);
     if (n_slabs == 1) hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 8, 1, 8>), grid, dim3(256), lds, st, a);
     else if (n_slabs == 2) hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 8, 1, 4>), grid, dim3(256), lds, st, a);
     else hipLaunchKernelGGL((attend_mfma_i8_kernel<SCHEME, 6, 1, 2>), grid, dim3(256), lds, st, a);
@@ -1361,7 +1380,8 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(slabs, rep * hps, grid, st, a);
       else launch_attend_mfma<PIKV_Q_I4_SYM>(slabs, rep * hps, grid, st, a);
-    } else if (eight && slabs >= 1 && slabs <= 8 && group % head_dim == 0 && rep * hps >= 2 && rep * hps <= 8) {
+    } else if (eight && slabs >= 1 && slabs <= 8 && group % head_dim == 0 && rep * hps >= 2 &&
+               (rep * hps <= 8 || (hps == 1 && rep <= 16 && n_q_heads <= 64))) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       if (scheme == PIKV_Q_I8_SYM) launch_attend_mfma8<PIKV_Q_I8_SYM>(slabs, hps, grid, st, a);
       else launch_attend_mfma8<PIKV_Q_I8_ASYM>(slabs, hps, grid, st, a);

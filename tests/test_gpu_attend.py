@@ -59,6 +59,9 @@ pytestmark = pytest.mark.gpu
     (O.Q_I4_ASYM, 32, 2, 32, 128),     # 16 q heads per kv head: two launches of two sets each
     (O.Q_I4_SYM, 32, 1, 12, 128),      # ... 12: the second launch with one set
     (O.Q_I4_ASYM, 32, 4, 36, 128),     # ... 9 on 4 kv heads
+    (O.Q_I8_SYM, 128, 2, 32, 128),     # 8-bit, 16 q heads per kv head: two launches of eight heads
+    (O.Q_I8_ASYM, 128, 1, 12, 128),    # ... 12: the second launch with four
+    (O.Q_I8_SYM, 128, 4, 40, 128),     # ... 10 on 4 kv heads (single rows)
 ])
 @pytest.mark.parametrize("form", ["stats", "probs"])
 def test_attend_values(dev, scheme, group, heads, hq, dh, form):
@@ -112,6 +115,7 @@ def test_attend_values(dev, scheme, group, heads, hq, dh, form):
     (O.Q_I4_ASYM, 32, 2, 12, 128),     # two kv heads x 6: pairs of rows, two sets
     (O.Q_I4_ASYM, 32, 3, 9, 128),      # three kv heads: pairs of rows, six slabs
     (O.Q_I4_ASYM, 32, 2, 24, 128),     # 12 q heads per kv head: two launches, the second adds to what the first decayed
+    (O.Q_I8_SYM, 128, 2, 24, 128),     # 8-bit, 12 q heads per kv head: two launches
     (O.Q_I8_ASYM, 128, 1, 8, 128),     # 8-bit, one kv head: eight neighbouring rows as one row
     (O.Q_I8_SYM, 128, 2, 4, 128),      # ... two kv heads: four rows
 ])
@@ -206,6 +210,7 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I4_SYM, 32, 1, 12, 128, "f32"),     # ... 12, float32 queries
     (O.Q_I4_ASYM, 32, 4, 40, 128, "bf16"),   # ... 10 on 4 kv heads
     (O.Q_I8_ASYM, 128, 2, 8, 128, "bf16"),   # 8-bit, 2 kv heads: four neighbouring rows as one row of eight slabs
+    (O.Q_I8_ASYM, 128, 2, 20, 128, "bf16"),  # ... 10 q heads per kv head: the attention output in two launches
     (O.Q_I8_SYM, 128, 1, 4, 128, "f32"),     # ... 1 kv head: eight rows as one
     (O.Q_I8_SYM, 128, 3, 12, 128, "bf16"),   # ... 3 kv heads x 4: pairs of rows, 24 staged probability rows
     # 3 kv heads x 8: this draw has scores up to 36, and the 8-bit matrix-core scores carry an absolute error
