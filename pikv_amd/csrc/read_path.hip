@@ -812,6 +812,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
 // k-steps of 16 dimensions per head); per 16-token slice a lane loads the two 16-byte
 // halves of its token's head row, so one load instruction fetches whole 128-byte lines.
 constexpr int kI8TilesPerBlock = 4;
+constexpr int kI8QsFloats = 4 * 4 * 4 * 16;   // query sums in LDS: 4 wavefronts x up to 4 kv head slots x up to 4 parts x 16
 
 // Heads narrower than 128 (HPS = 128 / head_dim = 2 or 4): a.n_kv_heads counts 128-dimension slabs of
 // the cached row, each the stored bytes of HPS neighbouring kv heads; the rep query heads of a slab
@@ -825,7 +826,8 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 8, "8-bit schemes only");
   extern __shared__ float i8_lds[];
-  float* stage = i8_lds;  // [q head][token in tile]
+  float* qs_lds = i8_lds;           // [wavefront][kv head slot][part][row group][4]: query sums (see NQ below)
+  float* stage = i8_lds + kI8QsFloats;  // [q head][token in tile]
 
   const int c = blockIdx.y;
   const int len = a.fill[c] < a.max_len ? a.fill[c] : a.max_len;
@@ -862,11 +864,17 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   // head item % n_kv_heads of tile item / n_kv_heads - so that all four load and multiply and 4 / n_kv_heads
   // tiles of the block are in flight at a time; a wavefront's kv head is the same in every round.
   const int spread = (NHW == 1 && a.n_kv_heads <= 2) ? a.n_kv_heads : 0;
+  // The accumulators carry the nibble offsets, 272 * (sum of q) - some 10^4 against scores of some 10 - and every
+  // k-step rounds at that magnitude.  The 128 dimensions are therefore accumulated in NQ parts, each with the
+  // offset of its own dimensions taken off before the parts are added (four parts: 1e-4 -> 1e-5 absolute at
+  // |score| 36); fewer parts where the registers of more kv heads per wavefront leave no room.
+  // The query sums of the parts live in LDS and are read where they are used: as registers they cost a resident
+  // wavefront per SIMD (8-bit scores at 8 kv heads x 32 q heads: 699 vs 588 us).
+  constexpr int NQ = NHW == 1 ? 4 : NHW == 2 ? 2 : 1;
   uint4 areg[NHW][8];
-  float qs[NHW][4];
 #pragma unroll
   for (int hs = 0; hs < NHW; ++hs) {
-    const int g = spread ? wave % spread : wave + 4 * hs;
+    const int g = spread ? wave % (spread ? spread : 1) : wave + 4 * hs;
     const bool on = g < a.n_kv_heads && (nl >> RSH) < rep;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
@@ -895,13 +903,17 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
     }
     // Qs of heads 4*rg .. 4*rg+3 (C rows) from a B operand that is 1 at the low-nibble slots
     const uint4 ones = make_uint4(0x3f803f80u, 0u, 0x3f803f80u, 0u);
-    pikv_f32x4 sumq = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks)
-      sumq = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, areg[hs][ks]),
-                                                     __builtin_bit_cast(pikv_bf16x8, ones), sumq, 0, 0, 0);
+    for (int part = 0; part < NQ; ++part) {
+      pikv_f32x4 sumq = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int qq = 0; qq < 4; ++qq) qs[hs][qq] = sumq[qq];
+      for (int ks = part * (8 / NQ); ks < (part + 1) * (8 / NQ); ++ks)
+        sumq = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, areg[hs][ks]),
+                                                       __builtin_bit_cast(pikv_bf16x8, ones), sumq, 0, 0, 0);
+      // lanes with the same row group hold the same four sums
+      if (nl == 0) *reinterpret_cast<float4*>(qs_lds + (((wave * NHW + hs) * NQ + part) * 4 + rg) * 4) =
+          make_float4(sumq[0], sumq[1], sumq[2], sumq[3]);
+    }
   }
 
   // kv head g (A operands of slot hs) against the tile that starts at token n0, scores into st
@@ -932,7 +944,9 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
       }
 #pragma unroll
       for (int sl = 0; sl < 4; ++sl) {
-        pikv_f32x4 pc = {0.f, 0.f, 0.f, 0.f};
+        pikv_f32x4 pc[NQ];
+#pragma unroll
+        for (int part = 0; part < NQ; ++part) pc[part] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
           const uint32_t wv[4] = {cv[sl][half].x, cv[sl][half].y, cv[sl][half].z, cv[sl][half].w};
@@ -941,9 +955,20 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
             const uint32_t w = Q::sym ? (wv[b2] ^ 0x80808080u) : wv[b2];
             const uint4 bb = make_uint4(and_or(w << 3, kNib, kExp), and_or(w >> 1, kNib, kExp),
                                         and_or(w >> 5, kNib, kExp), and_or(w >> 9, kNib, kExp));
-            pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, areg[hs][half * 4 + b2]),
-                                                         __builtin_bit_cast(pikv_bf16x8, bb), pc, 0, 0, 0);
+            constexpr int kPerPart = 8 / NQ;
+            pikv_f32x4& pp = pc[(half * 4 + b2) / kPerPart];
+            pp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, areg[hs][half * 4 + b2]),
+                                                         __builtin_bit_cast(pikv_bf16x8, bb), pp, 0, 0, 0);
           }
+        }
+        // (the offset is hidden from the compiler, which would otherwise keep the sums in registers across the slices)
+        int qoff = ((wave * NHW + hs) * NQ * 4 + rg) * 4;
+        asm volatile("" : "+v"(qoff));
+        float qsum[NQ][4];
+#pragma unroll
+        for (int part = 0; part < NQ; ++part) {
+          const float4 v = *reinterpret_cast<const float4*>(qs_lds + qoff + part * 16);
+          qsum[part][0] = v.x, qsum[part][1] = v.y, qsum[part][2] = v.z, qsum[part][3] = v.w;
         }
         float row_score[4];
 #pragma unroll
@@ -955,7 +980,10 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
             zrl = hh_c[qq] == k ? zr[sl][k] : zrl;
           }
           const float zz = 272.0f + (Q::sym ? 128.0f : zrl);
-          row_score[qq] = scl * fmaf(-zz, qs[hs][qq], pc[qq]) * a.scale_qk;
+          float dot = fmaf(-zz, qsum[0][qq], pc[0][qq]);
+#pragma unroll
+          for (int part = 1; part < NQ; ++part) dot = dot + fmaf(-zz, qsum[part][qq], pc[part][qq]);
+          row_score[qq] = scl * dot * a.scale_qk;
         }
         if constexpr (QF32) {
 #pragma unroll
@@ -975,6 +1003,10 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
       }
     }
   };
+  // the query sums were written by other lanes of this wavefront
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   if (spread) {
     const int tpr = kI8TilesPerBlock / spread;   // tiles per round, each with a staging area of its own
     for (int round = 0; round < spread; ++round) {
@@ -1010,7 +1042,8 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
 template <int SCHEME, int HPS, bool QF32>
 static void launch_i8_mfma_q(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
   // rows of 1 or 2 slabs stage 4 or 2 tiles at a time
-  const size_t lds = (size_t)a.n_q_heads * kTile * sizeof(float) * (a.n_kv_heads <= 2 ? kI8TilesPerBlock / a.n_kv_heads : 1);
+  const size_t lds = (size_t)a.n_q_heads * kTile * sizeof(float) * (a.n_kv_heads <= 2 ? kI8TilesPerBlock / a.n_kv_heads : 1) +
+                     kI8QsFloats * sizeof(float);
   const dim3 grid((unsigned)((n_tiles + kI8TilesPerBlock - 1) / kI8TilesPerBlock), (unsigned)n_caches);
   if (a.n_kv_heads <= 4)
     hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 1, HPS, QF32>), grid, dim3(256), lds, st, a);

@@ -213,11 +213,7 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I8_ASYM, 128, 2, 20, 128, "bf16"),  # ... 10 q heads per kv head: the attention output in two launches
     (O.Q_I8_SYM, 128, 1, 4, 128, "f32"),     # ... 1 kv head: eight rows as one
     (O.Q_I8_SYM, 128, 3, 12, 128, "bf16"),   # ... 3 kv heads x 4: pairs of rows, 24 staged probability rows
-    # 3 kv heads x 8: this draw has scores up to 36, and the 8-bit matrix-core scores carry an absolute error
-    # of about 1e-4 there (their nibble offsets make the accumulators ~250 times the score): the output misses
-    # the 1e-3 bar by the score side alone (1.4e-3 of its root-mean-square; the output side is 2.6e-4)
-    pytest.param(O.Q_I8_SYM, 128, 3, 24, 128, "bf16",
-                 marks=pytest.mark.xfail(reason="8-bit matrix-core scores: 1e-4 absolute at |score| 36", strict=False)),
+    (O.Q_I8_SYM, 128, 3, 24, 128, "bf16"),   # ... 3 kv heads x 8; scores up to 36 in this draw: needs the 8-bit scores' part-wise offsets
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.9])
 def test_decode_attend_one_call(dev, scheme, group, heads, hq, dh, qdtype, decay):
