@@ -866,7 +866,7 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   const int spread = (NHW == 1 && a.n_kv_heads <= 2) ? a.n_kv_heads : 0;
   // The accumulators carry the nibble offsets, 272 * (sum of q) - some 10^4 against scores of some 10 - and every
   // k-step rounds at that magnitude.  The 128 dimensions are therefore accumulated in NQ parts, each with the
-  // offset of its own dimensions taken off before the parts are added (four parts: 1e-4 -> 1e-5 absolute at
+  // offset of its own dimensions taken off before the parts are added (four parts: 1.4e-4 -> 4e-5 absolute at
   // |score| 36); fewer parts where the registers of more kv heads per wavefront leave no room.
   // The query sums of the parts live in LDS and are read where they are used: as registers they cost a resident
   // wavefront per SIMD (8-bit scores at 8 kv heads x 32 q heads: 699 vs 588 us).
