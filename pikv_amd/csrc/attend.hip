@@ -290,7 +290,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   constexpr int NH = (HK + 3) / 4;        // kv heads per wavefront
   constexpr int NI = NH * NSETS;          // (kv head, set of four query heads) pairs per wavefront
   static_assert(NSETS == 1 || (NSETS == 2 && HK <= 4), "two sets: the staged rows of 8 x 4 heads, accumulators of one kv head");
-  static_assert(TI == 1 || (!NARROW && !SPLIT && HK % TI == 0), "interleaved rows: whole rows of 128-wide heads");
+  static_assert(TI == 1 || (!SPLIT && HK % TI == 0), "interleaved rows: whole rows");
   constexpr int HR = HK / TI;             // slabs of a cached row
   constexpr int TT = kAttTile * TI;       // cached tokens per tile
   constexpr int RS = HK * 64 + 8;         // bytes per token row of staged codes
@@ -728,11 +728,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       }
       __syncthreads();
     }
-    const int heads = rep + rep_b;   // heads of a kv head in this launch
+    const int heads = rep + rep_b;   // heads of a slab in this launch
     for (int idx = threadIdx.x; idx < HR * 4 * NSETS * 128; idx += 256) {
-      const int row = idx >> 7, g = row / (4 * NSETS), hl = row % (4 * NSETS);
-      if (hl < heads)
-        a.partial[(((int64_t)xb * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + hl) * 128 + (idx & 127)] = ol[idx];
+      const int row = idx >> 7, g = row / (4 * NSETS), hl = row % (4 * NSETS), d = idx & 127;
+      if (hl >= heads) continue;
+      const int64_t ohead = ((int64_t)xb * a.n_caches + c) * a.n_q_heads + g * rep_all + a.head_off + hl;
+      if constexpr (!NARROW) {
+        a.partial[ohead * 128 + d] = ol[idx];
+      } else {
+        // a narrow head keeps the dimensions of its own kv head of the slab
+        const int hh = (a.head_off + hl) / rep1;
+        if (d / a.head_dim == hh) a.partial[ohead * a.head_dim + d - hh * a.head_dim] = ol[idx];
+      }
     }
     return;
   }
@@ -1257,7 +1264,7 @@ static void launch_attend_mfma(int n_slabs, int heads_per_slab, dim3 grid, hipSt
   const int nsets = (n_slabs <= 4 && heads_per_slab > 4) ? 2 : 1;
   // rows of few slabs: 8, 4 or 2 neighbouring rows as one (a block's token range must hold whole tiles of them)
   int ti = 1;
-  if (a.head_dim == 128 && n_slabs <= 4) {
+  if (n_slabs <= 4) {
     const int room = (nsets == 2 ? 4 : 8) / n_slabs;
     ti = room >= 8 ? 8 : room >= 4 ? 4 : room >= 2 ? 2 : 1;
     while (ti > 1 && a.tokens_per_block % (kAttTile * ti) != 0) ti >>= 1;
@@ -1271,8 +1278,12 @@ static void launch_attend_mfma(int n_slabs, int heads_per_slab, dim3 grid, hipSt
       const int hk = n_slabs * ti;
       const size_t lds = attend_mfma_lds_bytes(hk, a.n_q_heads, nsets);
 #define PIKV_ATT_ROWS(HKV, TIV, NS)                                                                              \
-  if (hk == HKV && ti == TIV && nsets == NS)                                                                     \
-    hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, HKV, EXCH, false, NS, false, TIV>), grid, dim3(256), lds, st, a);
+  if (hk == HKV && ti == TIV && nsets == NS) {                                                                   \
+    if (a.head_dim == 128)                                                                                       \
+      hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, HKV, EXCH, false, NS, false, TIV>), grid, dim3(256), lds, st, a); \
+    else                                                                                                         \
+      hipLaunchKernelGGL((attend_mfma_i4_kernel<SCHEME, HKV, EXCH, true, NS, false, TIV>), grid, dim3(256), lds, st, a);  \
+  }
       PIKV_ATT_ROWS(8, 8, 1)   // 1 kv head
       PIKV_ATT_ROWS(4, 4, 1)   // ... token ranges of 256
       PIKV_ATT_ROWS(8, 4, 1)   // 2
@@ -1481,7 +1492,7 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
   const bool hk_ok = (slabs >= 1 && slabs <= 8) || (hps == 1 && slabs > 8 && slabs % 8 == 0);
   const int64_t splits = attend_splits(n_caches, max_len);
   if ((scheme == PIKV_Q_I4_ASYM || scheme == PIKV_Q_I4_SYM) && group == 32 && rep >= 1 &&
-      (rep * hps <= 8 || (hps == 1 && slabs <= 4 && rep <= 16)) && hk_ok && (q_dtype == PIKV_BF16 || q_dtype == PIKV_F32) && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {
+      (rep * hps <= 8 || (slabs <= 4 && rep * hps <= 16)) && hk_ok && (q_dtype == PIKV_BF16 || q_dtype == PIKV_F32) && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {
     float* esc = reinterpret_cast<float*>(ws + w.scores);
     const int rc = scores_exchange_launch(k_codes, k_scale, k_zero, scheme, group, n_kv_heads, n_q_heads, head_dim, q,
                                           q_dtype, scale_qk, cache_row_base, cache_fill, n_caches, max_len, esc, tmax,

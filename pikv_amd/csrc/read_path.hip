@@ -584,7 +584,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   const int64_t tok0 = tile0 * kTile;
   if (tok0 >= len) return;  // uniform for the block
   // query heads per slab; a launch serves heads a.head_off .. a.head_off + rep - 1 of every slab, rep <= 4 NSET
-  // (more than 8 heads per slab: two launches; narrow heads and split rows are launched with head_off = 0 only)
+  // (more than 8 heads per slab: two launches; split rows are launched with head_off = 0 only)
   const int rep_all = a.n_q_heads / (SPLIT ? a.row_slabs : a.n_kv_heads);
   const int rep = rep_all - a.head_off < 4 * NSET ? rep_all - a.head_off : 4 * NSET;
   // Heads narrower than 128: a.n_kv_heads counts 128-dimension slabs of the cached row, each the
@@ -596,9 +596,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   // two tiles runs)
   const int head_dim = NARROW ? a.head_dim : 128;
   const int gshift = head_dim == 64 ? 1 : 0;          // log2 of a narrow head's groups of 32
-  const int rep1 = head_dim == 64 ? rep >> 1 : rep >> 2;
-  auto owns = [&](int r, int gq) {                    // group gq of the slab belongs to query head r's kv head
-    return !NARROW || (gq >> gshift) == (r >= rep1) + (r >= 2 * rep1) + (r >= 3 * rep1);
+  const int rep1 = head_dim == 64 ? rep_all >> 1 : rep_all >> 2;
+  auto owns = [&](int r, int gq) {                    // group gq of the slab belongs to the kv head of the launch's query head r
+    const int ra = r + a.head_off;                    // ... which is head ra of the slab
+    return !NARROW || (gq >> gshift) == (ra >= rep1) + (ra >= 2 * rep1) + (ra >= 3 * rep1);
   };
   auto group_in_head = [&](int gq) { return NARROW ? gq & ((1 << gshift) - 1) : gq; };
   const int lanes_per_row = SPLIT ? a.row_slabs * 4 : a.n_kv_heads * 4;   // 16-byte pieces of a whole cached row
@@ -1066,7 +1067,7 @@ static int launch_gqa_slabs(const ScoreArgs& a0, int n_caches, int64_t n_tiles, 
   const int nset = rep <= 4 ? 1 : 2;
   const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset, qf32 ? 2 * nset : nset);   // float32 queries: a copy of the A operands per limb
   // 9 to 16 query heads per kv head (heads of 128, up to 4 kv heads): two launches of eight heads over the same codes
-  if (rep > 8 && (NARROW || rep > 16 || a.n_kv_heads > 4)) return PIKV_ERR_UNSUPPORTED;
+  if (rep > 8 && (rep > 16 || a.n_kv_heads > 4)) return PIKV_ERR_UNSUPPORTED;
   if (lds > 64 * 1024 || a.n_kv_heads > (qf32 ? 8 : kGqaMaxKvHeads)) return PIKV_ERR_UNSUPPORTED;
   for (a.head_off = 0; a.head_off < rep; a.head_off += 4 * nset) {
   const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
@@ -1341,7 +1342,7 @@ int scores_exchange_launch(const void* k_codes, const void* k_scale, const void*
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
   if (hps == 0) return PIKV_ERR_UNSUPPORTED;
   const int slabs = n_kv_heads / hps;   // the kernel's kv heads are 128-dimension slabs of the row
-  if ((n_q_heads / slabs > 8 && !(hps == 1 && slabs <= 4 && n_q_heads / slabs <= 16 && q_dtype == PIKV_BF16)) ||
+  if ((n_q_heads / slabs > 8 && !(slabs <= 4 && n_q_heads / slabs <= 16 && q_dtype == PIKV_BF16)) ||
       n_q_heads > kMaxQHeads || max_len < 1)
     return PIKV_ERR_UNSUPPORTED;
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
@@ -1435,7 +1436,7 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   // (float32 queries: as two bf16 limbs on the same kernel, where its operands fit)
   // (9 to 16 bf16 query heads per kv head over up to 4 kv heads of 128: two launches of eight heads; float32
   // queries of such ratios stay on the vector form, which multiplies them exactly)
-  const bool two_launches = hps == 1 && n_kv_heads <= 4 && rep > 8 && rep <= 16;
+  const bool two_launches = hps > 0 && n_kv_heads / hps <= 4 && rep * hps > 8 && rep * hps <= 16;
   if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_F32 && rep * hps <= 8) {
     ScoreArgs as = a;
     as.n_kv_heads = n_kv_heads / hps;
@@ -1446,7 +1447,7 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
       return PIKV_OK;
     }
   }
-  if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_BF16 && rep * hps <= (hps == 1 ? 16 : 8)) {
+  if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_BF16 && (rep * hps <= (hps == 1 ? 16 : 8) || two_launches)) {
     int grc = PIKV_ERR_UNSUPPORTED;
     const size_t mlds = (size_t)n_q_heads * (kTile + 4) * sizeof(float);
     if (rep * hps <= 8 || two_launches) {

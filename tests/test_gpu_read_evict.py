@@ -80,6 +80,9 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I4_ASYM, 32, 2, 32, 128),     # 16 q heads per kv head: two launches of eight heads over the same codes
     (O.Q_I4_SYM, 32, 1, 12, 128),      # ... 12: the second launch with four heads
     (O.Q_I4_ASYM, 32, 4, 36, 128),     # ... 9: the second launch with one head
+    (O.Q_I4_ASYM, 32, 2, 14, 64),      # heads of 64, 14 q heads on the one slab (Qwen2.5-0.5B): two launches
+    (O.Q_I4_SYM, 32, 4, 20, 64),       # ... two slabs x 10
+    (O.Q_I4_ASYM, 32, 4, 12, 32),      # heads of 32: 12 q heads on the one slab
 ])
 @pytest.mark.parametrize("qdtype", ["f32", "bf16"])
 def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
