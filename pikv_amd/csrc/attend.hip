@@ -58,6 +58,7 @@ struct AttendArgs {
   int64_t n_tiles;
   int head_off;  // attend_mfma_i4_kernel: first query head of every kv group handled by this launch
   int tokens_per_block;  // cached tokens per block (a multiple of 64): block x covers tokens [x * tokens_per_block, ...)
+  int kv_window;         // attend_valu_kernel: kv heads per block when a whole row has more than 256 lanes (0: all)
   int row_slabs;         // attend_mfma_i4_kernel<SPLIT>: 128-dimension slabs of a whole cached row (the block takes 8 of them)
 };
 
@@ -67,6 +68,8 @@ __device__ __forceinline__ float prob_of(float s, float mx, float rz, bool norma
 
 // ---- vector-unit form --------------------------------------------------------------
 // RP query heads of every kv head per pass (blockIdx.z selects the pass).
+// Rows of more than 256 lanes (e.g. 40 kv heads of 128, 8-bit): a block takes a window of a.kv_window kv heads -
+// kv heads are independent here - and blockIdx.z = pass * windows + window.
 template <int SCHEME, int RP>
 __global__ __launch_bounds__(256) void attend_valu_kernel(AttendArgs a) {
   using Q = QScheme<SCHEME>;
@@ -77,15 +80,19 @@ __global__ __launch_bounds__(256) void attend_valu_kernel(AttendArgs a) {
   const int64_t t0 = (int64_t)blockIdx.x * a.tokens_per_block;
   const int64_t t1 = (t0 + a.tokens_per_block < len) ? t0 + a.tokens_per_block : len;
   const int rep = a.n_q_heads / a.n_kv_heads;
-  const int r0 = blockIdx.z * RP;
+  const int wk = a.kv_window ? a.kv_window : a.n_kv_heads;   // kv heads of this block
+  const int n_win = a.n_kv_heads / wk;
+  const int r0 = (blockIdx.z / n_win) * RP;
   const int D = a.n_kv_heads * a.head_dim;
-  const int lanes_per_row = D / EPL;
+  const int lanes_full = D / EPL;                 // 16-byte pieces of a whole cached row
   const int lanes_per_head = a.head_dim / EPL;
+  const int lanes_per_row = wk * lanes_per_head;  // ... of the block's window
   const int groups_per_row = D / a.group;
   const int tok_per_step = 256 / lanes_per_row;
   const int part = threadIdx.x % lanes_per_row;
+  const int gpart = (blockIdx.z % n_win) * lanes_per_row + part;   // piece of the whole row
   const int tok_in_step = threadIdx.x / lanes_per_row;
-  const int kvh = part / lanes_per_head;
+  const int kvh = gpart / lanes_per_head;
   const int d0 = (part % lanes_per_head) * EPL;
   const bool normalise = a.head_stats != nullptr;
 
@@ -121,8 +128,8 @@ __global__ __launch_bounds__(256) void attend_valu_kernel(AttendArgs a) {
       ok[u] = nn < t1;
       const int64_t nc = ok[u] ? nn : n;
       const int64_t row = base_row + nc;
-      v[u] = ld16(reinterpret_cast<const char*>(a.codes) + (row * lanes_per_row + part) * 16);
-      const int64_t mi = row * groups_per_row + (part * EPL) / a.group;
+      v[u] = ld16(reinterpret_cast<const char*>(a.codes) + (row * lanes_full + gpart) * 16);
+      const int64_t mi = row * groups_per_row + (gpart * EPL) / a.group;
       sc[u] = load_meta<SCHEME>(a.scale, mi);
       zu[u] = (Q::sym ? 0.f : load_meta<SCHEME>(a.zero, mi)) - (float)Q::qmin;
 #pragma unroll
@@ -1368,7 +1375,7 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
   if (D % group != 0) return PIKV_ERR_SHAPE;
   if (!is_pow2(head_dim) || head_dim < epl || group % epl != 0) return PIKV_ERR_UNSUPPORTED;
   const int lanes_per_row = D / epl;
-  if (lanes_per_row > 256) return PIKV_ERR_UNSUPPORTED;
+  if (head_dim / epl > 256) return PIKV_ERR_UNSUPPORTED;   // one kv head must fit a block of the vector form
   hipStream_t st = (hipStream_t)stream;
   const int64_t total = (int64_t)n_caches * n_q_heads * head_dim;
   const int64_t splits = attend_splits(n_caches, max_len);
@@ -1402,7 +1409,18 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
                            dim3(256), 0, st, a);
       // heads of a kv group per pass: the float accumulators of one lane must fit
       const int rp = eight ? (rep >= 8 ? 8 : rep >= 4 ? 4 : rep >= 2 ? 2 : 1) : (rep >= 2 ? 2 : 1);
-      const dim3 grid((unsigned)splits, (unsigned)n_caches, (unsigned)((rep + rp - 1) / rp));
+      // rows of more than 256 lanes: windows of kv heads, preferably of a lane count that divides the block
+      int n_win = 1;
+      if (lanes_per_row > 256) {
+        const int lph = head_dim / epl;
+        int wk = 0;
+        for (int w = n_kv_heads; w >= 1; --w)
+          if (n_kv_heads % w == 0 && w * lph <= 256 && (wk == 0 || (256 % (w * lph) == 0 && 256 % (wk * lph) != 0))) wk = w;
+        a.kv_window = wk;
+        n_win = n_kv_heads / wk;
+      }
+      if ((int64_t)((rep + rp - 1) / rp) * n_win > 65535) return PIKV_ERR_SHAPE;
+      const dim3 grid((unsigned)splits, (unsigned)n_caches, (unsigned)((rep + rp - 1) / rp * n_win));
 #define PIKV_ATTEND_CASE(S)                                                                        \
   case S:                                                                                          \
     if (rp == 8) hipLaunchKernelGGL((attend_valu_kernel<S, 8>), grid, dim3(256), 0, st, a);        \

@@ -59,6 +59,8 @@ pytestmark = pytest.mark.gpu
     (O.Q_I4_ASYM, 32, 2, 32, 128),     # 16 q heads per kv head: two launches of two sets each
     (O.Q_I4_SYM, 32, 1, 12, 128),      # ... 12: the second launch with one set
     (O.Q_I4_ASYM, 32, 4, 36, 128),     # ... 9 on 4 kv heads
+    (O.Q_I8_SYM, 128, 40, 40, 128),    # 40 kv heads of 128, 8-bit: rows of 320 lanes, the vector form in windows of 8 kv heads
+    (O.Q_I4_SYM, 64, 72, 72, 128),     # ... 4-bit, 288 lanes: windows of 8
     (O.Q_I4_ASYM, 32, 2, 14, 64),      # heads of 64, 14 q heads on the one slab: two launches
     (O.Q_I4_SYM, 32, 4, 12, 32),       # heads of 32, 12 q heads on the one slab
     (O.Q_I8_SYM, 128, 2, 32, 128),     # 8-bit, 16 q heads per kv head: two launches of eight heads
@@ -212,6 +214,7 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I4_ASYM, 32, 2, 32, 128, "bf16"),   # 16 q heads per kv head: both kernels in two launches of eight heads
     (O.Q_I4_SYM, 32, 1, 12, 128, "f32"),     # ... 12, float32 queries
     (O.Q_I4_ASYM, 32, 4, 40, 128, "bf16"),   # ... 10 on 4 kv heads
+    (O.Q_I8_ASYM, 128, 40, 40, 128, "bf16"), # 40 kv heads of 128, 8-bit: the vector forms in windows of kv heads
     (O.Q_I4_ASYM, 32, 2, 14, 64, "bf16"),    # ... heads of 64: 14 q heads on the one slab
     (O.Q_I4_SYM, 32, 4, 20, 64, "bf16"),     # ... two slabs x 10
     (O.Q_I8_ASYM, 128, 2, 8, 128, "bf16"),   # 8-bit, 2 kv heads: four neighbouring rows as one row of eight slabs
