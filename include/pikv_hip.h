@@ -392,8 +392,8 @@ int64_t pikv_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim,
  * 4-bit caches with group 32, rows that are 1 to 8 slabs of 128 dimensions, or whole groups
  * of 8 kv heads of 128 dimensions (a slab is one kv
  * head of 128 dimensions, two of 64 or four of 32) and up to 8 query heads per slab (5 to 8
- * heads with float32 queries: up to 7 slabs; 9 to 16 bf16 query heads per slab on rows of up to
- * 4 slabs, in two launches of each kernel) the two matrix-core kernels exchange exp(score - tile max)
+ * heads with float32 queries: up to 7 slabs; more than 8 bf16 query heads per slab on rows of up to
+ * 4 slabs, in launches of eight heads of each kernel) the two matrix-core kernels exchange exp(score - tile max)
  * with a tile's heads side by side, so that both sides stream contiguous 8 KB runs instead
  * of the 256-byte pieces of a [head][token] score matrix; every other format runs the three
  * steps with float scores in the workspace.

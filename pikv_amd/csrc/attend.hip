@@ -1394,7 +1394,7 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
     const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
     const int slabs = hps > 0 ? n_kv_heads / hps : 0;
     const bool slabs_ok = (slabs >= 1 && slabs <= 8) || (hps == 1 && slabs > 8 && slabs % 8 == 0 && splits * (slabs / 8) <= 0x7fffffffLL);
-    if (!eight && group == 32 && slabs_ok && (rep * hps <= 8 || (slabs <= 4 && rep * hps <= 16))) {
+    if (!eight && group == 32 && slabs_ok && (rep * hps <= 8 || slabs <= 4)) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(slabs, rep * hps, grid, st, a);
       else launch_attend_mfma<PIKV_Q_I4_SYM>(slabs, rep * hps, grid, st, a);
@@ -1510,7 +1510,7 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
   const bool hk_ok = (slabs >= 1 && slabs <= 8) || (hps == 1 && slabs > 8 && slabs % 8 == 0);
   const int64_t splits = attend_splits(n_caches, max_len);
   if ((scheme == PIKV_Q_I4_ASYM || scheme == PIKV_Q_I4_SYM) && group == 32 && rep >= 1 &&
-      (rep * hps <= 8 || (slabs <= 4 && rep * hps <= 16)) && hk_ok && (q_dtype == PIKV_BF16 || q_dtype == PIKV_F32) && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {
+      (rep * hps <= 8 || slabs <= 4) && hk_ok && (q_dtype == PIKV_BF16 || q_dtype == PIKV_F32) && n_caches <= 65535 && splits <= 65535 && (!asym || (k_zero && v_zero))) {
     float* esc = reinterpret_cast<float*>(ws + w.scores);
     const int rc = scores_exchange_launch(k_codes, k_scale, k_zero, scheme, group, n_kv_heads, n_q_heads, head_dim, q,
                                           q_dtype, scale_qk, cache_row_base, cache_fill, n_caches, max_len, esc, tmax,

@@ -1066,8 +1066,8 @@ static int launch_gqa_slabs(const ScoreArgs& a0, int n_caches, int64_t n_tiles, 
   const int rep = a.n_q_heads / a.n_kv_heads;
   const int nset = rep <= 4 ? 1 : 2;
   const size_t lds = gqa_lds_bytes(a.n_kv_heads, nset, qf32 ? 2 * nset : nset);   // float32 queries: a copy of the A operands per limb
-  // 9 to 16 query heads per kv head (heads of 128, up to 4 kv heads): two launches of eight heads over the same codes
-  if (rep > 8 && (rep > 16 || a.n_kv_heads > 4)) return PIKV_ERR_UNSUPPORTED;
+  // more than 8 query heads per slab (rows of up to 4 slabs): launches of eight heads each over the same codes
+  if (rep > 8 && a.n_kv_heads > 4) return PIKV_ERR_UNSUPPORTED;
   if (lds > 64 * 1024 || a.n_kv_heads > (qf32 ? 8 : kGqaMaxKvHeads)) return PIKV_ERR_UNSUPPORTED;
   for (a.head_off = 0; a.head_off < rep; a.head_off += 4 * nset) {
   const dim3 grid((unsigned)((n_tiles + kGqaTilesPerBlock - 1) / kGqaTilesPerBlock), (unsigned)n_caches);
@@ -1342,7 +1342,7 @@ int scores_exchange_launch(const void* k_codes, const void* k_scale, const void*
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
   if (hps == 0) return PIKV_ERR_UNSUPPORTED;
   const int slabs = n_kv_heads / hps;   // the kernel's kv heads are 128-dimension slabs of the row
-  if ((n_q_heads / slabs > 8 && !(slabs <= 4 && n_q_heads / slabs <= 16 && q_dtype == PIKV_BF16)) ||
+  if ((n_q_heads / slabs > 8 && !(slabs <= 4 && q_dtype == PIKV_BF16)) ||
       n_q_heads > kMaxQHeads || max_len < 1)
     return PIKV_ERR_UNSUPPORTED;
   const int64_t n_tiles = (max_len + kTile - 1) / kTile;
@@ -1434,9 +1434,9 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   // dimensions are served as 128-dimension slabs of two or four neighbouring kv heads
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);
   // (float32 queries: as two bf16 limbs on the same kernel, where its operands fit)
-  // (9 to 16 bf16 query heads per kv head over up to 4 kv heads of 128: two launches of eight heads; float32
+  // (more than 8 bf16 query heads per slab on rows of up to 4 slabs: launches of eight heads each; float32
   // queries of such ratios stay on the vector form, which multiplies them exactly)
-  const bool two_launches = hps > 0 && n_kv_heads / hps <= 4 && rep * hps > 8 && rep * hps <= 16;
+  const bool more_launches = hps > 0 && n_kv_heads / hps <= 4 && rep * hps > 8;
   if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_F32 && rep * hps <= 8) {
     ScoreArgs as = a;
     as.n_kv_heads = n_kv_heads / hps;
@@ -1447,10 +1447,10 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
       return PIKV_OK;
     }
   }
-  if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_BF16 && (rep * hps <= (hps == 1 ? 16 : 8) || two_launches)) {
+  if (!eight && group == 32 && hps > 0 && q_dtype == PIKV_BF16 && (rep * hps <= (hps == 1 ? 16 : 8) || more_launches)) {
     int grc = PIKV_ERR_UNSUPPORTED;
     const size_t mlds = (size_t)n_q_heads * (kTile + 4) * sizeof(float);
-    if (rep * hps <= 8 || two_launches) {
+    if (rep * hps <= 8 || more_launches) {
       ScoreArgs as = a;
       as.n_kv_heads = n_kv_heads / hps;
       grc = (scheme == PIKV_Q_I4_ASYM) ? launch_gqa<PIKV_Q_I4_ASYM>(as, n_caches, n_tiles, st)

@@ -83,6 +83,8 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I4_ASYM, 32, 2, 14, 64),      # heads of 64, 14 q heads on the one slab (Qwen2.5-0.5B): two launches
     (O.Q_I4_SYM, 32, 4, 20, 64),       # ... two slabs x 10
     (O.Q_I4_ASYM, 32, 4, 12, 32),      # heads of 32: 12 q heads on the one slab
+    (O.Q_I4_ASYM, 32, 1, 48, 128),     # multi-query: 48 q heads on one kv head, six launches
+    (O.Q_I4_SYM, 32, 2, 40, 64),       # ... 40 on one slab of two narrow heads
 ])
 @pytest.mark.parametrize("qdtype", ["f32", "bf16"])
 def test_scores_and_h2o(dev, scheme, group, heads, hq, dh, qdtype):
