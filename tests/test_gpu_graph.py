@@ -126,13 +126,19 @@ def test_decode_read_replays(dev):
         assert bool((pool.ts[~valid] == -1.0).all()), rep
 
 
-def test_decode_attend_replays(dev):
+@pytest.mark.parametrize("hkv,hq,dh", [
+    (8, 32, 128),     # the decode shape
+    (2, 24, 128),     # 12 q heads per kv head: two launches of each kernel, pairs of neighbouring rows as one
+    (1, 4, 128),      # one kv head: four neighbouring rows as one
+    (2, 14, 64),      # heads of 64, 14 q heads on the one slab
+])
+def test_decode_attend_replays(dev, hkv, hq, dh):
     """The one-call decode read under capture: its workspace is allocated before the capture, and every
     replay must rebuild the attention output and the H2O accumulators from scribbled memory."""
     import torch
     from pikv_amd import ops
     g = torch.Generator(device=dev).manual_seed(9)
-    B, N, hkv, hq, dh = 3, 4500, 8, 32, 128
+    B, N = 3, 4500
     D = hkv * dh
     lens = torch.tensor([4500, 2049, 64], dtype=torch.int32, device=dev)
 
