@@ -1399,7 +1399,7 @@ extern "C" int pikv_attend_values(const float* scores, const float* head_stats, 
       if (scheme == PIKV_Q_I4_ASYM) launch_attend_mfma<PIKV_Q_I4_ASYM>(slabs, rep * hps, grid, st, a);
       else launch_attend_mfma<PIKV_Q_I4_SYM>(slabs, rep * hps, grid, st, a);
     } else if (eight && slabs >= 1 && slabs <= 8 && group % head_dim == 0 && rep * hps >= 2 &&
-               (rep * hps <= 8 || (hps == 1 && rep <= 16 && n_q_heads <= 64))) {
+               (rep * hps <= 8 || (hps == 1 && (n_q_heads <= 64 || slabs <= 4)))) {
       const dim3 grid((unsigned)splits, (unsigned)n_caches);
       if (scheme == PIKV_Q_I8_SYM) launch_attend_mfma8<PIKV_Q_I8_SYM>(slabs, hps, grid, st, a);
       else launch_attend_mfma8<PIKV_Q_I8_ASYM>(slabs, hps, grid, st, a);

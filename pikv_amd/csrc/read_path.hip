@@ -444,12 +444,13 @@ __device__ __forceinline__ void tile_stats_store(const ScoreArgs& a, const float
                                                  int64_t n0, int len, int wave, int rg, int nl, int rep = 4,
                                                  int hq0 = 0,    // hq0: first query head of the block's kv heads
                                                  int rep_all = 0) {  // query heads per kv head when the launch serves only rep of them
-  const int n_pass_rows = GROUPED ? a.n_kv_heads * SLOTS : a.n_q_heads;
+  const int slots = SLOTS > 0 ? SLOTS : rep;                   // SLOTS = 0: compact rows, rep per kv head
+  const int n_pass_rows = GROUPED ? a.n_kv_heads * slots : a.n_q_heads;
   for (int h4 = wave * 4; h4 < n_pass_rows; h4 += 16) {
-    const int srow = h4 + rg;                                  // staged row = kv head * SLOTS + slot
-    const int slot = srow % SLOTS;
-    const int hq = hq0 + (GROUPED ? (srow / SLOTS) * (rep_all ? rep_all : rep) + slot : srow);  // query head
-    const bool hok = GROUPED ? slot < rep : hq < a.n_q_heads;
+    const int srow = h4 + rg;                                  // staged row = kv head * slots + slot
+    const int slot = srow % slots;
+    const int hq = hq0 + (GROUPED ? (srow / slots) * (rep_all ? rep_all : rep) + slot : srow);  // query head
+    const bool hok = GROUPED ? (slot < rep && srow < n_pass_rows) : hq < a.n_q_heads;
     float x[4];
     bool okk[4];
     float m = -__builtin_inff();
@@ -834,7 +835,10 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   const int len = a.fill[c] < a.max_len ? a.fill[c] : a.max_len;
   const int64_t tile0 = (int64_t)blockIdx.x * kI8TilesPerBlock;
   if (tile0 * kTile >= len) return;  // uniform for the block
-  const int rep = a.n_q_heads / a.n_kv_heads;  // <= 16
+  // a launch serves heads a.head_off .. a.head_off + rep - 1 of every kv head (more than 16 per kv head: several
+  // launches, heads of 128 only); the staged rows are those heads, rep per kv head
+  const int rep_all = a.n_q_heads / a.n_kv_heads;
+  const int rep = rep_all - a.head_off < 16 ? rep_all - a.head_off : 16;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nl = lane & 15;   // token of a slice (B, C column) / query head (A row)
@@ -882,7 +886,7 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
       uint2 qd = make_uint2(0, 0);
       const int ds = 64 * (ks >> 2) + 16 * rg + 4 * (ks & 3);   // dimension inside the slab
       if (on && (HPS == 1 || ds / (128 / HPS) == hh_a)) {
-        const int64_t qo = (int64_t)(g * rep + (nl >> RSH)) * (128 / HPS) + (ds - hh_a * (128 / HPS));
+        const int64_t qo = (int64_t)(g * rep_all + a.head_off + (nl >> RSH)) * (128 / HPS) + (ds - hh_a * (128 / HPS));
         if constexpr (QF32) {
           float f4[4];
           load_as_float<PIKV_F32, 4>(qfbase, qo, f4);
@@ -1017,8 +1021,10 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
       __syncthreads();
       for (int k = 0; k < tpr; ++k) {
         const int64_t tile = tile0 + round * tpr + k;
-        if (tile * kTile < len)  // uniform
-          tile_stats_store<false>(a, stage + k * a.n_q_heads * kTile, c, tile, tile * kTile, len, wave, rg, nl);
+        if (tile * kTile < len) {  // uniform
+          if (rep == rep_all) tile_stats_store<false>(a, stage + k * a.n_q_heads * kTile, c, tile, tile * kTile, len, wave, rg, nl);
+          else tile_stats_store<true, 0>(a, stage + k * a.n_q_heads * kTile, c, tile, tile * kTile, len, wave, rg, nl, rep, a.head_off, rep_all);
+        }
       }
       __syncthreads();  // the staging areas are reused by the next round
     }
@@ -1035,7 +1041,8 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
       head_tile(hs, g, n0, stage);
     }
     __syncthreads();
-    tile_stats_store<false>(a, stage, c, tile, n0, len, wave, rg, nl);
+    if (rep == rep_all) tile_stats_store<false>(a, stage, c, tile, n0, len, wave, rg, nl);
+    else tile_stats_store<true, 0>(a, stage, c, tile, n0, len, wave, rg, nl, rep, a.head_off, rep_all);
     __syncthreads();  // stage is reused by the next tile
   }
 }
@@ -1474,11 +1481,16 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   // (heads of 64 or 32 dimensions as 128-dimension slabs of two or four neighbouring kv heads)
   // (float32 queries as two bf16 limbs, two operand rows per head: up to 8 heads per slab)
   const bool qf32 = q_dtype == PIKV_F32;
-  if (eight && hps > 0 && group % head_dim == 0 && rep >= 2 && rep * hps <= (qf32 ? 8 : 16) && n_kv_heads / hps <= 16) {
+  // (more than 16 bf16 query heads per kv head of 128 on rows of up to 4 kv heads: launches of 16 heads each)
+  const bool many = hps == 1 && !qf32 && n_kv_heads <= 4 && rep > 16;
+  if (eight && hps > 0 && group % head_dim == 0 && rep >= 2 && (rep * hps <= (qf32 ? 8 : 16) || many) && n_kv_heads / hps <= 16) {
     ScoreArgs as = a;
     as.n_kv_heads = n_kv_heads / hps;
     const bool sym = scheme == PIKV_Q_I8_SYM;
-    if (hps == 1) sym ? launch_i8_mfma<PIKV_Q_I8_SYM>(as, n_caches, n_tiles, st, qf32) : launch_i8_mfma<PIKV_Q_I8_ASYM>(as, n_caches, n_tiles, st, qf32);
+    if (many) {
+      for (as.head_off = 0; as.head_off < rep; as.head_off += 16)
+        sym ? launch_i8_mfma<PIKV_Q_I8_SYM>(as, n_caches, n_tiles, st, false) : launch_i8_mfma<PIKV_Q_I8_ASYM>(as, n_caches, n_tiles, st, false);
+    } else if (hps == 1) sym ? launch_i8_mfma<PIKV_Q_I8_SYM>(as, n_caches, n_tiles, st, qf32) : launch_i8_mfma<PIKV_Q_I8_ASYM>(as, n_caches, n_tiles, st, qf32);
     else if (hps == 2) sym ? launch_i8_mfma<PIKV_Q_I8_SYM, 2>(as, n_caches, n_tiles, st, qf32) : launch_i8_mfma<PIKV_Q_I8_ASYM, 2>(as, n_caches, n_tiles, st, qf32);
     else sym ? launch_i8_mfma<PIKV_Q_I8_SYM, 4>(as, n_caches, n_tiles, st, qf32) : launch_i8_mfma<PIKV_Q_I8_ASYM, 4>(as, n_caches, n_tiles, st, qf32);
     PIKV_CHECK_LAUNCH();

@@ -64,6 +64,8 @@ pytestmark = pytest.mark.gpu
     (O.Q_I4_ASYM, 32, 2, 14, 64),      # heads of 64, 14 q heads on the one slab: two launches
     (O.Q_I4_SYM, 32, 4, 12, 32),       # heads of 32, 12 q heads on the one slab
     (O.Q_I4_ASYM, 32, 1, 48, 128),     # multi-query: 48 q heads on one kv head, six launches
+    (O.Q_I8_SYM, 128, 1, 48, 128),     # ... 8-bit
+    (O.Q_I8_ASYM, 128, 4, 80, 128),    # ... 8-bit, 20 per kv head on 4 kv heads
     (O.Q_I8_SYM, 128, 2, 32, 128),     # 8-bit, 16 q heads per kv head: two launches of eight heads
     (O.Q_I8_ASYM, 128, 1, 12, 128),    # ... 12: the second launch with four
     (O.Q_I8_SYM, 128, 4, 40, 128),     # ... 10 on 4 kv heads (single rows)
@@ -220,6 +222,7 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I4_ASYM, 32, 2, 14, 64, "bf16"),    # ... heads of 64: 14 q heads on the one slab
     (O.Q_I4_SYM, 32, 4, 20, 64, "bf16"),     # ... two slabs x 10
     (O.Q_I4_ASYM, 32, 1, 48, 128, "bf16"),   # multi-query: 48 q heads on one kv head
+    (O.Q_I8_SYM, 128, 1, 48, 128, "bf16"),   # ... 8-bit
     (O.Q_I8_ASYM, 128, 2, 8, 128, "bf16"),   # 8-bit, 2 kv heads: four neighbouring rows as one row of eight slabs
     (O.Q_I8_ASYM, 128, 2, 20, 128, "bf16"),  # ... 10 q heads per kv head: the attention output in two launches
     (O.Q_I8_SYM, 128, 1, 4, 128, "f32"),     # ... 1 kv head: eight rows as one
