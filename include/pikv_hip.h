@@ -310,8 +310,8 @@ int pikv_gather_dequant(const void* codes, const void* scale, const void* zero,
  *   n_tiles = ceil(max_len / PIKV_SCORE_TILE) with max_len <= score_stride
  *   the number of rows per cache the caller wants covered.
  *   D = n_kv_heads*head_dim; head_dim a power of two >= 16 (8-bit) / 32 (4-bit);
- *   any number of kv heads, any n_q_heads that is a multiple of n_kv_heads, for
- *   either q_dtype.  float32 queries against 4-bit group-32 caches, or 8-bit caches
+ *   any number of kv heads, any n_q_heads <= 128 that is a multiple of n_kv_heads, for
+ *   either q_dtype (more query heads: PIKV_ERR_UNSUPPORTED).  float32 queries against 4-bit group-32 caches, or 8-bit caches
  *   with a scale per kv head or coarser, with up to 8 query heads per 128 dimensions
  *   of kv heads are multiplied on the matrix cores as two bf16 limbs (q = hi + lo to
  *   2^-17 |q|; float32 accumulation). */
