@@ -284,6 +284,44 @@ def decode_read_int8_workload(torch, ops, dev, iters):
     }
 
 
+GEOMETRIES = [  # (model whose cache has this shape, kv heads, query heads, head_dim)
+    ("llama-3-8b", 8, 32, 128), ("llama-3-70b", 8, 64, 128), ("llama-2-7b", 32, 32, 128), ("llama-2-13b", 40, 40, 128),
+    ("qwen2.5-7b", 4, 28, 128), ("qwen2.5-3b", 2, 16, 128), ("qwen2.5-1.5b", 2, 12, 128), ("qwen2.5-0.5b", 2, 14, 64),
+    ("qwen2.5-14b", 8, 40, 128), ("chatglm3-6b", 2, 32, 128), ("gpt2", 12, 12, 64), ("gpt2-medium", 16, 16, 64),
+    ("gpt2-xl", 25, 25, 64), ("llama-3.2-1b", 8, 32, 64), ("llama-3.2-3b", 8, 24, 128), ("gemma-7b", 16, 16, 256),
+    ("gemma-2-9b", 8, 16, 256), ("falcon-7b", 1, 71, 64), ("starcoder2-7b", 4, 36, 128), ("starcoder-15b", 1, 48, 128),
+]
+
+
+def geometries_workload(torch, ops, dev, iters):
+    """pikv_decode_attend (the whole read of a decode step) over the cache geometries of published models:
+    64 sequences, about 0.6 GB of K + V codes each way, 4-bit group-32 and 8-bit per-head caches, bf16
+    queries.  Not part of the default run (`--workload geometries`); reported rates count the K and V bytes
+    only, the score traffic of many query heads comes on top."""
+    out, B = {}, 64
+    for eight in (False, True):
+        for name, hkv, hq, dh in GEOMETRIES:
+            row = hkv * dh * (1.0 if eight else 0.5) + (hkv * 4 if eight else hkv * dh // 32 * 4)
+            n_tok = int(min(32768, max(2048, (6e8 / B / row) // 512 * 512)))
+            pool = ops.CachePool([n_tok] * B, hkv, dh, dh if eight else 32, ops.Q_I8_SYM if eight else ops.Q_I4_ASYM,
+                                 dev, with_v=True)
+            if eight:
+                pool.k_codes.random_(-127, 127), pool.v_codes.random_(-127, 127)
+            else:
+                pool.k_codes.random_(0, 255), pool.v_codes.random_(0, 255)
+                pool.k_zero.fill_(7.0), pool.v_zero.fill_(7.0)
+            pool.k_scale.fill_(0.05), pool.v_scale.fill_(0.05)
+            pool.fill.fill_(n_tok)
+            q = torch.randn(B, hq, dh, device=dev).to(torch.bfloat16)
+            t = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=3.0), iters)
+            kv_bytes = 2 * row * n_tok * B
+            out[("int8 " if eight else "int4 ") + name] = {"kv_heads": hkv, "q_heads": hq, "head_dim": dh, "tokens": n_tok,
+                                                         "ms": t, "kv_GBps": kv_bytes / t / 1e6}
+            del pool
+            torch.cuda.empty_cache()
+    return out
+
+
 def wide_routing_workload(torch, ops, dev, iters):
     """Wide MoE routing: 65536 tokens, hidden 7168, 64 experts top-8, Zipf(1.2) expert
     popularity, EPLB-style per-expert logit scale; int8 KV of 8 heads x 128 scattered
@@ -364,7 +402,7 @@ def main():
     ap.add_argument("--only-headline", action="store_true",
                     help="skip the per-kernel figures of the decode, wide-routing and pyramid workloads")
     ap.add_argument("--workload", default="all",
-                    choices=["all", "prefill", "decode_read", "decode_read_int8_gqa8", "wide_routing", "pyramid"],
+                    choices=["all", "prefill", "decode_read", "decode_read_int8_gqa8", "wide_routing", "pyramid", "geometries"],
                     help="run one workload only (for profiling; the bench line proper is the default, all)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the streaming probes over 1 GiB (kernels of known traffic, to scale "
@@ -401,10 +439,11 @@ def main():
         return
     others = {"decode_read": decode_read_workload, "decode_read_int8_gqa8": decode_read_int8_workload,
               "wide_routing": wide_routing_workload, "pyramid": pyramid_workload}
-    if args.workload in others:
+    if args.workload in others or args.workload == "geometries":
         it = max(5, min(args.steps, 20))
+        fn = geometries_workload if args.workload == "geometries" else others[args.workload]
         print(json.dumps({"workload_only": args.workload, "hbm_ceiling": hbm_ceiling(torch, dev, 10),
-                          args.workload: others[args.workload](torch, ops, dev, it)}))
+                          args.workload: fn(torch, ops, dev, it)}))
         return
     w = WORKLOAD
     T, E, k = w["batch"] * w["seq"], w["experts"], w["top_k"]
