@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Profile one workload of bench.py with rocprofv3 and write its summary to profiles/.
 
-    python3 bench_profile.py <workload> [--out-dir gpurun_out/prof_<workload>]
+    python3 bench_profile.py <workload> [--out-dir prof_out/<workload>]
 
 <workload> is one of bench.py's --workload names (prefill, decode_read, decode_read_int8_gqa8,
 wide_routing, pyramid) or `ceilings` (the streaming probes alone).  Three profiler passes run,
@@ -77,7 +77,7 @@ def main():
     ap.add_argument("--out-dir", default=None)
     args = ap.parse_args()
     w = args.workload
-    out_dir = os.path.abspath(args.out_dir or os.path.join(ROOT, "gpurun_out", f"prof_{w}"))
+    out_dir = os.path.abspath(args.out_dir or os.path.join(ROOT, "prof_out", w))
     base = ["--calibrate-copy"] if w == "ceilings" else ["--workload", w, "--no-cpu-baseline"]
     short_run = [] if w == "ceilings" else ["--steps", "5", "--warmup", "2"]
     trace = read_trace(run_pass("trace", out_dir, base))
