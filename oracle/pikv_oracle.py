@@ -30,9 +30,17 @@ Pinning status (what, besides this file, fixes each function's output):
                                        hand-computed known answers (tie rounding, a shifted
                                        and a constant row; interior budgets from the integer
                                        formula; a literal 2-token dispatch)
-  fakequant_colblocks / _preset ...... hand-computed known answers; the preset form
-                                       given a block's own parameters must repeat
-                                       the block form bit for bit
+  scale_logits ....................... literals of a float32 case where (lg/T)*w and
+                                       (lg*w)/T differ in the last bit (one per reference
+                                       copy, re-derived with exact rationals), both mask
+                                       penalties as literals
+  fakequant_colblocks / _preset ...... hand-computed block scale / zero point / codes
+                                       ([-1,0,1] -> 2/255, 127; extremes in different rows;
+                                       two blocks; 4-bit; symmetric), identity with
+                                       quantize_groups on one-row inputs for all four
+                                       (bits, symmetric) pairs; the preset form given a
+                                       block's own parameters must repeat the block form
+                                       bit for bit
   all of the above ................... property tests (ranges, error bounds, total
                                        orders, conservation, monotone budgets) and the
                                        frozen digests of tests/golden

@@ -419,6 +419,141 @@ def test_fakequant_preset_known_answers():
     assert np.array_equal(dq, ref) and np.allclose(mse, mse_ref, rtol=0, atol=0)
 
 
+def _rn32(fr):
+    """Round an exact rational to the nearest float32, ties to even, without using any
+    float32 arithmetic: the independent arbiter of what one IEEE operation returns."""
+    from fractions import Fraction
+    fr = Fraction(fr)
+    if fr == 0:
+        return np.float32(0.0)
+    sign = -1 if fr < 0 else 1
+    a = abs(fr)
+    e = a.numerator.bit_length() - a.denominator.bit_length()
+    if Fraction(2) ** e > a:
+        e -= 1
+    e = max(e, -126)
+    q = a / Fraction(2) ** (e - 23)                 # significand in units of the last place
+    n = q.numerator // q.denominator
+    rem = q - n
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and n % 2 == 1):
+        n += 1
+    return np.float32(sign * float(Fraction(n) * Fraction(2) ** (e - 23)))
+
+
+def test_fakequant_colblocks_scale_and_zero_known_answers():
+    """core/single/pikv_compression.py:396-429 on a block: the block-wide scale and zero point
+    by hand.  [-1, 0, 1] (one row, then spread over three rows of one column block):
+    scale = RN(2/255) = 0.007843137718737125; -1/scale = -127.49999 in float32 (the real quotient
+    is -127.5 only for the unrounded scale), so round() gives -127 and zero = 0 - (-127) = 127
+    (floor would give 128; a range of 256 instead of 255 gives scale 0.0078125 and zero 128).
+    codes 0, 127, 254 -> dq = (q - 127) * scale."""
+    from fractions import Fraction as Fr
+    s_lit = np.float32(0.007843137718737125)
+    assert _rn32(Fr(2, 255)) == s_lit
+    assert _rn32(Fr(-1) / Fr(float(s_lit))) == np.float32(-127.49999237060547)   # not -127.5
+    for x in (np.array([[-1.0, 0.0, 1.0]], np.float32),
+              np.array([[-1.0], [0.0], [1.0]], np.float32)):
+        dq, st, mse = O.fakequant_colblocks(x, x.shape[1])
+        assert st.shape == (1, 4)
+        assert st[0, 0] == -1.0 and st[0, 1] == 1.0
+        assert st[0, 2] == s_lit, st
+        assert st[0, 3] == 127.0, st
+        want = np.array([-127, 0, 127], np.float32) * s_lit
+        assert want[2] == np.float32(0.9960784912109375)
+        assert np.array_equal(dq.reshape(-1), want)
+        assert abs(mse[0] - 2 * (1 - 0.9960784912109375) ** 2 / 3) < 1e-15
+    # min and max in different rows AND interior values: [[-1, 0.25], [0.5, 1]] as one block.
+    # 0.25/scale = 31.874998 -> +127 = 158.875 -> 159 -> 32*scale; 0.5/scale = 63.749996 -> 190.75 -> 191
+    dq, st, _ = O.fakequant_colblocks(np.array([[-1.0, 0.25], [0.5, 1.0]], np.float32), 2)
+    assert st[0, 2] == s_lit and st[0, 3] == 127.0
+    assert np.array_equal(dq, np.array([[-127, 32], [64, 127]], np.float32) * s_lit)
+    # two column blocks with different parameters: block 0 = {0, 51} -> scale 0.2, zero 0;
+    # block 1 = {10, 265} -> scale 1, zero = 0 - 10 = -10, codes round(x - 10), dq = code + 10
+    x = np.array([[0.0, 10.0], [51.0, 265.0], [25.5, 137.5]], np.float32)
+    dq, st, _ = O.fakequant_colblocks(x, 1)
+    assert st[0, 2] == _rn32(Fr(51, 255)) == np.float32(0.2) and st[0, 3] == 0.0
+    assert st[1, 2] == 1.0 and st[1, 3] == -10.0
+    # 25.5/0.2f: the real quotient 127.4999981 rounds to the float32 127.5 -> half to even -> 128
+    assert _rn32(Fr(51, 2) / Fr(float(np.float32(0.2)))) == np.float32(127.5)
+    assert dq[2, 0] == np.float32(128.0) * np.float32(0.2) and dq[1, 0] == np.float32(255.0) * np.float32(0.2)
+    assert dq[:, 1].tolist() == [10.0, 265.0, 138.0]                    # 137.5 - 10 = 127.5 -> 128 (even) -> 138
+    # 4-bit asymmetric and the symmetric variants (core/single/module/pikv_compression.py:945-1012)
+    dq, st, _ = O.fakequant_colblocks(np.array([[0.0, 1.0, 2.0, 3.75]], np.float32), 4, bits=4)
+    assert st[0, 2] == 0.25 and st[0, 3] == 0.0 and dq.tolist() == [[0.0, 1.0, 2.0, 3.75]]
+    dq, st, _ = O.fakequant_colblocks(np.array([[0.3, -0.7, 0.05, 0.7]], np.float32), 4, symmetric=True)
+    assert st[0, 2] == _rn32(Fr(float(np.float32(2.0) * np.float32(0.7))) / 255) and st[0, 3] == 0.0
+    assert np.array_equal(dq, np.array([[55, -128, 9, 127]], np.float32) * st[0, 2])
+    dq, st, _ = O.fakequant_colblocks(np.array([[-3.75, 1.0, 0.26, 3.0]], np.float32), 4, bits=4, symmetric=True)
+    assert st[0, 2] == 0.5 and dq.tolist() == [[-4.0, 1.0, 0.5, 3.0]]   # -7.5 -> -8 (even, in range) -> -4; 0.52 -> 1
+
+
+@pytest.mark.parametrize("bits,symmetric", [(8, False), (8, True), (4, False), (4, True)])
+def test_fakequant_one_row_block_equals_group_quantisation(bits, symmetric):
+    """With one row, the block domain of QuantizedCompressor.forward IS a per-row group: the result
+    must be quantize_groups + dequantize_groups (pinned by the known answers above) bit for bit.
+    The 4-bit group format rounds its metadata to float16, so those rows are built with extremes
+    whose scale and zero point are float16 numbers (range 15 * 2^-k)."""
+    scheme = {(8, False): O.Q_I8_ASYM, (8, True): O.Q_I8_SYM,
+              (4, False): O.Q_I4_ASYM, (4, True): O.Q_I4_SYM}[(bits, symmetric)]
+    r = rng(100 + bits + symmetric)
+    for trial in range(40):
+        G = [16, 32, 128][trial % 3]
+        if bits == 8:
+            x = (r.standard_normal((1, 3 * G)) * r.choice([1e-3, 1.0, 30.0])).astype(np.float32)
+            if trial % 5 == 0:
+                x += np.float32(r.uniform(-4, 4))
+        else:
+            step = np.float32(2.0 ** -r.integers(0, 6))
+            lo = np.float32(-r.integers(0, 16)) * step if not symmetric else np.float32(-7.5) * step
+            x = (lo + r.uniform(0, 15, (1, 3 * G)).astype(np.float32) * step).astype(np.float32)
+            for b in range(3):
+                x[0, b * G] = lo
+                x[0, b * G + 1] = lo + np.float32(15) * step
+        dq, st, _ = O.fakequant_colblocks(x, G, bits=bits, symmetric=symmetric)
+        q, s, z = O.quantize_groups(x, G, scheme)
+        want = O.dequantize_groups(q, s, z, G)
+        assert np.array_equal(st[:, 2], s[0]) and np.array_equal(st[:, 3], z[0]), (trial, st, s, z)
+        assert np.array_equal(dq, want), trial
+
+
+def test_scale_logits_order_and_penalty_known_answers():
+    """The two reference copies scale logits in different orders and mask with different
+    penalties; in float32 the orders differ in the last bit.  lg = 2.1f, T = 0.7f, w = 1.1f:
+      core/single/pikv_routing.py:653-656         (lg / T) * w = 3.3000001907348633
+      core/single/module/pikv_routing.py:596-600  (lg * w) / T = 3.299999952316284
+    (both literals re-derived below with exact rational arithmetic, one rounding per operation).
+    Penalties: single adds (1 - m) * -1e9 (:68-70), module adds (1 - m) * finfo(float32).min
+    (:133-134)."""
+    from fractions import Fraction as Fr
+    lg, T, w = np.float32(2.1), np.float32(0.7), np.float32(1.1)
+    single = _rn32(Fr(float(_rn32(Fr(float(lg)) / Fr(float(T))))) * Fr(float(w)))
+    module = _rn32(Fr(float(_rn32(Fr(float(lg)) * Fr(float(w))))) / Fr(float(T)))
+    assert single == np.float32(3.3000001907348633) and module == np.float32(3.299999952316284)
+    assert single != module
+    es = np.array([w, 1.0], np.float32)
+    row = np.array([[lg, lg]], np.float32)
+    out = O.scale_logits(row, temperature=float(T), expert_scale=es)
+    assert out[0, 0] == single and out[0, 1] == _rn32(Fr(float(lg)) / Fr(float(T)))
+    out = O.scale_logits(row, temperature=float(T), expert_scale=es, module_arithmetic=True)
+    assert out[0, 0] == module and out[0, 1] == _rn32(Fr(float(lg)) / Fr(float(T)))
+    # the C twin (single/ order only) through an identity gate
+    got = CO.router(row, np.eye(2, dtype=np.float32), None, 1, temperature=float(T), expert_scale=es)[1]
+    assert got[0, 0] == single
+    # penalties: 5 - 1e9 rounds to -1e9 (spacing 64 there); 5 + finfo.min rounds to finfo.min
+    m = np.array([0.0, 1.0], np.float32)
+    out = O.scale_logits(np.array([[5.0, -5.0]], np.float32), expert_mask=m)
+    assert out.tolist() == [[-1e9, -5.0]]
+    out = O.scale_logits(np.array([[5.0, -5.0]], np.float32), expert_mask=m, module_arithmetic=True)
+    assert out.tolist() == [[-3.4028234663852886e+38, -5.0]]
+    # a NEGATIVE masked logit overflows past finfo.min only when it is huge; an ordinary one stays finite
+    out = O.scale_logits(np.array([[-5.0, 1.0]], np.float32), expert_mask=m, module_arithmetic=True)
+    assert out[0, 0] == np.float32(-3.4028234663852886e+38) and np.isfinite(out[0, 0])
+    # the penalty is added after scaling in both copies: (lg / T) * w - 1e9, not (lg - 1e9) / T * w
+    out = O.scale_logits(np.array([[5.0, 1.0]], np.float32), temperature=0.5,
+                         expert_scale=np.array([2.0, 1.0], np.float32), expert_mask=m)
+    assert out.tolist() == [[-1e9, 2.0]]
+
+
 # ---------------------------------------------------------------- hand-computed pins of the facade / caller helpers
 def test_quant8_minshift_known_answers():
     """core/single/pikv_kernels.py:215-232 by hand.  Row 0: min 0, max 255, s = 1, so the
