@@ -103,7 +103,10 @@ int pikv_abi_version(void);
  *   logits     += (1-expert_mask[e])*-1e9 (if expert_mask != NULL)
  *                 (order and penalty of arithmetic = PIKV_ROUTER_SINGLE; see above)
  *   probs       = softmax_e(logits)
- *   topk_idx    = k largest logits, (value desc, index asc)
+ *   topk_idx    = k largest PROBABILITIES (the float32 values of `probs`, what the
+ *                 reference hands to torch.topk), (value desc, index asc, NaN last):
+ *                 distinct logits whose probabilities round to one float32 tie, and
+ *                 the lower expert wins
  *   topk_w      = probs[topk_idx] / (sum_j probs[topk_idx[j]] + renorm_eps)
  *   slot[t,j]   = number of assignments (t',j') < (t,j) in token-major order
  *                 with the same expert; -1 when that count >= capacity

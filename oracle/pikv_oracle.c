@@ -98,8 +98,9 @@ uint16_t pko_f32_to_half(float f) { return f32_to_half_sat(f); }
 float pko_half_to_f32(uint16_t h) { return half_to_f32(h); }
 
 /* ---- router --------------------------------------------------------------- */
-/* logits (double accumulation, rounded once), scaling, softmax, top-k by
- * (logit desc, index asc), renormalise.  probs/logits_out may be NULL. */
+/* logits (double accumulation, rounded once), scaling, softmax, top-k of the float32
+ * probabilities by (value desc, index asc, NaN last) as core/single/pikv_routing.py:73-76
+ * hands them to torch.topk, renormalise.  probs/logits_out may be NULL. */
 void pko_router(const void* x, const void* w, int dtype, const float* bias, const float* escale,
                 const float* emask, float temperature, float renorm_eps, int64_t T, int H, int E,
                 int k, float* probs, float* logits_out, int32_t* idx, float* wts) {
@@ -130,8 +131,10 @@ void pko_router(const void* x, const void* w, int dtype, const float* bias, cons
     float s = 0.f;
     for (int j = 0; j < k; ++j) {
       int best = -1;
-      for (int e = 0; e < E; ++e)
-        if (!used[e] && (best < 0 || lg[e] > lg[best])) best = e; /* strict >: lowest index wins ties */
+      for (int e = 0; e < E; ++e) { /* strict >: lowest index wins ties; a NaN never beats anything */
+        if (used[e]) continue;
+        if (best < 0 || pr[e] > pr[best] || (pr[best] != pr[best] && pr[e] == pr[e])) best = e;
+      }
       used[best] = 1;
       idx[t * k + j] = best;
       wts[t * k + j] = pr[best];

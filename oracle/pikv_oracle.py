@@ -10,8 +10,11 @@ Where the reference leaves a result implementation-defined the rule used here
 is stated in the docstring:
   * every top-k orders by (value, index) with the LOWER index first among
     equal values (torch.topk's tie order on CPU is unspecified);
-  * expert top-k is taken on the final logits, which orders exactly like the
-    probabilities except where float32 exp() collapses distinct logits.
+  * expert top-k is taken on what the reference hands to torch.topk, the float32
+    probabilities (core/single/pikv_routing.py:73-76): two distinct logits whose
+    probabilities round to the same float32 tie, and the lower expert wins; rows
+    whose probabilities are NaN (a NaN or +inf logit) select experts 0..k-1.
+    Without the softmax (PiKVKernels.top_k_routing) the key is the logit.
 
 Pinning status (what, besides this file, fixes each function's output):
   router_tail / capacity_slots ....... brute-force loops + invariants + the C
@@ -146,7 +149,7 @@ def softmax_rows(lg: np.ndarray) -> np.ndarray:
 
 def topk_desc(v: np.ndarray, k: int) -> np.ndarray:
     """Indices of the k largest entries of each row, largest first, lower
-    index first among equals (stable sort)."""
+    index first among equals (stable sort); NaN sorts after every number."""
     order = np.argsort(-v.astype(np.float64), axis=-1, kind="stable")
     return order[..., :k].astype(np.int32)
 
@@ -170,11 +173,12 @@ def router_tail(logits, top_k, temperature=1.0, expert_scale=None,
     lg = scale_logits(logits, temperature, expert_scale, expert_mask,
                       logits_b, select, module_arithmetic)
     k = min(int(top_k), lg.shape[-1])
-    idx = topk_desc(lg, k)
     if not use_softmax:
+        idx = topk_desc(lg, k)
         vals = np.take_along_axis(lg, idx.astype(np.int64), axis=-1)
         return None, idx, vals.astype(F32), lg
     probs = softmax_rows(lg)
+    idx = topk_desc(probs, k)
     vals = np.take_along_axis(probs, idx.astype(np.int64), axis=-1)
     s = np.zeros(vals.shape[:-1] + (1,), dtype=F32)
     for j in range(k):                       # left-to-right float32 sum

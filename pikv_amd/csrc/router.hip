@@ -121,6 +121,11 @@ __device__ __forceinline__ float final_logit(float lg, int e, const TailParams& 
 
 // Lane holds the raw logit of (token t, expert e); groups of EPAD adjacent lanes
 // form one token.  Writes probs / top-k for the token.
+// The top-k is taken on what the reference hands to torch.topk - the float32 probabilities
+// (core/single/pikv_routing.py:73-76), or the final logits without the softmax
+// (core/single/pikv_kernels.py:97) - in the total order (value descending, expert index
+// ascending, NaN last): two distinct logits whose probabilities round to the same float32
+// are a tie, and the lower expert wins it.
 // NTOK independent token groups go through the steps side by side: every step is a
 // chain of dependent cross-lane operations, and the chains of different tokens fill each
 // other's wait states.
@@ -171,7 +176,7 @@ __device__ __forceinline__ void router_tail_multi(float (&lg)[NTOK], const int64
   for (int j = 0; j < p.k; ++j) {
     float key[NTOK], mx[NTOK];
 #pragma unroll
-    for (int n = 0; n < NTOK; ++n) key[n] = remaining[n] ? lg[n] : -__builtin_inff();
+    for (int n = 0; n < NTOK; ++n) key[n] = remaining[n] ? carried[n] : -__builtin_inff();
 #pragma unroll
     for (int n = 0; n < NTOK; ++n) mx[n] = group_max_dpp(key[n], EPAD);
 #pragma unroll
@@ -555,22 +560,27 @@ __device__ __forceinline__ float tree16(const float* a) {
   return (q0 + q1) + (q2 + q3);
 }
 
-// Row `row` (stride RS floats) holds the final logits of one token, -inf in the padding
-// columns e >= E.  Leaves the probabilities in the row and writes the token's top-k
-// (without the softmax: the top-k of the logits, nothing else).
-// Same arithmetic, in the same order, as the lane-per-expert tail: max, expf(l - max), the
-// balanced sum, one division per expert; weights = p / (sum of the selected p, largest first).
-template <int EP, int RS>
-__device__ __forceinline__ void lane_token_tail(float* row, int64_t t, const TailParams& p) {
-  static_assert(EP == 16 || EP == 32 || EP == 64, "rows of 16, 32 or 64 columns");
-  uint64_t top[8];
+// Largest of 16 values, NaN ignored unless all are NaN (fmaxf), as a balanced tree
+__device__ __forceinline__ float max16(const float* a) {
+  const float q0 = fmaxf(fmaxf(a[0], a[1]), fmaxf(a[2], a[3])), q1 = fmaxf(fmaxf(a[4], a[5]), fmaxf(a[6], a[7]));
+  const float q2 = fmaxf(fmaxf(a[8], a[9]), fmaxf(a[10], a[11])), q3 = fmaxf(fmaxf(a[12], a[13]), fmaxf(a[14], a[15]));
+  return fmaxf(fmaxf(q0, q1), fmaxf(q2, q3));
+}
+// The value a key was made from (keys of values >= +0 or NaN only: probabilities)
+__device__ __forceinline__ float prob_of_key(uint64_t key) {
+  const uint32_t k = (uint32_t)(key >> 32);
+  return k == 1u ? __builtin_nanf("") : __uint_as_float(k & 0x7fffffffu);
+}
+// The eight largest of row[e0 .. e0 + 8*G) by (value desc, expert asc), sorted
+template <int G>
+__device__ __forceinline__ void top8_of_row(const float* row, int e0, int E, uint64_t (&top)[8]) {
 #pragma unroll
-  for (int g = 0; g < EP / 8; ++g) {
+  for (int g = 0; g < G; ++g) {
     uint64_t cur[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int e = 8 * g + i;
-      cur[i] = e < p.E ? lane_topk_key(row[e], e) : 0ull;
+      const int e = e0 + 8 * g + i;
+      cur[i] = e < E ? lane_topk_key(row[e], e) : 0ull;
     }
     sort8_desc(cur);
     if (g == 0) {
@@ -580,23 +590,44 @@ __device__ __forceinline__ void lane_token_tail(float* row, int64_t t, const Tai
       merge_top8(top, cur);
     }
   }
-  int idx[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) idx[j] = 63 - (int)(uint32_t)top[j];
-  float pv[8], wsum = 0.f;
+}
+
+// Row `row` (stride RS floats) holds the final logits of one token, -inf in the padding
+// columns e >= E.  Leaves the probabilities in the row and writes the token's top-k
+// (without the softmax: the top-k of the logits, nothing else).
+// Same arithmetic, in the same order, as the lane-per-expert tail: max, expf(l - max), the
+// balanced sum, one division per expert; the top-k is then taken on the PROBABILITIES (what
+// the reference passes to torch.topk, core/single/pikv_routing.py:73-76; value descending,
+// lower expert first among equal float32 values, NaN last); weights = p / (sum of the
+// selected p, largest first).
+template <int EP, int RS>
+__device__ __forceinline__ void lane_token_tail(float* row, int64_t t, const TailParams& p) {
+  static_assert(EP == 16 || EP == 32 || EP == 64, "rows of 16, 32 or 64 columns");
   if (p.use_softmax) {
-    const float m = row[idx[0]];
     float ex[EP];
 #pragma unroll
-    for (int e = 0; e < EP; ++e) ex[e] = expf(row[e] - m);  // padding: expf(-inf) = 0
+    for (int e = 0; e < EP; ++e) ex[e] = row[e];
+    float m = max16(ex);
+    if constexpr (EP >= 32) m = fmaxf(m, max16(ex + 16));
+    if constexpr (EP == 64) m = fmaxf(m, fmaxf(max16(ex + 32), max16(ex + 48)));
+#pragma unroll
+    for (int e = 0; e < EP; ++e) ex[e] = expf(ex[e] - m);  // padding: expf(-inf) = 0
     float sum = tree16(ex);
     if constexpr (EP == 32) sum = sum + tree16(ex + 16);
     if constexpr (EP == 64) sum = (sum + tree16(ex + 16)) + (tree16(ex + 32) + tree16(ex + 48));
 #pragma unroll
     for (int e = 0; e < EP; ++e) row[e] = ex[e] / sum;
+  }
+  uint64_t top[8];
+  top8_of_row<EP / 8>(row, 0, p.E, top);
+  int idx[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) idx[j] = 63 - (int)(uint32_t)top[j];
+  float pv[8], wsum = 0.f;
+  if (p.use_softmax) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      pv[j] = j < p.k ? row[idx[j]] : 0.f;
+      pv[j] = j < p.k ? prob_of_key(top[j]) : 0.f;
       if (j < p.k) wsum = wsum + pv[j];
     }
     if (p.renorm_eps != 0.f) wsum = wsum + p.renorm_eps;
@@ -632,75 +663,69 @@ __device__ __forceinline__ void lane_token_tail(float* row, int64_t t, const Tai
 }
 
 // The same for 64 columns with TWO lanes per token: `half` 0 takes experts 0..31, half 1 the
-// rest.  Each sorts its 32, the two top-8 lists meet in LDS and are merged by both; each takes
-// the exponentials, the partial sum (two 16-trees) and the divisions of its half - the total
-// is still (R0 + R1) + (R2 + R3) - and half 0 writes the token's top-k.  Every thread of the
-// block has to call this (three block barriers); `active` says whether it holds a token.
-// xkeys: [8][2][TB] 64-bit keys, xsum: [2][TB] floats.
+// rest.  The two maxima, then the two partial sums (two 16-trees each; the total is still
+// (R0 + R1) + (R2 + R3)) meet in LDS; each lane divides its half, sorts its 32 probabilities,
+// the two top-8 lists meet in LDS and half 0 merges them and writes the token's top-k.  Every
+// thread of the block has to call this (three block barriers, one without the softmax);
+// `active` says whether it holds a token.  xkeys: [8][2][TB] 64-bit keys (its first 2*TB
+// words also carry the two maxima), xsum: [2][TB] floats.
 template <int RS, int TB>
 __device__ __forceinline__ void pair_token_tail(float* row, int half, int tl, bool active, int64_t t,
                                                 const TailParams& p, uint64_t* xkeys, float* xsum) {
   uint64_t top[8];
-  if (active) {
+  if (p.use_softmax) {  // uniform for the block
+    float ex[32];
+    float* xmax = reinterpret_cast<float*>(xkeys);
+    if (active) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      uint64_t cur[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int e = 32 * half + 8 * g + i;
-        cur[i] = e < p.E ? lane_topk_key(row[e], e) : 0ull;
-      }
-      sort8_desc(cur);
-      if (g == 0) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) top[i] = cur[i];
-      } else {
-        merge_top8(top, cur);
-      }
+      for (int e = 0; e < 32; ++e) ex[e] = row[32 * half + e];
+      xmax[half * TB + tl] = fmaxf(max16(ex), max16(ex + 16));
     }
+    __syncthreads();
+    if (active) {
+      const float m = fmaxf(xmax[tl], xmax[TB + tl]);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) xkeys[(j * 2 + half) * TB + tl] = top[j];
-  }
-  __syncthreads();
-  int idx[8];
-  float ex[32];
-  if (active) {
-    uint64_t other[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) other[j] = xkeys[(j * 2 + (1 - half)) * TB + tl];
-    merge_top8(top, other);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) idx[j] = 63 - (int)(uint32_t)top[j];
-  }
-  if (!p.use_softmax) {  // raw top-k: the selected logits themselves (uniform for the block)
-    if (active && half == 0 && t < p.T) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        if (j < p.k) {
-          p.topk_idx[t * p.k + j] = idx[j];
-          p.topk_w[t * p.k + j] = row[idx[j]];
-        }
+      for (int e = 0; e < 32; ++e) ex[e] = expf(ex[e] - m);  // padding: expf(-inf) = 0
+      xsum[half * TB + tl] = tree16(ex) + tree16(ex + 16);
     }
-    return;
+    __syncthreads();  // also: every maximum has been read, xkeys may take the keys
+    if (active) {
+      const float sum = xsum[tl] + xsum[TB + tl];
+#pragma unroll
+      for (int e = 0; e < 32; ++e) row[32 * half + e] = ex[e] / sum;
+    }
   }
   if (active) {
-    const float m = row[idx[0]];
+    top8_of_row<4>(row, 32 * half, p.E, top);
+    if (half == 1) {
 #pragma unroll
-    for (int e = 0; e < 32; ++e) ex[e] = expf(row[32 * half + e] - m);  // padding: expf(-inf) = 0
-    xsum[half * TB + tl] = tree16(ex) + tree16(ex + 16);
-  }
-  __syncthreads();
-  if (active) {
-    const float sum = xsum[tl] + xsum[TB + tl];
-#pragma unroll
-    for (int e = 0; e < 32; ++e) row[32 * half + e] = ex[e] / sum;
+      for (int j = 0; j < 8; ++j) xkeys[j * TB + tl] = top[j];
+    }
   }
   __syncthreads();
   if (!active || half != 0 || t >= p.T) return;
+  {
+    uint64_t other[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) other[j] = xkeys[j * TB + tl];
+    merge_top8(top, other);
+  }
+  int idx[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) idx[j] = 63 - (int)(uint32_t)top[j];
+  if (!p.use_softmax) {  // raw top-k: the selected logits themselves
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < p.k) {
+        p.topk_idx[t * p.k + j] = idx[j];
+        p.topk_w[t * p.k + j] = row[idx[j]];
+      }
+    return;
+  }
   float pv[8], wsum = 0.f;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    pv[j] = j < p.k ? row[idx[j]] : 0.f;
+    pv[j] = j < p.k ? prob_of_key(top[j]) : 0.f;
     if (j < p.k) wsum = wsum + pv[j];
   }
   if (p.renorm_eps != 0.f) wsum = wsum + p.renorm_eps;

@@ -1,9 +1,11 @@
 """GPU parity: K1 router (gate projection, softmax, top-k, renormalise, capacity
 slots) through the C ABI against the numpy restatement.
 
-Bit-exact: expert indices and slots whenever the logits are given (tail entry
-point), including ties (lowest index wins), masks, scaling and the two-gate
-select.  For the fused gate projection the float32 summation order differs
+Expert indices: on every row the stable top-k (value descending, lower expert first
+among equal float32 values) of the probabilities the kernel returned - the tensor the
+reference hands to torch.topk - and equal to the restatement's selection except where
+the two sides' exp() round a near-tie differently (util.assert_topk_of_probs); slots
+bit-exact for the indices chosen; masks, scaling and the two-gate select included.  For the fused gate projection the float32 summation order differs
 from any CPU order, so indices are compared exactly wherever the float64 gap
 between the k-th and (k+1)-th logit exceeds 1e-4 (relative to the logit range)
 and the capacity slots are checked for exact consistency with the indices the
@@ -13,7 +15,7 @@ import numpy as np
 import pytest
 
 import pikv_oracle as O
-from util import np_of, rng, to_dev
+from util import assert_topk_of_probs, np_of, rng, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -45,10 +47,12 @@ def test_router_tail_bit_exact(dev, E, k):
             dkw["select"] = to_dev(sel.astype(np.uint8), dev)
         out = ops.router_tail(to_dev(lg, dev), top_k=k, capacity=cap, **dkw)
         probs, idx, w, _ = O.router_tail(lg, k, **okw)
-        assert np.array_equal(np_of(out.topk_idx), idx), kw.keys()
+        got = np_of(out.topk_idx)
+        assert_topk_of_probs(got, np_of(out.probs), k, idx, probs)
+        same = (got == idx).all(axis=1)
         assert np.allclose(np_of(out.probs), probs, atol=2e-6, rtol=1e-5)
-        assert np.allclose(np_of(out.topk_w), w, atol=2e-6, rtol=1e-5)
-        slot, count = O.capacity_slots(idx, E, cap)
+        assert np.allclose(np_of(out.topk_w)[same], w[same], atol=2e-6, rtol=1e-5)
+        slot, count = O.capacity_slots(got, E, cap)
         assert np.array_equal(np_of(out.slot), slot)
         assert np.array_equal(np_of(out.count), count)
     # raw top-k of logits (the facade's top_k_routing): values are the logits
@@ -56,6 +60,54 @@ def test_router_tail_bit_exact(dev, E, k):
     _, idx, vals, _ = O.router_tail(lg, k, use_softmax=False)
     assert np.array_equal(np_of(out.topk_idx), idx)
     assert np.array_equal(np_of(out.topk_w), vals)
+
+
+def _collapse_logits(E):
+    """Distinct logits whose float32 probabilities coincide: 2^-10 and its two predecessors
+    differ by 2^-34 - exp() of that difference is 1 to 2^-35, far inside one rounding - with
+    the LOWER logits at the LOWER expert indices (and, from 40 experts on, in the other half
+    of the row), everything else far below."""
+    hi = np.float32(2.0 ** -10)
+    lo = np.nextafter(hi, np.float32(0), dtype=np.float32)
+    lo2 = np.nextafter(lo, np.float32(0), dtype=np.float32)
+    row = np.linspace(-3.0, -6.0, E).astype(np.float32)
+    a, b, c = (3, 17, 40) if E > 40 else (0, 1, 2)
+    row[a], row[b], row[c] = lo2, lo, hi
+    return row, (a, b, c)
+
+
+@pytest.mark.parametrize("E,k", [(4, 1), (4, 2), (8, 2), (16, 3), (32, 2), (40, 1), (40, 2), (64, 1), (64, 2), (64, 8)])
+def test_topk_ties_on_probabilities_not_logits(dev, E, k):
+    """The reference takes torch.topk of the float32 PROBABILITIES (core/single/pikv_routing.py:
+    73-76).  Where exp() maps distinct logits to one float32 the experts tie and the lower index
+    wins, although its logit is the smaller one - in the restatement and in every form of the
+    kernel tail (standalone tail on given logits; the gate kernels fed the same logits through
+    the bias, for short, medium and long token streams, bf16 and float32 inputs)."""
+    import torch
+    from pikv_amd import ops
+    row, (a, b, c) = _collapse_logits(E)
+    want = [a, b, c][:k] + list(np.argsort(-row, kind="stable")[3:])[:max(0, k - 3)]
+    lg = np.tile(row, (300, 1))
+    probs, idx, w, _ = O.router_tail(lg, k)
+    assert probs[0, a] == probs[0, b] == probs[0, c] and row[a] < row[b] < row[c]
+    assert idx[0].tolist() == want
+    out = ops.router_tail(to_dev(lg, dev), top_k=k)
+    p = np_of(out.probs)
+    assert p[0, a] == p[0, b] == p[0, c]
+    assert (np_of(out.topk_idx) == np.array(want)).all()
+    raw = ops.router_tail(to_dev(lg, dev), top_k=k, use_softmax=False)      # without the softmax the key is the logit
+    assert np_of(raw.topk_idx)[0].tolist() == list(np.argsort(-row, kind="stable")[:k])
+    H = 256
+    for T, dt in [(300, torch.bfloat16), (300, torch.float32), (20480 + 64, torch.bfloat16), (32768 + 128, torch.bfloat16),
+                  (65536, torch.bfloat16)]:
+        if T == 65536 and E > 16:
+            continue
+        x = torch.randn(T, H, device=dev).to(dt)
+        out = ops.router_fused(x, torch.zeros(E, H, device=dev, dtype=dt), to_dev(row, dev), top_k=k, return_logits=True)
+        assert torch.equal(out.logits, to_dev(row, dev).expand(T, E))
+        got = np_of(out.topk_idx)
+        assert (got == np.array(want)).all(), (T, dt, got[0], want)
+        assert_topk_of_probs(got, np_of(out.probs), k)
 
 
 @pytest.mark.parametrize("E", [40, 64])
@@ -141,12 +193,13 @@ def test_router_fused(dev, dtype, T, H, E, k):
     assert np.allclose(np_of(out.logits), lg, atol=1e-5 * np.sqrt(H), rtol=1e-5)
     assert np.allclose(np_of(out.probs), probs, atol=1e-5)
     got = np_of(out.topk_idx)
-    # EVERY row: the selection is exactly the top-k (ties to the lower index) of the logits the
-    # kernel itself returned
+    # EVERY row: the selection is exactly the top-k (ties to the lower index) of the
+    # probabilities the kernel itself returned
     klg = np_of(out.logits)
-    _, idx_own, w_own, _ = O.router_tail(klg, k)
-    assert np.array_equal(got, idx_own)
-    assert np.allclose(np_of(out.topk_w), w_own, atol=1e-6)
+    p_own, idx_own, w_own, _ = O.router_tail(klg, k)
+    assert_topk_of_probs(got, np_of(out.probs), k, idx_own, p_own)
+    same = (got == idx_own).all(axis=1)
+    assert np.allclose(np_of(out.topk_w)[same], w_own[same], atol=1e-6)
     # and it is the float64 selection wherever the gap between neighbouring logits exceeds twice
     # the largest error the kernel's logits show against float64
     err = float(np.abs(klg.astype(np.float64) - lg64).max())
@@ -216,7 +269,7 @@ def test_router_long_stream(dev, T, H, E, k):
     lg = x.double() @ w.double().T + b.double()
     assert torch.allclose(out.logits.double(), lg, atol=1e-5 * H ** 0.5, rtol=1e-5)
     assert torch.allclose(out.probs, torch.softmax(out.logits, dim=1), atol=1e-6)
-    order = torch.sort(out.logits, dim=1, descending=True, stable=True).indices[:, :k]
+    order = torch.sort(out.probs, dim=1, descending=True, stable=True).indices[:, :k]
     assert torch.equal(out.topk_idx.long(), order)
     sel = torch.gather(out.probs, 1, order)
     assert torch.allclose(out.topk_w, sel / sel.sum(1, keepdim=True), atol=1e-6)
@@ -248,7 +301,7 @@ def test_router_short_stream_split(dev, T, H, E, k):
     if E >= 20:
         assert torch.equal(out.logits[:, 2], out.logits[:, 17])
     assert torch.allclose(out.probs, torch.softmax(out.logits, dim=1), atol=1e-6)
-    order = torch.sort(out.logits, dim=1, descending=True, stable=True).indices[:, :k]
+    order = torch.sort(out.probs, dim=1, descending=True, stable=True).indices[:, :k]
     assert torch.equal(out.topk_idx.long(), order)
     slot, count = O.capacity_slots(np_of(out.topk_idx), E, cap)
     assert np.array_equal(np_of(out.slot), slot)
@@ -277,9 +330,10 @@ def test_router_tiled_and_rows_forms_logit_arithmetic(dev, module):
     out = ops.router_tail(to_dev(lg, dev), top_k=k, temperature=0.7, expert_scale=to_dev(scale, dev),
                           expert_mask=to_dev(mask, dev), renorm_eps=kw["renorm_eps"], module_arithmetic=module)
     probs, idx, w, final = O.router_tail(lg, k, module_arithmetic=module, **kw)
-    assert np.array_equal(np_of(out.topk_idx), idx)
+    assert_topk_of_probs(np_of(out.topk_idx), np_of(out.probs), k, idx, probs)
+    same = (np_of(out.topk_idx) == idx).all(axis=1)
     assert np.allclose(np_of(out.probs), probs, atol=2e-6, rtol=1e-5)
-    assert np.allclose(np_of(out.topk_w), w, atol=2e-6, rtol=1e-5)
+    assert np.allclose(np_of(out.topk_w)[same], w[same], atol=2e-6, rtol=1e-5)
     assert not np.isin(np_of(out.topk_idx), [1, 9, 33]).any()
     # tiled gate kernel (more than 20480 tokens)
     T2, H = 20480 + 77, 256
@@ -296,12 +350,13 @@ def test_router_tiled_and_rows_forms_logit_arithmetic(dev, module):
     live = mask > 0
     assert np.allclose(fin[:, live], want[:, live], atol=2e-5 * H ** 0.5, rtol=2e-5)
     assert (fin[:, ~live] < (-1e38 if module else -1e8)).all()
-    order = torch.sort(o2.logits, dim=1, descending=True, stable=True).indices[:, :k]
+    order = torch.sort(o2.probs, dim=1, descending=True, stable=True).indices[:, :k]
     assert torch.equal(o2.topk_idx.long(), order)
     assert not np.isin(np_of(o2.topk_idx), [1, 9, 33]).any()
-    _, idx2, w2, _ = O.router_tail(fin, k, renorm_eps=kw["renorm_eps"])
-    assert np.array_equal(np_of(o2.topk_idx), idx2)
-    assert np.allclose(np_of(o2.topk_w), w2, atol=2e-6, rtol=1e-5)
+    p2, idx2, w2, _ = O.router_tail(fin, k, renorm_eps=kw["renorm_eps"])
+    assert_topk_of_probs(np_of(o2.topk_idx), np_of(o2.probs), k, idx2, p2)
+    same = (np_of(o2.topk_idx) == idx2).all(axis=1)
+    assert np.allclose(np_of(o2.topk_w)[same], w2[same], atol=2e-6, rtol=1e-5)
 
 
 def test_router_module_arithmetic(dev):
@@ -321,9 +376,10 @@ def test_router_module_arithmetic(dev):
     out = ops.router_tail(to_dev(lg, dev), top_k=k, capacity=900, temperature=0.7, expert_scale=to_dev(scale, dev),
                           expert_mask=to_dev(mask, dev), renorm_eps=1e-8, module_arithmetic=True)
     probs, idx, w, final = O.router_tail(lg, k, module_arithmetic=True, **kw)
-    assert np.array_equal(np_of(out.topk_idx), idx)
+    assert_topk_of_probs(np_of(out.topk_idx), np_of(out.probs), k, idx, probs)
+    same = (np_of(out.topk_idx) == idx).all(axis=1)
     assert np.allclose(np_of(out.probs), probs, atol=2e-6, rtol=1e-5)
-    assert np.allclose(np_of(out.topk_w), w, atol=2e-6, rtol=1e-5)
+    assert np.allclose(np_of(out.topk_w)[same], w[same], atol=2e-6, rtol=1e-5)
     assert not np.isin(np_of(out.topk_idx), [1, 9]).any()
     # the two orders really differ in the last bit for some logits
     other = O.scale_logits(lg, 0.7, scale, None)
@@ -336,9 +392,10 @@ def test_router_module_arithmetic(dev):
                            module_arithmetic=True, return_logits=True)
     fin = np_of(out.logits)
     assert (fin[:, [1, 9]] < -1e38).all()
-    _, idx2, w2, _ = O.router_tail(fin, k, renorm_eps=1e-8)
-    assert np.array_equal(np_of(out.topk_idx), idx2)
-    assert np.allclose(np_of(out.topk_w), w2, atol=2e-6, rtol=1e-5)
+    p2, idx2, w2, _ = O.router_tail(fin, k, renorm_eps=1e-8)
+    assert_topk_of_probs(np_of(out.topk_idx), np_of(out.probs), k, idx2, p2)
+    same = (np_of(out.topk_idx) == idx2).all(axis=1)
+    assert np.allclose(np_of(out.topk_w)[same], w2[same], atol=2e-6, rtol=1e-5)
 
 
 def test_router_empty_and_errors(dev):

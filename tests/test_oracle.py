@@ -151,6 +151,28 @@ def test_softmax_and_topk_closed_forms():
     assert np.allclose(w, 0.25)
 
 
+def test_topk_is_taken_on_probabilities():
+    """core/single/pikv_routing.py:73-76: torch.topk(softmax(logits)).  Distinct logits whose
+    float32 probabilities coincide tie, the lower expert wins (the build's tie rule), although
+    its logit is the smaller one; without the softmax (core/single/pikv_kernels.py:97) the
+    logits decide.  Both restatements."""
+    hi = np.float32(2.0 ** -10)
+    lo = np.nextafter(hi, np.float32(0), dtype=np.float32)
+    lg = np.array([[lo, hi, -3.0, -4.0], [-3.0, hi, -4.0, lo]], np.float32)
+    probs, idx, w, _ = O.router_tail(lg, 2)
+    assert probs[0, 0] == probs[0, 1] and probs[1, 1] == probs[1, 3]
+    assert idx.tolist() == [[0, 1], [1, 3]]
+    assert O.router_tail(lg, 1)[1].tolist() == [[0], [1]]
+    assert O.router_tail(lg, 1, use_softmax=False)[1].tolist() == [[1], [1]]
+    p2, _, i2, _ = CO.router(lg, np.eye(4, dtype=np.float32), None, 2)
+    assert p2[0, 0] == p2[0, 1] and i2.tolist() == [[0, 1], [1, 3]]
+    # rows whose probabilities are NaN (a NaN or +inf logit) select experts 0..k-1
+    bad = np.array([[0.0, np.nan, 1.0, 2.0], [0.0, 1.0, np.inf, 2.0]], np.float32)
+    with np.errstate(invalid="ignore"):
+        assert O.router_tail(bad, 2)[1].tolist() == [[0, 1], [0, 1]]
+    assert CO.router(bad, np.eye(4, dtype=np.float32), None, 2)[2].tolist() == [[0, 1], [0, 1]]
+
+
 def test_capacity_slots_vs_literal_loop_and_invariants():
     r = rng(12)
     for (T, k, E, cap) in [(50, 2, 4, 10), (64, 8, 64, 3), (31, 1, 3, 100), (40, 2, 4, 0)]:

@@ -101,17 +101,30 @@ def test_router_tail_invariants(lg, k, shift):
     assert np.allclose(probs.sum(1), 1.0, atol=1e-5)
     assert np.allclose(w.sum(1), 1.0, atol=1e-5)
     assert all(len(set(r)) == k for r in idx)
-    assert (np.diff(np.take_along_axis(lg, idx, 1), axis=1) <= 0).all()      # descending logits
-    # the C twin agrees
+    sel = np.take_along_axis(probs, idx, 1)
+    assert (np.diff(sel, axis=1) <= 0).all()                                  # descending probabilities
+    rest = probs.copy()
+    np.put_along_axis(rest, idx.astype(np.int64), -1.0, 1)
+    assert (rest.max(1) <= sel[:, -1]).all()                                  # nothing larger was left out
+    assert (np.diff(np.take_along_axis(lg, idx, 1), axis=1) <= 0).all() or \
+        (np.diff(sel, axis=1) == 0).any()                # logits descend too, except inside a run of equal probabilities
+    # the C twin: the stable top-k of ITS probabilities (libm's expf and numpy's exp may round
+    # differently), the same selection wherever numpy's probabilities are not within a rounding
     E = lg.shape[1]
-    _, _, i2, w2 = C.router(lg, np.eye(E, dtype=F32), None, k)     # identity gate: logits pass through
-    assert np.array_equal(i2, idx)
-    assert np.allclose(w2, w, atol=2e-6)
+    p2, _, i2, w2 = C.router(lg, np.eye(E, dtype=F32), None, k)    # identity gate: logits pass through
+    from util import assert_topk_of_probs
+    assert_topk_of_probs(i2, p2, k)
+    same = (i2 == idx).all(axis=1)
+    a = np.take_along_axis(probs, i2.astype(np.int64), 1)[~same]
+    assert (np.abs(a - sel[~same]) <= 4 * np.spacing(sel[~same])).all()
+    assert np.allclose(w2[same], w[same], atol=2e-6)
     # softmax is shift-invariant; a shift by a representable amount keeps the order
     lg2 = (lg.astype(np.float64) + np.float64(shift)).astype(F32)
     if np.array_equal((lg2.astype(np.float64) - np.float64(shift)).astype(F32), lg):
-        _, idx_s, _, _ = O.router_tail(lg2, k)
-        assert np.array_equal(idx_s, idx)
+        p_s, idx_s, _, _ = O.router_tail(lg2, k)
+        moved = (idx_s != idx).any(axis=1)               # only where probabilities sit within a rounding of each other
+        a = np.take_along_axis(probs, idx_s.astype(np.int64), 1)[moved]
+        assert (np.abs(a - sel[moved]) <= 4 * np.spacing(sel[moved])).all()
 
 
 @SET

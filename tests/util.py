@@ -48,3 +48,28 @@ def codes_np(pool_or_codes, scheme, D=None):
     if scheme in (O.Q_I4_ASYM, O.Q_I4_SYM):
         return O.unpack_int4(c.astype(np.uint8), signed=(scheme == O.Q_I4_SYM))
     return c.astype(np.int16)
+
+
+def assert_topk_of_probs(idx, probs, k, idx_ref=None, probs_ref=None, ulps=4):
+    """The routing contract: the selection is the stable top-k (value descending, lower
+    expert first among equal float32 values, NaN last) of the probabilities the same side
+    returned - on EVERY row.  Against a second implementation (idx_ref, probs_ref) rows may
+    differ only where exp() of the two sides can round differently: the reference's own
+    probabilities of the two choices are then within `ulps` units in the last place at every
+    rank, and such rows are rare."""
+    idx = np.asarray(idx)
+    probs = np.asarray(probs, dtype=np.float32)
+    own = O.topk_desc(probs, k)
+    assert np.array_equal(idx, own), f"{int((idx != own).any(axis=1).sum())} rows are not the top-k of their own probabilities"
+    if idx_ref is None:
+        return 0
+    idx_ref = np.asarray(idx_ref)
+    diff = (idx != idx_ref).any(axis=1)
+    n = int(diff.sum())
+    if n:
+        pr = np.asarray(probs_ref, dtype=np.float32)[diff]
+        a = np.take_along_axis(pr, idx[diff].astype(np.int64), 1)
+        b = np.take_along_axis(pr, idx_ref[diff].astype(np.int64), 1)
+        assert (np.abs(a - b) <= ulps * np.spacing(np.maximum(a, b))).all(), "selections differ beyond a rounding of exp()"
+        assert n <= max(2, len(idx) // 500), f"{n} near-tie rows of {len(idx)}"
+    return n
