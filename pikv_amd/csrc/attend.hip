@@ -1461,9 +1461,12 @@ static DecodeWs decode_ws(int n_caches, int n_q_heads, int head_dim, int64_t max
   w.n_tiles = (max_len + PIKV_SCORE_TILE - 1) / PIKV_SCORE_TILE;
   w.stride = w.n_tiles * PIKV_SCORE_TILE;
   w.scores = 0;  // float scores [cache][head][stride], or the exchange rows [cache][tile][head][64] (same size)
+  // (the two tile tables have room for one tile more than max_len holds: the one-pass form keeps a spare
+  // record per cache there, and its ranges' statistics - 8 bytes per head and range of at least 128 tokens -
+  // fit the second table)
   w.tmax = align256((int64_t)n_caches * n_q_heads * w.stride * 4);
-  w.tsum = w.tmax + align256((int64_t)n_caches * w.n_tiles * n_q_heads * 4);
-  w.stats = w.tsum + align256((int64_t)n_caches * w.n_tiles * n_q_heads * 4);
+  w.tsum = w.tmax + align256((int64_t)n_caches * (w.n_tiles + 1) * n_q_heads * 4);
+  w.stats = w.tsum + align256((int64_t)n_caches * (w.n_tiles + 1) * n_q_heads * 4);
   w.partial = w.stats + align256((int64_t)n_caches * n_q_heads * 2 * 4);
   w.total = w.partial + align256(pikv_attend_workspace_bytes(n_caches, n_q_heads, head_dim, max_len));
   return w;
@@ -1502,8 +1505,19 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
     return pikv_attend_values(reinterpret_cast<const float*>(out), nullptr, 0, v_codes, v_scale, v_zero, scheme, group,
                               n_kv_heads, n_q_heads, head_dim, cache_row_base, cache_fill, n_caches, 0, decay, now,
                               row_acc, row_ts, out, nullptr, 0, stream);
-  // fast form: the 4-bit matrix-core kernels meet in the exchange format
   const bool asym = scheme == PIKV_Q_I4_ASYM;
+  // one pass over K and V (no score matrix): 4-bit codes, heads of 128, up to 4 bf16 query heads per kv head.
+  // Its halves (n_q_heads * 128 bytes per tile and one spare tile per cache) lie where the float scores would
+  // (256 bytes per head and tile), the tiles' reference maxima in the tile-maximum table, the ranges' statistics
+  // in the tile-sum table.
+  if (decode_fused_serves(scheme, group, n_kv_heads, n_q_heads, head_dim, q_dtype, row_acc != nullptr) && (!asym || (k_zero && v_zero)) &&
+      n_caches <= 65535) {
+    const int tpb = fused_tokens_per_block(n_caches, n_kv_heads, max_len, attend_tokens_per_block(n_caches, max_len));
+    return decode_fused_launch(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, scheme, n_kv_heads, n_q_heads, q,
+                               scale_qk, cache_row_base, cache_fill, n_caches, max_len, tpb, decay, now, row_acc, row_ts,
+                               out, ws + w.scores, tmax, tsum, reinterpret_cast<float*>(partial), stats, st);
+  }
+  // the 4-bit matrix-core kernels meeting in the exchange format
   const int rep = n_q_heads % n_kv_heads == 0 ? n_q_heads / n_kv_heads : 0;
   const int hps = mfma_heads_per_slab(head_dim, n_kv_heads);   // 128-dimension slabs: one kv head, or 2 / 4 narrow ones
   const int slabs = hps > 0 ? n_kv_heads / hps : 0;
