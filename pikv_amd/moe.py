@@ -5,8 +5,15 @@ What stays in torch: the embedding, the dense experts (LoRAExpert,
 core/single/lora.py:31-52), the query/key projections and the vocabulary
 projection - dense GEMMs of the caller, not part of the cache data path.
 
+The router is the reference's routing_strategy.AdaptiveRouter (routing_strategy.py in this
+package: same parameter names, a reference state_dict loads), and the expert outputs are
+combined with its DENSE routing weights, as core/single/pikv_moe.py:281,312 does; on a model
+whose caches are empty the logits are the reference's up to the term its learned pyramid
+compressor adds for an all-zero cache (tests/test_gpu_moe_golden.py holds them to the output of
+the reference's own module).
+
 What runs natively, once per forward and for all experts together:
-  * the gate tail of the router (softmax, top-k, renormalise, capacity slots);
+  * every softmax + top-k + renormalise of the router, and the capacity slots of its top-k;
   * eviction of the rows that have to make room (LRU by default, H2O on request)
     and in-place compaction of every per-expert cache;
   * quantisation of the routed tokens' K/V rows and their scatter into the
@@ -34,7 +41,7 @@ import torch.nn.functional as F
 
 from . import ops
 from .config import config
-from .routing import TopKBalancedRouter
+from .routing_strategy import AdaptiveRouter
 from .scheduling import SchedulingPolicy
 
 _SCHEMES = {"int8": ops.Q_I8_SYM, "int8_asym": ops.Q_I8_ASYM, "int4": ops.Q_I4_ASYM,
@@ -113,14 +120,14 @@ class KVCache(nn.Module):
         k2 = key.reshape(-1, self.hidden_size).float().contiguous()
         v2 = value.reshape(-1, self.hidden_size).float().contiguous()
         pool = self._own_pool(k2.device)
-        if pool.n_caches != 1:
-            raise RuntimeError("caches of a PiKVMoE are updated together by the model's forward")
         n = k2.shape[0]
         dev = pool.device
-        n_new = torch.full((1,), min(n, self.size), dtype=torch.int32, device=dev)
+        # this cache takes n rows, the other caches of a shared pool none: they keep every row
+        n_new = torch.zeros(pool.n_caches, dtype=torch.int32, device=dev)
+        n_new[self.index] = min(n, self.size)
         _evict_for(pool, n_new, self._policy())
         self._time = max(self._time + 1, int(idx) + 1)
-        pool.quant_scatter(k2, v2, torch.zeros(n, dtype=torch.int32, device=dev),
+        pool.quant_scatter(k2, v2, torch.full((n,), self.index, dtype=torch.int32, device=dev),
                            torch.arange(n, dtype=torch.int32, device=dev), 1, now=float(self._time))
         pool.advance(n_new)
 
@@ -184,8 +191,7 @@ class PiKVMoE(nn.Module):
         H, E = config['hidden_size'], config['num_experts']
         self.embedding = nn.Embedding(config['vocab_size'], H)
         self.experts = nn.ModuleList([LoRAExpert(H, rank=rank, alpha=alpha) for _ in range(E)])
-        self.router = TopKBalancedRouter(H, E, top_k=config.get('top_k', 2),
-                                         capacity_factor=config.get('capacity_factor', 1.5))
+        self.router = AdaptiveRouter(hidden_size=H, num_experts=E, top_k=2, temperature=1.0)
         self.query_proj = nn.Linear(H, H)
         self.key_proj = nn.Linear(H, H)
         self.query_lora = LoRALayer(H, H, rank=rank, alpha=alpha)
@@ -231,9 +237,18 @@ class PiKVMoE(nn.Module):
         return torch.stack(means) / pool.fill.clamp_min(1).unsqueeze(1).float()
 
     def update_cache(self, expert_idx, key, value, importance):
-        """Single-expert update (core/single/pikv_moe.py:249-261); the forward pass
-        updates all experts together instead."""
-        raise RuntimeError("PiKVMoE.forward updates every expert's cache in one native call")
+        """Update one expert's cache with new key / value rows (core/single/pikv_moe.py:249-261).
+        The reference averages key and value over batch and sequence into ONE row and writes it at
+        the expert's ring pointer; here every given row ([n,H] or [B,S,H]) is quantised and appended,
+        the expert's policy (LRU, or H2O when scheduled so) evicting first when the cache is full.
+        `importance` has no part in either policy (the reference stores its mean and, with
+        scheduling, never reads it).  forward() updates all experts together instead."""
+        if not 0 <= int(expert_idx) < len(self.kv_caches):
+            raise IndexError(f"expert_idx {expert_idx} out of range")
+        self._ensure_pool(key.device)
+        self.clock += 1
+        self.kv_caches[int(expert_idx)].update(self.clock - 1, key, value, importance)
+        self.cache_ptrs = self.pool.fill.long()
 
     def forward(self, x, query=None, return_loss=False, targets=None, use_teacher=False):
         if x.dim() == 2:
@@ -246,15 +261,10 @@ class PiKVMoE(nn.Module):
         T, E = B * S, config['num_experts']
         pool = self._ensure_pool(x.device)
 
-        r, probs, lb_loss = self.router(x, return_compact=True)
-        k = r.topk_idx.shape[1]
-        routing_weights = torch.zeros(T, E, device=x.device)
-        routing_weights.scatter_(1, r.topk_idx.long(), r.topk_w)
-        routing_weights = routing_weights.view(B, S, E)
+        routing_weights, expert_indices, top_k_weights, lb_loss, importance = self.router(x)
+        k = expert_indices.shape[-1]
         if query is not None:
             importance = self.compute_token_importance(query.to(torch.float32), x)
-        else:
-            importance = probs.max(dim=-1).values
 
         cached = self._cached_means(pool)                              # [E, H]
         expert_output = torch.zeros(B, S, H, device=x.device)
@@ -271,28 +281,35 @@ class PiKVMoE(nn.Module):
             keys = (self.key_proj(x2) + self.key_lora(x2)).repeat_interleave(k, dim=0).contiguous()
             stacked = torch.stack([o.reshape(T, H) for o in outs])     # [E, T, H]
             tok = torch.arange(T, device=x.device).repeat_interleave(k)
-            values = stacked[r.topk_idx.reshape(-1).long(), tok].contiguous()
-            n_new = torch.minimum(torch.minimum(r.count, torch.full_like(r.count, r.capacity)), pool.cap)
+            # which token rows go to which expert's cache: the router's top-k, at most `capacity` per
+            # expert and forward in token order (core/single/pikv_routing.py:40-42,
+            # core/single/module/pikv_routing.py:93-104)
+            idx32 = expert_indices.reshape(T * k).to(torch.int32).contiguous()
+            capacity = int(B * S * config.get('capacity_factor', 1.5) * k / E)
+            slot, count = ops.capacity_slots(idx32, E, capacity)
+            values = stacked[idx32.long(), tok].contiguous()
+            n_new = torch.minimum(torch.minimum(count, torch.full_like(count, capacity)), pool.cap)
             policy = (ops.EVICT_H2O if self.use_cache_scheduling and
                       self.cache_scheduling_policy == SchedulingPolicy.H2O else ops.EVICT_LRU)
             _evict_for(pool, n_new, policy)
             self.clock += 1
             if self.debug_capture:
-                self.captured = dict(keys=keys, values=values, router=r, n_new=n_new,
-                                     cached=cached, fill_before=pool.fill.clone())
-            pool.quant_scatter(keys, values, r.topk_idx.reshape(-1), r.slot.reshape(-1), 1,
-                               now=float(self.clock))
-            pool.advance(r.count, r.capacity)
+                self.captured = dict(keys=keys, values=values, idx=idx32.view(T, k), slot=slot.view(T, k),
+                                     count=count, capacity=capacity, n_new=n_new, cached=cached,
+                                     fill_before=pool.fill.clone(), routing_weights=routing_weights,
+                                     top_k_weights=top_k_weights, importance=importance)
+            pool.quant_scatter(keys, values, idx32, slot, 1, now=float(self.clock))
+            pool.advance(count, capacity)
             self.cache_ptrs = pool.fill.long()
             if policy == ops.EVICT_H2O:
-                self._accumulate_h2o(pool, x2 if query is None else query.reshape(-1, H).float(), r)
+                self._accumulate_h2o(pool, x2 if query is None else query.reshape(-1, H).float())
 
         logits = self.vocab_proj(expert_output)
         if return_loss:
             return logits, lb_loss
         return logits
 
-    def _accumulate_h2o(self, pool, q_tokens, r):
+    def _accumulate_h2o(self, pool, q_tokens):
         """Scores of one query per expert (the mean projected query of the batch) over
         that expert's compressed cache feed the H2O accumulators."""
         H = config['hidden_size']
