@@ -33,23 +33,31 @@ METRIC = "routed KV tokens/s (quant+scatter+gather+dequant), 1 MI355X; % HBM pea
 HBM_PEAK_GBPS = 8000.0
 
 
-def profiled_traffic(kernel_prefix: str):
-    """HBM bytes per launch (fetched + written) of the roofline kernel as the rocprofv3 --pmc
-    runs recorded them: read from the machine-readable block at the end of profiles/prefill.md
-    (written by bench_profile.py, counters scaled by a streaming probe of known traffic in the
-    same run).  None when the summary is missing or has no such kernel."""
+def profiled_traffic(kernel_prefixes, summary="prefill.md"):
+    """HBM bytes per launch (fetched + written) of the named kernel(s), summed, as the rocprofv3
+    --pmc runs of the builder recorded them - NOT measured in this run: read from the
+    machine-readable block at the end of profiles/<summary> (written by bench_profile.py,
+    counters scaled by a streaming probe of known traffic in the same run).  None when the
+    summary is missing or lacks one of the kernels."""
     import re
+    if isinstance(kernel_prefixes, str):
+        kernel_prefixes = [kernel_prefixes]
     try:
-        text = open(os.path.join(ROOT, "profiles", "prefill.md")).read()
+        text = open(os.path.join(ROOT, "profiles", summary)).read()
         blob = json.loads(re.search(r"<!-- machine-readable: (.*) -->", text).group(1))
     except (OSError, AttributeError, ValueError):
         return None
-    best = None
-    for name, rec in blob.get("kernels", {}).items():
-        if name.startswith(kernel_prefix) and rec.get("fetch_bytes") is not None and rec.get("write_bytes") is not None:
-            if best is None or rec["calls"] > best["calls"]:
-                best = rec
-    return None if best is None else float(best["fetch_bytes"] + best["write_bytes"])
+    total = 0.0
+    for prefix in kernel_prefixes:
+        best = None
+        for name, rec in blob.get("kernels", {}).items():
+            if name.startswith(prefix) and rec.get("fetch_bytes") is not None and rec.get("write_bytes") is not None:
+                if best is None or rec["calls"] > best["calls"]:
+                    best = rec
+        if best is None:
+            return None
+        total += float(best["fetch_bytes"] + best["write_bytes"])
+    return total
 
 WORKLOAD = dict(name="prefill compress-write", batch=16, seq=2048, hidden=4096, experts=8, top_k=2,
                 capacity_factor=1.25, heads=32, head_dim=128, cache_slots=8192,
@@ -136,27 +144,34 @@ def _median_ms(torch, fn, iters, warm=3, setup=None):
     return ts[len(ts) // 2]
 
 
-def _entry(ms, nbytes, **extra):
+def _entry(ms, nbytes, traffic_bytes=None, **extra):
+    """nbytes: the ALGORITHMIC bytes of the step (what the cache format and the step's inputs and
+    outputs make unavoidable) - `GBps` and `hbm_frac` are on those alone.  traffic_bytes: what the
+    implementation moves on top of them or instead (score matrices, exchange rows, re-reads),
+    algorithmic bytes included; reported beside, never counted into hbm_frac."""
     d = {"ms": ms, "algorithmic_bytes": nbytes, "GBps": nbytes / (ms * 1e-3) / 1e9,
          "hbm_frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    if traffic_bytes is not None:
+        d["traffic_bytes"] = traffic_bytes
+        d["traffic_GBps"] = traffic_bytes / (ms * 1e-3) / 1e9
     d.update(extra)
     return d
 
 
 def hbm_ceiling(torch, dev, iters, nbytes=2 << 30):
     """Practical HBM rates of this machine with the library's own access pattern (16 bytes per
-    lane, 1 KiB per wavefront, 8 accesses in flight per lane): read only, write only, copy;
+    lane, 1 KiB per wavefront, 8 accesses in flight per lane; bench_probe.hip, a library of its
+    own beside this file): read only, write only, copy;
     plain and non-temporal stores.  Median of `iters` launches over `nbytes` (2 GiB: eight times
     the last-level cache), HIP events on the launch stream."""
-    from pikv_amd import _native as N
+    import bench_probe
     src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
     dst = torch.empty_like(src)
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
 
     def run(mode, nt):
         st = torch.cuda.current_stream().cuda_stream
-        return lambda: N.call("pikv_stream_probe", mode, src.data_ptr(), dst.data_ptr(), nbytes, nt,
-                              sink.data_ptr(), st)
+        return lambda: bench_probe.stream_probe(mode, src.data_ptr(), dst.data_ptr(), nbytes, nt, sink.data_ptr(), st)
     gb = nbytes / 1e9
     ms = {name: _median_ms(torch, run(mode, nt), iters)
           for name, mode, nt in (("read", 0, 0), ("write", 1, 0), ("write_nt", 1, 1), ("copy", 2, 0), ("copy_nt", 2, 1))}
@@ -208,6 +223,7 @@ def decode_read_workload(torch, ops, dev, iters):
     # every step starts from caches of N - 1 rows: the reset is the bench's, not the step's
     t_step = _median_ms(torch, decode_step, iters, setup=lambda: pool.fill.fill_(N - 1))
     t_fused = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=2.0), iters)
+    t_fused_nb = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=2.0, accumulate=False), iters)
     t_att_acc = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats, accumulate=True, now=1.0), iters)
     pool.fill.fill_(N)
 
@@ -231,22 +247,42 @@ def decode_read_workload(torch, ops, dev, iters):
     t_evict = _median_ms(torch, evict, iters) - t_restore
     kept_rows = int(pool.fill.sum())
     rows = B * N
-    k_bytes = rows * (D // 2 + (D // 32) * 4)
+    k_bytes = rows * (D // 2 + (D // 32) * 4)          # codes + half scale / zero point of one of K, V
+    q_bytes = B * hq * dh * 2
+    acc_rw = rows * 8                                   # H2O accumulator read + written
+    # algorithmic bytes of a decode step: K (1.36 GB with queries and accumulators) / K + V (2.70 GB)
+    alg_k, alg_kv = k_bytes + q_bytes + acc_rw, 2 * k_bytes + q_bytes + acc_rw
+    score_bytes = rows * hq * 4                         # the float score matrix of the public three-step form
+    half_bytes = rows * hq * 2                          # the half-precision importance exchange of the one-pass form
     return {
         "workload": "decode read: 64 seq x 32768 cached tokens, 8 KV heads x 128 (32 q heads), int4 asym g32",
+        "algorithmic_bytes_K": alg_k, "algorithmic_bytes_KV": alg_kv,
         "quant_scatter_i4": _entry(t_write, chunk * N * (2 * (D * 2 + D // 2 + (D // 32) * 4) + 8),
                                    rows=chunk * N),
-        "gather_dequant_scores": _entry(t_scores, k_bytes, cached_tokens_per_s=rows / (t_scores * 1e-3),
-                                        bytes_with_score_store=k_bytes + rows * hq * 4),
-        "h2o_accumulate": _entry(t_h2o, rows * hq * 4 + rows * 12),
-        "attend_values": _entry(t_att, k_bytes + rows * hq * 4),
-        "attend_values_with_h2o": _entry(t_att_acc, k_bytes + rows * hq * 4 + rows * 12),
-        "decode_attend": _entry(t_fused, 2 * k_bytes + 2 * rows * hq * 4 + rows * 12,
-                                what="pikv_decode_attend: scores + softmax + attention output + H2O accumulate in one call"),
-        "decode_step": {"ms": t_step, "what": "append 1 token per sequence + pikv_decode_attend",
-                        "cached_tokens_per_s": rows / (t_step * 1e-3),
-                        "algorithmic_bytes": 2 * k_bytes + 2 * rows * hq * 4 + rows * 12,
-                        "GBps": (2 * k_bytes + 2 * rows * hq * 4 + rows * 12) / (t_step * 1e-3) / 1e9},
+        "gather_dequant_scores": _entry(t_scores, k_bytes + q_bytes, traffic_bytes=k_bytes + q_bytes + score_bytes,
+                                        cached_tokens_per_s=rows / (t_scores * 1e-3),
+                                        what="public float score matrix [cache, head, token] + tile statistics"),
+        "h2o_accumulate": _entry(t_h2o, acc_rw, traffic_bytes=score_bytes + acc_rw + rows * 4,
+                                 what="reads the float score matrix; only the accumulators are algorithmic"),
+        "attend_values": _entry(t_att, k_bytes, traffic_bytes=k_bytes + score_bytes),
+        "attend_values_with_h2o": _entry(t_att_acc, k_bytes + acc_rw, traffic_bytes=k_bytes + score_bytes + acc_rw + rows * 4),
+        "decode_attend": _entry(t_fused, alg_kv, traffic_bytes=alg_kv + 2 * half_bytes + rows * 4,
+                                what="pikv_decode_attend: scores + softmax + attention output + H2O accumulate in "
+                                     "one call (one pass over K and V; halves written and read back for the importance)"),
+        "decode_attend_without_h2o": _entry(t_fused_nb, 2 * k_bytes + q_bytes,
+                                            what="pikv_decode_attend with row_acc = row_ts = NULL: attention output only"),
+        "decode_step": _entry(t_step, alg_kv, traffic_bytes=alg_kv + 2 * half_bytes + rows * 4,
+                              what="append 1 token per sequence + pikv_decode_attend",
+                              cached_tokens_per_s=rows / (t_step * 1e-3)),
+        "roofline": {"bound": "hbm", "kernel": "decode_fused_i4_kernel<I4_ASYM, bookkeeping> + decode_finish_kernel + "
+                                               "decode_importance_kernel (one pikv_decode_attend call)",
+                     "achieved": alg_kv / (t_fused * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": alg_kv / (t_fused * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": profiled_traffic(["decode_fused_i4_kernel<2, true>", "decode_finish_kernel",
+                                                  "decode_importance_kernel"], "decode_read.md"),
+                     "traffic_source": "profiles/decode_read.md (builder's rocprofv3 --pmc runs, not this run)",
+                     "algorithmic_bytes": alg_kv, "avg_launch_ms": t_fused,
+                     "note": "time of the whole call (three launches) by HIP events on its stream"},
         "evict_select": _entry(t_sel, rows * 8 + rows * 5),
         "evict_select_plus_compact": {"ms": t_evict, "kept_rows": kept_rows,
                                       "moved_bytes": 2 * kept_rows * (2 * (D // 2 + (D // 32) * 4) + 8)},
@@ -275,12 +311,17 @@ def decode_read_int8_workload(torch, ops, dev, iters):
     sc, tm, tsu = pool.scores(q, hq)
     pool.h2o_accumulate(sc, tm, tsu, now=1.0, stats_only=True)
     t_att = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats, accumulate=True, now=1.0), iters)
+    t_call = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=2.0), iters)
     rows = B * N
     k_bytes = rows * (D + hkv * 4)
     return {
         "workload": "decode read, int8 per token per head: 64 seq x 32768 cached tokens, 8 KV heads x 128 (64 q heads)",
-        "gather_dequant_scores": _entry(t_scores, k_bytes, bytes_with_score_store=k_bytes + rows * hq * 4),
-        "attend_values_with_h2o": _entry(t_att, k_bytes + rows * hq * 4 + rows * 12),
+        "gather_dequant_scores": _entry(t_scores, k_bytes + B * hq * dh * 2,
+                                        traffic_bytes=k_bytes + B * hq * dh * 2 + rows * hq * 4),
+        "attend_values_with_h2o": _entry(t_att, k_bytes + rows * 8, traffic_bytes=k_bytes + rows * hq * 4 + rows * 12),
+        "decode_attend": _entry(t_call, 2 * k_bytes + B * hq * dh * 2 + rows * 8,
+                                traffic_bytes=2 * k_bytes + 2 * rows * hq * 4 + rows * 12,
+                                what="pikv_decode_attend: the three public steps inside one call for this format"),
     }
 
 
@@ -422,14 +463,14 @@ def main():
     if args.calibrate_copy:
         # five launches each of the read, write and copy probes over 1 GiB: kernels of exactly
         # known traffic for scaling FETCH_SIZE / WRITE_SIZE, and the ceilings as a JSON line
-        from pikv_amd import _native as N
+        import bench_probe
         n = 1 << 30
         src = torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
         st = torch.cuda.current_stream().cuda_stream
         for mode in (0, 1, 2):
             for _ in range(5):
-                N.call("pikv_stream_probe", mode, src.data_ptr(), dst.data_ptr(), n, 0, None, st)
+                bench_probe.stream_probe(mode, src.data_ptr(), dst.data_ptr(), n, 0, None, st)
         torch.cuda.synchronize()
         del src, dst
         print(json.dumps({"calibrate_bytes_per_launch": n,
@@ -495,6 +536,11 @@ def main():
         return sum(ev[a].elapsed_time(ev[b]) for ev in events) / len(events)
 
     t_router, t_scores, t_h2o = avg(0, 1), avg(2, 3), avg(3, 4)
+    # the plain gather + dequantise of the metric's name (pikv_gather_dequant): every K row the step cached,
+    # to float32 and to bf16
+    n_rows = pool.rows
+    t_gd32 = _median_ms(torch, lambda: pool.gather_dequant("k"), max(5, min(args.steps, 20)))
+    t_gd16 = _median_ms(torch, lambda: pool.gather_dequant("k", out_dtype=torch.bfloat16), max(5, min(args.steps, 20)))
     A = T * k
     # algorithmic bytes of one launch
     b_quant = T * 2 * D * 2 + kept * (2 * D + 2 * heads * 4) + A * 8
@@ -514,6 +560,7 @@ def main():
                      "achieved": gbps(b_quant, t_quant), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": gbps(b_quant, t_quant) / HBM_PEAK_GBPS,
                      "traffic": profiled_traffic("quant_scatter_kernel<0, 1, 2, true>"),
+                     "traffic_source": "profiles/prefill.md (builder's rocprofv3 --pmc runs, not this run)",
                      "algorithmic_bytes": b_quant, "avg_launch_ms": t_quant},
         "kernels": {
             "router": {"ms": t_router, "GBps": gbps(b_router, t_router)},
@@ -522,6 +569,11 @@ def main():
             "scores": {"ms": t_scores, "GBps": gbps(b_scores, t_scores),
                        "cached_token_reads_per_s": kept / (t_scores * 1e-3)},
             "h2o_accumulate": {"ms": t_h2o, "GBps": gbps(b_h2o, t_h2o)},
+            "gather_dequant_f32": _entry(t_gd32, n_rows * (D + heads * 4) + n_rows * D * 4, rows=n_rows,
+                                         cached_tokens_per_s=n_rows / (t_gd32 * 1e-3),
+                                         what="pikv_gather_dequant over all 65536 slots of the 8 caches, K plane -> float32"),
+            "gather_dequant_bf16": _entry(t_gd16, n_rows * (D + heads * 4) + n_rows * D * 2, rows=n_rows,
+                                          cached_tokens_per_s=n_rows / (t_gd16 * 1e-3)),
         },
     }
     out["hbm_ceiling"] = ceiling

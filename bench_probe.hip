@@ -1,11 +1,19 @@
-// Streaming probes with the access pattern every kernel of this library uses for its bulk
-// data: 16 bytes per lane, 1 KiB contiguous per wavefront, several accesses in flight per
-// lane.  They put the practical HBM rates of the machine at hand (read only, write only,
-// read + write) on record next to the kernels' own figures, and give profiler counters a
-// launch of exactly known traffic to be scaled by.  Not part of the data path.
-#include "common.hpp"
+// Streaming probes for bench.py / bench_profile.py (libbench_probe.so; NOT part of libpikv_hip.so
+// and not declared in include/pikv_hip.h): the access pattern every kernel of the library uses for
+// its bulk data - 16 bytes per lane, 1 KiB contiguous per wavefront, several accesses in flight per
+// lane - over a plain buffer.  They put the practical HBM rates of the machine at hand (read only,
+// write only, read + write) on record next to the kernels' own figures, and give profiler counters a
+// launch of exactly known traffic to be scaled by.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
 namespace pikv {
+
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void st16_stream(void* p, uint4 v) {
+  probe_u32x4 t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<probe_u32x4*>(p));
+}
 
 constexpr int kProbeUnroll = 8;                              // 16-byte accesses in flight per lane
 constexpr int64_t kProbeBlockBytes = 256 * 16 * kProbeUnroll;  // 32 KiB per block
@@ -45,15 +53,16 @@ __global__ __launch_bounds__(256) void stream_probe_kernel(const uint4* __restri
 
 using namespace pikv;
 
-extern "C" int pikv_stream_probe(int mode, const void* src, void* dst, int64_t bytes, int streaming_stores,
+// 0 on success, negative on a bad argument or a refused launch.
+extern "C" int bench_stream_probe(int mode, const void* src, void* dst, int64_t bytes, int streaming_stores,
                                  void* sink, void* stream) {
-  if (mode < 0 || mode > 2) return PIKV_ERR_UNSUPPORTED;
-  if ((mode != 1 && !src) || (mode != 0 && !dst)) return PIKV_ERR_NULL;
-  if (bytes < 0 || bytes % 16 != 0) return PIKV_ERR_SHAPE;
-  if ((reinterpret_cast<uintptr_t>(src) & 15) || (reinterpret_cast<uintptr_t>(dst) & 15)) return PIKV_ERR_SHAPE;
-  if (bytes == 0) return PIKV_OK;
+  if (mode < 0 || mode > 2) return -3;
+  if ((mode != 1 && !src) || (mode != 0 && !dst)) return -1;
+  if (bytes < 0 || bytes % 16 != 0) return -2;
+  if ((reinterpret_cast<uintptr_t>(src) & 15) || (reinterpret_cast<uintptr_t>(dst) & 15)) return -2;
+  if (bytes == 0) return 0;
   const int64_t blocks = (bytes + kProbeBlockBytes - 1) / kProbeBlockBytes;
-  if (blocks > 0x7fffffffLL) return PIKV_ERR_SHAPE;
+  if (blocks > 0x7fffffffLL) return -2;
   const int64_t n16 = bytes / 16;
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid((unsigned)blocks);
@@ -65,6 +74,6 @@ extern "C" int pikv_stream_probe(int mode, const void* src, void* dst, int64_t b
   else if (mode == 1) hipLaunchKernelGGL((stream_probe_kernel<1, false>), grid, dim3(256), 0, st, s, d, n16, sk);
   else if (streaming_stores) hipLaunchKernelGGL((stream_probe_kernel<2, true>), grid, dim3(256), 0, st, s, d, n16, sk);
   else hipLaunchKernelGGL((stream_probe_kernel<2, false>), grid, dim3(256), 0, st, s, d, n16, sk);
-  PIKV_CHECK_LAUNCH();
-  return PIKV_OK;
+  if (hipGetLastError() != hipSuccess) return -5;
+  return 0;
 }

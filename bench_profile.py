@@ -11,7 +11,7 @@ each as a process of its own with the program directly after `--`:
     rocprofv3 --pmc FETCH_SIZE --output-format csv -d <dir>/fetch -o p -- python3 bench.py --workload <w> --no-cpu-baseline --steps 5 --warmup 2
     rocprofv3 --pmc WRITE_SIZE --output-format csv -d <dir>/write -o p -- python3 bench.py --workload <w> --no-cpu-baseline --steps 5 --warmup 2
 
-Every run also executes the streaming probes of `bench.py` (pikv_stream_probe: kernels that read,
+Every run also executes the streaming probes of `bench.py` (bench_probe.hip: kernels that read,
 write or copy exactly 2 GiB), so each counter is scaled inside its own run by what it reads for a
 launch of known traffic.  Rows are keyed by (kernel, grid size): launches of one kernel at
 different sizes are never averaged together.  The summary goes to profiles/<workload>.md and ends

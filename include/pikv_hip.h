@@ -497,20 +497,6 @@ int pikv_fakequant_preset(const float* x, int64_t N, int H, int group,
                           void* workspace, int64_t workspace_bytes,
                           void* stream);
 
-/* ------------------------------------------------------------------------
- * Streaming probe: the library's bulk access pattern (16 bytes per lane, 1 KiB
- * per wavefront, 8 accesses in flight per lane) over a plain buffer, to put the
- * practical HBM rates of the machine on record beside the kernels' figures and
- * to give profiler counters a launch of exactly known traffic.
- * No counterpart in the reference.
- *   mode 0: read `bytes` of src (nothing is written); sink (4 bytes, may be NULL)
- *           is the pro-forma destination of the running checksum
- *   mode 1: write `bytes` of dst      mode 2: copy src to dst
- *   streaming_stores != 0: non-temporal stores, as the code planes are written.
- *   bytes % 16 == 0, pointers 16-byte aligned. */
-int pikv_stream_probe(int mode, const void* src, void* dst, int64_t bytes,
-                      int streaming_stores, void* sink, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

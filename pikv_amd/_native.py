@@ -60,7 +60,6 @@ SIGNATURES = {
     "pikv_evict_workspace_bytes": (_l, [_i, _l]),
     "pikv_h2o_budget": (_i, [_p, _i, _d, _d, _p, _p, _p]),
     "pikv_compact_rows": (_i, [C.POINTER(_p), C.POINTER(_l), _i, _p, _p, _p, _p, _i, _p]),
-    "pikv_stream_probe": (_i, [_i, _p, _p, _l, _i, _p, _p]),
     "pikv_fakequant_colblocks": (_i, [_p, _l, _i, _i, _i, _i, _p, _p, _p, _p, _l, _p]),
     "pikv_fakequant_workspace_bytes": (_l, [_l, _i, _i]),
     "pikv_fakequant_preset": (_i, [_p, _l, _i, _i, _i, _i, _p, _p, _p, _p, _l, _p]),

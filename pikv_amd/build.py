@@ -18,7 +18,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libpikv_hip.so")
 
 SOURCES = ["status.hip", "quant_scatter.hip", "router.hip", "read_path.hip", "attend.hip", "decode_fused.hip",
-           "evict.hip", "fakequant.hip", "minshift.hip", "stream_probe.hip"]
+           "evict.hip", "fakequant.hip", "minshift.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

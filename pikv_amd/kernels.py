@@ -10,8 +10,13 @@ order and return tuples, dispatching into libpikv_hip.so.
       clamped to 0..255, dq = q*s+min, :215-232) in pikv_quant8_minshift; meta holds
       k_scale, k_min, v_scale, v_min as [N,1] like the reference, plus the uint8
       codes (k_codes, v_codes), which the reference computes and throws away.
-      NONE returns the inputs; LORA and MASK are dense/elementwise torch and not
-      part of the native path.
+      NONE returns the inputs.  LORA (K + (K A) B * rank/hidden, :185-204) and MASK
+      (entries below 0.1 x the row's mean magnitude set to zero, :248-275) are a dense
+      product and an elementwise pass, done by torch on the GPU as the reference's own
+      fallback does them - no kernel of this library is involved; they exist so that a
+      caller of the facade finds every mode.  (The reference's LORA fallback multiplies
+      by B through F.linear, which only accepts B as [hidden, rank]; both that layout and
+      the [rank, hidden] one its own default allocates are taken here.)
   evict_cache(keys, values, timestamps, usage, now, policy, window, thr)
       -> (keys, values, timestamps, usage, new_size)                   :289-422
       SLIDING keeps rows with now - ts <= window; QUEST keeps rows with
@@ -63,10 +68,37 @@ class PiKVKernels:
         mode = CompressionMode(compression_mode)
         if mode == CompressionMode.NONE:
             return keys, values, {"compression_type": "none"}
-        if mode != CompressionMode.QUANT8:
-            raise NotImplementedError(f"{mode.name}: only NONE and QUANT8 run on the native path")
         if keys.dim() != 2 or values.shape != keys.shape:
             raise ValueError("keys and values must be [batch, hidden] of one shape")
+        if keys.device.type != "cuda":
+            raise ValueError("compress_kv needs GPU tensors; there is no CPU path")
+        hidden = keys.shape[1]
+        if mode == CompressionMode.LORA:
+            rank = max(int(hidden * 0.1), 1)
+            if lora_params is None:      # the reference's default: random A, zero B - the identity
+                a_k = torch.randn(hidden, rank, device=keys.device) * 0.1
+                a_v = torch.randn(hidden, rank, device=keys.device) * 0.1
+                b_k = torch.zeros(rank, hidden, device=keys.device)
+                b_v = torch.zeros(rank, hidden, device=keys.device)
+            else:
+                a_k, b_k = lora_params.get('lora_a_k'), lora_params.get('lora_b_k')
+                a_v, b_v = lora_params.get('lora_a_v'), lora_params.get('lora_b_v')
+                rank = a_k.shape[1]
+
+            def adapt(x, a, b):
+                if b.shape == (hidden, rank) and hidden != rank:
+                    b = b.t()
+                return x + ((x.float() @ a.float()) @ b.float()).to(x.dtype) * (rank / hidden)
+            return adapt(keys, a_k, b_k), adapt(values, a_v, b_v), {
+                "compression_type": "lora", "lora_rank": rank, "lora_ratio": rank / hidden}
+        if mode == CompressionMode.MASK:
+            threshold = 0.1
+            k_mask = keys.abs() >= threshold * keys.abs().mean(dim=1, keepdim=True)
+            v_mask = values.abs() >= threshold * values.abs().mean(dim=1, keepdim=True)
+            return keys * k_mask.to(keys.dtype), values * v_mask.to(values.dtype), {
+                "compression_type": "mask", "threshold": threshold,
+                "k_sparsity": 1.0 - k_mask.float().mean().item(),
+                "v_sparsity": 1.0 - v_mask.float().mean().item()}
         ck, kc, ks, kmin = ops.quant8_minshift(keys)
         cv, vc, vs, vmin = ops.quant8_minshift(values)
         meta = {"compression_type": "quant8", "k_scale": ks, "k_min": kmin, "v_scale": vs, "v_min": vmin,

@@ -32,7 +32,7 @@ def test_header_declares_expected_surface():
                  "pikv_router_fused_workspace_bytes", "pikv_quant_gather", "pikv_attend_values",
                  "pikv_attend_workspace_bytes", "pikv_evict_workspace_bytes",
                  "pikv_decode_attend", "pikv_decode_attend_workspace_bytes", "pikv_quant8_minshift",
-                 "pikv_capacity_slots_static", "pikv_capacity_slots_static_max", "pikv_stream_probe",
+                 "pikv_capacity_slots_static", "pikv_capacity_slots_static_max",
                  "pikv_status_string", "pikv_abi_version"]:
         assert need in d
 

@@ -362,8 +362,23 @@ def test_kernels_facade(dev):
     assert out[4] == m and out[0].data_ptr() == tens[0].data_ptr()
     assert np.array_equal(np_of(tens[0][:m]), keys[valid]) and np.array_equal(np_of(tens[1][:m]), vals[valid])
     assert np.array_equal(np_of(tens[2][:m]), ts[valid]) and np.array_equal(np_of(tens[3][:m]), use[valid])
-    with pytest.raises(NotImplementedError):
-        K.compress_kv(torch.zeros(4, 64, device=dev), torch.zeros(4, 64, device=dev), CompressionMode.LORA)
+    # LORA and MASK (core/single/pikv_kernels.py:185-204, 248-275): hand-checkable cases
+    kk = torch.tensor([[1.0, -2.0, 0.05, 4.0], [0.0, 0.0, 0.0, 3.0]], device=dev)
+    a = torch.tensor([[1.0], [0.0], [0.0], [1.0]], device=dev)            # rank 1: K A = k0 + k3
+    b = torch.tensor([[0.0, 1.0, 0.0, 2.0]], device=dev)
+    ck, cv, meta = K.compress_kv(kk, kk * 2, CompressionMode.LORA,
+                                 dict(lora_a_k=a, lora_b_k=b, lora_a_v=a, lora_b_v=b.t().contiguous()))
+    assert meta == {"compression_type": "lora", "lora_rank": 1, "lora_ratio": 0.25}
+    assert ck.tolist() == [[1.0, -2.0 + 5 * 0.25, 0.05, 4.0 + 10 * 0.25], [0.0, 3 * 0.25, 0.0, 3.0 + 6 * 0.25]]
+    assert torch.equal(cv, 2 * ck)                                         # B given as [hidden, rank] for the values
+    ck, cv, meta = K.compress_kv(kk, kk, CompressionMode.LORA)             # default: zero B, the identity
+    assert torch.equal(ck, kk) and meta["lora_rank"] == 1
+    ck, cv, meta = K.compress_kv(kk, -kk, CompressionMode.MASK)
+    # row 0: mean |k| = 1.7625, threshold 0.17625 -> 0.05 goes; row 1: mean 0.75 -> the zeros stay zero
+    assert ck.tolist() == [[1.0, -2.0, 0.0, 4.0], [0.0, 0.0, 0.0, 3.0]] and torch.equal(cv, -ck)
+    assert meta["compression_type"] == "mask" and abs(meta["k_sparsity"] - 0.5) < 1e-6
+    with pytest.raises(ValueError):
+        K.compress_kv(torch.zeros(4, 64), torch.zeros(4, 64), CompressionMode.MASK)
 
 
 @pytest.mark.parametrize("trim", [True, False])
