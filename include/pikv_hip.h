@@ -112,6 +112,12 @@ int pikv_abi_version(void);
  *                 with the same expert; -1 when that count >= capacity
  *   count[e]    = number of assignments to e (kept or not)
  *
+ *   The float32 summation order of the projection depends on T (short, medium and long
+ *   token streams take different kernels) and on the token's position in the batch (a
+ *   block starts its walk along H at a block-dependent offset): the same token row gives
+ *   logits that agree to within 1e-5 * sqrt(H) of the exact value, not bit for bit, and a
+ *   near-tie can resolve differently.  For one (T, position) the result is deterministic.
+ *
  *   x        [T,H]  x_dtype (PIKV_F32|PIKV_BF16)   w [E,H] same dtype
  *   bias     [E] float or NULL        expert_scale, expert_mask [E] float|NULL
  *   probs    [T,E] float or NULL      logits_out [T,E] float or NULL
@@ -176,7 +182,12 @@ int pikv_capacity_slots(const int32_t* expert_idx, int64_t A, int E,
  *   a larger A returns PIKV_ERR_WORKSPACE and enqueues nothing.
  *   All calls on one GPU share the array: calls that overlap on one GPU (two
  *   streams, two threads) race; calls on one stream are ordered and safe.
- *   The device that is current at the call must be the one that owns the pointers. */
+ *   The device that is current at the call must be the one that owns the pointers.
+ *   Set-up: the first use on a device looks up the array's address there, which can
+ *   make the HIP runtime load the library's code object - not something to do inside an
+ *   open graph capture.  pikv_capacity_slots_static_max() performs that look-up for the
+ *   current device (and returns the limit): call it, or make one eager call, on every
+ *   device before capturing. */
 int pikv_capacity_slots_static(const int32_t* expert_idx, int64_t A, int E,
                                int64_t capacity, int32_t* slot, int32_t* count,
                                void* stream);

@@ -26,6 +26,7 @@ cache objects (transformers' DynamicCache); `past_key_values` returns the Huggin
 from __future__ import annotations
 
 import math
+import warnings
 from typing import Optional, Tuple
 
 import torch
@@ -69,7 +70,7 @@ class PiKVAttention(nn.Module):
                  max_position_embeddings: int = 2048, cache_size: int = 4096, *,
                  num_kv_heads: Optional[int] = None, kv_quant: str = "int4", kv_group: int = 32,
                  heavy_ratio: float = 0.0625, recent_ratio: float = 0.0078125,
-                 on_overflow: str = "h2o", layer_idx: int = 0, past_layout: str = "hf"):
+                 on_overflow: str = "h2o", layer_idx: int = 0, past_layout: str = "reference"):
         super().__init__()
         self.hidden_size = hidden_size
         self.num_heads = num_heads
@@ -178,7 +179,11 @@ class PiKVAttention(nn.Module):
         ref = t.shape[2] == self.num_kv_heads         # [B, S, kv_heads, head_dim]
         if layout == "auto":
             if hf and ref:
-                layout = self.past_layout             # S == kv_heads: the shape cannot tell
+                # S == kv_heads: the shape cannot tell.  past_layout decides - it is also the layout
+                # forward() returns `present` in, so the module's own output always reads back right
+                warnings.warn(f"{name} {tuple(t.shape)} fits both layouts; read as '{self.past_layout}' "
+                              "(the module's past_layout) - pass layout= to say which", stacklevel=3)
+                layout = self.past_layout
             elif hf or ref:
                 layout = "hf" if hf else "reference"
             else:
@@ -318,5 +323,9 @@ class PiKVAttention(nn.Module):
                 self._update_cache(k.detach(), v.detach())
             context = self._dense_attention(q, k, v, attention_mask, causal_mask, past)
         output = self.o_proj(context.reshape(B, S, self.num_heads * self.head_dim).to(hidden_states.dtype))
-        present = (k, v) if use_cache else None
+        # `present` in the module's past_layout: [B,S,kv_heads,head_dim] as the reference returns it
+        # (core/single/pikv_attention.py:240-247), or [B,kv_heads,S,head_dim] for past_layout="hf"
+        present = None
+        if use_cache:
+            present = (k, v) if self.past_layout == "reference" else (k.transpose(1, 2), v.transpose(1, 2))
         return output, present

@@ -1047,11 +1047,18 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
   }
 }
 
+// LDS of scores_mfma_i8_kernel: the staged score rows of every query head of the cache, for 4 or 2 tiles at
+// a time on rows of 1 or 2 slabs, plus the query sums.  (The kernel strides its staging areas by
+// n_q_heads * 64 floats, whatever part of the heads a launch serves.)
+static size_t i8_mfma_lds_bytes(int n_slabs, int n_q_heads) {
+  return (size_t)n_q_heads * kTile * sizeof(float) * (n_slabs <= 2 ? kI8TilesPerBlock / n_slabs : 1) +
+         kI8QsFloats * sizeof(float);
+}
+constexpr size_t kI8MfmaMaxLds = 64 * 1024;   // beyond it the vector form serves the cache (one block per compute unit otherwise)
+
 template <int SCHEME, int HPS, bool QF32>
 static void launch_i8_mfma_q(const ScoreArgs& a, int n_caches, int64_t n_tiles, hipStream_t st) {
-  // rows of 1 or 2 slabs stage 4 or 2 tiles at a time
-  const size_t lds = (size_t)a.n_q_heads * kTile * sizeof(float) * (a.n_kv_heads <= 2 ? kI8TilesPerBlock / a.n_kv_heads : 1) +
-                     kI8QsFloats * sizeof(float);
+  const size_t lds = i8_mfma_lds_bytes(a.n_kv_heads, a.n_q_heads);
   const dim3 grid((unsigned)((n_tiles + kI8TilesPerBlock - 1) / kI8TilesPerBlock), (unsigned)n_caches);
   if (a.n_kv_heads <= 4)
     hipLaunchKernelGGL((scores_mfma_i8_kernel<SCHEME, 1, HPS, QF32>), grid, dim3(256), lds, st, a);
@@ -1483,7 +1490,8 @@ extern "C" int pikv_gather_dequant_scores(const void* k_codes, const void* k_sca
   const bool qf32 = q_dtype == PIKV_F32;
   // (more than 16 bf16 query heads per kv head of 128 on rows of up to 4 kv heads: launches of 16 heads each)
   const bool many = hps == 1 && !qf32 && n_kv_heads <= 4 && rep > 16;
-  if (eight && hps > 0 && group % head_dim == 0 && rep >= 2 && (rep * hps <= (qf32 ? 8 : 16) || many) && n_kv_heads / hps <= 16) {
+  if (eight && hps > 0 && group % head_dim == 0 && rep >= 2 && (rep * hps <= (qf32 ? 8 : 16) || many) && n_kv_heads / hps <= 16 &&
+      i8_mfma_lds_bytes(n_kv_heads / hps, n_q_heads) <= kI8MfmaMaxLds) {
     ScoreArgs as = a;
     as.n_kv_heads = n_kv_heads / hps;
     const bool sym = scheme == PIKV_Q_I8_SYM;

@@ -1194,7 +1194,14 @@ static int scratch_of_current_device(int32_t** out) {
   return PIKV_OK;
 }
 
-extern "C" int64_t pikv_capacity_slots_static_max(void) { return kSlotStaticMaxAssignments; }
+// The limit of the static form - and its set-up call: asking for the limit also looks up the array's
+// address on the current device (which may make the runtime load the code object, a host-side step that
+// does not belong inside an open graph capture).  A caller that captures asks here first, per device.
+extern "C" int64_t pikv_capacity_slots_static_max(void) {
+  int32_t* p = nullptr;
+  (void)scratch_of_current_device(&p);   // no device current / no GPU: the limit is still the answer
+  return kSlotStaticMaxAssignments;
+}
 
 extern "C" int pikv_capacity_slots_static(const int32_t* expert_idx, int64_t A, int E, int64_t capacity,
                                           int32_t* slot, int32_t* count, void* stream) {

@@ -185,13 +185,17 @@ class BaseRouter(nn.Module):
         B, S, H = hidden_states.shape
         seq = self.router if seq is None else seq
         x2d = hidden_states.reshape(B * S, H)
-        with torch.no_grad():
+        # ONE pass through the gate's hidden layers (one dropout mask, if any is active): the kernel gets
+        # the activation's values, the torch tail - when gradients are wanted - continues from the same
+        # tensor, so values and gradients belong to the same function
+        grad = _wants_grad(hidden_states, *seq.parameters())
+        with torch.set_grad_enabled(grad):
             h = self._hidden_before_gate(seq, x2d)
         cap = self._compute_capacity(B, S)
-        r = _gate_tail(h, seq[-1], top_k=self.top_k, capacity=cap, expert_mask=expert_mask,
+        r = _gate_tail(h.detach(), seq[-1], top_k=self.top_k, capacity=cap, expert_mask=expert_mask,
                        **self._arith_kw(), **scale_kw)
-        if _wants_grad(hidden_states, *seq.parameters()):
-            r = _attach_grad(r, seq(x2d), expert_mask=expert_mask, **self._arith_kw(), **scale_kw)
+        if grad:
+            r = _attach_grad(r, seq[-1](h), expert_mask=expert_mask, **self._arith_kw(), **scale_kw)
         return r
 
     def _aux_loss(self, router_probs: torch.Tensor) -> torch.Tensor:
@@ -270,17 +274,19 @@ class EPLBRouter(BaseRouter):
         # /temperature, then *expert_weights, then mask: the order of :653-660
         seq = self.router
         x2d = hidden_states.reshape(B_S, -1)
-        with torch.no_grad():
+        # one pass through the hidden layers and their dropout: values (kernel) and gradients (torch tail)
+        # come from the same activation, drawn with one mask
+        grad = _wants_grad(hidden_states, *seq.parameters())
+        with torch.set_grad_enabled(grad):
             h = self._hidden_before_gate(seq, x2d)
         cap = self._compute_capacity(B, S)
-        r = ops.router_fused(h.contiguous(), seq[-1].weight.detach().to(h.dtype).contiguous(),
+        hv = h.detach()
+        r = ops.router_fused(hv.contiguous(), seq[-1].weight.detach().to(hv.dtype).contiguous(),
                              seq[-1].bias.detach().float(), top_k=self.top_k, capacity=cap,
                              expert_scale=self.expert_weights, expert_mask=expert_mask,
                              temperature=self.temperature, return_logits=True, **self._arith_kw())
-        if _wants_grad(hidden_states, *seq.parameters()):
-            # (dropout layers: the torch pass draws its own mask; in training the values are the
-            # kernel's for the eval-mode activations only when dropout is inactive)
-            r = _attach_grad(r, seq(x2d), temperature=self.temperature, expert_scale=self.expert_weights,
+        if grad:
+            r = _attach_grad(r, seq[-1](h), temperature=self.temperature, expert_scale=self.expert_weights,
                              expert_mask=expert_mask, **self._arith_kw())
         out, probs = self._finish(r, B, S, return_compact)
         aux = torch.zeros((), device=probs.device)
@@ -315,19 +321,20 @@ class AdaptiveRouter(BaseRouter):
     def _two_gate_route(self, hidden_states, importance, expert_mask, expert_scale=None):
         B, S, H = hidden_states.shape
         x2 = hidden_states.reshape(B * S, H)
-        with torch.no_grad():
-            la = self.router_important(x2).float().contiguous()
-            lb = self.router_unimportant(x2).float().contiguous()
+        grad = _wants_grad(hidden_states, expert_scale, *self.router_important.parameters(),
+                           *self.router_unimportant.parameters())
+        with torch.set_grad_enabled(grad):      # both gates run once; the kernel takes their values
+            la_t = self.router_important(x2).float()
+            lb_t = self.router_unimportant(x2).float()
+        la, lb = la_t.detach().contiguous(), lb_t.detach().contiguous()
         sel = (importance.reshape(-1) > self.imp_threshold)
         cap = self._compute_capacity(B, S)
         scale_v = None if expert_scale is None else expert_scale.detach()
         r = ops.router_tail(la, top_k=self.top_k, capacity=cap, logits_b=lb, select=sel,
                             expert_scale=scale_v, expert_mask=expert_mask, **self._arith_kw())
-        if _wants_grad(hidden_states, expert_scale, *self.router_important.parameters(),
-                       *self.router_unimportant.parameters()):
+        if grad:
             # the per-token choice between the two gates (core/single/pikv_routing.py:450-458)
-            lg = torch.where(sel.unsqueeze(1), self.router_important(x2).float(),
-                             self.router_unimportant(x2).float())
+            lg = torch.where(sel.unsqueeze(1), la_t, lb_t)
             r = _attach_grad(r, lg, expert_scale=expert_scale, expert_mask=expert_mask, **self._arith_kw())
         return r
 

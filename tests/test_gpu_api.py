@@ -363,18 +363,18 @@ def test_kernels_facade(dev):
     assert np.array_equal(np_of(tens[0][:m]), keys[valid]) and np.array_equal(np_of(tens[1][:m]), vals[valid])
     assert np.array_equal(np_of(tens[2][:m]), ts[valid]) and np.array_equal(np_of(tens[3][:m]), use[valid])
     # LORA and MASK (core/single/pikv_kernels.py:185-204, 248-275): hand-checkable cases
-    kk = torch.tensor([[1.0, -2.0, 0.05, 4.0], [0.0, 0.0, 0.0, 3.0]], device=dev)
+    kk = torch.tensor([[1.0, -2.0, 0.0625, 4.0], [0.0, 0.0, 0.0, 3.0]], device=dev)
     a = torch.tensor([[1.0], [0.0], [0.0], [1.0]], device=dev)            # rank 1: K A = k0 + k3
     b = torch.tensor([[0.0, 1.0, 0.0, 2.0]], device=dev)
     ck, cv, meta = K.compress_kv(kk, kk * 2, CompressionMode.LORA,
                                  dict(lora_a_k=a, lora_b_k=b, lora_a_v=a, lora_b_v=b.t().contiguous()))
     assert meta == {"compression_type": "lora", "lora_rank": 1, "lora_ratio": 0.25}
-    assert ck.tolist() == [[1.0, -2.0 + 5 * 0.25, 0.05, 4.0 + 10 * 0.25], [0.0, 3 * 0.25, 0.0, 3.0 + 6 * 0.25]]
+    assert ck.tolist() == [[1.0, -2.0 + 5 * 0.25, 0.0625, 4.0 + 10 * 0.25], [0.0, 3 * 0.25, 0.0, 3.0 + 6 * 0.25]]
     assert torch.equal(cv, 2 * ck)                                         # B given as [hidden, rank] for the values
     ck, cv, meta = K.compress_kv(kk, kk, CompressionMode.LORA)             # default: zero B, the identity
     assert torch.equal(ck, kk) and meta["lora_rank"] == 1
     ck, cv, meta = K.compress_kv(kk, -kk, CompressionMode.MASK)
-    # row 0: mean |k| = 1.7625, threshold 0.17625 -> 0.05 goes; row 1: mean 0.75 -> the zeros stay zero
+    # row 0: mean |k| = 1.765625, threshold 0.1765625 -> 0.0625 goes; row 1: mean 0.75 -> the zeros stay zero
     assert ck.tolist() == [[1.0, -2.0, 0.0, 4.0], [0.0, 0.0, 0.0, 3.0]] and torch.equal(cv, -ck)
     assert meta["compression_type"] == "mask" and abs(meta["k_sparsity"] - 0.5) < 1e-6
     with pytest.raises(ValueError):
@@ -501,3 +501,26 @@ def test_moe_load_balance_loss_backpropagates(dev):
     # (expert_capacity takes no part in the forward, here as in core/single/routing_strategy.py:22)
     g = [p.grad for n, p in model.router.named_parameters() if not n.endswith('expert_capacity')]
     assert all(t is not None for t in g) and any(float(t.abs().sum()) > 0 for t in g)
+
+
+def test_eplb_router_training_with_dropout_uses_one_mask(dev):
+    """EPLBRouter's gate has dropout layers (core/single/pikv_routing.py:596-610).  In training the
+    values of the native tail and the gradients of the torch tail must belong to ONE draw of the
+    dropout masks: the returned logits (kernel values) equal the torch tail applied to the very
+    activation that carries the gradient, which a second pass through the gate would not give."""
+    import torch
+    from pikv_amd.routing import EPLBRouter
+    torch.manual_seed(11)
+    r = EPLBRouter(64, 8, top_k=2).to(dev).train()
+    x = torch.randn(2, 40, 64, device=dev, requires_grad=True)
+    seen = {}
+    hook = r.router[-1].register_forward_hook(lambda m, inp, out: seen.setdefault("calls", []).append(out))
+    out, probs, aux = r(x, return_compact=True)
+    hook.remove()
+    assert len(seen["calls"]) == 1                       # the gate's last layer ran once, on the one activation
+    lg_t = seen["calls"][0].float() / r.temperature      # expert_weights are ones on the first call
+    assert torch.allclose(probs.reshape(-1, 8), torch.softmax(lg_t, -1), atol=2e-6)
+    (probs.square().sum() + out.topk_w.sum()).backward()
+    assert x.grad is not None and float(x.grad.abs().sum()) > 0
+    dropped = [m for m in r.router if isinstance(m, torch.nn.Dropout)]
+    assert dropped and all(m.p > 0 for m in dropped)

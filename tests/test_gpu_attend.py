@@ -223,6 +223,8 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I4_SYM, 32, 4, 20, 64, "bf16"),     # ... two slabs x 10
     (O.Q_I4_ASYM, 32, 1, 48, 128, "bf16"),   # multi-query: 48 q heads on one kv head
     (O.Q_I8_SYM, 128, 1, 48, 128, "bf16"),   # ... 8-bit
+    (O.Q_I8_SYM, 128, 1, 128, 128, "bf16"),  # ... 128 q heads on one 8-bit kv head: the staged rows exceed the matrix-core kernel's LDS, vector scores
+    (O.Q_I8_ASYM, 128, 2, 128, 128, "bf16"), # ... 2 kv x 64 q heads each, same limit
     (O.Q_I8_ASYM, 128, 2, 8, 128, "bf16"),   # 8-bit, 2 kv heads: four neighbouring rows as one row of eight slabs
     (O.Q_I8_ASYM, 128, 2, 20, 128, "bf16"),  # ... 10 q heads per kv head: the attention output in two launches
     (O.Q_I8_SYM, 128, 1, 4, 128, "f32"),     # ... 1 kv head: eight rows as one

@@ -214,13 +214,31 @@ def test_past_key_values_shape_is_checked(dev):
         att(torch.randn(3, 2, 128, device=dev))                                      # 3 sequences, 2 caches in use
     with pytest.raises(ValueError):
         att(torch.randn(2, 2, 128, device=dev), attention_mask=torch.ones(2, 7, device=dev))
-    # S == kv_heads: the shape cannot tell the layouts apart, past_layout decides
+    # S == kv_heads: the shape cannot tell the layouts apart, past_layout decides (with a warning)
     sq = torch.randn(1, 2, 2, 32, device=dev)
-    att.load_past_key_values((sq, sq))
+    att.load_past_key_values((sq, sq), layout="hf")
     k_hf, _ = att.past_key_values()
     att.load_past_key_values((sq, sq), layout="reference")
     k_ref, _ = att.past_key_values()
     assert torch.equal(k_hf.transpose(1, 2), k_ref)
+    with pytest.warns(UserWarning, match="fits both layouts"):
+        att.load_past_key_values((sq, sq))
+    k_auto, _ = att.past_key_values()
+    assert att.past_layout == "reference" and torch.equal(k_auto, k_ref)
+    # the module reads its own `present` back correctly in either layout, also when S == kv_heads
+    for lay in ("reference", "hf"):
+        a2 = PiKVAttention(128, 4, head_dim=32, dropout=0.0, cache_size=64, num_kv_heads=2, kv_quant="int8",
+                           kv_group=32, past_layout=lay).to(dev).eval()
+        x = torch.randn(1, 2, 128, device=dev)                                       # S = 2 = kv heads
+        with torch.no_grad():
+            _, present = a2(x, use_cache=True)
+        assert tuple(present[0].shape) == (1, 2, 2, 32)
+        want_k, _ = a2.past_key_values()
+        a2.reset_cache()
+        with pytest.warns(UserWarning):
+            a2.load_past_key_values(present)
+        got_k, _ = a2.past_key_values()
+        assert torch.equal(got_k, want_k), lay
 
 
 def test_hf_dynamic_cache_drives_the_adapter(dev):

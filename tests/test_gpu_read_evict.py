@@ -86,6 +86,8 @@ def _fill_pool(dev, r, caps, lens, heads, dh, group, scheme, dtype="bf16"):
     (O.Q_I4_ASYM, 32, 1, 48, 128),     # multi-query: 48 q heads on one kv head, six launches
     (O.Q_I4_SYM, 32, 2, 40, 64),       # ... 40 on one slab of two narrow heads
     (O.Q_I8_SYM, 128, 1, 48, 128),     # 8-bit multi-query: three launches of 16 heads
+    (O.Q_I8_SYM, 128, 1, 128, 128),    # ... 128 heads: beyond the matrix-core kernel's staging, the vector form
+    (O.Q_I8_ASYM, 128, 2, 122, 128),   # ... 2 kv x 61 q heads
     (O.Q_I8_ASYM, 128, 2, 40, 128),    # ... 20 per kv head: launches of 16 and 4
 ])
 @pytest.mark.parametrize("qdtype", ["f32", "bf16"])

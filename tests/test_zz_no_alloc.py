@@ -62,3 +62,43 @@ def test_static_slots_reject_oversize(dev):
     idx = r.integers(0, 64, size=limit).astype(np.int32)
     (s_ws, c_ws), (s_st, c_st) = _both(idx, 64, 1 << 14, dev)
     assert np.array_equal(s_st, s_ws) and np.array_equal(c_st, c_ws)
+
+
+def test_static_slots_allocate_nothing_and_replay_from_a_graph(dev):
+    """After the set-up call (pikv_capacity_slots_static_max on this device) the entry point leaves the
+    device's free memory untouched, and it can be captured into a HIP graph: every replay, with slot and
+    count scribbled over in between and eager work of the program around it, gives the eager result."""
+    lib = N.lib()
+    assert int(lib.pikv_capacity_slots_static_max()) == 1 << 20       # set-up: address looked up outside any capture
+    r = np.random.default_rng(23)
+    A, E, cap = 70_001, 24, 2500
+    idx_np = r.integers(0, E, size=A).astype(np.int32)
+    idx = torch.from_numpy(idx_np).to(dev)
+    slot = torch.empty(A, dtype=torch.int32, device=dev)
+    count = torch.empty(E, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info(dev)
+    st = torch.cuda.current_stream().cuda_stream
+    for _ in range(3):
+        assert lib.pikv_capacity_slots_static(idx.data_ptr(), A, E, cap, slot.data_ptr(), count.data_ptr(), st) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info(dev)
+    assert free1 == free0
+    s_ref, c_ref = O.capacity_slots(idx_np.reshape(-1, 1), E, cap)
+    assert np.array_equal(slot.cpu().numpy(), s_ref.reshape(-1)) and np.array_equal(count.cpu().numpy(), c_ref)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = lib.pikv_capacity_slots_static(idx.data_ptr(), A, E, cap, slot.data_ptr(), count.data_ptr(),
+                                                torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    for rep in range(3):
+        slot.fill_(-9 - rep)
+        count.fill_(-9 - rep)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(slot.cpu().numpy(), s_ref.reshape(-1)), rep
+        assert np.array_equal(count.cpu().numpy(), c_ref), rep
+        (idx.float().sum() + 1).item()                                    # eager work between the replays
