@@ -465,13 +465,13 @@ __global__ __launch_bounds__(256) void decode_finish_kernel(const float* __restr
 
 // H2O bookkeeping from the halves the fused pass left: one wavefront per tile of 64 cached tokens.
 //   acc[n] = acc[n] * decay + sum_h e[h,n] * exp(m_tile[h] - M[h]) / Z[h];  ts[n] = now
+// with (M, Z) of every head as decode_finish_kernel merged them into head_stats [cache][q head][2].
 __global__ __launch_bounds__(256) void decode_importance_kernel(const uint2* __restrict__ e16,
                                                                const float* __restrict__ tref,
-                                                               const float* __restrict__ pstats,
+                                                               const float* __restrict__ head_stats,
                                                                const int64_t* __restrict__ row_base,
                                                                const int32_t* __restrict__ fill, int64_t max_len,
-                                                               int64_t n_tiles, int n_caches, int n_kv_heads,
-                                                               int n_q_heads, int n_splits, int tokens_per_block,
+                                                               int64_t n_tiles, int n_kv_heads, int n_q_heads,
                                                                float decay, float now, float* __restrict__ row_acc,
                                                                float* __restrict__ row_ts) {
   const int lane = threadIdx.x & 63;
@@ -486,8 +486,11 @@ __global__ __launch_bounds__(256) void decode_importance_kernel(const uint2* __r
   const int64_t n = tile * kFTile + tok;
   const int64_t row = row_base[c] + n;
   float val = 0.f;
+  float acc0 = 0.f;
+  if (row_acc != nullptr && n < len) acc0 = row_acc[row];
   if (row_acc != nullptr) {
-    // the tile's halves are asked for first: nothing below depends on them until the statistics are merged
+    // everything the wavefront reads is asked for at once: the tile's halves, the heads' merged statistics
+    // (decode_finish_kernel left them in head_stats), the tile's reference maxima, the accumulators
     uint2 hv[8];
     const uint2* ep = e16 + ((int64_t)c * n_tiles + tile) * n_kv_heads * (rep * 16) + lane;
 #pragma unroll
@@ -497,17 +500,9 @@ __global__ __launch_bounds__(256) void decode_importance_kernel(const uint2* __r
     }
     float fac = 0.f;   // lane h: what turns a stored half of head h in this tile into a probability
     if (lane < n_q_heads) {
-      const int64_t used = (len + tokens_per_block - 1) / tokens_per_block;
-      const int lim = used < n_splits ? (int)used : n_splits;
-      float M = -__builtin_inff();
-      for (int sp = 0; sp < lim; ++sp) M = fmaxf(M, pstats[(((int64_t)sp * n_caches + c) * n_q_heads + lane) * 2]);
-      float Z = 0.f;
-      for (int sp = 0; sp < lim; ++sp) {
-        const int64_t pi = ((int64_t)sp * n_caches + c) * n_q_heads + lane;
-        Z = fmaf(pstats[pi * 2 + 1], __builtin_amdgcn_exp2f((pstats[pi * 2] - M) * kLog2e), Z);
-      }
+      const float2 mz = *reinterpret_cast<const float2*>(head_stats + ((int64_t)c * n_q_heads + lane) * 2);
       const float mt = tref[((int64_t)c * n_tiles + tile) * n_q_heads + lane];
-      fac = __builtin_amdgcn_exp2f((mt - M) * kLog2e) / (Z * kHalfScale);
+      fac = __builtin_amdgcn_exp2f((mt - mz.x) * kLog2e) / (mz.y * kHalfScale);
     }
     float imp[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -529,7 +524,7 @@ __global__ __launch_bounds__(256) void decode_importance_kernel(const uint2* __r
   }
   if (n < len) {
     if (row_acc != nullptr) {
-      float acc = row_acc[row];
+      float acc = acc0;
       if (decay != 1.0f) acc = acc * decay;
       row_acc[row] = acc + val;
     }
@@ -623,9 +618,8 @@ int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_
                      cache_fill, max_len, n_caches, n_q_heads, (int)splits, tokens_per_block, out, head_stats);
   if (book)
     hipLaunchKernelGGL(decode_importance_kernel, dim3((unsigned)((n_tiles + 3) / 4), (unsigned)n_caches), dim3(256), 0,
-                       st, reinterpret_cast<const uint2*>(e16), tref, pstats, cache_row_base, cache_fill, max_len,
-                       n_tiles, n_caches, n_kv_heads, n_q_heads, (int)splits, tokens_per_block, decay, now, row_acc,
-                       row_ts);
+                       st, reinterpret_cast<const uint2*>(e16), tref, head_stats, cache_row_base, cache_fill, max_len,
+                       n_tiles, n_kv_heads, n_q_heads, decay, now, row_acc, row_ts);
   PIKV_CHECK_LAUNCH();
   return PIKV_OK;
 }
