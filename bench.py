@@ -312,16 +312,23 @@ def decode_read_int8_workload(torch, ops, dev, iters):
     pool.h2o_accumulate(sc, tm, tsu, now=1.0, stats_only=True)
     t_att = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats, accumulate=True, now=1.0), iters)
     t_call = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=2.0), iters)
+    t_call_nb = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=2.0, accumulate=False), iters)
     rows = B * N
     k_bytes = rows * (D + hkv * 4)
+    q_bytes = B * hq * dh * 2
+    half_bytes = rows * hq * 2                          # the half-precision importance exchange of the one-pass form
     return {
         "workload": "decode read, int8 per token per head: 64 seq x 32768 cached tokens, 8 KV heads x 128 (64 q heads)",
-        "gather_dequant_scores": _entry(t_scores, k_bytes + B * hq * dh * 2,
-                                        traffic_bytes=k_bytes + B * hq * dh * 2 + rows * hq * 4),
+        "algorithmic_bytes_KV": 2 * k_bytes + q_bytes + rows * 8,
+        "gather_dequant_scores": _entry(t_scores, k_bytes + q_bytes,
+                                        traffic_bytes=k_bytes + q_bytes + rows * hq * 4),
         "attend_values_with_h2o": _entry(t_att, k_bytes + rows * 8, traffic_bytes=k_bytes + rows * hq * 4 + rows * 12),
-        "decode_attend": _entry(t_call, 2 * k_bytes + B * hq * dh * 2 + rows * 8,
-                                traffic_bytes=2 * k_bytes + 2 * rows * hq * 4 + rows * 12,
-                                what="pikv_decode_attend: the three public steps inside one call for this format"),
+        "decode_attend": _entry(t_call, 2 * k_bytes + q_bytes + rows * 8,
+                                traffic_bytes=2 * k_bytes + q_bytes + 2 * half_bytes + rows * 12,
+                                what="pikv_decode_attend: one pass over K and V (decode_fused_i8_kernel), halves written "
+                                     "and read back for the H2O importance"),
+        "decode_attend_without_h2o": _entry(t_call_nb, 2 * k_bytes + q_bytes,
+                                            what="pikv_decode_attend with row_acc = row_ts = NULL: attention output only"),
     }
 
 

@@ -1506,14 +1506,16 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
                               n_kv_heads, n_q_heads, head_dim, cache_row_base, cache_fill, n_caches, 0, decay, now,
                               row_acc, row_ts, out, nullptr, 0, stream);
   const bool asym = scheme == PIKV_Q_I4_ASYM;
-  // one pass over K and V (no score matrix): 4-bit codes, heads of 128, up to 4 bf16 query heads per kv head.
+  const bool any_asym = asym || scheme == PIKV_Q_I8_ASYM;
+  // one pass over K and V (no score matrix): heads of 128, bf16 queries; 4-bit codes with up to 4 query heads per
+  // kv head, 8-bit codes (scale per kv head or coarser) with up to 8.
   // Its halves (n_q_heads * 128 bytes per tile and one spare tile per cache) lie where the float scores would
   // (256 bytes per head and tile), the tiles' reference maxima in the tile-maximum table, the ranges' statistics
   // in the tile-sum table.
-  if (decode_fused_serves(scheme, group, n_kv_heads, n_q_heads, head_dim, q_dtype, row_acc != nullptr) && (!asym || (k_zero && v_zero)) &&
+  if (decode_fused_serves(scheme, group, n_kv_heads, n_q_heads, head_dim, q_dtype, row_acc != nullptr) && (!any_asym || (k_zero && v_zero)) &&
       n_caches <= 65535) {
     const int tpb = fused_tokens_per_block(n_caches, n_kv_heads, max_len, attend_tokens_per_block(n_caches, max_len));
-    return decode_fused_launch(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, scheme, n_kv_heads, n_q_heads, q,
+    return decode_fused_launch(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, scheme, group, n_kv_heads, n_q_heads, q,
                                scale_qk, cache_row_base, cache_fill, n_caches, max_len, tpb, decay, now, row_acc, row_ts,
                                out, ws + w.scores, tmax, tsum, reinterpret_cast<float*>(partial), stats, st);
   }

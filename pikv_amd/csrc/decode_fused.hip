@@ -431,6 +431,409 @@ __global__ __launch_bounds__(512) void decode_fused_i4_kernel(FusedArgs a) {
   }
 }
 
+// ---- the same pass over an 8-bit cache ----------------------------------------------------------
+// Codes of one byte, a float scale (and zero point) per (token, kv head) or coarser, heads of 128
+// dimensions, 2..8 kv heads, 1..8 bf16 query heads per kv head.  The plan is the 4-bit kernel's - a
+// wavefront per kv head, 64-token tiles, K from memory into matrix-core operands, V through a private
+// piece of LDS and ds_read_b64_tr_b8, running softmax, ranges merged by decode_finish_kernel - with
+// these differences:
+//  * A stored byte u (the code, or code + 128 for the symmetric scheme: one XOR per word) IS a bf16
+//    number - integers up to 255 need eight significant bits - so it goes to the matrix cores as
+//    itself (v_cvt_f32_ubyteN + v_cvt_pk_bf16_f32, three instructions per two codes): no nibble
+//    split, no offset beyond the zero point.  score = s (sum q u - zz sum q), the two halves of the
+//    head dimension accumulated apart, each with its own query sum taken off first.
+//  * The A operand of the score product holds the query heads as rows (up to 8 of 16), so a result
+//    lane holds FOUR heads of one token; lanes 32..63 (rows of no head) take over two of the four
+//    16-token slices from lanes 0..31 (v_permlane32_swap), and every lane runs the softmax of four
+//    heads x two neighbouring tokens.  Slice s of lane column n is token 4 n + s.
+//  * One register set: the V codes of the next tile are asked for as soon as this tile's are staged,
+//    the K codes as soon as this tile's scores are done (a tile is 16 KB per wavefront).
+//  * Bookkeeping records: 16 bytes per lane - 2 tokens x 4 heads as halves - from every lane (5..8
+//    query heads per kv head: 1 KB per tile and kv head) or from the lanes of heads 0..3 (512 B).
+constexpr int k8CodeRow = 144;    // bytes per staged V row: 128 code bytes + 16 (bank spread, 16-byte aligned)
+constexpr int k8VCodes = 0;                                    // [64 tokens][k8CodeRow]
+constexpr int k8Meta = k8VCodes + kFTile * k8CodeRow;          // two sets of {K (scale, zz), V (scale, zz)} float2 per token
+constexpr int k8MetaSet = 2 * kFTile * 8;
+constexpr int k8ABuf = k8Meta + 2 * k8MetaSet;                 // [16 rows][kFARow]
+constexpr int k8AZero = k8ABuf + 16 * kFARow;                  // 32 zero bytes
+constexpr int k8WaveLds = (k8AZero + 32 + 255) & ~255;
+static_assert(k8WaveLds * 8 <= 160 * 1024, "eight wavefronts per block fit the LDS of a compute unit");
+
+struct Fused8Args {
+  const void* k_codes;
+  const void* k_scale;
+  const void* k_zero;
+  const void* v_codes;
+  const void* v_scale;
+  const void* v_zero;
+  const void* q;            // bf16 [cache][n_q_heads][128]
+  const int64_t* row_base;
+  const int32_t* fill;
+  float* partial;           // [range][cache][q head][128]
+  float* pstats;            // [range][cache][q head][2]
+  uint4* e16;               // [cache][tile][kv head][64 or 32 lanes]: 8 halves per lane
+  float* tref;              // [cache][tile][q head]
+  int64_t n_tiles;          // records per cache
+  int64_t max_len;
+  int n_caches;
+  int n_kv_heads;
+  int n_q_heads;
+  int tokens_per_block;     // a multiple of 64
+  float scale_qk;
+  int group;                // elements per scale: a multiple of 128 that divides the row
+  int blocks_per_range;     // each block takes n_kv_heads / blocks_per_range neighbouring kv heads
+};
+
+// four bytes of a word as bf16, in order: {b0, b1}, {b2, b3}
+__device__ __forceinline__ uint2 bytes_to_bf16(uint32_t w) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  f2 lo, hi;
+  lo[0] = (float)(w & 0xffu);
+  lo[1] = (float)((w >> 8) & 0xffu);
+  hi[0] = (float)((w >> 16) & 0xffu);
+  hi[1] = (float)(w >> 24);
+  return make_uint2(__builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf2)),
+                    __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf2)));
+}
+
+template <int SCHEME, bool BOOK>
+__global__ __launch_bounds__(512) void decode_fused_i8_kernel(Fused8Args a) {
+  using Q = QScheme<SCHEME>;
+  static_assert(Q::bits == 8, "8-bit schemes only");
+  extern __shared__ __align__(16) unsigned char fused_lds[];
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  unsigned char* const lds = fused_lds + wv * k8WaveLds;
+  unsigned char* const vcodes = lds + k8VCodes;
+  unsigned char* const abuf = lds + k8ABuf;
+  unsigned char* const azero = lds + k8AZero;
+
+  const int c = blockIdx.x;
+  const int xr = blockIdx.y / a.blocks_per_range;   // token range
+  const int HK = a.n_kv_heads;
+  const int nwb = blockDim.x >> 6;                  // wavefronts (kv heads) of this block
+  const int g0 = (blockIdx.y % a.blocks_per_range) * nwb;
+  const int g = g0 + wv;                            // this wavefront's kv head
+  const int rep = a.n_q_heads / HK;
+  const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
+  const int64_t t0 = (int64_t)xr * a.tokens_per_block;
+  if (t0 >= len) return;   // the merge skips ranges that hold no token
+  const int span = (int)((t0 + a.tokens_per_block < len ? t0 + a.tokens_per_block : len) - t0);
+  const int last = span - 1;
+
+  // roles.  Score product: lane = (column nl: a token, k-slice rg: 16 dimensions of each half of the head);
+  // result lane (nl, rg) holds heads 4 rg .. 4 rg + 3 of its token.  Softmax and weights: heads
+  // hq0 .. hq0 + 3, tokens tp, tp + 1.  Output product: lane = (A row / dimension i, k-slice kg: 8 tokens).
+  const int nl = lane & 15, rg = lane >> 4;
+  const int i = nl, kg = rg;
+  const int hq0 = 4 * (rg & 1);
+  const int tp = 4 * nl + 2 * (rg >> 1);
+  const int row_codes = HK * 128;                       // bytes per cached row in the code planes
+  const int gpr = row_codes / a.group;                  // metadata entries per cached row
+  const int64_t urow = a.row_base[c] + t0;
+  const char* const kc = reinterpret_cast<const char*>(a.k_codes) + urow * row_codes + g * 128;
+  const char* const vc = reinterpret_cast<const char*>(a.v_codes) + urow * row_codes + g * 128;
+
+  if (lane < 8) reinterpret_cast<uint32_t*>(azero)[lane] = 0u;
+
+  // metadata: thread e takes entry (token e / heads, head e % heads) of the next tile's rows and writes
+  // it into the owning wavefront's piece of LDS; the barrier at the top of the next tile publishes it
+  const int m_tok = threadIdx.x / nwb, m_hd = threadIdx.x - m_tok * nwb;
+  unsigned char* const m_lds = fused_lds + m_hd * k8WaveLds + k8Meta;
+  const int m_ent = ((g0 + m_hd) * 128) / a.group;
+  const float* const ksb = reinterpret_cast<const float*>(a.k_scale) + urow * gpr + m_ent;
+  const float* const kzb = reinterpret_cast<const float*>(a.k_zero) + urow * gpr + m_ent;
+  const float* const vsb = reinterpret_cast<const float*>(a.v_scale) + urow * gpr + m_ent;
+  const float* const vzb = reinterpret_cast<const float*>(a.v_zero) + urow * gpr + m_ent;
+
+  // ---- queries: A rows = the kv head's query heads, k-step (half, o) = dimensions 64 half + 16 rg + 8 o .. + 7 ----
+  uint4 aq[4];
+  float qs0, qs1;   // sum of the head's query over the dimensions of half 0 / half 1 (lane's row nl)
+  {
+    const bool a_on = nl < rep;
+    const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)c * a.n_q_heads + g * rep + (a_on ? nl : 0)) * 128 + rg * 16;
+    float part[2] = {0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      uint4 d = make_uint4(0, 0, 0, 0);
+      if (a_on) d = ld16(qp + (k >> 1) * 64 + (k & 1) * 8);
+      aq[k] = d;
+      const uint32_t w[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        part[k >> 1] += __uint_as_float(w[e] << 16);
+        part[k >> 1] += __uint_as_float(w[e] & 0xffff0000u);
+      }
+    }
+    part[0] += __shfl_xor(part[0], 16, PIKV_WAVE);
+    part[0] += __shfl_xor(part[0], 32, PIKV_WAVE);
+    part[1] += __shfl_xor(part[1], 16, PIKV_WAVE);
+    part[1] += __shfl_xor(part[1], 32, PIKV_WAVE);
+    qs0 = part[0];
+    qs1 = part[1];
+  }
+  // ... of the four heads in this lane's result rows 4 rg .. 4 rg + 3 (rows past the heads: zero)
+  float4 q0v, q1v;
+  q0v.x = __shfl(qs0, 4 * rg + 0, PIKV_WAVE); q0v.y = __shfl(qs0, 4 * rg + 1, PIKV_WAVE);
+  q0v.z = __shfl(qs0, 4 * rg + 2, PIKV_WAVE); q0v.w = __shfl(qs0, 4 * rg + 3, PIKV_WAVE);
+  q1v.x = __shfl(qs1, 4 * rg + 0, PIKV_WAVE); q1v.y = __shfl(qs1, 4 * rg + 1, PIKV_WAVE);
+  q1v.z = __shfl(qs1, 4 * rg + 2, PIKV_WAVE); q1v.w = __shfl(qs1, 4 * rg + 3, PIKV_WAVE);
+
+  pikv_f32x4 C[8];
+#pragma unroll
+  for (int d = 0; d < 8; ++d) C[d] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
+  float zacc[4] = {0.f, 0.f, 0.f, 0.f};
+  float lsum[4] = {0.f, 0.f, 0.f, 0.f};
+  float m_run[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) m_run[j] = -__builtin_inff();
+
+  // A-operand piece of this lane in the output product: row i = (head i / 2, part i % 2), or the zero piece
+  const bool arow_on = i < 2 * rep;
+  const unsigned char* const a_row = arow_on ? abuf + i * kFARow + kg * 16 : azero;
+  const int a_half = arow_on ? 64 : 0;   // bytes from the first 32 tokens of a row to the second
+
+  uint4 rk[8], rv[8];
+  float mks, mkz, mvs, mvz;
+  auto clamp_row = [&](int tok) { return tok < last ? tok : last; };
+  auto issue_meta = [&](int n0) {   // this thread's metadata entry of the tile that starts at n0
+    const uint32_t mo = (uint32_t)(clamp_row(n0 + m_tok) * gpr);
+    mks = ksb[mo];
+    mvs = vsb[mo];
+    mkz = 128.0f;
+    mvz = 128.0f;
+    if constexpr (!Q::sym) {
+      mkz = kzb[mo];
+      mvz = vzb[mo];
+    }
+  };
+  auto stage_meta = [&](int set) {
+    float2* const mb = reinterpret_cast<float2*>(m_lds + set * k8MetaSet);
+    mb[m_tok] = make_float2(mks, mkz);
+    mb[kFTile + m_tok] = make_float2(mvs, mvz);
+  };
+  auto issue_v = [&](int n0) {   // whole 128-byte rows: 8 tokens per instruction
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      rv[k] = ld16(vc + (uint32_t)(clamp_row(n0 + 8 * k + (lane >> 3)) * row_codes + (lane & 7) * 16));
+  };
+  auto issue_k = [&](int n0) {   // slice s: token 4 nl + s, the lane's 16 bytes of each half
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const uint32_t ro = (uint32_t)(clamp_row(n0 + 4 * nl + s) * row_codes + rg * 16);
+      rk[2 * s] = ld16(kc + ro);
+      rk[2 * s + 1] = ld16(kc + ro + 64);
+    }
+  };
+  auto wave_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  auto pin_order = [] { asm volatile("" ::: "memory"); };
+  auto both_halves_max = [](float v) {   // max over lanes l and l ^ 32
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+  };
+  auto both_halves_sum = [](float v) {
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+  };
+
+  issue_meta(0);
+  stage_meta(0);
+  pin_order();
+  issue_meta(kFTile);
+  issue_v(0);
+  pin_order();
+  issue_k(0);
+  pin_order();
+
+  for (int n0 = 0; n0 < span; n0 += kFTile) {
+    const int par = (n0 / kFTile) & 1;
+    // one block barrier per tile: it publishes the metadata other wavefronts' threads wrote
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      *reinterpret_cast<uint4*>(vcodes + (8 * k + (lane >> 3)) * k8CodeRow + (lane & 7) * 16) = rv[k];
+    stage_meta(par ^ 1);   // the NEXT tile's metadata, into the other set
+    wave_sync();
+    const float2* const kmeta = reinterpret_cast<const float2*>(lds + k8Meta + par * k8MetaSet);
+    const float2* const vmeta = kmeta + kFTile;
+    pin_order();
+    issue_v(n0 + kFTile);
+    issue_meta(n0 + 2 * kFTile);
+    pin_order();
+
+    // ---- scores: heads 4 rg .. 4 rg + 3 of tokens 4 nl + s ----
+    float sc[4][4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      pikv_f32x4 pc0 = pikv_f32x4{0.f, 0.f, 0.f, 0.f}, pc1 = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const uint4 cw = rk[2 * s + half];
+        const uint32_t w0 = Q::sym ? cw.x ^ 0x80808080u : cw.x, w1 = Q::sym ? cw.y ^ 0x80808080u : cw.y;
+        const uint32_t w2 = Q::sym ? cw.z ^ 0x80808080u : cw.z, w3 = Q::sym ? cw.w ^ 0x80808080u : cw.w;
+        const uint2 b0 = bytes_to_bf16(w0), b1 = bytes_to_bf16(w1), b2 = bytes_to_bf16(w2), b3 = bytes_to_bf16(w3);
+        const uint4 bo0 = make_uint4(b0.x, b0.y, b1.x, b1.y), bo1 = make_uint4(b2.x, b2.y, b3.x, b3.y);
+        pikv_f32x4& pc = half ? pc1 : pc0;
+        pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, aq[2 * half]),
+                                                     __builtin_bit_cast(pikv_bf16x8, bo0), pc, 0, 0, 0);
+        pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, aq[2 * half + 1]),
+                                                     __builtin_bit_cast(pikv_bf16x8, bo1), pc, 0, 0, 0);
+      }
+      const float2 km = kmeta[4 * nl + s];
+      const float f = km.x * a.scale_qk;
+      sc[s][0] = f * (fmaf(-km.y, q0v.x, pc0[0]) + fmaf(-km.y, q1v.x, pc1[0]));
+      sc[s][1] = f * (fmaf(-km.y, q0v.y, pc0[1]) + fmaf(-km.y, q1v.y, pc1[1]));
+      sc[s][2] = f * (fmaf(-km.y, q0v.z, pc0[2]) + fmaf(-km.y, q1v.z, pc1[2]));
+      sc[s][3] = f * (fmaf(-km.y, q0v.w, pc0[3]) + fmaf(-km.y, q1v.w, pc1[3]));
+    }
+    pin_order();
+    issue_k(n0 + kFTile);
+    pin_order();
+    // lanes 32..63 take slices 2, 3 of lanes 0..31: afterwards every lane holds heads hq0 .. hq0 + 3 of
+    // tokens tp (e0) and tp + 1 (e1)
+    float e0[4], e1[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      auto s02 = __builtin_amdgcn_permlane32_swap(__float_as_uint(sc[0][j]), __float_as_uint(sc[2][j]), false, false);
+      auto s13 = __builtin_amdgcn_permlane32_swap(__float_as_uint(sc[1][j]), __float_as_uint(sc[3][j]), false, false);
+      const bool head_on = hq0 + j < rep;
+      e0[j] = (head_on && n0 + tp <= last) ? __uint_as_float(s02[0]) : -__builtin_inff();
+      e1[j] = (head_on && n0 + tp + 1 <= last) ? __uint_as_float(s13[0]) : -__builtin_inff();
+    }
+
+    // ---- running softmax of the four heads ----
+    float alpha[4], m_ref[4];
+    bool moved = false;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float m_tile = both_halves_max(group_max_dpp(fmaxf(e0[j], e1[j]), 16));
+      const float m_new = fmaxf(m_run[j], m_tile);
+      m_ref[j] = m_new == -__builtin_inff() ? 0.f : m_new;
+      alpha[j] = m_run[j] == m_new ? 1.0f : __builtin_amdgcn_exp2f((m_run[j] - m_ref[j]) * kLog2e);
+      moved = moved || alpha[j] != 1.0f;
+      m_run[j] = m_new;
+    }
+    if (__ballot(moved) != 0ull) {   // some head's maximum moved: scale what has been added so far
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        lsum[j] *= alpha[j];
+        zacc[j] *= alpha[j];
+      }
+      // result rows 4 kg + q of the output product: heads 2 kg (q = 0, 1) and 2 kg + 1 (q = 2, 3); head h
+      // is slot h % 4 of the lanes with rg % 2 == h / 4
+      const int src = 16 * (kg >> 1);
+      const float al0 = __shfl(alpha[0], src, PIKV_WAVE), al1 = __shfl(alpha[1], src, PIKV_WAVE);
+      const float al2 = __shfl(alpha[2], src, PIKV_WAVE), al3 = __shfl(alpha[3], src, PIKV_WAVE);
+      const float a0 = (kg & 1) ? al2 : al0, a1 = (kg & 1) ? al3 : al1;
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {
+        C[d][0] *= a0; C[d][1] *= a0;
+        C[d][2] *= a1; C[d][3] *= a1;
+      }
+    }
+    float p0[4], p1[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      p0[j] = __builtin_amdgcn_exp2f((e0[j] - m_ref[j]) * kLog2e);
+      p1[j] = __builtin_amdgcn_exp2f((e1[j] - m_ref[j]) * kLog2e);
+      lsum[j] += p0[j] + p1[j];
+    }
+    if constexpr (BOOK) {
+      const int64_t tile = (t0 + n0) / kFTile;
+      auto hb = [](float p) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(p * kHalfScale)); };
+      const uint4 ev = make_uint4(hb(p0[0]) | (hb(p1[0]) << 16), hb(p0[1]) | (hb(p1[1]) << 16),
+                                  hb(p0[2]) | (hb(p1[2]) << 16), hb(p0[3]) | (hb(p1[3]) << 16));
+      float* const rrec = a.tref + ((int64_t)c * a.n_tiles + tile) * a.n_q_heads + g * rep;
+      if (rep > 4) {
+        a.e16[(((int64_t)c * a.n_tiles + tile) * HK + g) * 64 + lane] = ev;
+      } else if (hq0 == 0) {
+        a.e16[(((int64_t)c * a.n_tiles + tile) * HK + g) * 32 + 16 * (rg >> 1) + nl] = ev;
+      }
+      if (nl == 0 && rg < 2) {   // (one store of the eight maxima from lanes nl < 4 measured slower: 1053 vs 1040 us)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (hq0 + j < rep) rrec[hq0 + j] = m_ref[j];
+      }
+    }
+
+    // ---- weights: p * scale of the token's V row as a bf16 high part and a bf16 remainder ----
+    {
+      const float2 vm0 = vmeta[tp], vm1 = vmeta[tp + 1];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float w0 = p0[j] * vm0.x, w1 = p1[j] * vm1.x;
+        const float h0 = __uint_as_float(__float_as_uint(w0) & 0xffff0000u);
+        const float h1 = __uint_as_float(__float_as_uint(w1) & 0xffff0000u);
+        const float l0 = __uint_as_float(__float_as_uint(w0 - h0) & 0xffff0000u);
+        const float l1 = __uint_as_float(__float_as_uint(w1 - h1) & 0xffff0000u);
+        // the zero-point sum uses the SAME two-part values the matrix core multiplies with the codes
+        zacc[j] = fmaf(h0 + l0, vm0.y, zacc[j]);
+        zacc[j] = fmaf(h1 + l1, vm1.y, zacc[j]);
+        if (hq0 + j < rep) {
+          unsigned char* const rowp = abuf + (2 * (hq0 + j)) * kFARow + tp * 2;
+          *reinterpret_cast<uint32_t*>(rowp) = (__float_as_uint(h0) >> 16) | __float_as_uint(h1);
+          *reinterpret_cast<uint32_t*>(rowp + kFARow) = (__float_as_uint(l0) >> 16) | __float_as_uint(l1);
+        }
+      }
+    }
+    wave_sync();   // the rows were written by other lanes of this wavefront
+
+    // ---- output product: A rows (head, part) against 16 dimensions of 2 x 32 tokens ----
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const uint4 aw = *reinterpret_cast<const uint4*>(a_row + hf * a_half);
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+        // source lane i points at token 32 hf + 8 kg + i / 2, dims 16 db + 8 (i % 2) .. + 7; result lane i
+        // holds dimension 16 db + i of tokens 32 hf + 8 kg .. + 7
+        const pikv_i32x2 tr = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+            (pikv_i32x2 __attribute__((address_space(3)))*)(vcodes + (32 * hf + 8 * kg + (i >> 1)) * k8CodeRow + db * 16 + 8 * (i & 1)));
+        const uint32_t x0 = Q::sym ? ((uint32_t)tr[0] ^ 0x80808080u) : (uint32_t)tr[0];
+        const uint32_t x1 = Q::sym ? ((uint32_t)tr[1] ^ 0x80808080u) : (uint32_t)tr[1];
+        const uint2 b0 = bytes_to_bf16(x0), b1 = bytes_to_bf16(x1);
+        C[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, aw),
+                                                        __builtin_bit_cast(pikv_bf16x8, make_uint4(b0.x, b0.y, b1.x, b1.y)),
+                                                        C[db], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- what the range leaves: (maximum, sum, unnormalised output) of each head ----
+  wave_sync();
+  float* const zl = reinterpret_cast<float*>(lds);   // [head]: zero-point sums
+  float ltot[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    ltot[j] = both_halves_sum(group_sum_dpp(lsum[j], 16));
+    const float z = both_halves_sum(group_sum_dpp(zacc[j], 16));
+    if (nl == 0 && rg < 2) zl[hq0 + j] = z;
+  }
+  wave_sync();
+  const int64_t pbase = ((int64_t)xr * a.n_caches + c) * a.n_q_heads + g * rep;
+  if (nl == 0 && rg < 2) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (hq0 + j < rep) {
+        a.pstats[(pbase + hq0 + j) * 2] = m_run[j];
+        a.pstats[(pbase + hq0 + j) * 2 + 1] = ltot[j];
+      }
+  }
+  // C: lane (dimension i, rows 4 kg + q): rows 2 h / 2 h + 1 are the two parts of head h
+#pragma unroll
+  for (int rr = 0; rr < 2; ++rr) {
+    const int ho = 2 * kg + rr;
+    if (ho >= rep) continue;
+    float* o = a.partial + (pbase + ho) * 128;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) o[db * 16 + i] = (C[db][2 * rr] + C[db][2 * rr + 1]) - zl[ho];
+  }
+}
+
 // out[c,h,:] = sum over ranges of partial * exp(m_range - M) / Z,  M = max of the ranges' maxima,
 // Z = sum of their sums scaled alike.  One thread per output element; caches without a token give 0.
 __global__ __launch_bounds__(256) void decode_finish_kernel(const float* __restrict__ partial,
@@ -532,6 +935,85 @@ __global__ __launch_bounds__(256) void decode_importance_kernel(const uint2* __r
   }
 }
 
+// The same for the records of the 8-bit pass: lane (nl, rg) of a record holds heads 4 (rg % 2) .. + 3 of
+// tokens 4 nl + 2 (rg / 2) and the next one, two tokens x four heads as halves {token, token + 1} per
+// head; with up to four query heads per kv head a record is the 32 lanes of heads 0..3 only.
+__global__ __launch_bounds__(256) void decode_importance8_kernel(const uint4* __restrict__ e16,
+                                                                const float* __restrict__ tref,
+                                                                const float* __restrict__ head_stats,
+                                                                const int64_t* __restrict__ row_base,
+                                                                const int32_t* __restrict__ fill, int64_t max_len,
+                                                                int64_t n_tiles, int n_kv_heads, int n_q_heads,
+                                                                float decay, float now, float* __restrict__ row_acc,
+                                                                float* __restrict__ row_ts) {
+  const int lane = threadIdx.x & 63;
+  const int c = blockIdx.y;
+  const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t len = fill[c] < max_len ? (int64_t)fill[c] : max_len;
+  if (tile * kFTile >= len) return;
+  const int rep = n_q_heads / n_kv_heads;
+  const int nl = lane & 15, rg = lane >> 4;
+  const int hq0 = 4 * (rg & 1);
+  const int64_t n = tile * kFTile + 4 * nl + 2 * (rg >> 1);   // first of this lane's two tokens
+  const int64_t row = row_base[c] + n;
+  const bool writer = hq0 == 0;
+  float acc0 = 0.f, acc1 = 0.f;
+  if (row_acc != nullptr && writer) {
+    if (n < len) acc0 = row_acc[row];
+    if (n + 1 < len) acc1 = row_acc[row + 1];
+  }
+  float i0 = 0.f, i1 = 0.f;
+  if (row_acc != nullptr) {
+    const int lanes = rep > 4 ? 64 : 32;
+    const bool have = rep > 4 || hq0 == 0;
+    const uint4* ep = e16 + ((int64_t)c * n_tiles + tile) * n_kv_heads * lanes + (rep > 4 ? lane : 16 * (rg >> 1) + nl);
+    uint4 hv[8];
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      hv[g] = make_uint4(0, 0, 0, 0);
+      if (g < n_kv_heads && have) hv[g] = ep[(int64_t)g * lanes];
+    }
+    float fac = 0.f;   // lane h: what turns a stored half of head h in this tile into a probability
+    if (lane < n_q_heads) {
+      const float2 mz = *reinterpret_cast<const float2*>(head_stats + ((int64_t)c * n_q_heads + lane) * 2);
+      const float mt = tref[((int64_t)c * n_tiles + tile) * n_q_heads + lane];
+      fac = __builtin_amdgcn_exp2f((mt - mz.x) * kLog2e) / (mz.y * kHalfScale);
+    }
+    auto lo = [](uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu)); };
+    auto hi = [](uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); };
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      if (g >= n_kv_heads) break;
+      const uint32_t w[4] = {hv[g].x, hv[g].y, hv[g].z, hv[g].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int h = g * rep + hq0 + j;
+        const float f = __shfl(fac, hq0 + j < rep ? h : 0, PIKV_WAVE);
+        const float ff = hq0 + j < rep ? f : 0.f;
+        i0 = fmaf(lo(w[j]), ff, i0);
+        i1 = fmaf(hi(w[j]), ff, i1);
+      }
+    }
+    // heads 4..7 of the same tokens sit 16 lanes up
+    i0 += __shfl_xor(i0, 16, PIKV_WAVE);
+    i1 += __shfl_xor(i1, 16, PIKV_WAVE);
+  }
+  if (writer) {
+    if (row_acc != nullptr) {
+      if (decay != 1.0f) {
+        acc0 = acc0 * decay;
+        acc1 = acc1 * decay;
+      }
+      if (n < len) row_acc[row] = acc0 + i0;
+      if (n + 1 < len) row_acc[row + 1] = acc1 + i1;
+    }
+    if (row_ts != nullptr) {
+      if (n < len) row_ts[row] = now;
+      if (n + 1 < len) row_ts[row + 1] = now;
+    }
+  }
+}
+
 }  // namespace pikv
 
 using namespace pikv;
@@ -545,6 +1027,8 @@ namespace pikv {
 // Rows of 8 (6) kv heads go as two blocks of 4 (3) wavefronts per token range: two independent blocks per
 // compute unit fill each other's waits, where one block of eight wavefronts meets at one barrier per tile.
 static int fused_groups(int n_kv_heads) { (void)n_kv_heads; return 1; }
+// the 8-bit pass: its wavefronts share no code lines (a kv head's 128 bytes of a row are a line of their own)
+static int fused8_blocks_per_range(int n_kv_heads) { return (n_kv_heads == 8 || n_kv_heads == 6) ? 2 : 1; }
 
 int fused_tokens_per_block(int n_caches, int n_kv_heads, int64_t max_len, int min_tpb) {
   const int groups = fused_groups(n_kv_heads);
@@ -573,10 +1057,16 @@ int fused_tokens_per_block(int n_caches, int n_kv_heads, int64_t max_len, int mi
 // 6 x 24: 552 -> 537, 8 x 32: 675 vs 677 - the halves cost the pass 0.1 ms, see the kernel's comment; with
 // fewer query heads per kv head the float rows of the two-kernel form are the smaller exchange).
 bool decode_fused_serves(int scheme, int group, int n_kv_heads, int n_q_heads, int head_dim, int q_dtype, bool bookkeeping) {
-  if (scheme != PIKV_Q_I4_ASYM && scheme != PIKV_Q_I4_SYM) return false;
-  if (group != 32 || head_dim != 128 || q_dtype != PIKV_BF16) return false;
+  if (head_dim != 128 || q_dtype != PIKV_BF16) return false;
   if (n_kv_heads < 2 || n_kv_heads > 8 || n_q_heads % n_kv_heads != 0) return false;
   const int rep = n_q_heads / n_kv_heads;
+  if (scheme == PIKV_Q_I8_SYM || scheme == PIKV_Q_I8_ASYM) {
+    // a scale per (token, kv head) or coarser; with bookkeeping the records must fit where the float scores would
+    if (group < 128 || group % 128 != 0 || (n_kv_heads * 128) % group != 0) return false;
+    if (bookkeeping) return rep >= 2 && rep <= 8;
+    return rep >= 1 && rep <= 8;
+  }
+  if (group != 32) return false;
   if (bookkeeping) return rep == 4 && n_kv_heads >= 3;
   return rep >= 1 && rep <= 4;
 }
@@ -587,7 +1077,7 @@ bool decode_fused_serves(int scheme, int group, int n_kv_heads, int n_q_heads, i
 //   e16     n_caches * n_tiles * n_q_heads * 128 bytes       tref   n_caches * n_tiles * n_q_heads floats
 //   pstats  splits * n_caches * n_q_heads * 2 floats          partial splits * n_caches * n_q_heads * 128 floats
 int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_zero, const void* v_codes,
-                        const void* v_scale, const void* v_zero, int scheme, int n_kv_heads, int n_q_heads,
+                        const void* v_scale, const void* v_zero, int scheme, int group, int n_kv_heads, int n_q_heads,
                         const void* q, float scale_qk, const int64_t* cache_row_base, const int32_t* cache_fill,
                         int n_caches, int64_t max_len, int tokens_per_block, float decay, float now, float* row_acc,
                         float* row_ts, float* out, void* e16, float* tref, float* pstats, float* partial,
@@ -596,6 +1086,34 @@ int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_
   const int64_t splits = (max_len + tokens_per_block - 1) / tokens_per_block;
   if (splits > 65535 || (tokens_per_block & 127) != 0) return PIKV_ERR_SHAPE;
   const bool book = row_acc != nullptr || row_ts != nullptr;
+  if (scheme == PIKV_Q_I8_SYM || scheme == PIKV_Q_I8_ASYM) {
+    const int64_t n_tiles8 = (max_len + kFTile - 1) / kFTile;   // this pass never touches a tile past a range's end
+    Fused8Args a8{k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, q, cache_row_base, cache_fill, partial, pstats,
+                  reinterpret_cast<uint4*>(e16), tref, n_tiles8, max_len, n_caches, n_kv_heads, n_q_heads,
+                  tokens_per_block, scale_qk, group,
+                  splits * fused8_blocks_per_range(n_kv_heads) <= 65535 ? fused8_blocks_per_range(n_kv_heads) : 1};
+    const dim3 grid8((unsigned)n_caches, (unsigned)(splits * a8.blocks_per_range));
+    const dim3 block8((unsigned)(n_kv_heads / a8.blocks_per_range * 64));
+    const size_t lds8 = (size_t)(n_kv_heads / a8.blocks_per_range) * k8WaveLds;
+    const bool wr8 = row_acc != nullptr;
+    if (scheme == PIKV_Q_I8_SYM) {
+      if (wr8) hipLaunchKernelGGL((decode_fused_i8_kernel<PIKV_Q_I8_SYM, true>), grid8, block8, lds8, st, a8);
+      else hipLaunchKernelGGL((decode_fused_i8_kernel<PIKV_Q_I8_SYM, false>), grid8, block8, lds8, st, a8);
+    } else {
+      if (wr8) hipLaunchKernelGGL((decode_fused_i8_kernel<PIKV_Q_I8_ASYM, true>), grid8, block8, lds8, st, a8);
+      else hipLaunchKernelGGL((decode_fused_i8_kernel<PIKV_Q_I8_ASYM, false>), grid8, block8, lds8, st, a8);
+    }
+    PIKV_CHECK_LAUNCH();
+    const int64_t total8 = (int64_t)n_caches * n_q_heads * 128;
+    hipLaunchKernelGGL(decode_finish_kernel, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, st, partial, pstats,
+                       cache_fill, max_len, n_caches, n_q_heads, (int)splits, tokens_per_block, out, head_stats);
+    if (book)
+      hipLaunchKernelGGL(decode_importance8_kernel, dim3((unsigned)((n_tiles8 + 3) / 4), (unsigned)n_caches), dim3(256), 0,
+                         st, reinterpret_cast<const uint4*>(e16), tref, head_stats, cache_row_base, cache_fill, max_len,
+                         n_tiles8, n_kv_heads, n_q_heads, decay, now, row_acc, row_ts);
+    PIKV_CHECK_LAUNCH();
+    return PIKV_OK;
+  }
   FusedArgs a{k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, q, cache_row_base, cache_fill, partial, pstats,
               reinterpret_cast<uint2*>(e16), tref, n_tiles, max_len, n_caches, n_kv_heads, n_q_heads, tokens_per_block,
               scale_qk, fused_groups(n_kv_heads)};

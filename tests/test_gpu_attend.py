@@ -230,6 +230,12 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I8_SYM, 128, 1, 4, 128, "f32"),     # ... 1 kv head: eight rows as one
     (O.Q_I8_SYM, 128, 3, 12, 128, "bf16"),   # ... 3 kv heads x 4: pairs of rows, 24 staged probability rows
     (O.Q_I8_SYM, 128, 3, 24, 128, "bf16"),   # ... 3 kv heads x 8; scores up to 36 in this draw: needs the 8-bit scores' part-wise offsets
+    (O.Q_I8_SYM, 128, 8, 64, 128, "bf16"),   # 8-bit one-pass form: 8 q heads per kv head, every lane of a record
+    (O.Q_I8_ASYM, 128, 6, 42, 128, "bf16"),  # ... 7 q heads per kv head, zero points
+    (O.Q_I8_ASYM, 256, 4, 20, 128, "bf16"),  # ... a scale per pair of kv heads, 5 q heads per kv head
+    (O.Q_I8_SYM, 512, 4, 8, 128, "bf16"),    # ... a scale per token, 2 q heads per kv head: records of 32 lanes
+    (O.Q_I8_ASYM, 128, 7, 14, 128, "bf16"),  # ... 7 kv heads x 2
+    (O.Q_I8_SYM, 128, 5, 5, 128, "bf16"),    # ... one q head per kv head: one pass only without the bookkeeping
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.9])
 def test_decode_attend_one_call(dev, scheme, group, heads, hq, dh, qdtype, decay):
