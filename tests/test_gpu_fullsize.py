@@ -167,18 +167,21 @@ def test_decode_read_full(dev):
     assert torch.equal(pool.k_codes, k0)
 
 
-def test_decode_attend_full(dev):
-    """Attention output and the one-call decode read at the full decode shape (64 x 32768 tokens,
-    blocks of 4096 cached tokens), through properties: with every cached V row equal the output IS
+@pytest.mark.parametrize("fmt", ["int4_asym_g32_x32q", "int8_sym_per_head_x64q"])
+def test_decode_attend_full(dev, fmt):
+    """Attention output and the one-call decode read at the full decode shape (64 x 32768 tokens; the
+    4-bit cache of the decode configuration, and the same tokens as 8-bit codes read by 64 query
+    heads), through properties: with every cached V row equal the output IS
     that row whatever the probabilities are (they sum to one over all 32768 tokens); the
     accumulators grow by one per query head and cache; the one call agrees with the three public
     steps; two sequences are checked against dequantise + softmax + matmul in float32."""
     import torch
     from pikv_amd import ops
-    B, N, hkv, hq, dh = 64, 32768, 8, 32, 128
+    B, N, hkv, dh = 64, 32768, 8, 128
+    hq, group, scheme = (32, 32, ops.Q_I4_ASYM) if fmt.startswith("int4") else (64, 128, ops.Q_I8_SYM)
     D = hkv * dh
     g = torch.Generator(device=dev).manual_seed(22)
-    pool = ops.CachePool([N] * B, hkv, dh, 32, ops.Q_I4_ASYM, dev, with_v=True)
+    pool = ops.CachePool([N] * B, hkv, dh, group, scheme, dev, with_v=True)
     chunk = 8
     slot = torch.arange(N, device=dev, dtype=torch.int32).repeat(chunk)
     for b0 in range(0, B, chunk):
@@ -212,7 +215,8 @@ def test_decode_attend_full(dev):
     # every V row the same: the output is that row, bit patterns of the probabilities do not matter
     pool.v_codes.copy_(pool.v_codes[:1].expand_as(pool.v_codes))
     pool.v_scale.copy_(pool.v_scale[:1].expand_as(pool.v_scale))
-    pool.v_zero.copy_(pool.v_zero[:1].expand_as(pool.v_zero))
+    if pool.v_zero is not None:
+        pool.v_zero.copy_(pool.v_zero[:1].expand_as(pool.v_zero))
     row = pool.gather_dequant("v", row0=0, n=1).view(hkv, dh).repeat_interleave(hq // hkv, dim=0)
     out_c = pool.decode_attend(q, hq, now=4.0, accumulate=False)
     assert float((out_c - row.unsqueeze(0)).abs().max()) <= 2e-5 * float(row.abs().max())
