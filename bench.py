@@ -162,7 +162,7 @@ def hbm_ceiling(torch, dev, iters, nbytes=2 << 30):
     """Practical HBM rates of this machine with the library's own access pattern (16 bytes per
     lane, 1 KiB per wavefront, 8 accesses in flight per lane; bench_probe.hip, a library of its
     own beside this file): read only, write only, copy;
-    plain and non-temporal stores.  Median of `iters` launches over `nbytes` (2 GiB: eight times
+    plain and non-temporal stores; and a read stream in a tile loop without and with small stores.  Median of `iters` launches over `nbytes` (2 GiB: eight times
     the last-level cache), HIP events on the launch stream."""
     import bench_probe
     src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
@@ -174,14 +174,20 @@ def hbm_ceiling(torch, dev, iters, nbytes=2 << 30):
         return lambda: bench_probe.stream_probe(mode, src.data_ptr(), dst.data_ptr(), nbytes, nt, sink.data_ptr(), st)
     gb = nbytes / 1e9
     ms = {name: _median_ms(torch, run(mode, nt), iters)
-          for name, mode, nt in (("read", 0, 0), ("write", 1, 0), ("write_nt", 1, 1), ("copy", 2, 0), ("copy_nt", 2, 1))}
+          for name, mode, nt in (("read", 0, 0), ("write", 1, 0), ("write_nt", 1, 1), ("copy", 2, 0), ("copy_nt", 2, 1),
+                                 ("tile_loop_read", 3, 0), ("tile_loop_read_with_stores", 4, 0))}
     del src, dst
     torch.cuda.empty_cache()
     return {"buffer_bytes": nbytes, "pattern": "16 B per lane, 1 KiB per wavefront, 8 in flight per lane",
             "read_GBps": gb / (ms["read"] * 1e-3), "write_GBps": gb / (ms["write"] * 1e-3),
             "write_nontemporal_GBps": gb / (ms["write_nt"] * 1e-3),
             "copy_GBps": 2 * gb / (ms["copy"] * 1e-3), "copy_nontemporal_GBps": 2 * gb / (ms["copy_nt"] * 1e-3),
-            "ms": ms, "note": "copy rates count bytes read + bytes written"}
+            "tile_loop_read_GBps": gb / (ms["tile_loop_read"] * 1e-3),
+            "tile_loop_read_with_6pct_stores_GBps": gb / (ms["tile_loop_read_with_stores"] * 1e-3),
+            "ms": ms, "note": "copy rates count bytes read + bytes written; tile_loop_*: persistent blocks of eight "
+                              "wavefronts reading 64 KiB tiles, two in flight per block (the loop shape of the one-pass "
+                              "decode kernels), without and with 8 bytes stored per lane and tile (1/16 of the bytes read); "
+                              "both rates count the bytes read only"}
 
 
 def decode_read_workload(torch, ops, dev, iters):

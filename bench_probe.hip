@@ -49,13 +49,72 @@ __global__ __launch_bounds__(256) void stream_probe_kernel(const uint4* __restri
   }
 }
 
+// modes 3 / 4: what small stores cost a saturated read stream.  Persistent blocks of eight wavefronts
+// walk `tiles` tiles of 64 KiB each (16 bytes per lane and access, two tiles in flight per block: the
+// shape of the one-pass decode kernels' tile loop); mode 4 additionally stores 8 bytes per lane and tile
+// (4 KiB per block and tile, 6 % of what it reads) to dst, as those kernels do for the H2O bookkeeping.
+constexpr int kMixTileBytes = 512 * 8 * 16;
+template <bool STORES>
+__global__ __launch_bounds__(512) void mixed_probe_kernel(const uint4* __restrict__ src, uint2* __restrict__ dst,
+                                                          int tiles, uint32_t* __restrict__ sink) {
+  const int tid = threadIdx.x;
+  const uint4* s = src + (int64_t)blockIdx.x * tiles * (kMixTileBytes / 16);
+  uint2* d = dst + (int64_t)blockIdx.x * tiles * 512;
+  uint4 a[8], b[8];
+  uint32_t acc = 0;
+  auto issue = [&](int t, uint4* r) {   // a tile past the end repeats the last one
+    const int tt = t < tiles ? t : tiles - 1;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) r[u] = s[(int64_t)tt * (kMixTileBytes / 16) + u * 512 + tid];
+  };
+  auto use = [&](const uint4* r) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= r[u].x ^ r[u].y ^ r[u].z ^ r[u].w;
+  };
+  issue(0, a);
+  asm volatile("" ::: "memory");
+  issue(1, b);
+  asm volatile("" ::: "memory");
+  for (int t = 0; t < tiles; t += 2) {   // tiles is even
+    use(a);
+    asm volatile("" ::: "memory");
+    issue(t + 2, a);
+    asm volatile("" ::: "memory");
+    if constexpr (STORES) d[(int64_t)t * 512 + tid] = make_uint2(acc, (uint32_t)t);
+    use(b);
+    asm volatile("" ::: "memory");
+    issue(t + 3, b);
+    asm volatile("" ::: "memory");
+    if constexpr (STORES) d[(int64_t)(t + 1) * 512 + tid] = make_uint2(acc, (uint32_t)t);
+  }
+  if (acc == 0x9e3779b9u && sink) sink[0] = acc;
+}
+
 }  // namespace pikv
 
 using namespace pikv;
 
-// 0 on success, negative on a bad argument or a refused launch.
+// 0 on success, negative on a bad argument or a refused launch.  Modes 3 and 4: `bytes` (read from src) must be a
+// multiple of 8 MiB; mode 4 writes bytes / 16 to the front of dst.
 extern "C" int bench_stream_probe(int mode, const void* src, void* dst, int64_t bytes, int streaming_stores,
                                  void* sink, void* stream) {
+  if (mode == 3 || mode == 4) {
+    // 128 tiles per block; every address the kernel forms lies inside src[0, bytes) and dst[0, bytes / 16)
+    constexpr int tiles = 128;
+    if (!src || (mode == 4 && !dst) || bytes <= 0 || bytes % ((int64_t)tiles * kMixTileBytes) != 0) return -2;
+    const int64_t nb = bytes / ((int64_t)tiles * kMixTileBytes);
+    if (nb > 0x7fffffffLL) return -2;
+    hipStream_t st3 = (hipStream_t)stream;
+    if (mode == 3)
+      hipLaunchKernelGGL((mixed_probe_kernel<false>), dim3((unsigned)nb), dim3(512), 0, st3,
+                         reinterpret_cast<const uint4*>(src), reinterpret_cast<uint2*>(dst), tiles,
+                         reinterpret_cast<uint32_t*>(sink));
+    else
+      hipLaunchKernelGGL((mixed_probe_kernel<true>), dim3((unsigned)nb), dim3(512), 0, st3,
+                         reinterpret_cast<const uint4*>(src), reinterpret_cast<uint2*>(dst), tiles,
+                         reinterpret_cast<uint32_t*>(sink));
+    return hipGetLastError() == hipSuccess ? 0 : -5;
+  }
   if (mode < 0 || mode > 2) return -3;
   if ((mode != 1 && !src) || (mode != 0 && !dst)) return -1;
   if (bytes < 0 || bytes % 16 != 0) return -2;
