@@ -48,8 +48,10 @@ Pinning status (what, besides this file, fixes each function's output):
                                        orders, conservation, monotone budgets) and the
                                        frozen digests of tests/golden
 The reference's own tests hold no golden vectors for any of these.  Parity
-unpinned: none of the functions here; the end-to-end logits of the reference's
-PiKVMoE module graph are not restated in this file.
+unpinned: none of the functions here.  The end-to-end outputs of the reference's
+PiKVMoE module graph are not restated in this file: they are held as a fixture written
+by the reference's own module (tests/golden/make_ref_moe_golden.py ->
+tests/golden/ref_moe_forward.npz).
 """
 from __future__ import annotations
 
