@@ -232,6 +232,10 @@ def decode_read_workload(torch, ops, dev, iters):
     t_fused_nb = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=2.0, accumulate=False), iters)
     t_att_acc = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats, accumulate=True, now=1.0), iters)
     pool.fill.fill_(N)
+    # the plain gather + dequantise of the metric's name over this cache format: the K rows of 8 of the 64 sequences
+    gd_rows = 8 * N
+    t_gd32 = _median_ms(torch, lambda: pool.gather_dequant("k", row0=0, n=gd_rows), iters)
+    t_gd16 = _median_ms(torch, lambda: pool.gather_dequant("k", row0=0, n=gd_rows, out_dtype=torch.bfloat16), iters)
 
     # Eviction with a realistic state every time: importance as accumulated above, timestamps =
     # token positions (the recent rows are the tail).  Without the restore the second call would
@@ -268,6 +272,10 @@ def decode_read_workload(torch, ops, dev, iters):
         "gather_dequant_scores": _entry(t_scores, k_bytes + q_bytes, traffic_bytes=k_bytes + q_bytes + score_bytes,
                                         cached_tokens_per_s=rows / (t_scores * 1e-3),
                                         what="public float score matrix [cache, head, token] + tile statistics"),
+        "gather_dequant_f32": _entry(t_gd32, gd_rows * (D // 2 + (D // 32) * 4) + gd_rows * D * 4, rows=gd_rows,
+                                     what="pikv_gather_dequant, K rows of 8 sequences (262144 rows) -> float32: "
+                                          "640 B read and 4096 B written per row"),
+        "gather_dequant_bf16": _entry(t_gd16, gd_rows * (D // 2 + (D // 32) * 4) + gd_rows * D * 2, rows=gd_rows),
         "h2o_accumulate": _entry(t_h2o, acc_rw, traffic_bytes=score_bytes + acc_rw + rows * 4,
                                  what="reads the float score matrix; only the accumulators are algorithmic"),
         "attend_values": _entry(t_att, k_bytes, traffic_bytes=k_bytes + score_bytes),
