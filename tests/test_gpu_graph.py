@@ -126,13 +126,15 @@ def test_decode_read_replays(dev):
         assert bool((pool.ts[~valid] == -1.0).all()), rep
 
 
-@pytest.mark.parametrize("hkv,hq,dh", [
-    (8, 32, 128),     # the decode shape
-    (2, 24, 128),     # 12 q heads per kv head: two launches of each kernel, pairs of neighbouring rows as one
-    (1, 4, 128),      # one kv head: four neighbouring rows as one
-    (2, 14, 64),      # heads of 64, 14 q heads on the one slab
+@pytest.mark.parametrize("hkv,hq,dh,eight", [
+    (8, 32, 128, False),     # the decode shape: one pass over K and V
+    (2, 24, 128, False),     # 12 q heads per kv head: two launches of each kernel, pairs of neighbouring rows as one
+    (1, 4, 128, False),      # one kv head: four neighbouring rows as one
+    (2, 14, 64, False),      # heads of 64, 14 q heads on the one slab
+    (8, 64, 128, True),      # 8-bit codes, 8 q heads per kv head: the one-pass form, two blocks per token range
+    (3, 12, 128, True),      # ... 3 kv heads x 4: records of 32 lanes
 ])
-def test_decode_attend_replays(dev, hkv, hq, dh):
+def test_decode_attend_replays(dev, hkv, hq, dh, eight):
     """The one-call decode read under capture: its workspace is allocated before the capture, and every
     replay must rebuild the attention output and the H2O accumulators from scribbled memory."""
     import torch
@@ -143,7 +145,8 @@ def test_decode_attend_replays(dev, hkv, hq, dh):
     lens = torch.tensor([4500, 2049, 64], dtype=torch.int32, device=dev)
 
     def filled():
-        pool = ops.CachePool([N] * B, hkv, dh, 32, ops.Q_I4_ASYM, dev, with_v=True)
+        pool = (ops.CachePool([N] * B, hkv, dh, dh, ops.Q_I8_ASYM, dev, with_v=True) if eight else
+                ops.CachePool([N] * B, hkv, dh, 32, ops.Q_I4_ASYM, dev, with_v=True))
         gg = torch.Generator(device=dev).manual_seed(10)
         ks = torch.randn(B * N, D, generator=gg, device=dev).to(torch.bfloat16)
         vs = torch.randn(B * N, D, generator=gg, device=dev).to(torch.bfloat16)
