@@ -1,4 +1,4 @@
-// The decode read over a 4-bit cache as ONE pass: scores, running softmax and attention
+// The decode read over a compressed cache as ONE pass: scores, running softmax and attention
 // output in the same kernel, so that no score matrix ever exists in memory.
 //
 // Replaces, for one new token per sequence, the reference's
@@ -6,18 +6,20 @@
 // (core/single/pikv_attention.py:123,163,188) over the dequantised cache, and feeds
 // H2OScheduler.update_attention_scores (core/single/cache_scheduling.py:69-73).
 //
-// Served here: 4-bit codes in groups of 32 (half scale / zero point), heads of 128 dimensions,
-// 1..8 kv heads, 1..4 query heads per kv head, bf16 queries.  Everything else keeps the
-// two-kernel forms of read_path.hip / attend.hip.
+// Served here: heads of 128 dimensions, 2..8 kv heads, bf16 queries; 4-bit codes in groups of 32
+// (half scale / zero point) with 1..4 query heads per kv head (decode_fused_i4_kernel), 8-bit
+// codes with a float scale per kv head or coarser and 1..8 (decode_fused_i8_kernel, further
+// down).  Everything else keeps the two-kernel forms of read_path.hip / attend.hip.
 //
 // Division of labour: a WAVEFRONT owns one kv head of one token range of one cache and walks it
 // in tiles of 64 cached tokens - its K codes go straight from memory into matrix-core operands,
 // its V codes through a wavefront-private piece of LDS (they are needed transposed), its scores
 // never leave registers: the lane that receives the score of (head r, token t) from the
-// matrix core is the lane that turns it into the weight rows of the second product.  Nothing is
-// shared between the wavefronts of a block, so the tile loop has no block barrier; a block is
-// the kv heads of one token range only so that whole cached rows are in flight together.
-// Two tiles are on their way from memory per wavefront (two register sets).
+// matrix core is the lane that turns it into the weight rows of the second product.  The
+// wavefronts of a block share no data, but they share cache lines (the pieces of a cached row,
+// the metadata rows): one block barrier per tile keeps them on the same tile, and the
+// metadata of a tile is loaded once for the whole block, a tile ahead.  The 4-bit kernel has two
+// tiles on their way from memory per wavefront (two register sets), the 8-bit kernel one.
 //
 // Softmax over a token range that is still being read: the running maximum m of every head
 // (flash-decoding).  When a tile raises it, the accumulators are scaled by exp(m_old - m_new)
@@ -30,7 +32,10 @@
 // and m_at_that_tile per (tile, head); decode_importance_kernel turns them into probabilities
 // (e * exp(m_tile - M) / Z) and adds them to the accumulators.  A sum of positive terms each
 // within 2^-11 stays within 2^-11: inside the 1e-3 bar of the accumulators.  The attention
-// output never sees the halves.
+// output never sees the halves.  These stores are what the bookkeeping costs: a compute unit
+// whose read stream is saturated takes about 17 cycles per 64-byte write request, during which
+// it issues no load addresses (0.8 us per MB written, whatever the size, place or scope of the
+// stores; the bare loop shape shows the same in bench_probe.hip).
 #include "common.hpp"
 
 namespace pikv {
@@ -1024,8 +1029,8 @@ namespace pikv {
 // LDS, so a compute unit holds 8 / n_kv_heads of them (at most 8 wavefronts' pieces fit); the longest
 // range that still fills the chip wins, and it is never shorter than `min_tpb` (the workspace is
 // laid out for that many ranges).
-// Rows of 8 (6) kv heads go as two blocks of 4 (3) wavefronts per token range: two independent blocks per
-// compute unit fill each other's waits, where one block of eight wavefronts meets at one barrier per tile.
+// (4-bit rows as two blocks of half the kv heads per token range measured slower - 662 vs 632 us at 8 kv
+// heads: the halves of a 128-byte line then belong to different blocks and the metadata is fetched 1.75 x.)
 static int fused_groups(int n_kv_heads) { (void)n_kv_heads; return 1; }
 // the 8-bit pass: its wavefronts share no code lines (a kv head's 128 bytes of a row are a line of their own)
 static int fused8_blocks_per_range(int n_kv_heads) { return (n_kv_heads == 8 || n_kv_heads == 6) ? 2 : 1; }
@@ -1051,11 +1056,16 @@ int fused_tokens_per_block(int n_caches, int n_kv_heads, int64_t max_len, int mi
 }
 
 // Which calls take the one-pass form (measured against the two-kernel forms at 64 caches x 32768 tokens,
-// one process, alternating): without bookkeeping every geometry from 2 kv heads on (8 kv x 32 q heads
-// 625 -> 524 us, 4 x 16: 333 -> 266, 6 x 24: 499 -> 418, 2 x 8: 194 -> 177; 1 x 4: 122 vs 128, left alone);
+// one process, alternating).  4-bit: without bookkeeping every geometry from 2 kv heads on (8 kv x 32 q heads
+// 625 -> 502 us, 4 x 16: 333 -> 266, 6 x 24: 499 -> 418, 2 x 8: 194 -> 177; 1 x 4: 122 vs 128, left alone);
 // with bookkeeping only four query heads per kv head on at least 3 kv heads (3 x 12: 306 -> 297,
-// 6 x 24: 552 -> 537, 8 x 32: 675 vs 677 - the halves cost the pass 0.1 ms, see the kernel's comment; with
+// 6 x 24: 552 -> 537, 8 x 32: 660-680 -> 643 - the halves cost the pass 0.1 ms, see the top of this file; with
 // fewer query heads per kv head the float rows of the two-kernel form are the smaller exchange).
+// 8-bit: everything it can hold, with / without bookkeeping - 8 kv x 64 q heads 1225 -> 1032 / 1148 -> 788 us,
+// 8 x 32: 1107 -> 956 / 1031 -> 786, 8 x 16: 1053 -> 962 / 981 -> 779, 6 x 24: 972 -> 743 / 898 -> 580,
+// 4 x 16: 619 -> 516 / 541 -> 391, 3 x 12: 519 -> 392 / 442 -> 304, 2 x 8: 361 -> 292 / 297 -> 244,
+// 8 x 8 without bookkeeping 826 -> 777 (with it the records of one head per kv head do not fit the workspace
+// piece the float scores would take: two-kernel form, 853 us).
 bool decode_fused_serves(int scheme, int group, int n_kv_heads, int n_q_heads, int head_dim, int q_dtype, bool bookkeeping) {
   if (head_dim != 128 || q_dtype != PIKV_BF16) return false;
   if (n_kv_heads < 2 || n_kv_heads > 8 || n_q_heads % n_kv_heads != 0) return false;
