@@ -403,7 +403,8 @@ int64_t pikv_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim,
  *   H2OScheduler.update_attention_scores (core/single/cache_scheduling.py:69-73).
  * Same results as pikv_gather_dequant_scores + pikv_h2o_accumulate + pikv_attend_values
  * (to the float tolerance of those), but the score matrix never leaves the library.
- * Caches of 2 to 8 kv heads of 128 dimensions read by bf16 queries take ONE pass over K and V
+ * Caches of 2 to 8 kv heads of 128 dimensions read by bf16 queries (8-bit codes: float32 queries
+ * too, as two bf16 limbs) take ONE pass over K and V
  * (scores, running softmax and attention output per 64-token tile, no score matrix at all;
  * exp(score - running maximum) leaves the pass as a half per head and token for the
  * accumulators only): 4-bit codes in groups of 32 with up to 4 query heads per kv head

@@ -1516,7 +1516,7 @@ extern "C" int pikv_decode_attend(const void* k_codes, const void* k_scale, cons
       n_caches <= 65535) {
     const int tpb = fused_tokens_per_block(n_caches, n_kv_heads, max_len, attend_tokens_per_block(n_caches, max_len));
     return decode_fused_launch(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, scheme, group, n_kv_heads, n_q_heads, q,
-                               scale_qk, cache_row_base, cache_fill, n_caches, max_len, tpb, decay, now, row_acc, row_ts,
+                               q_dtype, scale_qk, cache_row_base, cache_fill, n_caches, max_len, tpb, decay, now, row_acc, row_ts,
                                out, ws + w.scores, tmax, tsum, reinterpret_cast<float*>(partial), stats, st);
   }
   // the 4-bit matrix-core kernels meeting in the exchange format

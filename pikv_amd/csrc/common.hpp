@@ -444,12 +444,12 @@ int scores_exchange_launch(const void* k_codes, const void* k_scale, const void*
 
 // decode_fused.hip, for pikv_decode_attend in attend.hip: the one-pass decode read (heads of 128, 2 to 8
 // kv heads, bf16 queries; 4-bit codes in groups of 32 with up to 4 query heads per kv head - with the H2O
-// bookkeeping exactly 4 -, 8-bit codes with a scale per kv head or coarser and up to 8).
+// bookkeeping exactly 4 -, 8-bit codes with a scale per kv head or coarser and up to 8, float32 queries too).
 bool decode_fused_serves(int scheme, int group, int n_kv_heads, int n_q_heads, int head_dim, int q_dtype, bool bookkeeping);
 int fused_tokens_per_block(int n_caches, int n_kv_heads, int64_t max_len, int min_tpb);
 int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_zero, const void* v_codes,
                         const void* v_scale, const void* v_zero, int scheme, int group, int n_kv_heads, int n_q_heads,
-                        const void* q, float scale_qk, const int64_t* cache_row_base, const int32_t* cache_fill,
+                        const void* q, int q_dtype, float scale_qk, const int64_t* cache_row_base, const int32_t* cache_fill,
                         int n_caches, int64_t max_len, int tokens_per_block, float decay, float now, float* row_acc,
                         float* row_ts, float* out, void* e16, float* tref, float* pstats, float* partial,
                         float* head_stats, hipStream_t st);

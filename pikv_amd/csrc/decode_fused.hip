@@ -471,7 +471,7 @@ struct Fused8Args {
   const void* v_codes;
   const void* v_scale;
   const void* v_zero;
-  const void* q;            // bf16 [cache][n_q_heads][128]
+  const void* q;            // bf16 (float32 for the QF32 kernels) [cache][n_q_heads][128]
   const int64_t* row_base;
   const int32_t* fill;
   float* partial;           // [range][cache][q head][128]
@@ -502,7 +502,9 @@ __device__ __forceinline__ uint2 bytes_to_bf16(uint32_t w) {
                     __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf2)));
 }
 
-template <int SCHEME, bool BOOK>
+// QF32: float32 queries as two bf16 limbs, q = hi + lo to 2^-17 |q| (hi = the float cut to its upper 16 bits, lo = the
+// rest rounded to bf16); both limbs are multiplied with the same converted codes into the same accumulators.
+template <int SCHEME, bool BOOK, bool QF32 = false>
 __global__ __launch_bounds__(512) void decode_fused_i8_kernel(Fused8Args a) {
   using Q = QScheme<SCHEME>;
   static_assert(Q::bits == 8, "8-bit schemes only");
@@ -553,22 +555,40 @@ __global__ __launch_bounds__(512) void decode_fused_i8_kernel(Fused8Args a) {
   const float* const vzb = reinterpret_cast<const float*>(a.v_zero) + urow * gpr + m_ent;
 
   // ---- queries: A rows = the kv head's query heads, k-step (half, o) = dimensions 64 half + 16 rg + 8 o .. + 7 ----
-  uint4 aq[4];
+  uint4 aq[4], aql[QF32 ? 4 : 1];
   float qs0, qs1;   // sum of the head's query over the dimensions of half 0 / half 1 (lane's row nl)
   {
     const bool a_on = nl < rep;
-    const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)c * a.n_q_heads + g * rep + (a_on ? nl : 0)) * 128 + rg * 16;
+    const int64_t qoff = ((int64_t)c * a.n_q_heads + g * rep + (a_on ? nl : 0)) * 128 + rg * 16;
     float part[2] = {0.f, 0.f};
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      uint4 d = make_uint4(0, 0, 0, 0);
-      if (a_on) d = ld16(qp + (k >> 1) * 64 + (k & 1) * 8);
-      aq[k] = d;
-      const uint32_t w[4] = {d.x, d.y, d.z, d.w};
+      const int64_t eo = qoff + (k >> 1) * 64 + (k & 1) * 8;
+      if constexpr (QF32) {
+        const float* qf = reinterpret_cast<const float*>(a.q) + eo;
+        uint32_t hb[8], lb[8];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        part[k >> 1] += __uint_as_float(w[e] << 16);
-        part[k >> 1] += __uint_as_float(w[e] & 0xffff0000u);
+        for (int e = 0; e < 8; ++e) {
+          const float f = a_on ? qf[e] : 0.f;
+          const uint32_t h = __float_as_uint(f) & 0xffff0000u;
+          const uint32_t l = float_to_bf16_bits(f - __uint_as_float(h));
+          hb[e] = h >> 16;
+          lb[e] = l;
+          part[k >> 1] += __uint_as_float(h);
+          part[k >> 1] += __uint_as_float(l << 16);
+        }
+        aq[k] = make_uint4(hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16), hb[4] | (hb[5] << 16), hb[6] | (hb[7] << 16));
+        aql[k] = make_uint4(lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16), lb[4] | (lb[5] << 16), lb[6] | (lb[7] << 16));
+      } else {
+        uint4 d = make_uint4(0, 0, 0, 0);
+        if (a_on) d = ld16(reinterpret_cast<const uint16_t*>(a.q) + eo);
+        aq[k] = d;
+        const uint32_t w[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          part[k >> 1] += __uint_as_float(w[e] << 16);
+          part[k >> 1] += __uint_as_float(w[e] & 0xffff0000u);
+        }
       }
     }
     part[0] += __shfl_xor(part[0], 16, PIKV_WAVE);
@@ -688,6 +708,12 @@ __global__ __launch_bounds__(512) void decode_fused_i8_kernel(Fused8Args a) {
                                                      __builtin_bit_cast(pikv_bf16x8, bo0), pc, 0, 0, 0);
         pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, aq[2 * half + 1]),
                                                      __builtin_bit_cast(pikv_bf16x8, bo1), pc, 0, 0, 0);
+        if constexpr (QF32) {
+          pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, aql[2 * half]),
+                                                       __builtin_bit_cast(pikv_bf16x8, bo0), pc, 0, 0, 0);
+          pc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, aql[2 * half + 1]),
+                                                       __builtin_bit_cast(pikv_bf16x8, bo1), pc, 0, 0, 0);
+        }
       }
       const float2 km = kmeta[4 * nl + s];
       const float f = km.x * a.scale_qk;
@@ -1067,7 +1093,8 @@ int fused_tokens_per_block(int n_caches, int n_kv_heads, int64_t max_len, int mi
 // 8 x 8 without bookkeeping 826 -> 777 (with it the records of one head per kv head do not fit the workspace
 // piece the float scores would take: two-kernel form, 853 us).
 bool decode_fused_serves(int scheme, int group, int n_kv_heads, int n_q_heads, int head_dim, int q_dtype, bool bookkeeping) {
-  if (head_dim != 128 || q_dtype != PIKV_BF16) return false;
+  const bool eight = scheme == PIKV_Q_I8_SYM || scheme == PIKV_Q_I8_ASYM;
+  if (head_dim != 128 || !(q_dtype == PIKV_BF16 || (eight && q_dtype == PIKV_F32))) return false;
   if (n_kv_heads < 2 || n_kv_heads > 8 || n_q_heads % n_kv_heads != 0) return false;
   const int rep = n_q_heads / n_kv_heads;
   if (scheme == PIKV_Q_I8_SYM || scheme == PIKV_Q_I8_ASYM) {
@@ -1088,7 +1115,7 @@ bool decode_fused_serves(int scheme, int group, int n_kv_heads, int n_q_heads, i
 //   pstats  splits * n_caches * n_q_heads * 2 floats          partial splits * n_caches * n_q_heads * 128 floats
 int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_zero, const void* v_codes,
                         const void* v_scale, const void* v_zero, int scheme, int group, int n_kv_heads, int n_q_heads,
-                        const void* q, float scale_qk, const int64_t* cache_row_base, const int32_t* cache_fill,
+                        const void* q, int q_dtype, float scale_qk, const int64_t* cache_row_base, const int32_t* cache_fill,
                         int n_caches, int64_t max_len, int tokens_per_block, float decay, float now, float* row_acc,
                         float* row_ts, float* out, void* e16, float* tref, float* pstats, float* partial,
                         float* head_stats, hipStream_t st) {
@@ -1096,6 +1123,8 @@ int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_
   const int64_t splits = (max_len + tokens_per_block - 1) / tokens_per_block;
   if (splits > 65535 || (tokens_per_block & 127) != 0) return PIKV_ERR_SHAPE;
   const bool book = row_acc != nullptr || row_ts != nullptr;
+  if (q_dtype != PIKV_BF16 && !(q_dtype == PIKV_F32 && (scheme == PIKV_Q_I8_SYM || scheme == PIKV_Q_I8_ASYM)))
+    return PIKV_ERR_UNSUPPORTED;
   if (scheme == PIKV_Q_I8_SYM || scheme == PIKV_Q_I8_ASYM) {
     const int64_t n_tiles8 = (max_len + kFTile - 1) / kFTile;   // this pass never touches a tile past a range's end
     Fused8Args a8{k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, q, cache_row_base, cache_fill, partial, pstats,
@@ -1106,13 +1135,20 @@ int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_
     const dim3 block8((unsigned)(n_kv_heads / a8.blocks_per_range * 64));
     const size_t lds8 = (size_t)(n_kv_heads / a8.blocks_per_range) * k8WaveLds;
     const bool wr8 = row_acc != nullptr;
+#define PIKV_FUSED8(S, F)                                                                                   \
+  do {                                                                                                      \
+    if (wr8) hipLaunchKernelGGL((decode_fused_i8_kernel<S, true, F>), grid8, block8, lds8, st, a8);         \
+    else hipLaunchKernelGGL((decode_fused_i8_kernel<S, false, F>), grid8, block8, lds8, st, a8);            \
+  } while (0)
+    const bool qf = q_dtype == PIKV_F32;
     if (scheme == PIKV_Q_I8_SYM) {
-      if (wr8) hipLaunchKernelGGL((decode_fused_i8_kernel<PIKV_Q_I8_SYM, true>), grid8, block8, lds8, st, a8);
-      else hipLaunchKernelGGL((decode_fused_i8_kernel<PIKV_Q_I8_SYM, false>), grid8, block8, lds8, st, a8);
+      if (qf) PIKV_FUSED8(PIKV_Q_I8_SYM, true);
+      else PIKV_FUSED8(PIKV_Q_I8_SYM, false);
     } else {
-      if (wr8) hipLaunchKernelGGL((decode_fused_i8_kernel<PIKV_Q_I8_ASYM, true>), grid8, block8, lds8, st, a8);
-      else hipLaunchKernelGGL((decode_fused_i8_kernel<PIKV_Q_I8_ASYM, false>), grid8, block8, lds8, st, a8);
+      if (qf) PIKV_FUSED8(PIKV_Q_I8_ASYM, true);
+      else PIKV_FUSED8(PIKV_Q_I8_ASYM, false);
     }
+#undef PIKV_FUSED8
     PIKV_CHECK_LAUNCH();
     const int64_t total8 = (int64_t)n_caches * n_q_heads * 128;
     hipLaunchKernelGGL(decode_finish_kernel, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, st, partial, pstats,

@@ -236,6 +236,9 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I8_SYM, 512, 4, 8, 128, "bf16"),    # ... a scale per token, 2 q heads per kv head: records of 32 lanes
     (O.Q_I8_ASYM, 128, 7, 14, 128, "bf16"),  # ... 7 kv heads x 2
     (O.Q_I8_SYM, 128, 5, 5, 128, "bf16"),    # ... one q head per kv head: one pass only without the bookkeeping
+    (O.Q_I8_SYM, 128, 8, 32, 128, "f32"),    # ... float32 queries as two bf16 limbs
+    (O.Q_I8_ASYM, 128, 4, 32, 128, "f32"),   # ... 8 q heads per kv head, zero points
+    (O.Q_I8_ASYM, 256, 6, 18, 128, "f32"),   # ... 6 kv heads x 3: two blocks of three wavefronts, a scale per pair of heads
 ])
 @pytest.mark.parametrize("decay", [1.0, 0.9])
 def test_decode_attend_one_call(dev, scheme, group, heads, hq, dh, qdtype, decay):
