@@ -328,7 +328,7 @@ int pikv_gather_dequant(const void* codes, const void* scale, const void* zero,
  *   either q_dtype (more query heads: PIKV_ERR_UNSUPPORTED).  float32 queries against 4-bit group-32 caches, or 8-bit caches
  *   with a scale per kv head or coarser, with up to 8 query heads per 128 dimensions
  *   of kv heads are multiplied on the matrix cores as two bf16 limbs (q = hi + lo to
- *   2^-17 |q|; float32 accumulation). */
+ *   2^-18 |q|; float32 accumulation). */
 #define PIKV_SCORE_TILE 64
 int pikv_gather_dequant_scores(const void* k_codes, const void* k_scale,
                                const void* k_zero, int scheme, int group,
@@ -403,13 +403,13 @@ int64_t pikv_attend_workspace_bytes(int n_caches, int n_q_heads, int head_dim,
  *   H2OScheduler.update_attention_scores (core/single/cache_scheduling.py:69-73).
  * Same results as pikv_gather_dequant_scores + pikv_h2o_accumulate + pikv_attend_values
  * (to the float tolerance of those), but the score matrix never leaves the library.
- * Caches of 2 to 8 kv heads of 128 dimensions read by bf16 queries (8-bit codes: float32 queries
- * too, as two bf16 limbs) take ONE pass over K and V
- * (scores, running softmax and attention output per 64-token tile, no score matrix at all;
- * exp(score - running maximum) leaves the pass as a half per head and token for the
- * accumulators only): 4-bit codes in groups of 32 with up to 4 query heads per kv head
- * (with row_acc: exactly 4, on 3 or more kv heads), 8-bit codes with a scale per kv head or
- * coarser and up to 8 (with row_acc: 2 to 8).  Otherwise, for
+ * Caches of 2 to 8 kv heads of 128 dimensions take ONE pass over K and V (scores, running
+ * softmax and attention output per 64-token tile, no score matrix at all; exp(score - running
+ * maximum) leaves the pass as a half per head and token for the accumulators only): 4-bit
+ * codes in groups of 32 with up to 4 bf16 or float32 query heads per kv head (with row_acc:
+ * exactly 4, on 3 or more kv heads) or 5 to 8 bf16 ones (3 or more kv heads), 8-bit codes
+ * with a scale per kv head or coarser and up to 8 bf16 or float32 ones (with row_acc: 2 to 8);
+ * float32 queries go in as two bf16 limbs.  Otherwise, for
  * 4-bit caches with group 32, rows that are 1 to 8 slabs of 128 dimensions, or whole groups
  * of 8 kv heads of 128 dimensions (a slab is one kv
  * head of 128 dimensions, two of 64 or four of 32) and up to 8 query heads per slab (5 to 8

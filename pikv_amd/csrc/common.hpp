@@ -29,6 +29,15 @@ __device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
   return u >> 16;
 }
 
+// A float32 value as two bf16 limbs, f = hi + lo to 2^-18 |f|: hi = f rounded to bf16 (cut to its upper 16
+// bits instead where rounding would carry a finite value to infinity), lo = the rest rounded to bf16.  A value
+// that is a bf16 number gives (itself, 0).  Returns the bits of limb `which`.
+__device__ __forceinline__ uint32_t bf16_limb_bits(float f, int which) {
+  uint32_t h = float_to_bf16_bits(f);
+  if ((h & 0x7f80u) == 0x7f80u && (__float_as_uint(f) & 0x7f800000u) != 0x7f800000u) h = __float_as_uint(f) >> 16;
+  return which == 0 ? h : float_to_bf16_bits(f - __uint_as_float(h << 16));
+}
+
 // float -> half, round to nearest even, finite values saturate at +-65504.
 __device__ __forceinline__ _Float16 float_to_half_sat(float f) {
   if (f > 65504.0f && f < __builtin_inff()) return (_Float16)65504.0f;
@@ -443,8 +452,8 @@ int scores_exchange_launch(const void* k_codes, const void* k_scale, const void*
                            float* escores, float* tile_max, float* tile_sum, float* head_stats, hipStream_t st);
 
 // decode_fused.hip, for pikv_decode_attend in attend.hip: the one-pass decode read (heads of 128, 2 to 8
-// kv heads, bf16 queries; 4-bit codes in groups of 32 with up to 4 query heads per kv head - with the H2O
-// bookkeeping exactly 4 -, 8-bit codes with a scale per kv head or coarser and up to 8, float32 queries too).
+// kv heads; 4-bit codes in groups of 32 with up to 4 bf16 or float32 query heads per kv head, or 5 to 8 bf16
+// ones; 8-bit codes with a scale per kv head or coarser and up to 8 bf16 or float32 ones).
 bool decode_fused_serves(int scheme, int group, int n_kv_heads, int n_q_heads, int head_dim, int q_dtype, bool bookkeeping);
 int fused_tokens_per_block(int n_caches, int n_kv_heads, int64_t max_len, int min_tpb);
 int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_zero, const void* v_codes,

@@ -6,10 +6,11 @@
 // (core/single/pikv_attention.py:123,163,188) over the dequantised cache, and feeds
 // H2OScheduler.update_attention_scores (core/single/cache_scheduling.py:69-73).
 //
-// Served here: heads of 128 dimensions, 2..8 kv heads, bf16 queries; 4-bit codes in groups of 32
-// (half scale / zero point) with 1..4 query heads per kv head (decode_fused_i4_kernel), 8-bit
-// codes with a float scale per kv head or coarser and 1..8 (decode_fused_i8_kernel, further
-// down).  Everything else keeps the two-kernel forms of read_path.hip / attend.hip.
+// Served here: heads of 128 dimensions, 2..8 kv heads; 4-bit codes in groups of 32 (half scale /
+// zero point) with 1..4 bf16 query heads per kv head (decode_fused_i4_kernel), with 5..8, or with
+// 1..4 float32 ones (decode_fused_i4w_kernel); 8-bit codes with a float scale per kv head or
+// coarser and 1..8 bf16 or float32 ones (decode_fused_i8_kernel).  Everything else keeps the
+// two-kernel forms of read_path.hip / attend.hip.
 //
 // Division of labour: a WAVEFRONT owns one kv head of one token range of one cache and walks it
 // in tiles of 64 cached tokens - its K codes go straight from memory into matrix-core operands,
@@ -436,6 +437,385 @@ __global__ __launch_bounds__(512) void decode_fused_i4_kernel(FusedArgs a) {
   }
 }
 
+// ---- the 4-bit pass with TWO sets of query operands ------------------------------------------------
+// The block-diagonal A operand above holds four query heads (rows = 4 groups x 4 heads).  A second operand
+// set, multiplied with the same expanded codes, serves either heads 4..7 of the kv head (5 to 8 bf16 query
+// heads per kv head) or the low limbs of float32 queries (QF32: q = hi + lo to 2^-18 |q|, hi = the float rounded
+// to bf16, lo = the rest rounded to bf16; the two sets' scores of a head are added, everything
+// after that is the one-set kernel's).  What changes besides: a lane runs the softmax of TWO heads (rg and
+// 4 + rg) x four tokens; the weight rows of eight heads x two parts fill all 16 A rows of the output product,
+// which therefore runs in two passes of two groups each through the same 4.6 KB of LDS; and there is ONE
+// register set for the codes on their way (the second operand set and the second head's state take the
+// registers of the other one), refilled as in the 8-bit kernel: V as soon as the tile's codes are staged, K
+// as soon as its scores are done.  Bookkeeping records: one per (kv head, operand set), each laid out as the
+// one-set kernel's (QF32: that kernel's records exactly).
+template <int SCHEME, bool BOOK, bool QF32>
+__global__ __launch_bounds__(512) void decode_fused_i4w_kernel(FusedArgs a) {
+  using Q = QScheme<SCHEME>;
+  static_assert(Q::bits == 4, "4-bit schemes only");
+  constexpr int NH = QF32 ? 1 : 2;   // query heads per lane: rg (and 4 + rg)
+  extern __shared__ __align__(16) unsigned char fused_lds[];
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  unsigned char* const lds = fused_lds + wv * kFWaveLds;
+  unsigned char* const vcodes = lds + kFVCodes;
+  unsigned char* const abuf = lds + kFABuf;     // [2 groups][16 rows][kFARow]
+  unsigned char* const azero = lds + kFAZero;
+
+  const int c = blockIdx.x;
+  const int xr = blockIdx.y;
+  const int HK = a.n_kv_heads;
+  const int g = wv;
+  const int rep = a.n_q_heads / HK;
+  const int64_t len = a.fill[c] < a.max_len ? (int64_t)a.fill[c] : a.max_len;
+  const int64_t t0 = (int64_t)xr * a.tokens_per_block;
+  if (t0 >= len) return;   // the merge skips ranges that hold no token
+  const int span = (int)((t0 + a.tokens_per_block < len ? t0 + a.tokens_per_block : len) - t0);
+  const int last = span - 1;
+
+  const int nl = lane & 15, rg = lane >> 4;
+  const int i = nl, kg = rg;
+  const int wkg = nl >> 2, qd = nl & 3;
+  const int tk = wkg * 16 + qd;
+  bool row_on[NH];
+#pragma unroll
+  for (int k = 0; k < NH; ++k) row_on[k] = rg + 4 * k < rep;
+  const float zbias = 128.0f - (float)Q::qmin;
+  const int row_codes = HK * 64, row_meta = HK * 8;
+  const int64_t urow = a.row_base[c] + t0;
+  const char* const kc = reinterpret_cast<const char*>(a.k_codes) + urow * row_codes + g * 64;
+  const char* const vc = reinterpret_cast<const char*>(a.v_codes) + urow * row_codes + g * 64;
+
+  if (lane < 8) reinterpret_cast<uint32_t*>(azero)[lane] = 0u;
+
+  // metadata: thread e takes entry (token e / heads, head e % heads) of a tile's rows, one tile ahead
+  const int m_tok = threadIdx.x / HK, m_hd = threadIdx.x - m_tok * HK;
+  unsigned char* const m_lds = fused_lds + m_hd * kFWaveLds;
+  const char* const ksb = reinterpret_cast<const char*>(a.k_scale) + urow * row_meta + m_hd * 8;
+  const char* const kzb = reinterpret_cast<const char*>(a.k_zero) + urow * row_meta + m_hd * 8;
+  const char* const vsb = reinterpret_cast<const char*>(a.v_scale) + urow * row_meta + m_hd * 8;
+  const char* const vzb = reinterpret_cast<const char*>(a.v_zero) + urow * row_meta + m_hd * 8;
+
+  // ---- queries: two block-diagonal A operand sets.  Row nl = 4 * group + head of the set; a lane's k-slice
+  // rg meets its row's group only when nl / 4 == rg.  Set s holds heads 4 s .. 4 s + 3 (QF32: limb s of heads 0..3).
+  uint4 aq[2][4];
+  float4 qv[2];
+#pragma unroll
+  for (int st = 0; st < 2; ++st) {
+    const int head = QF32 ? (nl & 3) : 4 * st + (nl & 3);
+    const bool a_on = (nl >> 2) == rg && head < rep;
+    const int64_t qo = ((int64_t)c * a.n_q_heads + g * rep + (head < rep ? head : 0)) * 128 + rg * 32;
+    float qsum = 0.f;
+#pragma unroll
+    for (int b2 = 0; b2 < 4; ++b2) {
+      uint4 d = make_uint4(0, 0, 0, 0);
+      if constexpr (QF32) {
+        if (a_on) {
+          const float* qf = reinterpret_cast<const float*>(a.q) + qo + b2 * 8;
+          uint32_t e[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            e[k] = bf16_limb_bits(qf[k], st);
+          }
+          d = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
+        }
+      } else {
+        if (a_on) d = ld16(reinterpret_cast<const uint16_t*>(a.q) + qo + b2 * 8);
+      }
+      const uint32_t w[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        qsum += __uint_as_float(w[k] << 16);
+        qsum += __uint_as_float(w[k] & 0xffff0000u);
+      }
+      // element order inside a k-slice is {0,4,1,5,2,6,3,7}: what the nibble expansion yields
+      aq[st][b2] = make_uint4((d.x & 0xffffu) | (d.z << 16), (d.x >> 16) | (d.z & 0xffff0000u),
+                              (d.y & 0xffffu) | (d.w << 16), (d.y >> 16) | (d.w & 0xffff0000u));
+    }
+    // group sums of the set's four rows for this lane's group rg: held by lanes 20 * rg + row
+    qv[st].x = __shfl(qsum, 20 * rg + 0, PIKV_WAVE);
+    qv[st].y = __shfl(qsum, 20 * rg + 1, PIKV_WAVE);
+    qv[st].z = __shfl(qsum, 20 * rg + 2, PIKV_WAVE);
+    qv[st].w = __shfl(qsum, 20 * rg + 3, PIKV_WAVE);
+  }
+
+  pikv_f32x4 C[8];
+#pragma unroll
+  for (int d = 0; d < 8; ++d) C[d] = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
+  float zacc[NH][4], lsum[NH], m_run[NH];
+#pragma unroll
+  for (int k = 0; k < NH; ++k) {
+    lsum[k] = 0.f;
+    m_run[k] = -__builtin_inff();
+#pragma unroll
+    for (int sg = 0; sg < 4; ++sg) zacc[k][sg] = 0.f;
+  }
+
+  // A-operand piece of this lane in the output product: row i = (head i / 2, part i % 2) of a group's 16 rows
+  const bool arow_on = i < 2 * rep;
+  const unsigned char* const a_row = arow_on ? abuf + i * kFARow + kg * 32 : azero;
+  const int a_gstep = arow_on ? 16 * kFARow : 0;
+  uint32_t kNib = 0x000f000fu, kExp = 0x43004300u;
+  asm volatile("" : "+v"(kNib), "+v"(kExp));   // both constants in vector registers: the and-or stays one instruction
+
+  uint4 rk[4], rv[4];
+  uint2 mks, mkz, mvs, mvz;
+  auto clamp_row = [&](int tok) { return tok < last ? tok : last; };
+  auto issue_meta = [&](int n0) {
+    const uint32_t mo = (uint32_t)(clamp_row(n0 + m_tok) * row_meta);
+    mks = *reinterpret_cast<const uint2*>(ksb + mo);
+    mvs = *reinterpret_cast<const uint2*>(vsb + mo);
+    mkz = make_uint2(0, 0);
+    mvz = make_uint2(0, 0);
+    if constexpr (!Q::sym) {
+      mkz = *reinterpret_cast<const uint2*>(kzb + mo);
+      mvz = *reinterpret_cast<const uint2*>(vzb + mo);
+    }
+  };
+  auto issue_v = [&](int n0) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      rv[k] = ld16(vc + (uint32_t)(clamp_row(n0 + 16 * k + (lane >> 2)) * row_codes + (lane & 3) * 16));
+  };
+  auto issue_k = [&](int n0) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      rk[s] = ld16(kc + (uint32_t)(clamp_row(n0 + tk + 4 * s) * row_codes + rg * 16));
+  };
+  auto h2f = [](uint32_t w, int hi) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> (16 * hi))); };
+  auto wave_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  auto pin_order = [] { asm volatile("" ::: "memory"); };
+  auto stage_meta = [&](int set) {
+    unsigned char* const mb = m_lds + set * kFMetaSet;
+    const int mo = fused_vmeta_off(m_tok);
+    *reinterpret_cast<float4*>(mb + kFVScale + mo) = make_float4(h2f(mvs.x, 0), h2f(mvs.x, 1), h2f(mvs.y, 0), h2f(mvs.y, 1));
+    *reinterpret_cast<float4*>(mb + kFVZterm + mo) = make_float4(h2f(mvz.x, 0) + zbias, h2f(mvz.x, 1) + zbias,
+                                                                 h2f(mvz.y, 0) + zbias, h2f(mvz.y, 1) + zbias);
+    float4* km = reinterpret_cast<float4*>(mb + kFKMeta + fused_kmeta_off(m_tok, 0));
+    km[0] = make_float4(h2f(mks.x, 0), h2f(mkz.x, 0) + zbias, h2f(mks.x, 1), h2f(mkz.x, 1) + zbias);
+    km[1] = make_float4(h2f(mks.y, 0), h2f(mkz.y, 0) + zbias, h2f(mks.y, 1), h2f(mkz.y, 1) + zbias);
+  };
+
+  issue_meta(0);
+  stage_meta(0);
+  pin_order();
+  issue_meta(kFTile);
+  issue_v(0);
+  pin_order();
+  issue_k(0);
+  pin_order();
+
+  for (int n0 = 0; n0 < span; n0 += kFTile) {
+    const int par = (n0 / kFTile) & 1;
+    __syncthreads();   // keeps the wavefronts on one tile, and publishes the metadata their threads wrote for each other
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      *reinterpret_cast<uint4*>(vcodes + (16 * k + (lane >> 2)) * kFCodeRow + (lane & 3) * 16) = rv[k];
+    stage_meta(par ^ 1);   // the NEXT tile's metadata, into the other set
+    wave_sync();
+    const unsigned char* const vscale = lds + kFVScale + par * kFMetaSet;
+    const unsigned char* const vzterm = lds + kFVZterm + par * kFMetaSet;
+    const unsigned char* const kmeta = lds + kFKMeta + par * kFMetaSet;
+    pin_order();
+    issue_v(n0 + kFTile);
+    issue_meta(n0 + 2 * kFTile);
+    pin_order();
+
+    // ---- scores of heads rg (and 4 + rg), tokens tk + 4 s ----
+    float sc[NH][4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const uint32_t wv4[4] = {rk[s].x, rk[s].y, rk[s].z, rk[s].w};
+      pikv_f32x4 pc0 = pikv_f32x4{0.f, 0.f, 0.f, 0.f}, pc1 = pikv_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int b2 = 0; b2 < 4; ++b2) {
+        const uint32_t w = Q::sym ? (wv4[b2] ^ 0x88888888u) : wv4[b2];
+        const uint4 bb = make_uint4(and_or(w, kNib, kExp), and_or(w >> 4, kNib, kExp), and_or(w >> 8, kNib, kExp),
+                                    and_or(w >> 12, kNib, kExp));
+        pc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, aq[0][b2]),
+                                                      __builtin_bit_cast(pikv_bf16x8, bb), pc0, 0, 0, 0);
+        pc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, aq[1][b2]),
+                                                      __builtin_bit_cast(pikv_bf16x8, bb), pc1, 0, 0, 0);
+      }
+      const int tok = tk + 4 * s;
+      const float2 km = *reinterpret_cast<const float2*>(kmeta + fused_kmeta_off(tok, rg));
+      float set_score[2];
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const pikv_f32x4 pc = st ? pc1 : pc0;
+        const float4 q4 = qv[st];
+        const float u0 = km.x * fmaf(-km.y, q4.x, pc[0]), u1 = km.x * fmaf(-km.y, q4.y, pc[1]);
+        const float u2 = km.x * fmaf(-km.y, q4.z, pc[2]), u3 = km.x * fmaf(-km.y, q4.w, pc[3]);
+        // sum over the four groups; row-group r ends with row r of the set
+        auto s01 = __builtin_amdgcn_permlane16_swap(__float_as_uint(u0), __float_as_uint(u1), false, false);
+        auto s23 = __builtin_amdgcn_permlane16_swap(__float_as_uint(u2), __float_as_uint(u3), false, false);
+        const float u01 = __uint_as_float(s01[0]) + __uint_as_float(s01[1]);
+        const float u23 = __uint_as_float(s23[0]) + __uint_as_float(s23[1]);
+        auto sf = __builtin_amdgcn_permlane32_swap(__float_as_uint(u01), __float_as_uint(u23), false, false);
+        set_score[st] = __uint_as_float(sf[0]) + __uint_as_float(sf[1]);
+      }
+      const bool tok_on = n0 + tok <= last;
+      if constexpr (QF32) {
+        sc[0][s] = (tok_on && row_on[0]) ? (set_score[0] + set_score[1]) * a.scale_qk : -__builtin_inff();
+      } else {
+        sc[0][s] = (tok_on && row_on[0]) ? set_score[0] * a.scale_qk : -__builtin_inff();
+        sc[NH - 1][s] = (tok_on && row_on[NH - 1]) ? set_score[1] * a.scale_qk : -__builtin_inff();
+      }
+    }
+    pin_order();
+    issue_k(n0 + kFTile);
+    pin_order();
+
+    // ---- running softmax of the lane's heads (all 16 lanes of a row-group hold the same statistics) ----
+    float alpha[NH], m_ref[NH], p4[NH][4];
+    bool moved = false;
+#pragma unroll
+    for (int k = 0; k < NH; ++k) {
+      const float m_tile = group_max_dpp(fmaxf(fmaxf(sc[k][0], sc[k][1]), fmaxf(sc[k][2], sc[k][3])), 16);
+      const float m_new = fmaxf(m_run[k], m_tile);
+      m_ref[k] = m_new == -__builtin_inff() ? 0.f : m_new;
+      alpha[k] = m_run[k] == m_new ? 1.0f : __builtin_amdgcn_exp2f((m_run[k] - m_ref[k]) * kLog2e);
+      moved = moved || alpha[k] != 1.0f;
+      m_run[k] = m_new;
+    }
+    if (__ballot(moved) != 0ull) {   // some head's maximum moved: scale what has been added so far
+#pragma unroll
+      for (int k = 0; k < NH; ++k) {
+        lsum[k] *= alpha[k];
+#pragma unroll
+        for (int sg = 0; sg < 4; ++sg) zacc[k][sg] *= alpha[k];
+      }
+      // result rows 4 kg + q: heads 2 kg (q = 0, 1) and 2 kg + 1 (q = 2, 3); head h is slot h / 4 of the lanes with rg = h % 4
+      const int src0 = 16 * ((2 * kg) & 3), src1 = 16 * ((2 * kg + 1) & 3);
+      const float t00 = __shfl(alpha[0], src0, PIKV_WAVE), t01 = __shfl(alpha[NH - 1], src0, PIKV_WAVE);
+      const float t10 = __shfl(alpha[0], src1, PIKV_WAVE), t11 = __shfl(alpha[NH - 1], src1, PIKV_WAVE);
+      const float a0 = (kg >> 1) ? t01 : t00, a1 = (kg >> 1) ? t11 : t10;
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {
+        C[d][0] *= a0; C[d][1] *= a0;
+        C[d][2] *= a1; C[d][3] *= a1;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < NH; ++k)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        p4[k][j] = __builtin_amdgcn_exp2f((sc[k][j] - m_ref[k]) * kLog2e);
+        lsum[k] += p4[k][j];
+      }
+    if constexpr (BOOK) {
+      const int64_t tile = (t0 + n0) / kFTile;
+      auto hb = [](float p) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(p * kHalfScale)); };
+#pragma unroll
+      for (int k = 0; k < NH; ++k) {
+        const uint2 ev = make_uint2(hb(p4[k][0]) | (hb(p4[k][1]) << 16), hb(p4[k][2]) | (hb(p4[k][3]) << 16));
+        if constexpr (QF32) a.e16[(((int64_t)c * a.n_tiles + tile) * HK + g) * (rep * 16) + lane] = ev;
+        else a.e16[((((int64_t)c * a.n_tiles + tile) * HK + g) * 2 + k) * 64 + lane] = ev;
+        if (nl == 0 && row_on[k])
+          a.tref[((int64_t)c * a.n_tiles + tile) * a.n_q_heads + g * rep + rg + 4 * k] = m_ref[k];
+      }
+    }
+
+    // ---- weights and output product, two groups of 32 dimensions at a time ----
+#pragma unroll
+    for (int pp = 0; pp < 2; ++pp) {
+      float2 s2[4], z2[4];   // scale and zero term of this pass's two groups, tokens tk + 4 j
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s2[j] = *reinterpret_cast<const float2*>(vscale + fused_vmeta_off(tk + 4 * j) + 8 * pp);
+        z2[j] = *reinterpret_cast<const float2*>(vzterm + fused_vmeta_off(tk + 4 * j) + 8 * pp);
+      }
+#pragma unroll
+      for (int sgl = 0; sgl < 2; ++sgl) {
+        const int sg = 2 * pp + sgl;
+#pragma unroll
+        for (int k = 0; k < NH; ++k) {
+          float hi[4], lo[4];
+          float zsum = 0.f;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float scl = sgl == 0 ? s2[j].x : s2[j].y;
+            const float zt = sgl == 0 ? z2[j].x : z2[j].y;
+            const float w = p4[k][j] * scl;
+            hi[j] = __uint_as_float(__float_as_uint(w) & 0xffff0000u);
+            lo[j] = __uint_as_float(__float_as_uint(w - hi[j]) & 0xffff0000u);
+            // the zero-point sum uses the SAME two-part value the matrix core multiplies with 128 + code
+            zsum = fmaf(hi[j] + lo[j], zt, zsum);
+          }
+          zacc[k][sg] += zsum;
+          if (row_on[k]) {
+            const int h = rg + 4 * k;
+            // operand order inside 8 tokens is {0,4,1,5,2,6,3,7}: tokens (k, k+4) share a dword
+            uint32_t* rowh = reinterpret_cast<uint32_t*>(abuf + (sgl * 16 + 2 * h) * kFARow + wkg * 32) + qd;
+            uint32_t* rowl = reinterpret_cast<uint32_t*>(abuf + (sgl * 16 + 2 * h + 1) * kFARow + wkg * 32) + qd;
+            rowh[0] = (__float_as_uint(hi[0]) >> 16) | __float_as_uint(hi[1]);
+            rowh[4] = (__float_as_uint(hi[2]) >> 16) | __float_as_uint(hi[3]);
+            rowl[0] = (__float_as_uint(lo[0]) >> 16) | __float_as_uint(lo[1]);
+            rowl[4] = (__float_as_uint(lo[2]) >> 16) | __float_as_uint(lo[3]);
+          }
+        }
+      }
+      wave_sync();   // the rows were written by other lanes of this wavefront
+#pragma unroll
+      for (int sgl = 0; sgl < 2; ++sgl) {
+        const int sg = 2 * pp + sgl;
+        const uint4* ap = reinterpret_cast<const uint4*>(a_row + sgl * a_gstep);
+        const uint4 a1 = ap[0], a2 = ap[1];
+#pragma unroll
+        for (int dbl = 0; dbl < 2; ++dbl) {
+          const int db = 2 * sg + dbl;
+          const pikv_i32x2 tr = __builtin_amdgcn_ds_read_tr4_b64_v2i32(
+              (pikv_i32x2 __attribute__((address_space(3)))*)(vcodes + (kg * 16 + i) * kFCodeRow + db * 8));
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const uint32_t u = Q::sym ? ((uint32_t)tr[half] ^ 0x88888888u) : (uint32_t)tr[half];
+            const uint4 bb = make_uint4(and_or(u, kNib, kExp), and_or(u >> 4, kNib, kExp), and_or(u >> 8, kNib, kExp),
+                                        and_or(u >> 12, kNib, kExp));
+            C[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pikv_bf16x8, half ? a2 : a1),
+                                                            __builtin_bit_cast(pikv_bf16x8, bb), C[db], 0, 0, 0);
+          }
+        }
+      }
+      wave_sync();   // the rows are rewritten by the next pass / the next tile
+    }
+  }
+
+  // ---- what the range leaves: (maximum, sum, unnormalised output) of each head ----
+  wave_sync();
+  float* const zl = reinterpret_cast<float*>(lds);   // [head][group]
+  float ltot[NH];
+#pragma unroll
+  for (int k = 0; k < NH; ++k) {
+    ltot[k] = group_sum_dpp(lsum[k], 16);
+#pragma unroll
+    for (int sg = 0; sg < 4; ++sg) {
+      const float z = group_sum_dpp(zacc[k][sg], 16);
+      if (nl == 0) zl[(rg + 4 * k) * 4 + sg] = z;
+    }
+  }
+  wave_sync();
+  const int64_t pbase = ((int64_t)xr * a.n_caches + c) * a.n_q_heads + g * rep;
+#pragma unroll
+  for (int k = 0; k < NH; ++k)
+    if (row_on[k] && nl == 0) {
+      a.pstats[(pbase + rg + 4 * k) * 2] = m_run[k];
+      a.pstats[(pbase + rg + 4 * k) * 2 + 1] = ltot[k];
+    }
+  // C: lane (dimension i, rows 4 kg + q): rows 2 h / 2 h + 1 are the two parts of head h
+#pragma unroll
+  for (int rr = 0; rr < 2; ++rr) {
+    const int ho = 2 * kg + rr;
+    if (ho >= rep) continue;
+    float* o = a.partial + (pbase + ho) * 128;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) o[db * 16 + i] = (C[db][2 * rr] + C[db][2 * rr + 1]) - zl[ho * 4 + (db >> 1)];
+  }
+}
+
 // ---- the same pass over an 8-bit cache ----------------------------------------------------------
 // Codes of one byte, a float scale (and zero point) per (token, kv head) or coarser, heads of 128
 // dimensions, 2..8 kv heads, 1..8 bf16 query heads per kv head.  The plan is the 4-bit kernel's - a
@@ -502,7 +882,7 @@ __device__ __forceinline__ uint2 bytes_to_bf16(uint32_t w) {
                     __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf2)));
 }
 
-// QF32: float32 queries as two bf16 limbs, q = hi + lo to 2^-17 |q| (hi = the float cut to its upper 16 bits, lo = the
+// QF32: float32 queries as two bf16 limbs, q = hi + lo to 2^-18 |q| (hi = the float rounded to bf16, lo = the
 // rest rounded to bf16); both limbs are multiplied with the same converted codes into the same accumulators.
 template <int SCHEME, bool BOOK, bool QF32 = false>
 __global__ __launch_bounds__(512) void decode_fused_i8_kernel(Fused8Args a) {
@@ -570,12 +950,10 @@ __global__ __launch_bounds__(512) void decode_fused_i8_kernel(Fused8Args a) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float f = a_on ? qf[e] : 0.f;
-          const uint32_t h = __float_as_uint(f) & 0xffff0000u;
-          const uint32_t l = float_to_bf16_bits(f - __uint_as_float(h));
-          hb[e] = h >> 16;
-          lb[e] = l;
-          part[k >> 1] += __uint_as_float(h);
-          part[k >> 1] += __uint_as_float(l << 16);
+          hb[e] = bf16_limb_bits(f, 0);
+          lb[e] = bf16_limb_bits(f, 1);
+          part[k >> 1] += __uint_as_float(hb[e] << 16);
+          part[k >> 1] += __uint_as_float(lb[e] << 16);
         }
         aq[k] = make_uint4(hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16), hb[4] | (hb[5] << 16), hb[6] | (hb[7] << 16));
         aql[k] = make_uint4(lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16), lb[4] | (lb[5] << 16), lb[6] | (lb[7] << 16));
@@ -907,7 +1285,9 @@ __global__ __launch_bounds__(256) void decode_importance_kernel(const uint2* __r
                                                                const int32_t* __restrict__ fill, int64_t max_len,
                                                                int64_t n_tiles, int n_kv_heads, int n_q_heads,
                                                                float decay, float now, float* __restrict__ row_acc,
-                                                               float* __restrict__ row_ts) {
+                                                               float* __restrict__ row_ts, int sets) {
+  // sets = 1: one record of rep * 16 lanes per kv head (heads 0 .. rep - 1); sets = 2 (the two-set kernel with
+  // 5 to 8 heads per kv head): two records of 64 lanes, heads 0..3 and 4..7
   const int lane = threadIdx.x & 63;
   const int c = blockIdx.y;
   const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -925,12 +1305,13 @@ __global__ __launch_bounds__(256) void decode_importance_kernel(const uint2* __r
   if (row_acc != nullptr) {
     // everything the wavefront reads is asked for at once: the tile's halves, the heads' merged statistics
     // (decode_finish_kernel left them in head_stats), the tile's reference maxima, the accumulators
-    uint2 hv[8];
-    const uint2* ep = e16 + ((int64_t)c * n_tiles + tile) * n_kv_heads * (rep * 16) + lane;
+    uint2 hv[16];
+    const int rec = sets == 2 ? 64 : rep * 16;        // lanes per record
+    const uint2* ep = e16 + ((int64_t)c * n_tiles + tile) * n_kv_heads * sets * rec + lane;
 #pragma unroll
-    for (int g = 0; g < 8; ++g) {
-      hv[g] = make_uint2(0, 0);
-      if (g < n_kv_heads && r < rep) hv[g] = ep[(int64_t)g * (rep * 16)];
+    for (int gs = 0; gs < 16; ++gs) {
+      hv[gs] = make_uint2(0, 0);
+      if (gs < n_kv_heads * sets && (sets == 2 ? 4 * (gs & 1) + r : r) < rep) hv[gs] = ep[(int64_t)gs * rec];
     }
     float fac = 0.f;   // lane h: what turns a stored half of head h in this tile into a probability
     if (lane < n_q_heads) {
@@ -940,10 +1321,12 @@ __global__ __launch_bounds__(256) void decode_importance_kernel(const uint2* __r
     }
     float imp[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int g = 0; g < 8; ++g) {
-      if (g >= n_kv_heads) break;
-      const float f = __shfl(fac, r < rep ? g * rep + r : 0, PIKV_WAVE);
-      const uint2 v = hv[g];
+    for (int gs = 0; gs < 16; ++gs) {
+      if (gs >= n_kv_heads * sets) break;
+      const int g = sets == 2 ? gs >> 1 : gs;
+      const int hr = sets == 2 ? 4 * (gs & 1) + r : r;   // head of this lane's row group inside the kv head
+      const float f = __shfl(fac, hr < rep ? g * rep + hr : 0, PIKV_WAVE);
+      const uint2 v = hv[gs];
       imp[0] = fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(v.x & 0xffffu)), f, imp[0]);
       imp[1] = fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(v.x >> 16)), f, imp[1]);
       imp[2] = fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(v.y & 0xffffu)), f, imp[2]);
@@ -1087,6 +1470,11 @@ int fused_tokens_per_block(int n_caches, int n_kv_heads, int64_t max_len, int mi
 // with bookkeeping only four query heads per kv head on at least 3 kv heads (3 x 12: 306 -> 297,
 // 6 x 24: 552 -> 537, 8 x 32: 660-680 -> 643 - the halves cost the pass 0.1 ms, see the top of this file; with
 // fewer query heads per kv head the float rows of the two-kernel form are the smaller exchange).
+// 4-bit, two operand sets, with / without bookkeeping: float32 queries 8 kv x 32 q heads 919 -> 710 / 887 -> 551 us,
+// 6 x 24: 738 -> 601 / 664 -> 445, 4 x 16: 470 -> 422 / 426 -> 280, 3 x 12: 399 -> 340 / 357 -> 235, 2 x 8: 282 vs 298
+// (left alone) / 261 -> 210, 8 x 16 without bookkeeping 847 -> 554; bf16, 5 to 8 heads per kv head: 8 x 64
+// 1040 -> 826 / 873 -> 615, 8 x 40: 970 -> 804 / 807 -> 602, 4 x 28: 481 -> 465 / 420 -> 305, 2 x 16: 271 vs 343 /
+// 233 vs 241 (left alone).
 // 8-bit: everything it can hold, with / without bookkeeping - 8 kv x 64 q heads 1225 -> 1032 / 1148 -> 788 us,
 // 8 x 32: 1107 -> 956 / 1031 -> 786, 8 x 16: 1053 -> 962 / 981 -> 779, 6 x 24: 972 -> 743 / 898 -> 580,
 // 4 x 16: 619 -> 516 / 541 -> 391, 3 x 12: 519 -> 392 / 442 -> 304, 2 x 8: 361 -> 292 / 297 -> 244,
@@ -1094,7 +1482,8 @@ int fused_tokens_per_block(int n_caches, int n_kv_heads, int64_t max_len, int mi
 // piece the float scores would take: two-kernel form, 853 us).
 bool decode_fused_serves(int scheme, int group, int n_kv_heads, int n_q_heads, int head_dim, int q_dtype, bool bookkeeping) {
   const bool eight = scheme == PIKV_Q_I8_SYM || scheme == PIKV_Q_I8_ASYM;
-  if (head_dim != 128 || !(q_dtype == PIKV_BF16 || (eight && q_dtype == PIKV_F32))) return false;
+  if (head_dim != 128 || !(q_dtype == PIKV_BF16 || q_dtype == PIKV_F32)) return false;
+  (void)eight;
   if (n_kv_heads < 2 || n_kv_heads > 8 || n_q_heads % n_kv_heads != 0) return false;
   const int rep = n_q_heads / n_kv_heads;
   if (scheme == PIKV_Q_I8_SYM || scheme == PIKV_Q_I8_ASYM) {
@@ -1104,6 +1493,9 @@ bool decode_fused_serves(int scheme, int group, int n_kv_heads, int n_q_heads, i
     return rep >= 1 && rep <= 8;
   }
   if (group != 32) return false;
+  // two operand sets: the limbs of four float32 heads, or eight bf16 heads
+  if (q_dtype == PIKV_F32) return bookkeeping ? (rep == 4 && n_kv_heads >= 3) : rep <= 4;
+  if (rep >= 5 && rep <= 8) return n_kv_heads >= 3;
   if (bookkeeping) return rep == 4 && n_kv_heads >= 3;
   return rep >= 1 && rep <= 4;
 }
@@ -1119,12 +1511,12 @@ int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_
                         int n_caches, int64_t max_len, int tokens_per_block, float decay, float now, float* row_acc,
                         float* row_ts, float* out, void* e16, float* tref, float* pstats, float* partial,
                         float* head_stats, hipStream_t st) {
-  const int64_t n_tiles = (max_len + kFTile - 1) / kFTile + 1;   // one spare record per cache
+  // one spare record per cache for the one-set 4-bit kernel (it walks tiles in pairs); the others touch no tile past a range's end
+  const int64_t n_tiles = (max_len + kFTile - 1) / kFTile + ((q_dtype == PIKV_F32 || n_q_heads > 4 * n_kv_heads) ? 0 : 1);
   const int64_t splits = (max_len + tokens_per_block - 1) / tokens_per_block;
   if (splits > 65535 || (tokens_per_block & 127) != 0) return PIKV_ERR_SHAPE;
   const bool book = row_acc != nullptr || row_ts != nullptr;
-  if (q_dtype != PIKV_BF16 && !(q_dtype == PIKV_F32 && (scheme == PIKV_Q_I8_SYM || scheme == PIKV_Q_I8_ASYM)))
-    return PIKV_ERR_UNSUPPORTED;
+  if (q_dtype != PIKV_BF16 && q_dtype != PIKV_F32) return PIKV_ERR_UNSUPPORTED;
   if (scheme == PIKV_Q_I8_SYM || scheme == PIKV_Q_I8_ASYM) {
     const int64_t n_tiles8 = (max_len + kFTile - 1) / kFTile;   // this pass never touches a tile past a range's end
     Fused8Args a8{k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, q, cache_row_base, cache_fill, partial, pstats,
@@ -1167,10 +1559,17 @@ int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_
   const dim3 block((unsigned)(n_kv_heads / a.groups * 64));
   const size_t lds = (size_t)(n_kv_heads / a.groups) * kFWaveLds;
   const bool wr = row_acc != nullptr;
-  if (wr && n_q_heads != 4 * n_kv_heads) return PIKV_ERR_UNSUPPORTED;
+  const int rep4 = n_q_heads / n_kv_heads;
+  const bool qf = q_dtype == PIKV_F32;
+  const bool wide = qf || rep4 > 4;   // two operand sets: float32 limbs, or 5 to 8 heads per kv head
+  if (wide ? (qf ? (rep4 > 4 || (wr && rep4 != 4)) : rep4 > 8) : (wr && rep4 != 4)) return PIKV_ERR_UNSUPPORTED;
 #define PIKV_FUSED(S)                                                                                   \
   do {                                                                                                  \
-    if (wr) hipLaunchKernelGGL((decode_fused_i4_kernel<S, true>), grid, block, lds, st, a);             \
+    if (wide && qf && wr) hipLaunchKernelGGL((decode_fused_i4w_kernel<S, true, true>), grid, block, lds, st, a);        \
+    else if (wide && qf) hipLaunchKernelGGL((decode_fused_i4w_kernel<S, false, true>), grid, block, lds, st, a);        \
+    else if (wide && wr) hipLaunchKernelGGL((decode_fused_i4w_kernel<S, true, false>), grid, block, lds, st, a);        \
+    else if (wide) hipLaunchKernelGGL((decode_fused_i4w_kernel<S, false, false>), grid, block, lds, st, a);             \
+    else if (wr) hipLaunchKernelGGL((decode_fused_i4_kernel<S, true>), grid, block, lds, st, a);        \
     else hipLaunchKernelGGL((decode_fused_i4_kernel<S, false>), grid, block, lds, st, a);               \
   } while (0)
   if (scheme == PIKV_Q_I4_ASYM) PIKV_FUSED(PIKV_Q_I4_ASYM);
@@ -1183,7 +1582,7 @@ int decode_fused_launch(const void* k_codes, const void* k_scale, const void* k_
   if (book)
     hipLaunchKernelGGL(decode_importance_kernel, dim3((unsigned)((n_tiles + 3) / 4), (unsigned)n_caches), dim3(256), 0,
                        st, reinterpret_cast<const uint2*>(e16), tref, head_stats, cache_row_base, cache_fill, max_len,
-                       n_tiles, n_kv_heads, n_q_heads, decay, now, row_acc, row_ts);
+                       n_tiles, n_kv_heads, n_q_heads, decay, now, row_acc, row_ts, (wide && !qf) ? 2 : 1);
   PIKV_CHECK_LAUNCH();
   return PIKV_OK;
 }

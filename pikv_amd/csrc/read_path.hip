@@ -555,7 +555,7 @@ static size_t gqa_lds_bytes(int n_kv_heads, int nset, int na) {
 // of a kv head are multiplied with one block-diagonal A operand per set.
 // NARROW: heads of 64 or 32 dimensions (below); the kernel for heads of 128 carries none of it.
 // QF32: float32 queries.  A query element goes in as two bf16 limbs, q = hi + lo + (at most
-// 2^-17 |q|), hi = the float cut to its upper 16 bits, lo = the rest rounded to bf16: two copies of a
+// 2^-18 |q|), hi = the float rounded to bf16, lo = the rest rounded to bf16: two copies of a
 // set's A operands, one per limb, are multiplied with the same unpacked codes into the same
 // accumulators, and the group sums of q are those of hi + lo.
 // SPLIT (rows of more than 16 slabs, e.g. 32 kv heads of 128): a block takes a group of a.n_kv_heads slabs
@@ -613,10 +613,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NKV * NSET 
   const uint16_t* qbase = reinterpret_cast<const uint16_t*>(a.q) + ((int64_t)c * a.n_q_heads + kv_off * rep_all + a.head_off) * head_dim;
   const float* qfbase = reinterpret_cast<const float*>(a.q) + ((int64_t)c * a.n_q_heads + kv_off * rep_all + a.head_off) * head_dim;
   // bf16 bits of limb `set` of a float32 query element
-  auto limb_bits = [](float v, int set) -> uint32_t {
-    const uint32_t hb = __float_as_uint(v) & 0xffff0000u;
-    return set == 0 ? hb >> 16 : float_to_bf16_bits(v - __uint_as_float(hb));
-  };
+  auto limb_bits = [](float v, int set) -> uint32_t { return bf16_limb_bits(v, set); };
   const int64_t base_row = a.row_base[c];
 
   // Code vectors of this wavefront's slice of tile tt (one 16-byte load per kv
@@ -821,7 +818,7 @@ constexpr int kI8QsFloats = 4 * 4 * 4 * 16;   // query sums in LDS: 4 wavefronts
 // are the heads of those kv heads, rep / HPS each, in order.  A query head's A rows are zero outside
 // its own kv head's dimensions, and its scores take that kv head's scale and zero point.
 // QF32 (up to 8 query heads per slab): float32 queries as two bf16 limbs, q = hi + lo + (at most
-// 2^-17 |q|): A rows 2r and 2r+1 hold the limbs of head r, and the two rows' scores - they sit in
+// 2^-18 |q|): A rows 2r and 2r+1 hold the limbs of head r, and the two rows' scores - they sit in
 // the same lane - are added before they are staged.
 template <int SCHEME, int NHW, int HPS = 1, bool QF32 = false>  // NHW = kv heads per wavefront: ceil(n_kv_heads / 4), 1, 2 or 4
 __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
@@ -892,10 +889,7 @@ __global__ __launch_bounds__(256) void scores_mfma_i8_kernel(ScoreArgs a) {
           load_as_float<PIKV_F32, 4>(qfbase, qo, f4);
           uint32_t lb[4];
 #pragma unroll
-          for (int k = 0; k < 4; ++k) {   // limb nl & 1: the float cut to its upper 16 bits, or the rest rounded to bf16
-            const uint32_t hb = __float_as_uint(f4[k]) & 0xffff0000u;
-            lb[k] = (nl & 1) ? float_to_bf16_bits(f4[k] - __uint_as_float(hb)) : hb >> 16;
-          }
+          for (int k = 0; k < 4; ++k) lb[k] = bf16_limb_bits(f4[k], nl & 1);   // limb nl & 1: the float rounded to bf16, or the rest
           qd = make_uint2(lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16));
         } else {
           qd = *reinterpret_cast<const uint2*>(qbase + qo);

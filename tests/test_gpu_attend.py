@@ -236,6 +236,11 @@ def test_attend_peaked_distribution(dev):
     (O.Q_I8_SYM, 512, 4, 8, 128, "bf16"),    # ... a scale per token, 2 q heads per kv head: records of 32 lanes
     (O.Q_I8_ASYM, 128, 7, 14, 128, "bf16"),  # ... 7 kv heads x 2
     (O.Q_I8_SYM, 128, 5, 5, 128, "bf16"),    # ... one q head per kv head: one pass only without the bookkeeping
+    (O.Q_I4_ASYM, 32, 8, 40, 128, "bf16"),   # 4-bit one-pass form with two operand sets: 5 q heads per kv head
+    (O.Q_I4_SYM, 32, 5, 40, 128, "bf16"),    # ... 8 on 5 kv heads, symmetric codes
+    (O.Q_I4_SYM, 32, 4, 16, 128, "f32"),     # ... float32 queries: the sets are the limbs
+    (O.Q_I4_ASYM, 32, 6, 18, 128, "f32"),    # ... 3 q heads per kv head
+    (O.Q_I4_ASYM, 32, 3, 3, 128, "f32"),     # ... one
     (O.Q_I8_SYM, 128, 8, 32, 128, "f32"),    # ... float32 queries as two bf16 limbs
     (O.Q_I8_ASYM, 128, 4, 32, 128, "f32"),   # ... 8 q heads per kv head, zero points
     (O.Q_I8_ASYM, 256, 6, 18, 128, "f32"),   # ... 6 kv heads x 3: two blocks of three wavefronts, a scale per pair of heads

@@ -133,6 +133,7 @@ def test_decode_read_replays(dev):
     (2, 14, 64, False),      # heads of 64, 14 q heads on the one slab
     (8, 64, 128, True),      # 8-bit codes, 8 q heads per kv head: the one-pass form, two blocks per token range
     (3, 12, 128, True),      # ... 3 kv heads x 4: records of 32 lanes
+    (8, 64, 128, False),     # 4-bit, 8 q heads per kv head: the one-pass form with two operand sets
 ])
 def test_decode_attend_replays(dev, hkv, hq, dh, eight):
     """The one-call decode read under capture: its workspace is allocated before the capture, and every
