@@ -1321,12 +1321,11 @@ __global__ __launch_bounds__(256) void decode_importance_kernel(const uint2* __r
     }
     float imp[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int gs = 0; gs < 16; ++gs) {
-      if (gs >= n_kv_heads * sets) break;
+    for (int gs = 0; gs < 16; ++gs) {   // (no early exit: the loop must unroll, or the records live in scratch memory)
       const int g = sets == 2 ? gs >> 1 : gs;
       const int hr = sets == 2 ? 4 * (gs & 1) + r : r;   // head of this lane's row group inside the kv head
-      const float f = __shfl(fac, hr < rep ? g * rep + hr : 0, PIKV_WAVE);
-      const uint2 v = hv[gs];
+      const float f = __shfl(fac, (gs < n_kv_heads * sets && hr < rep) ? g * rep + hr : 0, PIKV_WAVE);
+      const uint2 v = hv[gs];   // zero beyond the last record
       imp[0] = fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(v.x & 0xffffu)), f, imp[0]);
       imp[1] = fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(v.x >> 16)), f, imp[1]);
       imp[2] = fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(v.y & 0xffffu)), f, imp[2]);
@@ -1470,11 +1469,11 @@ int fused_tokens_per_block(int n_caches, int n_kv_heads, int64_t max_len, int mi
 // with bookkeeping only four query heads per kv head on at least 3 kv heads (3 x 12: 306 -> 297,
 // 6 x 24: 552 -> 537, 8 x 32: 660-680 -> 643 - the halves cost the pass 0.1 ms, see the top of this file; with
 // fewer query heads per kv head the float rows of the two-kernel form are the smaller exchange).
-// 4-bit, two operand sets, with / without bookkeeping: float32 queries 8 kv x 32 q heads 919 -> 710 / 887 -> 551 us,
-// 6 x 24: 738 -> 601 / 664 -> 445, 4 x 16: 470 -> 422 / 426 -> 280, 3 x 12: 399 -> 340 / 357 -> 235, 2 x 8: 282 vs 298
-// (left alone) / 261 -> 210, 8 x 16 without bookkeeping 847 -> 554; bf16, 5 to 8 heads per kv head: 8 x 64
-// 1040 -> 826 / 873 -> 615, 8 x 40: 970 -> 804 / 807 -> 602, 4 x 28: 481 -> 465 / 420 -> 305, 2 x 16: 271 vs 343 /
-// 233 vs 241 (left alone).
+// 4-bit, two operand sets, with / without bookkeeping: float32 queries 8 kv x 32 q heads 919 -> 674 / 887 -> 537 us,
+// 6 x 24: 738 -> 540 / 664 -> 446, 4 x 16: 470 -> 371 / 426 -> 281, 3 x 12: 399 -> 293 / 357 -> 236, 2 x 8 without
+// bookkeeping 261 -> 210, 8 x 16 without bookkeeping 847 -> 554; bf16, 5 to 8 heads per kv head: 8 x 64
+// 1040 -> 741 / 873 -> 608, 8 x 40: 970 -> 726 / 807 -> 592, 4 x 28: 481 -> 401 / 420 -> 312; 2 kv heads are left
+// on the two-kernel form (2 x 16 bf16 without bookkeeping: 233 vs 241 us).
 // 8-bit: everything it can hold, with / without bookkeeping - 8 kv x 64 q heads 1225 -> 1032 / 1148 -> 788 us,
 // 8 x 32: 1107 -> 956 / 1031 -> 786, 8 x 16: 1053 -> 962 / 981 -> 779, 6 x 24: 972 -> 743 / 898 -> 580,
 // 4 x 16: 619 -> 516 / 541 -> 391, 3 x 12: 519 -> 392 / 442 -> 304, 2 x 8: 361 -> 292 / 297 -> 244,
