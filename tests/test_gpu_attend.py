@@ -361,3 +361,81 @@ def test_attend_block_lengths(dev, n_caches, length, scheme, heads, hq):
         assert np.abs(out3[c] - want).max() <= tol, (c, "three steps")
         np.testing.assert_allclose(acc1[rows], imp, rtol=1e-3, atol=1e-6)
         np.testing.assert_allclose(acc3[rows], imp, rtol=1e-3, atol=1e-6)
+
+
+def _decode_reference(ref, q, lens_now, acc_before, heads, group, scale_qk, decay):
+    """softmax(q k^T) v and the H2O sums of every cache in float64 on the restatement's dequantised rows."""
+    outs, accs = [], acc_before.copy()
+    hq, dh = q.shape[1], q.shape[2]
+    for c, L in enumerate(lens_now):
+        if L == 0:
+            outs.append(np.zeros((hq, dh), np.float32))
+            continue
+        rows = ref.valid_rows(c)[:L]
+        k_hat = O.dequantize_groups(ref.k_codes[rows], ref.k_scale[rows], ref.k_zero[rows], group)
+        v_hat = O.dequantize_groups(ref.v_codes[rows], ref.v_scale[rows], ref.v_zero[rows], group)
+        s = O.attention_scores(q[c], k_hat, heads, scale_qk)
+        p, imp = O.h2o_importance(s)
+        outs.append(O.attend_values(p, v_hat, heads))
+        accs[rows] = accs[rows] * np.float32(decay) + imp
+    return np.stack(outs), accs
+
+
+@pytest.mark.parametrize("draw", range(20))
+def test_decode_attend_one_pass_sweep(dev, draw):
+    """Seeded random draws over the shapes the one-pass decode kernels take (2 to 8 kv heads of 128
+    dimensions; 4-bit: 1 to 8 bf16 or 1 to 4 float32 query heads per kv head; 8-bit: 1 to 8 of either):
+    ragged cache lengths around the 64-token tile and the token-range boundaries, empty caches, reads cut
+    by max_len, queries scaled up to peaked distributions (scores of +-80: the running maximum moves, most
+    halves of the bookkeeping underflow), with and without the bookkeeping.  Same bars as
+    test_decode_attend_one_call."""
+    r = rng(1000 + draw)
+    eight = bool(draw % 2)
+    sym = bool((draw // 2) % 2)
+    scheme = (O.Q_I8_SYM if sym else O.Q_I8_ASYM) if eight else (O.Q_I4_SYM if sym else O.Q_I4_ASYM)
+    heads = int(r.integers(2, 9))
+    qdtype = "f32" if r.random() < 0.4 else "bf16"
+    max_rep = 8 if (eight or qdtype == "bf16") else 4
+    rep = int(r.integers(1, max_rep + 1))
+    if draw % 5 == 0:
+        rep = 4          # the shape the 4-bit bookkeeping path takes
+    hq, dh = heads * rep, 128
+    group = 32 if not eight else int(r.choice([128, 128, heads * 128 if (heads & (heads - 1)) == 0 else 128]))
+    n_caches = int(r.integers(1, 6))
+    edge = [0, 1, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 513]
+    lens = [int(r.choice(edge)) if r.random() < 0.5 else int(r.integers(1, 2600)) for _ in range(n_caches)]
+    caps = [max(L + int(r.integers(0, 70)), 1) for L in lens]
+    pool, ref = _fill_pool(dev, r, caps, lens, heads, dh, group, scheme)
+    acc0 = r.random(pool.rows).astype(np.float32)
+    pool.acc.copy_(to_dev(acc0, dev))
+    pool.ts.fill_(-3.0)
+    scale_qk = 1.0 / np.sqrt(dh)
+    qscale = float(r.choice([1.0, 2.0, 6.0]))
+    q = r.standard_normal((n_caches, hq, dh)).astype(np.float32) * qscale
+    if qdtype == "bf16":
+        q = O.bf16_round(q)
+    decay = float(r.choice([1.0, 0.9]))
+    cut = int(r.integers(1, max(caps) + 1)) if r.random() < 0.3 else None
+    lens_now = [min(L, cut) for L in lens] if cut else lens
+    out = np_of(pool.decode_attend(to_dev(q, dev, qdtype), hq, now=7.0, decay=decay, max_len=cut))
+    want, acc_ref = _decode_reference(ref, q, lens_now, acc0, heads, group, scale_qk, decay)
+    for c, L in enumerate(lens_now):
+        if L == 0:
+            assert not out[c].any()
+            continue
+        rms = np.sqrt((want[c].astype(np.float64) ** 2).mean()) + 1e-12
+        assert np.abs(out[c] - want[c]).max() <= 1e-3 * rms, (c, L, np.abs(out[c] - want[c]).max(), rms)
+    np.testing.assert_allclose(np_of(pool.acc), acc_ref, rtol=1e-3, atol=1e-5)
+    ts = np_of(pool.ts)
+    touched = np.zeros(pool.rows, bool)
+    for c, L in enumerate(lens_now):
+        touched[ref.valid_rows(c)[:L]] = True
+    assert (ts[touched] == 7.0).all() and (ts[~touched] == -3.0).all()
+    # without the bookkeeping: same output path, accumulators untouched
+    acc_now = np_of(pool.acc).copy()
+    out_nb = np_of(pool.decode_attend(to_dev(q, dev, qdtype), hq, now=8.0, accumulate=False, max_len=cut))
+    for c, L in enumerate(lens_now):
+        if L:
+            rms = np.sqrt((want[c].astype(np.float64) ** 2).mean()) + 1e-12
+            assert np.abs(out_nb[c] - want[c]).max() <= 1e-3 * rms, (c, L)
+    assert np.array_equal(np_of(pool.acc), acc_now)
