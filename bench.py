@@ -297,7 +297,9 @@ def decode_read_workload(torch, ops, dev, iters):
                      "traffic_source": "profiles/decode_read.md (builder's rocprofv3 --pmc runs, not this run)",
                      "algorithmic_bytes": alg_kv, "avg_launch_ms": t_fused,
                      "note": "time of the whole call (three launches) by HIP events on its stream"},
-        "evict_select": _entry(t_sel, rows * 8 + rows * 5),
+        "evict_select": _entry(t_sel, rows * 8 + rows * 5,
+                               what="exact top-k selection, six dependent launches over 17 MB of keys: latency-bound, "
+                                    "hbm_frac is not its measure"),
         "evict_select_plus_compact": {"ms": t_evict, "kept_rows": kept_rows,
                                       "moved_bytes": 2 * kept_rows * (2 * (D // 2 + (D // 32) * 4) + 8)},
     }
@@ -449,7 +451,8 @@ def pyramid_workload(torch, ops, dev, iters):
     rows = sum(keep)
     return {
         "workload": "pyramid compression: 32 layers x 131072 tokens, 8 heads x 128 bf16, budget 100% -> 25%, int8",
-        "select_top_rows": _entry(t_sel, L * N * 4 + L * N * 5),
+        "select_top_rows": _entry(t_sel, L * N * 4 + L * N * 5,
+                                  what="exact top-k selection over small key arrays: latency-bound, hbm_frac is not its measure"),
         "quant_gather": _entry(t_g, rows * (2 * D * 2 + 2 * D + 2 * heads * 4), rows=rows,
                                rows_per_s=rows / (t_g * 1e-3)),
     }
