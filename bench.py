@@ -230,6 +230,9 @@ def decode_read_workload(torch, ops, dev, iters):
     t_step = _median_ms(torch, decode_step, iters, setup=lambda: pool.fill.fill_(N - 1))
     t_fused = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=2.0), iters)
     t_fused_nb = _median_ms(torch, lambda: pool.decode_attend(q, hq, now=2.0, accumulate=False), iters)
+    qf = q.float()
+    t_fused_f32 = _median_ms(torch, lambda: pool.decode_attend(qf, hq, now=2.0), iters)
+    t_fused_f32_nb = _median_ms(torch, lambda: pool.decode_attend(qf, hq, now=2.0, accumulate=False), iters)
     t_att_acc = _median_ms(torch, lambda: pool.attend_values(sc, pool.head_stats, accumulate=True, now=1.0), iters)
     pool.fill.fill_(N)
     # the plain gather + dequantise of the metric's name over this cache format: the K rows of 8 of the 64 sequences
@@ -285,6 +288,10 @@ def decode_read_workload(torch, ops, dev, iters):
                                      "one call (one pass over K and V; halves written and read back for the importance)"),
         "decode_attend_without_h2o": _entry(t_fused_nb, 2 * k_bytes + q_bytes,
                                             what="pikv_decode_attend with row_acc = row_ts = NULL: attention output only"),
+        "decode_attend_f32_queries": _entry(t_fused_f32, alg_kv + q_bytes, traffic_bytes=alg_kv + q_bytes + 2 * half_bytes + rows * 4,
+                                            what="the same call with float32 queries (the reference modules' own dtype): two bf16 limbs "
+                                                 "per query element, decode_fused_i4w_kernel"),
+        "decode_attend_f32_queries_without_h2o": _entry(t_fused_f32_nb, 2 * k_bytes + 2 * q_bytes),
         "decode_step": _entry(t_step, alg_kv, traffic_bytes=alg_kv + 2 * half_bytes + rows * 4,
                               what="append 1 token per sequence + pikv_decode_attend",
                               cached_tokens_per_s=rows / (t_step * 1e-3)),
